@@ -1,0 +1,317 @@
+/*
+ * wgml_hip — C ABI of the MI355X (gfx950) batch-1 token-decode path behind
+ * dimforge/wgml's operator API.
+ *
+ * The reference has no FFI layer: its boundary is the Rust API of `wgml::ops`,
+ * `wgml::models` and `wgml::quantized_matrix` running on wgpu.  Each entry
+ * point below names the reference interface it replaces (paths relative to the
+ * reference's `crates/wgml/src/`).  A Rust `wgml-hip-sys` crate would bind
+ * exactly these symbols with `extern "C"` declarations.
+ *
+ * Conventions
+ *   - every call returns a status (0 = WGML_OK); wgml_last_error() returns the
+ *     message of the last failure on the calling thread;
+ *   - handles are opaque, owned by the caller, freed by the matching _destroy;
+ *   - a context owns one in-order HIP stream: ops are *enqueued* in program
+ *     order and return immediately, like `dispatch()` recording into one
+ *     wgpu compute pass.  Only *_download, *_read_*, wgml_argmax, the timers'
+ *     stop call and wgml_ctx_synchronize block;
+ *   - tensors are f32 *views*: buffer + element offset + length, so an output
+ *     may alias a sub-range such as one KV-cache column
+ *     (models/llama2/transformer.rs:326-341);
+ *   - a context is not thread-safe; use one per thread;
+ *   - there is no CPU fallback: without a HIP device wgml_ctx_create fails.
+ */
+#ifndef WGML_HIP_H
+#define WGML_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WGML_API __attribute__((visibility("default")))
+
+/* ---- status ------------------------------------------------------------ */
+enum {
+    WGML_OK = 0,
+    WGML_E_INVALID = 1,     /* bad argument / shape mismatch (the reference panics) */
+    WGML_E_UNSUPPORTED = 2, /* quantization tag or op outside this path */
+    WGML_E_HIP = 3,         /* a HIP runtime call failed */
+    WGML_E_NO_DEVICE = 4,   /* no usable gfx950 device */
+    WGML_E_OOM = 5,
+};
+
+WGML_API const char *wgml_last_error(void);
+WGML_API const char *wgml_version(void);
+
+/* ---- quantization tags (GGUF tensor-type ids, gguf.rs:70-103) ------------ */
+enum {
+    WGML_F32 = 0,
+    WGML_F16 = 1,
+    WGML_Q4_0 = 2,
+    WGML_Q4_1 = 3,
+    WGML_Q5_0 = 6,
+    WGML_Q5_1 = 7,
+    WGML_Q8_0 = 8,
+    WGML_Q4_K = 12,
+    WGML_Q5_K = 13,
+    WGML_Q6_K = 14,
+    WGML_Q8_K = 15,
+};
+
+typedef struct wgml_ctx wgml_ctx;
+typedef struct wgml_buf wgml_buf;
+typedef struct wgml_qmat wgml_qmat;
+
+/* An f32 vector view: GpuVectorView<f32> (wgcore), `.column()`, `.rows()`. */
+typedef struct {
+    wgml_buf *buf;
+    uint64_t offset; /* in f32 elements */
+    uint32_t len;    /* in f32 elements */
+} wgml_view;
+
+/* ---- context: GpuInstance::new + every `X::from_device` ------------------ */
+WGML_API int wgml_ctx_create(int device, wgml_ctx **out);
+WGML_API int wgml_ctx_destroy(wgml_ctx *ctx);
+WGML_API int wgml_ctx_synchronize(wgml_ctx *ctx);
+/* Device name and compute-unit count (diagnostics). */
+WGML_API int wgml_ctx_info(wgml_ctx *ctx, char *name, size_t name_len, int *n_cu);
+
+/* GPU timestamps over the context's stream (wgcore GpuTimestamps as used by
+ * wgml-bench/src/main.rs:201,225-244).  stop() blocks and returns milliseconds. */
+WGML_API int wgml_timer_start(wgml_ctx *ctx);
+WGML_API int wgml_timer_stop(wgml_ctx *ctx, float *ms);
+
+/* ---- buffers: GpuVector / GpuMatrix / GpuScalar -------------------------- */
+WGML_API int wgml_buf_create(wgml_ctx *ctx, uint64_t bytes, wgml_buf **out); /* ::uninit */
+WGML_API int wgml_buf_destroy(wgml_buf *buf);
+WGML_API uint64_t wgml_buf_size(const wgml_buf *buf);
+WGML_API int wgml_buf_upload(wgml_buf *buf, uint64_t offset_bytes, const void *src,
+                             uint64_t bytes); /* ::init / queue.write_buffer */
+WGML_API int wgml_buf_download(wgml_buf *buf, uint64_t offset_bytes, void *dst,
+                               uint64_t bytes); /* ::read / read_to (blocks) */
+WGML_API int wgml_buf_copy(wgml_buf *dst, uint64_t dst_offset_bytes, const wgml_buf *src,
+                           uint64_t src_offset_bytes, uint64_t bytes); /* copy_from{,_view} */
+WGML_API int wgml_buf_zero(wgml_buf *buf);
+
+/* ---- quantized matrices: GpuQuantMatrix (quantized_matrix.rs:9-75) and
+ *      GgufTensorData::to_gpu_matrix (gguf.rs:131-184) ---------------------- *
+ * `gguf_bytes` is the tensor exactly as stored in a GGUF file: row-major,
+ * nrows rows of ncols/elems_per_block blocks.  Supported tags: WGML_F32,
+ * WGML_Q8_0, WGML_Q4_K, WGML_Q6_K; others give WGML_E_UNSUPPORTED.  Unlike
+ * the reference there is no pairing rule (ncols % 64 / % 512) and no silent
+ * fall-back to f32: any ncols that is a multiple of the block length stays
+ * quantized.  The bytes are re-laid out on the device (see the layout notes
+ * in csrc/quant.hip); the values are unchanged. */
+WGML_API int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t ncols,
+                                      const void *gguf_bytes, wgml_qmat **out);
+WGML_API int wgml_quant_matrix_destroy(wgml_qmat *m);
+WGML_API int wgml_quant_matrix_shape(const wgml_qmat *m, int *type, uint32_t *nrows,
+                                     uint32_t *ncols); /* GpuQuantMatrix::shape */
+/* Size of the tensor in GGUF bytes (the algorithmic weight traffic of one GEMV). */
+WGML_API uint64_t wgml_quant_matrix_gguf_bytes(const wgml_qmat *m);
+
+/* Host helpers (no device needed): bytes of `nelems` elements in a format
+ * (0 if unsupported / not a whole number of blocks). */
+WGML_API uint64_t wgml_quant_bytes(int type, uint64_t nelems);
+WGML_API uint32_t wgml_quant_block_elems(int type); /* QuantizedValue::DEQUANTIZED_LEN per GGUF block */
+
+/* ---- ops ------------------------------------------------------------------ */
+
+/* GemvQuant::dispatch (ops/gemv_quant.rs:243-348): out = m * v, fp32 accumulate.
+ * out.len == nrows, v.len == ncols. */
+WGML_API int wgml_gemv_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, wgml_view v);
+
+/* Quantization shader `dequantize_*` (ops/quantization.wgsl, exercised by
+ * ops/quantization.rs:37-408) == Block*::dequantize (quantization.rs): writes
+ * the nrows*ncols f32 values, row-major, bit-exact with the CPU twin. */
+WGML_API int wgml_dequantize(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m);
+
+/* BlockF16::dequantize (quantization.rs:16-24): n IEEE half bit patterns
+ * (uint16, at `in_offset_bytes` of `in`) -> f32. */
+WGML_API int wgml_f16_to_f32(wgml_ctx *ctx, wgml_view out, const wgml_buf *in,
+                             uint64_t in_offset_bytes);
+
+/* wgebra Gemv / GemvTr on f32 (call sites ops/gemv_quant.rs:119,305,
+ * models/gpt2/transformer.rs:243-476).  `a` is row-major nrows x ncols;
+ * transposed != 0 computes out = a^T v (out.len == ncols, v.len == nrows). */
+WGML_API int wgml_gemv_f32(wgml_ctx *ctx, wgml_view out, wgml_view a, uint32_t nrows,
+                           uint32_t ncols, int transposed, wgml_view v);
+
+/* RmsNorm::dispatch (ops/rms_norm.rs:24-53); eps = RmsNormConfig.nudge_factor. */
+WGML_API int wgml_rms_norm(wgml_ctx *ctx, float eps, wgml_view out, wgml_view x, wgml_view w);
+
+/* LayerNorm::dispatch (ops/layernorm.rs:18-41): no affine, eps 1e-5. */
+WGML_API int wgml_layernorm(wgml_ctx *ctx, wgml_view out, wgml_view x);
+
+enum { WGML_ROPE_ORIGINAL = 0, WGML_ROPE_NEOX = 1 }; /* ops/rope.rs:10-16 */
+typedef struct {
+    uint32_t head_size, kv_dim, pos;
+    float base_freq;
+} wgml_rope_config; /* ops/rope.rs:30-35 */
+/* RoPE::dispatch (ops/rope.rs:38-76): rotates q (all pairs) and k (pairs below
+ * kv_dim) in place.  Errors where the reference asserts: odd lengths, q shorter
+ * than k. */
+WGML_API int wgml_rope(wgml_ctx *ctx, int variant, const wgml_rope_config *cfg, wgml_view q,
+                       wgml_view k);
+
+/* SoftMax::dispatch (ops/softmax.rs:18-30): independent softmax of each of the
+ * ncols columns of length nrows; column j starts at offset + j*col_stride. */
+WGML_API int wgml_softmax(wgml_ctx *ctx, wgml_view mat, uint32_t nrows, uint32_t ncols,
+                          uint32_t col_stride);
+
+typedef struct {
+    uint32_t seq_len, kv_dim, kv_mul, n_heads, head_size, pos;
+} wgml_attn_params; /* ops/batched_multiquery_attention.rs:30-37 */
+/* BatchedMultiqueryAttention::{dispatch, dispatch_multi}
+ * (ops/batched_multiquery_attention.rs:55-139).  key/value cache: position t at
+ * [t*kv_dim, (t+1)*kv_dim).  If att.buf != NULL the normalised weights of head
+ * h are also written to att[h*seq_len + t] as `dispatch` does; pass a null
+ * view to skip them (as `dispatch_multi`, whose scratch layout is private). */
+WGML_API int wgml_attention(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
+                            wgml_view key_cache, wgml_view value_cache, wgml_view att,
+                            wgml_view xb);
+
+/* Silu::dispatch (ops/silu.rs:18-34): h1 = h2 * h1 / (1 + exp(-h1)). */
+WGML_API int wgml_silu(wgml_ctx *ctx, wgml_view h1, wgml_view h2);
+
+/* UnaryOp (ops/unary.rs:16-38), same order. */
+enum {
+    WGML_UNARY_ABS = 0, WGML_UNARY_SGN, WGML_UNARY_NEG, WGML_UNARY_STEP, WGML_UNARY_ELU,
+    WGML_UNARY_GELU, WGML_UNARY_GELU_QUICK, WGML_UNARY_SILU, WGML_UNARY_TANH, WGML_UNARY_RELU,
+    WGML_UNARY_SIGMOID, WGML_UNARY_HARD_SIGMOID, WGML_UNARY_HARD_SWISH, WGML_UNARY_SQR,
+    WGML_UNARY_SQRT, WGML_UNARY_LOG, WGML_UNARY_LEAKY_RELU, WGML_UNARY_CLAMP, WGML_UNARY_SCALE,
+    WGML_UNARY_ADD_SCALAR,
+};
+/* UnaryInplace::dispatch (ops/unary.rs:207-261); args may be NULL for ops
+ * without arguments. */
+WGML_API int wgml_unary_inplace(wgml_ctx *ctx, int op, wgml_view x, const float *args4);
+
+enum { WGML_ASSIGN_ADD = 0, WGML_ASSIGN_MUL = 1, WGML_ASSIGN_COPY = 2 };
+/* wgebra OpAssign (call sites models/llama2/transformer.rs:293,344-353,383,406;
+ * models/gpt2/transformer.rs:277-452): a op= b elementwise. */
+WGML_API int wgml_op_assign(wgml_ctx *ctx, int op, wgml_view a, wgml_view b);
+
+/* Sampler::sample_argmax (models/sampler.rs:54-56): first index of the
+ * maximum, computed on the device; blocks and returns it. */
+WGML_API int wgml_argmax(wgml_ctx *ctx, wgml_view logits, uint32_t *out_index);
+
+/* ---- Llama-family model: Llama2 / Llama2State / Llama2Weights ------------- */
+typedef struct {
+    uint32_t dim, hidden_dim, n_layers, n_q_heads, n_kv_heads, vocab_size, seq_len;
+    float rope_base_freq, rms_norm_eps;
+} wgml_llama2_config; /* models/llama2/cpu.rs:46-67 */
+
+enum { WGML_MODEL_LLAMA = 0, WGML_MODEL_QWEN2 = 1 }; /* models/llama2/mod.rs:13-33 */
+
+enum { /* matrices of Llama2LayerWeights / Llama2Weights (transformer.rs:128-148) */
+    WGML_LLAMA2_ATTN_Q = 0, WGML_LLAMA2_ATTN_K, WGML_LLAMA2_ATTN_V, WGML_LLAMA2_ATTN_OUTPUT,
+    WGML_LLAMA2_FFN_GATE, WGML_LLAMA2_FFN_UP, WGML_LLAMA2_FFN_DOWN,
+    WGML_LLAMA2_OUTPUT, /* layer ignored */
+};
+enum { /* f32 vectors */
+    WGML_LLAMA2_ATTN_NORM = 0, WGML_LLAMA2_FFN_NORM,
+    WGML_LLAMA2_ATTN_Q_BIAS, WGML_LLAMA2_ATTN_K_BIAS, WGML_LLAMA2_ATTN_V_BIAS,
+    WGML_LLAMA2_OUTPUT_NORM, /* layer ignored */
+};
+
+typedef struct wgml_llama2 wgml_llama2;
+
+/* Llama2::new + Llama2State::new (models/llama2/transformer.rs:47-105,283-296):
+ * allocates activations and the per-layer f32 KV caches (kv_dim x seq_len). */
+WGML_API int wgml_llama2_create(wgml_ctx *ctx, const wgml_llama2_config *cfg, int model_type,
+                                wgml_llama2 **out);
+WGML_API int wgml_llama2_destroy(wgml_llama2 *m);
+/* Llama2Weights fields (models/llama2/transformer.rs:151-268).  The model
+ * borrows the matrix; it must outlive the model.  Shapes are checked. */
+WGML_API int wgml_llama2_set_matrix(wgml_llama2 *m, int which, uint32_t layer,
+                                    const wgml_qmat *mat);
+WGML_API int wgml_llama2_set_vector(wgml_llama2 *m, int which, uint32_t layer, const float *host,
+                                    uint32_t len);
+/* token_embd: f32, dim x vocab, token t at [t*dim, (t+1)*dim)
+ * (models/llama2/transformer.rs:239-242). */
+WGML_API int wgml_llama2_set_token_embd(wgml_llama2 *m, const float *host);
+/* One decode step: ChatLlama2::forward_logits minus the read-back
+ * (wgml-chat/src/chat_llama2.rs:155-213) = embedding copy + Llama2::dispatch
+ * (models/llama2/transformer.rs:298-431).  Enqueues and returns. */
+WGML_API int wgml_llama2_forward(wgml_llama2 *m, uint32_t token, uint32_t pos);
+/* logits_readback.read_to (chat_llama2.rs:216-220): blocks. */
+WGML_API int wgml_llama2_read_logits(wgml_llama2 *m, float *host_out);
+/* The token loop of ChatLlama2::forward + sample_next_token with temperature 0
+ * (chat_llama2.rs:51-153, wgml-chat/src/sampler.rs:91-111): positions
+ * 0..n_total-1; position p consumes prompt[p] while p < n_prompt, else the
+ * arg-max of the previous step.  out_tokens[p] receives the arg-max after
+ * position p (n_total entries).  The arg-max runs on the device; only the
+ * 4-byte index crosses to the host. */
+WGML_API int wgml_llama2_generate_greedy(wgml_llama2 *m, const uint32_t *prompt,
+                                         uint32_t n_prompt, uint32_t n_total,
+                                         uint32_t *out_tokens);
+/* As above from an arbitrary start position with the KV cache already filled
+ * for positions < start_pos; first consumed token is `first_token`. */
+WGML_API int wgml_llama2_decode_greedy(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos,
+                                       uint32_t n_steps, uint32_t *out_tokens);
+/* Direct KV-cache access (tests; pre-filled long-context runs). which: 0 = key,
+ * 1 = value; `n_pos` positions starting at `first_pos`, kv_dim floats each. */
+WGML_API int wgml_llama2_kv_upload(wgml_llama2 *m, uint32_t layer, int which, uint32_t first_pos,
+                                   uint32_t n_pos, const float *host);
+WGML_API int wgml_llama2_kv_download(wgml_llama2 *m, uint32_t layer, int which,
+                                     uint32_t first_pos, uint32_t n_pos, float *host);
+/* Number of kernel launches one forward enqueues (diagnostics). */
+WGML_API int wgml_llama2_launches_per_token(const wgml_llama2 *m);
+/* 0: one launch per reference op (mirrors Llama2::dispatch one to one);
+ * 1 (default): fused kernels.  Both give the same results to fp32 rounding. */
+WGML_API int wgml_llama2_set_fusion(wgml_llama2 *m, int level);
+
+/* ---- GPT-2: Gpt2 / Gpt2State / Gpt2Weights -------------------------------- */
+typedef struct {
+    uint32_t n_vocab, n_seq, n_embd, n_head, n_layer, ff_len, attn_b;
+} wgml_gpt2_params; /* models/gpt2/cpu.rs:18-33 */
+
+enum { /* matrices (models/gpt2/transformer.rs:72-106) */
+    WGML_GPT2_ATTN_W = 0, WGML_GPT2_ATTN_PROJ_W, WGML_GPT2_MLP_FC_W, WGML_GPT2_MLP_PROJ_W,
+    WGML_GPT2_LM_HEAD, /* layer ignored */
+};
+enum { /* f32 vectors */
+    WGML_GPT2_LN_1_G = 0, WGML_GPT2_LN_1_B, WGML_GPT2_LN_2_G, WGML_GPT2_LN_2_B,
+    WGML_GPT2_ATTN_B, WGML_GPT2_ATTN_PROJ_B, WGML_GPT2_MLP_FC_B, WGML_GPT2_MLP_PROJ_B,
+    WGML_GPT2_LN_F_G, WGML_GPT2_LN_F_B, /* layer ignored */
+};
+
+typedef struct wgml_gpt2 wgml_gpt2;
+
+/* Gpt2::new + Gpt2State::new (+ the per-layer KV caches of Gpt2LayerWeights,
+ * models/gpt2/transformer.rs:27-57,86-87,252-263). */
+WGML_API int wgml_gpt2_create(wgml_ctx *ctx, const wgml_gpt2_params *p, wgml_gpt2 **out);
+WGML_API int wgml_gpt2_destroy(wgml_gpt2 *m);
+WGML_API int wgml_gpt2_set_matrix(wgml_gpt2 *m, int which, uint32_t layer, const wgml_qmat *mat);
+WGML_API int wgml_gpt2_set_vector(wgml_gpt2 *m, int which, uint32_t layer, const float *host,
+                                  uint32_t len);
+/* wte: n_embd x n_vocab, wpe: n_embd x n_seq, column c at [c*n_embd ..]. */
+WGML_API int wgml_gpt2_set_embeddings(wgml_gpt2 *m, const float *wte, const float *wpe);
+/* Gpt2::dispatch (models/gpt2/transformer.rs:265-477). */
+WGML_API int wgml_gpt2_forward(wgml_gpt2 *m, uint32_t token, uint32_t pos);
+WGML_API int wgml_gpt2_read_logits(wgml_gpt2 *m, float *host_out);
+/* ChatGpt2::forward's loop with greedy sampling (wgml-chat/src/chat_gpt2.rs:43-151). */
+WGML_API int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_prompt,
+                                       uint32_t n_total, uint32_t *out_tokens);
+
+/* ---- host-side input makers (no device needed) ---------------------------- *
+ * The reference only de-quantizes; its inputs come from GGUF files written by
+ * ggml.  These restate ggml's reference quantizers (quantize_row_q8_0_ref,
+ * quantize_row_q4_K_ref, quantize_row_q6_K_ref) so that synthetic weights can
+ * be produced in-process.  nthreads <= 0 picks the available cores. */
+WGML_API int wgml_quantize(int type, const float *src, void *dst, uint64_t nelems, int nthreads);
+/* Counter-based generator: element i depends only on (seed, i).
+ * normal: mean + std * N(0,1) by Box-Muller in f32. */
+WGML_API int wgml_rng_normal(uint64_t seed, float *out, uint64_t n, float mean, float std,
+                             int nthreads);
+/* uniform integers in [0, bound). */
+WGML_API int wgml_rng_uniform_u32(uint64_t seed, uint32_t *out, uint64_t n, uint32_t bound);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

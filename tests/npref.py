@@ -1,0 +1,207 @@
+"""Independent numpy restatements used to pin the C oracle.
+
+These follow ggml's published dequantizers (dequantize_row_q8_0 / q4_K / q6_K)
+in vectorised form: a different code shape from oracle/wgml_oracle.c, so a
+wrong index, shift or sign in either one shows up as a bit mismatch.  Every
+arithmetic step is done in float32 with one rounding per operation, as the
+reference's scalar Rust code does.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+f32 = np.float32
+
+
+def half_bits_to_f32(bits: np.ndarray) -> np.ndarray:
+    return np.asarray(bits, dtype=np.uint16).view(np.float16).astype(np.float32)
+
+
+def dequant_q8_0(raw: np.ndarray) -> np.ndarray:
+    b = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1, 34)
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])
+    qs = b[:, 2:].view(np.int8).astype(np.float32)
+    return (qs * d[:, None]).astype(np.float32).reshape(-1)
+
+
+def _scale_min_k4(scales: np.ndarray):
+    """scales: (nb, 12) uint8 -> sc, m: (nb, 8) uint8 (ggml get_scale_min_k4)."""
+    s = scales.astype(np.uint8)
+    sc = np.empty((s.shape[0], 8), dtype=np.uint8)
+    m = np.empty_like(sc)
+    sc[:, :4] = s[:, 0:4] & 63
+    m[:, :4] = s[:, 4:8] & 63
+    sc[:, 4:] = (s[:, 8:12] & 0x0F) | ((s[:, 0:4] >> 6) << 4)
+    m[:, 4:] = (s[:, 8:12] >> 4) | ((s[:, 4:8] >> 6) << 4)
+    return sc, m
+
+
+def dequant_q4_k(raw: np.ndarray) -> np.ndarray:
+    b = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1, 144)
+    nb = b.shape[0]
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])
+    dmin = half_bits_to_f32(b[:, 2:4].copy().view(np.uint16)[:, 0])
+    sc, m = _scale_min_k4(b[:, 4:16])
+    qs = b[:, 16:].reshape(nb, 4, 32)
+    # sub-block 2j = low nibbles of group j, 2j+1 = high nibbles
+    q = np.empty((nb, 8, 32), dtype=np.float32)
+    q[:, 0::2, :] = (qs & 0x0F).astype(np.float32)
+    q[:, 1::2, :] = (qs >> 4).astype(np.float32)
+    dl = (d[:, None] * sc.astype(np.float32)).astype(np.float32)     # d * sc
+    ml = (dmin[:, None] * m.astype(np.float32)).astype(np.float32)   # min * m
+    prod = (dl[:, :, None] * q).astype(np.float32)
+    return (prod - ml[:, :, None]).astype(np.float32).reshape(-1)
+
+
+def dequant_q6_k(raw: np.ndarray) -> np.ndarray:
+    b = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1, 210)
+    nb = b.shape[0]
+    ql = b[:, 0:128].reshape(nb, 2, 64)
+    qh = b[:, 128:192].reshape(nb, 2, 32)
+    sc = b[:, 192:208].view(np.int8).reshape(nb, 2, 8).astype(np.float32)
+    d = half_bits_to_f32(b[:, 208:210].copy().view(np.uint16)[:, 0])
+    out = np.empty((nb, 2, 4, 32), dtype=np.float32)
+    lo = [ql[:, :, 0:32] & 0x0F, ql[:, :, 32:64] & 0x0F, ql[:, :, 0:32] >> 4, ql[:, :, 32:64] >> 4]
+    for k in range(4):
+        hi = (qh >> (2 * k)) & 3
+        q = (lo[k] | (hi << 4)).astype(np.int16) - 32          # (nb, 2, 32)
+        # scale index: is = l // 16, + 2k
+        s = np.repeat(sc[:, :, 2 * k:2 * k + 2], 16, axis=2)   # (nb, 2, 32)
+        ds = (d[:, None, None] * s).astype(np.float32)         # d * scale
+        out[:, :, k, :] = (ds * q.astype(np.float32)).astype(np.float32)
+    return out.reshape(-1)
+
+
+DEQUANT = {8: dequant_q8_0, 12: dequant_q4_k, 14: dequant_q6_k}
+BLOCK_BYTES = {8: 34, 12: 144, 14: 210}
+BLOCK_ELEMS = {8: 32, 12: 256, 14: 256}
+
+
+def random_blocks(qtype: int, nblocks: int, seed: int) -> np.ndarray:
+    """Random block *bits* (as wgml-bench does, ops/gemv_quant.rs:83-101) with
+    the half-precision scale fields forced finite and moderate (exponent bits
+    in 1..24, i.e. |d| < 1024) so that outputs are finite numbers."""
+    rng = np.random.default_rng(seed)
+    raw = rng.integers(0, 256, size=(nblocks, BLOCK_BYTES[qtype]), dtype=np.uint8)
+
+    def fix_half(col: int):
+        h = raw[:, col:col + 2].copy().view(np.uint16)[:, 0]
+        exp = (h >> 10) & 0x1F
+        exp = (exp % 24) + 1
+        h = (h & 0x83FF) | (exp.astype(np.uint16) << 10)
+        raw[:, col:col + 2] = h.view(np.uint8).reshape(-1, 2)
+
+    if qtype == 8:
+        fix_half(0)
+    elif qtype == 12:
+        fix_half(0)
+        fix_half(2)
+    else:
+        fix_half(208)
+    return raw.reshape(-1)
+
+
+# ---- float64 model forwards (composition check for the oracle) ---------------
+
+def llama_forward_f64(w, tokens, rope_variant: int = 0):
+    """Straight numpy float64 Llama forward over dequantized weights; returns the
+    logits after consuming `tokens` at positions 0..len-1."""
+    import oracle as orc
+
+    c = w.config
+    hs, kv_dim, kv_mul = c.head_size, c.kv_dim, c.n_q_heads // c.n_kv_heads
+
+    def deq(hm):
+        return orc.dequantize(hm.qtype, hm.data, hm.nrows * hm.ncols).reshape(
+            hm.nrows, hm.ncols).astype(np.float64)
+
+    L = [{k: (deq(v) if hasattr(v, "qtype") else np.asarray(v, dtype=np.float64))
+          for k, v in l.items()} for l in w.layers]
+    out_w = deq(w.output)
+    kc = np.zeros((c.n_layers, c.seq_len, kv_dim))
+    vc = np.zeros_like(kc)
+
+    def rms(x, g):
+        return x / np.sqrt((x * x).mean() + c.rms_norm_eps) * g
+
+    logits = None
+    for pos, tok in enumerate(tokens):
+        x = w.token_embd[tok].astype(np.float64)
+        for l, wl in enumerate(L):
+            xb = rms(x, wl["attn_norm"])
+            q, k, v = wl["attn_q"] @ xb, wl["attn_k"] @ xb, wl["attn_v"] @ xb
+            for name, vec in (("attn_q_bias", q), ("attn_k_bias", k), ("attn_v_bias", v)):
+                if name in wl:
+                    vec += wl[name]
+            i = np.arange(0, c.dim, 2)
+            theta = float(c.rope_base_freq) ** (-(i % hs) / hs)
+            ang = pos * theta
+            cs, sn = np.cos(ang), np.sin(ang)
+            if rope_variant == 0:
+                a, b = i, i + 1
+            else:
+                a = i // 2 + (i // hs) * hs // 2
+                b = a + hs // 2
+            qa, qb = q[a].copy(), q[b].copy()
+            q[a], q[b] = cs * qa - sn * qb, sn * qa + cs * qb
+            nk = kv_dim // 2
+            ka, kb = k[a[:nk]].copy(), k[b[:nk]].copy()
+            k[a[:nk]], k[b[:nk]] = cs[:nk] * ka - sn[:nk] * kb, sn[:nk] * ka + cs[:nk] * kb
+            kc[l, pos], vc[l, pos] = k, v
+            att_out = np.zeros(c.dim)
+            for h in range(c.n_q_heads):
+                g = h // kv_mul
+                qh = q[h * hs:(h + 1) * hs]
+                s = kc[l, :pos + 1, g * hs:(g + 1) * hs] @ qh / np.sqrt(hs)
+                p = np.exp(s - s.max())
+                p /= p.sum()
+                att_out[h * hs:(h + 1) * hs] = p @ vc[l, :pos + 1, g * hs:(g + 1) * hs]
+            x = x + wl["attn_output"] @ att_out
+            xb = rms(x, wl["ffn_norm"])
+            g_, u_ = wl["ffn_gate"] @ xb, wl["ffn_up"] @ xb
+            x = x + wl["ffn_down"] @ (u_ * (g_ / (1 + np.exp(-g_))))
+        logits = out_w @ rms(x, w.output_norm.astype(np.float64))
+    return logits
+
+
+def gpt2_forward_f64(w, tokens):
+    import oracle as orc
+
+    p = w.params
+    n, hs = p.n_embd, p.n_embd // p.n_head
+
+    def deq(hm):
+        return orc.dequantize(hm.qtype, hm.data, hm.nrows * hm.ncols).reshape(
+            hm.nrows, hm.ncols).astype(np.float64)
+
+    L = [{k: (deq(v) if hasattr(v, "qtype") else np.asarray(v, dtype=np.float64))
+          for k, v in l.items()} for l in w.layers]
+    head = deq(w.lm_head)
+    kc = np.zeros((p.n_layer, p.n_seq, n))
+    vc = np.zeros_like(kc)
+
+    def ln(x, g, b):
+        mu = x.mean()
+        return (x - mu) / np.sqrt(((x - mu) ** 2).mean() + 1e-5) * g + b
+
+    logits = None
+    for pos, tok in enumerate(tokens):
+        x = w.wte[tok].astype(np.float64) + w.wpe[pos].astype(np.float64)
+        for l, wl in enumerate(L):
+            cur = ln(x, wl["ln_1_g"], wl["ln_1_b"])
+            qkv = wl["attn_w"] @ cur + wl["attn_b"]
+            q, kc[l, pos], vc[l, pos] = qkv[:n], qkv[n:2 * n], qkv[2 * n:]
+            att = np.zeros(n)
+            for h in range(p.n_head):
+                sl = slice(h * hs, (h + 1) * hs)
+                s = kc[l, :pos + 1, sl] @ q[sl] / np.sqrt(hs)
+                pr = np.exp(s - s.max())
+                pr /= pr.sum()
+                att[sl] = pr @ vc[l, :pos + 1, sl]
+            x = x + wl["attn_proj_w"] @ att + wl["attn_proj_b"]
+            cur = ln(x, wl["ln_2_g"], wl["ln_2_b"])
+            hdn = wl["mlp_fc_w"] @ cur + wl["mlp_fc_b"]
+            hdn = 0.5 * hdn * (1 + np.tanh(0.7978845608028654 * hdn * (1 + 0.044715 * hdn * hdn)))
+            x = x + wl["mlp_proj_w"] @ hdn + wl["mlp_proj_b"]
+        logits = head @ ln(x, w.ln_f_g.astype(np.float64), w.ln_f_b.astype(np.float64))
+    return logits

@@ -1,0 +1,89 @@
+"""GPU parity: KV-cache attention against the oracle's restatement of
+BatchedMultiqueryAttention::run_cpu.  Shapes follow the reference tests
+(crates/wgml/src/ops/batched_multiquery_attention.rs:210-413: seq 1024, kv_dim
+768, 12 heads x 64, pos 0..8, epsilon 1e-5) plus the grouped-query and
+long-context cases of the benchmark configurations."""
+import numpy as np
+import pytest
+
+import oracle as orc
+import wgml_amd as W
+
+pytestmark = pytest.mark.gpu
+
+
+def rnd(n, seed, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal(n) * scale).astype(np.float32)
+
+
+def run(gpu, seq_len, kv_mul, n_heads, hs, pos, with_att, seed=0):
+    kv_dim = n_heads // kv_mul * hs
+    q = rnd(n_heads * hs, seed + 1)
+    kc, vc = rnd(seq_len * kv_dim, seed + 2), rnd(seq_len * kv_dim, seed + 3)
+    p = W.BatchedMultiqueryAttentionParams(seq_len, kv_dim, kv_mul, n_heads, hs, pos)
+    gq, gk, gv = (W.GpuVector.init(gpu, a) for a in (q, kc, vc))
+    att = W.GpuVector.init(gpu, np.zeros(seq_len * n_heads, dtype=np.float32)) if with_att else None
+    xb = W.GpuVector.init(gpu, np.full(n_heads * hs, np.nan, dtype=np.float32))
+    W.BatchedMultiqueryAttention.from_device(gpu).dispatch(p, gq, gk, gv, att, xb)
+    want_xb, want_att = orc.attention(seq_len, kv_dim, kv_mul, n_heads, hs, pos, q, kc, vc)
+    got_att = att.read().reshape(n_heads, seq_len) if with_att else None
+    return xb.read(), want_xb, got_att, want_att
+
+
+@pytest.mark.parametrize("pos", list(range(9)))
+def test_attention_reference_shape_with_weights(gpu, pos):  # `gpu_attention`: xb and att
+    xb, wxb, att, watt = run(gpu, 1024, 1, 12, 64, pos, True)
+    np.testing.assert_allclose(xb, wxb, rtol=0, atol=1e-5)
+    np.testing.assert_allclose(att[:, :pos + 1], watt[:, :pos + 1], rtol=0, atol=1e-5)
+    assert not att[:, pos + 1:].any()  # nothing written past pos
+
+
+@pytest.mark.parametrize("pos", [0, 1, 8, 63, 64, 100, 1023])
+def test_attention_multi(gpu, pos):  # `gpu_attention_multi`: xb only
+    xb, wxb, _, _ = run(gpu, 1024, 1, 12, 64, pos, False)
+    np.testing.assert_allclose(xb, wxb, rtol=0, atol=1e-5)
+
+
+@pytest.mark.parametrize("kv_mul,n_heads,hs", [(4, 32, 128), (2, 8, 64), (8, 16, 128), (3, 6, 32),
+                                               (1, 6, 48), (1, 32, 128), (1, 2, 256), (6, 12, 128)])
+@pytest.mark.parametrize("pos", [5, 383])
+def test_attention_grouped_and_head_sizes(gpu, kv_mul, n_heads, hs, pos):
+    xb, wxb, _, _ = run(gpu, 512, kv_mul, n_heads, hs, pos, False, seed=kv_mul)
+    np.testing.assert_allclose(xb, wxb, rtol=0, atol=2e-5)
+
+
+@pytest.mark.parametrize("with_att", [False, True])
+def test_attention_long_context_gqa(gpu, with_att):
+    # Llama-3-8B-like head layout at a long position: many workgroups per KV head + merge
+    xb, wxb, att, watt = run(gpu, 8448, 4, 32, 128, 8300, with_att, seed=9)
+    np.testing.assert_allclose(xb, wxb, rtol=0, atol=2e-5)
+    if with_att:
+        np.testing.assert_allclose(att[:, :8301], watt[:, :8301], rtol=0, atol=1e-6)
+
+
+def test_attention_invariants(gpu):
+    seq_len, n_heads, hs, kv_mul = 64, 8, 64, 2
+    kv_dim = n_heads // kv_mul * hs
+    q = rnd(n_heads * hs, 1)
+    vc = rnd(seq_len * kv_dim, 3)
+    kc = np.tile(rnd(kv_dim, 2), seq_len)  # identical keys -> uniform weights -> mean of V
+    p = W.BatchedMultiqueryAttentionParams(seq_len, kv_dim, kv_mul, n_heads, hs, 39)
+    xb = W.GpuVector.uninit(gpu, n_heads * hs)
+    W.BatchedMultiqueryAttention.from_device(gpu).dispatch_multi(
+        p, W.GpuVector.init(gpu, q), W.GpuVector.init(gpu, kc), W.GpuVector.init(gpu, vc), xb)
+    vm = vc.reshape(seq_len, kv_dim)[:40].astype(np.float64).mean(0)
+    got = xb.read()
+    for h in range(n_heads):
+        g = h // kv_mul
+        np.testing.assert_allclose(got[h * hs:(h + 1) * hs], vm[g * hs:(g + 1) * hs], atol=1e-5)
+
+
+def test_attention_argument_checks(gpu):
+    a = W.BatchedMultiqueryAttention.from_device(gpu)
+    v = W.GpuVector.uninit(gpu, 1024)
+    with pytest.raises(W.WgmlError):  # pos outside seq_len
+        a.dispatch(W.BatchedMultiqueryAttentionParams(4, 64, 1, 1, 64, 4), v.rows(0, 64), v, v,
+                   None, v.rows(0, 64))
+    with pytest.raises(W.WgmlError):  # kv_dim inconsistent with heads
+        a.dispatch(W.BatchedMultiqueryAttentionParams(4, 32, 1, 1, 64, 0), v.rows(0, 64), v, v,
+                   None, v.rows(0, 64))

@@ -1,0 +1,172 @@
+"""GPU parity: quantized GEMV (GemvQuant) and dense f32 GEMV against the oracle.
+
+Tolerance (stated by the task): relative 1e-3 with fp32 accumulation.  It is
+applied as |gpu - ref| <= 1e-3 * |ref| + 1e-3 * rms(ref), with ref the float64
+dot product of the bit-exact dequantized weights; the observed error is
+typically 1e-6 * rms.  The reference has no numerical GEMV test of its own
+(only a shader-compilation check, crates/wgml/src/ops/gemv_quant.rs:350).
+"""
+import numpy as np
+import pytest
+
+import npref
+import oracle as orc
+import wgml_amd as W
+
+pytestmark = pytest.mark.gpu
+QT = [W.Q8_0, W.Q4_K, W.Q6_K]
+
+
+def close(got, ref):
+    ref = np.asarray(ref, dtype=np.float64)
+    rms = float(np.sqrt((ref ** 2).mean())) or 1.0
+    err = np.abs(got.astype(np.float64) - ref)
+    ok = err <= 1e-3 * np.abs(ref) + 1e-3 * rms
+    return bool(ok.all()), float(err.max() / rms)
+
+
+def gemv(gpu, qtype, raw, nrows, ncols, x):
+    m = W.GpuQuantMatrix(gpu, qtype, nrows, ncols, raw)
+    xv = W.GpuVector.init(gpu, x)
+    out = W.GpuVector.init(gpu, np.full(nrows, np.nan, dtype=np.float32))
+    W.GemvQuant.from_device(gpu).dispatch(out, m, xv)
+    return out.read()
+
+
+def weights(qtype, nrows, ncols, seed):
+    return W.quantize(qtype, W.rng_normal(seed, nrows * ncols, 0, 0.02))
+
+
+@pytest.mark.parametrize("qtype", QT)
+@pytest.mark.parametrize("nrows,ncols", [(4, 256), (8, 512), (1, 256), (5, 768), (13, 2304),
+                                         (33, 4096), (260, 11008), (7, 14336)])
+def test_gemv_small_and_ragged(gpu, qtype, nrows, ncols):
+    raw = weights(qtype, nrows, ncols, 100 + nrows)
+    x = W.rng_normal(200 + ncols, ncols)
+    _, ref = orc.gemv_quant(qtype, raw, nrows, ncols, x)
+    ok, e = close(gemv(gpu, qtype, raw, nrows, ncols, x), ref)
+    assert ok, e
+    assert e < 1e-4
+
+
+@pytest.mark.parametrize("ncols", [32, 288, 96])
+def test_gemv_q8_0_unpaired_block_counts(gpu, ncols):
+    # the reference needs ncols % 64 == 0 (% 128 in its kernel) and otherwise falls back to f32
+    # (gguf.rs:146-159); the tiny Llama has 288 columns = 9 blocks
+    nrows = 50
+    raw = weights(W.Q8_0, nrows, ncols, 3)
+    x = W.rng_normal(4, ncols)
+    _, ref = orc.gemv_quant(W.Q8_0, raw, nrows, ncols, x)
+    ok, e = close(gemv(gpu, W.Q8_0, raw, nrows, ncols, x), ref)
+    assert ok, e
+
+
+@pytest.mark.parametrize("qtype", QT)
+@pytest.mark.parametrize("r", [1, 2, 4])
+def test_gemv_rows_per_wave_variants(gpu, qtype, r):
+    nrows, ncols = 1030, 1024  # not a multiple of rows-per-workgroup
+    raw = weights(qtype, nrows, ncols, 8)
+    x = W.rng_normal(9, ncols)
+    _, ref = orc.gemv_quant(qtype, raw, nrows, ncols, x)
+    W._lib.call("wgml_debug_set_gemv_rows_per_wave", r)
+    try:
+        ok, e = close(gemv(gpu, qtype, raw, nrows, ncols, x), ref)
+    finally:
+        W._lib.call("wgml_debug_set_gemv_rows_per_wave", 0)
+    assert ok, e
+
+
+@pytest.mark.parametrize("qtype", QT)
+def test_gemv_one_hot_gives_dequantized_column(gpu, qtype):
+    nrows, ncols = 16, 512
+    be = npref.BLOCK_ELEMS[qtype]
+    raw = npref.random_blocks(qtype, nrows * ncols // be, seed=5)
+    deq = orc.dequantize(qtype, raw, nrows * ncols).reshape(nrows, ncols)
+    for j in (0, 31, 32, 100, 255, 256, 511):
+        x = np.zeros(ncols, dtype=np.float32)
+        x[j] = 1.0
+        got = gemv(gpu, qtype, raw, nrows, ncols, x)
+        # same value up to the rounding of the regrouped scale arithmetic
+        np.testing.assert_allclose(got, deq[:, j], rtol=2e-6, atol=1e-30)
+
+
+@pytest.mark.parametrize("qtype", QT)
+def test_gemv_random_block_bits(gpu, qtype):
+    # wgml-bench feeds random raw bits (gemv_quant.rs:83-101): every scale/min pattern occurs
+    nrows, ncols = 64, 1024
+    raw = npref.random_blocks(qtype, nrows * ncols // npref.BLOCK_ELEMS[qtype], seed=21)
+    x = W.rng_normal(22, ncols)
+    _, ref = orc.gemv_quant(qtype, raw, nrows, ncols, x)
+    ok, e = close(gemv(gpu, qtype, raw, nrows, ncols, x), ref)
+    assert ok, e
+
+
+@pytest.mark.parametrize("qtype", QT)
+@pytest.mark.parametrize("nrows,ncols", [(4096, 4096), (11008, 4096), (4096, 11008),
+                                         (32000, 4096)])
+def test_gemv_benchmark_shapes(gpu, qtype, nrows, ncols):
+    raw = weights(qtype, nrows, ncols, 1000 + qtype)
+    x = W.rng_normal(31, ncols)
+    m = W.GpuQuantMatrix(gpu, qtype, nrows, ncols, raw)
+    op = W.GemvQuant.from_device(gpu)
+    xv, out = W.GpuVector.init(gpu, x), W.GpuVector.uninit(gpu, nrows)
+    op.dispatch(out, m, xv)
+    got = out.read()
+    _, ref = orc.gemv_quant(qtype, raw, nrows, ncols, x)
+    ok, e = close(got, ref)
+    assert ok, e
+    # linearity at full size: M(2x - 3y) = 2 Mx - 3 My
+    y = W.rng_normal(32, ncols)
+    yv = W.GpuVector.init(gpu, y)
+    zv = W.GpuVector.init(gpu, 2 * x - 3 * y)
+    oy, oz = W.GpuVector.uninit(gpu, nrows), W.GpuVector.uninit(gpu, nrows)
+    op.dispatch(oy, m, yv)
+    op.dispatch(oz, m, zv)
+    ok, e = close(oz.read(), 2.0 * got.astype(np.float64) - 3.0 * oy.read().astype(np.float64))
+    assert ok, e
+    # repeatable bit for bit (fixed reduction order)
+    op.dispatch(oy, m, xv)
+    assert np.array_equal(oy.read(), got)
+
+
+def test_gemv_output_into_view(gpu):
+    # the K/V GEMVs write straight into a cache column (models/llama2/transformer.rs:326-341)
+    nrows, ncols = 64, 256
+    raw = weights(W.Q8_0, nrows, ncols, 1)
+    x = W.rng_normal(2, ncols)
+    cache = W.GpuMatrix(gpu, nrows, 8)
+    cache.write(np.zeros(nrows * 8, dtype=np.float32))
+    m = W.GpuQuantMatrix(gpu, W.Q8_0, nrows, ncols, raw)
+    W.GemvQuant.from_device(gpu).dispatch(cache.column(3), m, W.GpuVector.init(gpu, x))
+    full = cache.read().reshape(8, nrows)
+    _, ref = orc.gemv_quant(W.Q8_0, raw, nrows, ncols, x)
+    assert close(full[3], ref)[0]
+    assert not full[[0, 1, 2, 4, 5, 6, 7]].any()
+
+
+def test_gemv_f32_matrix_and_dense_op(gpu):
+    rng = np.random.default_rng(0)
+    nrows, ncols = 37, 288
+    a = rng.standard_normal((nrows, ncols)).astype(np.float32)
+    x = rng.standard_normal(ncols).astype(np.float32)
+    ref = orc.gemv_f64(a, x)
+    assert close(gemv(gpu, W.F32, a.view(np.uint8), nrows, ncols, x), ref)[0]
+    g = W.Gemv.from_device(gpu)
+    av, xv, out = W.GpuVector.init(gpu, a), W.GpuVector.init(gpu, x), W.GpuVector.uninit(gpu, nrows)
+    g.dispatch(out, av, nrows, ncols, xv)
+    assert close(out.read(), ref)[0]
+    # transposed (GemvTr): out = A^T v
+    v = rng.standard_normal(nrows).astype(np.float32)
+    out_t = W.GpuVector.uninit(gpu, ncols)
+    g.dispatch(out_t, av, nrows, ncols, W.GpuVector.init(gpu, v), transposed=True)
+    assert close(out_t.read(), a.astype(np.float64).T @ v.astype(np.float64))[0]
+
+
+def test_gemv_dimension_mismatch(gpu):
+    raw = weights(W.Q8_0, 8, 64, 1)
+    m = W.GpuQuantMatrix(gpu, W.Q8_0, 8, 64, raw)
+    op = W.GemvQuant.from_device(gpu)
+    with pytest.raises(W.WgmlError, match="dimension mismatch"):
+        op.dispatch(W.GpuVector.uninit(gpu, 8), m, W.GpuVector.uninit(gpu, 32))
+    with pytest.raises(W.WgmlError, match="dimension mismatch"):
+        op.dispatch(W.GpuVector.uninit(gpu, 4), m, W.GpuVector.uninit(gpu, 64))

@@ -1,0 +1,143 @@
+"""GPU parity: whole decode steps of the Llama-family and GPT-2 assemblies against
+the oracle's restatement of the reference's CPU transformers, on identical
+quantized bytes.  Logits: |gpu - ref| <= 1e-3 * max|ref| (fp32 accumulate).
+Greedy token ids on the tiny model must be identical."""
+import numpy as np
+import pytest
+
+import oracle as orc
+import wgml_amd as W
+from wgml_amd.models import (GPT2_124M, TINY_LLAMA, Gpt2, Gpt2Params, Llama2, Llama2Config,
+                             LlamaModelType, synth_gpt2, synth_llama)
+
+pytestmark = pytest.mark.gpu
+
+MICRO = Llama2Config(dim=256, hidden_dim=512, n_layers=2, n_q_heads=4, n_kv_heads=2,
+                     vocab_size=320, seq_len=32, rope_base_freq=10000.0, rms_norm_eps=1e-5)
+
+
+def logits_close(got, ref):
+    scale = float(np.abs(ref).max())
+    err = float(np.abs(got.astype(np.float64) - ref).max())
+    return err <= 1e-3 * scale, err / scale
+
+
+def spice(w, cfg, seed, biases):
+    rng = np.random.default_rng(seed)
+    for l in w.layers:
+        l["attn_norm"] = (1 + 0.1 * rng.standard_normal(cfg.dim)).astype(np.float32)
+        l["ffn_norm"] = (1 + 0.1 * rng.standard_normal(cfg.dim)).astype(np.float32)
+        if biases:
+            l["attn_q_bias"] = (0.1 * rng.standard_normal(cfg.dim)).astype(np.float32)
+            l["attn_k_bias"] = (0.1 * rng.standard_normal(cfg.kv_dim)).astype(np.float32)
+            l["attn_v_bias"] = (0.1 * rng.standard_normal(cfg.kv_dim)).astype(np.float32)
+    w.output_norm = (1 + 0.1 * rng.standard_normal(cfg.dim)).astype(np.float32)
+
+
+@pytest.mark.parametrize("scheme", ["q8_0", "q4_k", "q6_k", "q4_k_m", "f32"])
+@pytest.mark.parametrize("model_type", [LlamaModelType.Llama, LlamaModelType.Qwen2])
+@pytest.mark.parametrize("fusion", [0, 1])
+def test_llama_micro_logits_and_kv(gpu, scheme, model_type, fusion):
+    w = synth_llama(MICRO, seed=21, scheme=scheme)
+    spice(w, MICRO, 5, biases=model_type == LlamaModelType.Qwen2)
+    ref = orc.Llama2(w, rope_variant=model_type)
+    m = Llama2(gpu, MICRO, model_type).load(w)
+    m.set_fusion(fusion)
+    toks = [3, 300, 17, 17, 250, 9, 1, 77, 12]
+    for pos, t in enumerate(toks):
+        want = ref.forward(t, pos)
+        got = m.forward_logits(pos, t)
+        ok, e = logits_close(got, want)
+        assert ok, (pos, e)
+    for layer in range(MICRO.n_layers):
+        np.testing.assert_allclose(m.kv_download(layer, 0, 0, len(toks)),
+                                   ref.key_cache(layer)[:len(toks)], atol=1e-4)
+        np.testing.assert_allclose(m.kv_download(layer, 1, 0, len(toks)),
+                                   ref.value_cache(layer)[:len(toks)], atol=1e-4)
+
+
+def test_tiny_llama_greedy_tokens_identical(gpu):
+    # the tiny Llama-2 configuration: Q8_0 weights, 16-token seeded prompt, 128 greedy tokens
+    cfg = TINY_LLAMA
+    w = synth_llama(cfg, seed=1, scheme="q8_0")
+    prompt = W.prompt_tokens(1, 16, cfg.vocab_size)
+    n_total = 16 + 128
+    want, margins = orc.Llama2(w, predequantize=True).generate_greedy(prompt, n_total)
+    m = Llama2(gpu, cfg).load(w)
+    got = m.generate_greedy(prompt, n_total)
+    print(f"top-2 logit margin: min {margins.min():.3e}, median {np.median(margins):.3e}; "
+          f"{m.launches_per_token()} launches/token")
+    assert np.array_equal(got, want)
+    # and once more without the fused epilogues
+    m2 = Llama2(gpu, cfg).load(w)
+    m2.set_fusion(0)
+    assert np.array_equal(m2.generate_greedy(prompt, n_total), want)
+
+
+def test_llama_decode_from_uploaded_kv(gpu):
+    # pre-filled cache then decode, as the long-context configuration does
+    w = synth_llama(MICRO, seed=23, scheme="q6_k")
+    ref = orc.Llama2(w)
+    m = Llama2(gpu, MICRO).load(w)
+    rng = np.random.default_rng(1)
+    n_pre = 20
+    for layer in range(MICRO.n_layers):
+        k = rng.standard_normal((n_pre, MICRO.kv_dim)).astype(np.float32)
+        v = rng.standard_normal((n_pre, MICRO.kv_dim)).astype(np.float32)
+        ref.key_cache(layer)[:n_pre] = k
+        ref.value_cache(layer)[:n_pre] = v
+        m.kv_upload(layer, 0, 0, k)
+        m.kv_upload(layer, 1, 0, v)
+    tok = 7
+    want = []
+    for pos in range(n_pre, n_pre + 6):
+        tok = orc.argmax(ref.forward(tok, pos))
+        want.append(tok)
+    got = m.decode_greedy(7, n_pre, 6)
+    assert list(got) == want
+
+
+def test_llama_argument_checks(gpu):
+    m = Llama2(gpu, MICRO)
+    with pytest.raises(W.WgmlError, match="unset weights"):
+        m.forward(0, 0)
+    w = synth_llama(MICRO, seed=2, scheme="q8_0")
+    bad = w.layers[0]["ffn_down"]
+    with pytest.raises(W.WgmlError, match="expected"):
+        m.set_matrix("attn_q", 0, bad)
+    m.load(w)
+    with pytest.raises(W.WgmlError):
+        m.forward(MICRO.vocab_size, 0)
+    with pytest.raises(W.WgmlError):
+        m.forward(0, MICRO.seq_len)
+
+
+def test_gpt2_micro_logits(gpu):
+    p = Gpt2Params(n_vocab=300, n_seq=32, n_embd=64, n_head=4, n_layer=2, ff_len=256, attn_b=192)
+    w = synth_gpt2(p, seed=5)
+    rng = np.random.default_rng(4)
+    for l in w.layers:
+        for g in ("ln_1_g", "ln_2_g"):
+            l[g] = (1 + 0.1 * rng.standard_normal(p.n_embd)).astype(np.float32)
+        for b in ("ln_1_b", "ln_2_b"):
+            l[b] = (0.1 * rng.standard_normal(p.n_embd)).astype(np.float32)
+    ref = orc.Gpt2(w)
+    m = Gpt2(gpu, p).load(w)
+    for pos, t in enumerate([1, 250, 33, 7, 7, 100]):
+        want = ref.forward(t, pos)
+        m.forward(t, pos)
+        ok, e = logits_close(m.logits(), want)
+        assert ok, (pos, e)
+
+
+def test_gpt2_124m_greedy_prefix(gpu):
+    # GPT-2 124M shape, Q8_0; a 32-token prompt and the first 24 generated tokens against the
+    # oracle (the full run to position 1024 is a benchmark, not a CPU-checkable case)
+    p = GPT2_124M
+    w = synth_gpt2(p, seed=3)
+    prompt = W.prompt_tokens(3, 32, p.n_vocab)
+    n_total = 32 + 24
+    want, margins = orc.Gpt2(w, predequantize=True).generate_greedy(prompt, n_total)
+    got = Gpt2(gpu, p).load(w).generate_greedy(prompt, n_total)
+    print(f"gpt2 top-2 logit margin: min {margins.min():.3e}")
+    assert np.array_equal(got, want)

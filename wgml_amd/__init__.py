@@ -1,0 +1,11 @@
+"""wgml_amd — MI355X (gfx950) batch-1 token-decode path behind wgml's operator API.
+
+Everything computes in `lib/libwgml_hip.so` (hand-written HIP kernels behind a C
+ABI, see include/wgml_hip.h); this package is the thin host-side mirror of the
+reference's `wgml::ops` / `wgml::models` names.  Importing fails if the library
+has not been built: there is no CPU fallback.
+"""
+from ._lib import (F32, Q4_K, Q6_K, Q8_0, LIB_PATH, WgmlError, lib)  # noqa: F401
+from .ops import *  # noqa: F401,F403
+from .models import *  # noqa: F401,F403
+from .models import prompt_tokens  # noqa: F401

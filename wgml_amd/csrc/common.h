@@ -1,0 +1,128 @@
+// Internal declarations shared by the library's translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../include/wgml_hip.h"
+
+namespace wgml {
+
+// ---- errors ---------------------------------------------------------------
+int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define WGML_CHECK_HIP(expr)                                                              \
+    do {                                                                                  \
+        hipError_t e__ = (expr);                                                          \
+        if (e__ != hipSuccess)                                                            \
+            return ::wgml::set_error(WGML_E_HIP, "%s failed: %s (%s:%d)", #expr,          \
+                                     hipGetErrorString(e__), __FILE__, __LINE__);         \
+    } while (0)
+
+#define WGML_REQUIRE(cond, ...)                                                           \
+    do {                                                                                  \
+        if (!(cond)) return ::wgml::set_error(WGML_E_INVALID, __VA_ARGS__);               \
+    } while (0)
+
+#define WGML_TRY(expr)                                                                    \
+    do {                                                                                  \
+        int rc__ = (expr);                                                                \
+        if (rc__ != WGML_OK) return rc__;                                                 \
+    } while (0)
+
+// Reports a launch-configuration error of the kernel just launched.
+#define WGML_CHECK_LAUNCH() WGML_CHECK_HIP(hipGetLastError())
+
+}  // namespace wgml
+
+// ---- handles ----------------------------------------------------------------
+struct wgml_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    int n_cu = 0;
+    char name[128] = {0};
+    // scratch for device-side arg-max results (2 x u32) + pinned mirror
+    uint32_t *d_scalar = nullptr;
+    uint32_t *h_scalar = nullptr;
+    // scratch for split attention partials, grown on demand
+    float *attn_ws = nullptr;
+    size_t attn_ws_bytes = 0;
+    uint64_t launches = 0;  // kernels enqueued so far (diagnostics)
+};
+
+struct wgml_buf {
+    wgml_ctx *ctx = nullptr;
+    void *ptr = nullptr;
+    uint64_t bytes = 0;
+};
+
+// Device layout of a quantized matrix.
+//   F32 : row-major f32.
+//   Q4_K: the GGUF bytes unchanged (144-byte super-blocks, 16-byte aligned).
+//   Q8_0: two planes: `qs` (nrows*ncols int8, row-major) then `d`
+//         (nrows*ncols/32 f16), so that quants load as aligned 128-bit words.
+//   Q6_K: four planes: ql (128 B/block), qh (64 B/block), scales (16 B/block),
+//         d (2 B/block), each row-major in block order.
+// Plane offsets are multiples of 256 bytes; the byte total equals the GGUF size
+// up to that padding.
+struct wgml_qmat {
+    wgml_ctx *ctx = nullptr;
+    int type = 0;
+    uint32_t nrows = 0, ncols = 0;
+    uint64_t gguf_bytes = 0;
+    uint8_t *base = nullptr;  // device allocation
+    uint64_t alloc_bytes = 0;
+    uint8_t *p0 = nullptr, *p1 = nullptr, *p2 = nullptr, *p3 = nullptr;  // planes
+};
+
+namespace wgml {
+
+inline float *view_ptr(const wgml_view &v) {
+    return reinterpret_cast<float *>(v.buf->ptr) + v.offset;
+}
+
+// Validates that a view lies inside its buffer.
+int check_view(const wgml_view &v, const char *what);
+
+// Dynamic per-token scalars read by kernels from device memory so that one
+// captured launch sequence can be replayed for every position.
+struct DynPos {
+    const uint32_t *ptr;  // if non-null, *ptr is used
+    uint32_t val;
+};
+__device__ __forceinline__ uint32_t dyn_pos(const DynPos &p) { return p.ptr ? *p.ptr : p.val; }
+
+// ---- internal launchers (async on ctx->stream, raw device pointers) --------
+struct GemvEpilogue {
+    // out[r] = acc (+ bias[r]) (+ out[r] if accumulate)
+    const float *bias = nullptr;
+    int accumulate = 0;
+};
+
+int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float *v,
+                      const GemvEpilogue &ep);
+int launch_gemv_f32(wgml_ctx *ctx, float *out, const float *a, uint32_t nrows, uint32_t ncols,
+                    int transposed, const float *v);
+int launch_rms_norm(wgml_ctx *ctx, float eps, float *out, const float *x, const float *w,
+                    uint32_t n);
+int launch_layernorm(wgml_ctx *ctx, float *out, const float *x, const float *gamma,
+                     const float *beta, uint32_t n);
+int launch_rope(wgml_ctx *ctx, int variant, uint32_t head_size, uint32_t kv_dim, DynPos pos,
+                float base_freq, float *q, uint32_t q_len, float *k, uint64_t k_pos_stride);
+int launch_softmax(wgml_ctx *ctx, float *mat, uint32_t nrows, uint32_t ncols, uint32_t col_stride);
+int launch_attention(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos, const float *q,
+                     const float *kc, const float *vc, float *att, float *xb);
+int launch_silu(wgml_ctx *ctx, float *h1, const float *h2, uint32_t n);
+int launch_unary(wgml_ctx *ctx, int op, float *x, uint32_t n, const float *args4);
+int launch_op_assign(wgml_ctx *ctx, int op, float *a, const float *b, uint32_t n);
+int launch_argmax(wgml_ctx *ctx, const float *v, uint32_t n, uint32_t *d_out);
+int launch_dequantize(wgml_ctx *ctx, float *out, const wgml_qmat *m);
+
+}  // namespace wgml

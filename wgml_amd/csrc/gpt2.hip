@@ -1,0 +1,266 @@
+// GPT-2 decoder: state, weights and the per-token launch sequence.  Mirrors
+// Gpt2State / Gpt2Weights / Gpt2::dispatch (models/gpt2/transformer.rs:14-477 of
+// the reference) and ChatGpt2's token loop (wgml-chat/src/chat_gpt2.rs:43-151).
+// Unlike the reference, which expands every weight to f32 at load
+// (models/gpt2/transformer.rs:133-141), the matrices stay in their GGUF
+// quantization and go through the quantized GEMV.
+#include "common.h"
+
+using namespace wgml;
+
+namespace wgml {
+int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
+                             uint32_t plan_positions, const float *q, const float *kc,
+                             const float *vc, float *att, float *xb);
+}
+
+struct Gpt2Layer {
+    const wgml_qmat *attn_w = nullptr, *proj_w = nullptr, *fc_w = nullptr, *mlp_proj_w = nullptr;
+    float *ln_1_g = nullptr, *ln_1_b = nullptr, *ln_2_g = nullptr, *ln_2_b = nullptr;
+    float *attn_b = nullptr, *proj_b = nullptr, *fc_b = nullptr, *mlp_proj_b = nullptr;
+    float *key_cache = nullptr, *value_cache = nullptr;
+};
+
+struct wgml_gpt2 {
+    wgml_ctx *ctx = nullptr;
+    wgml_gpt2_params p{};
+    std::vector<Gpt2Layer> layers;
+    const wgml_qmat *lm_head = nullptr;
+    float *ln_f_g = nullptr, *ln_f_b = nullptr, *wte = nullptr, *wpe = nullptr;
+    // Gpt2State (models/gpt2/transformer.rs:14-25)
+    float *layer_input = nullptr, *curr_768 = nullptr, *curr_768_b = nullptr, *curr_2304 = nullptr,
+          *curr_3072 = nullptr, *curr_vocab = nullptr;
+    std::vector<void *> allocs;
+};
+
+namespace {
+
+int dev_alloc(wgml_gpt2 *m, float **p, uint64_t n_floats, bool zero) {
+    void *d = nullptr;
+    hipError_t e = hipMalloc(&d, n_floats * 4);
+    if (e != hipSuccess)
+        return set_error(WGML_E_OOM, "wgml_gpt2: hipMalloc(%llu) failed: %s",
+                         (unsigned long long)(n_floats * 4), hipGetErrorString(e));
+    m->allocs.push_back(d);
+    if (zero) WGML_CHECK_HIP(hipMemsetAsync(d, 0, n_floats * 4, m->ctx->stream));
+    *p = (float *)d;
+    return WGML_OK;
+}
+
+int check_ready(const wgml_gpt2 *m) {
+    for (size_t l = 0; l < m->layers.size(); ++l) {
+        const Gpt2Layer &w = m->layers[l];
+        WGML_REQUIRE(w.attn_w && w.proj_w && w.fc_w && w.mlp_proj_w && w.ln_1_g && w.ln_1_b &&
+                         w.ln_2_g && w.ln_2_b && w.attn_b && w.proj_b && w.fc_b && w.mlp_proj_b,
+                     "wgml_gpt2: layer %zu has unset weights", l);
+    }
+    WGML_REQUIRE(m->lm_head && m->ln_f_g && m->ln_f_b && m->wte && m->wpe,
+                 "wgml_gpt2: lm_head / ln_f / embeddings not set");
+    return WGML_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int wgml_gpt2_create(wgml_ctx *ctx, const wgml_gpt2_params *p, wgml_gpt2 **out) {
+    WGML_REQUIRE(ctx && p && out, "wgml_gpt2_create: null argument");
+    *out = nullptr;
+    WGML_REQUIRE(p->n_vocab && p->n_seq && p->n_embd && p->n_head && p->n_layer && p->ff_len,
+                 "wgml_gpt2_create: zero field in params");
+    WGML_REQUIRE(p->n_embd % p->n_head == 0 && p->attn_b == 3 * p->n_embd,
+                 "wgml_gpt2_create: n_embd %u, n_head %u, attn_b %u are inconsistent", p->n_embd,
+                 p->n_head, p->attn_b);
+    WGML_REQUIRE(p->n_embd % 4 == 0 && p->ff_len % 4 == 0,
+                 "wgml_gpt2_create: n_embd and ff_len must be multiples of 4");
+    WGML_REQUIRE(p->n_embd / p->n_head <= 256, "wgml_gpt2_create: head size above 256");
+    wgml_gpt2 *m = new wgml_gpt2();
+    m->ctx = ctx;
+    m->p = *p;
+    m->layers.resize(p->n_layer);
+    int rc = WGML_OK;
+    auto A = [&](float **q, uint64_t n, bool z) {
+        if (rc == WGML_OK) rc = dev_alloc(m, q, n, z);
+    };
+    A(&m->layer_input, p->n_embd, true);
+    A(&m->curr_768, p->n_embd, true);
+    A(&m->curr_768_b, p->n_embd, true);
+    A(&m->curr_2304, p->attn_b, true);
+    A(&m->curr_3072, p->ff_len, true);
+    A(&m->curr_vocab, p->n_vocab, true);
+    for (auto &l : m->layers) {
+        A(&l.key_cache, (uint64_t)p->n_embd * p->n_seq, true);
+        A(&l.value_cache, (uint64_t)p->n_embd * p->n_seq, true);
+    }
+    if (rc == WGML_OK && hipStreamSynchronize(ctx->stream) != hipSuccess)
+        rc = set_error(WGML_E_HIP, "wgml_gpt2_create: synchronize failed");
+    if (rc != WGML_OK) {
+        wgml_gpt2_destroy(m);
+        return rc;
+    }
+    *out = m;
+    return WGML_OK;
+}
+
+int wgml_gpt2_destroy(wgml_gpt2 *m) {
+    if (!m) return WGML_OK;
+    if (m->ctx && m->ctx->stream) (void)hipStreamSynchronize(m->ctx->stream);
+    for (void *p : m->allocs) (void)hipFree(p);
+    delete m;
+    return WGML_OK;
+}
+
+int wgml_gpt2_set_matrix(wgml_gpt2 *m, int which, uint32_t layer, const wgml_qmat *mat) {
+    WGML_REQUIRE(m && mat, "wgml_gpt2_set_matrix: null argument");
+    const wgml_gpt2_params &p = m->p;
+    uint32_t er = 0, ec = 0;
+    switch (which) {  // models/gpt2/cpu.rs:150-158,193-196
+    case WGML_GPT2_ATTN_W: er = p.attn_b; ec = p.n_embd; break;
+    case WGML_GPT2_ATTN_PROJ_W: er = p.n_embd; ec = p.n_embd; break;
+    case WGML_GPT2_MLP_FC_W: er = p.ff_len; ec = p.n_embd; break;
+    case WGML_GPT2_MLP_PROJ_W: er = p.n_embd; ec = p.ff_len; break;
+    case WGML_GPT2_LM_HEAD: er = p.n_vocab; ec = p.n_embd; break;
+    default: return set_error(WGML_E_INVALID, "wgml_gpt2_set_matrix: unknown matrix %d", which);
+    }
+    WGML_REQUIRE(mat->nrows == er && mat->ncols == ec,
+                 "wgml_gpt2_set_matrix: matrix %d is %ux%u, expected %ux%u", which, mat->nrows,
+                 mat->ncols, er, ec);
+    if (which == WGML_GPT2_LM_HEAD) {
+        m->lm_head = mat;
+        return WGML_OK;
+    }
+    WGML_REQUIRE(layer < p.n_layer, "wgml_gpt2_set_matrix: layer %u of %u", layer, p.n_layer);
+    Gpt2Layer &l = m->layers[layer];
+    switch (which) {
+    case WGML_GPT2_ATTN_W: l.attn_w = mat; break;
+    case WGML_GPT2_ATTN_PROJ_W: l.proj_w = mat; break;
+    case WGML_GPT2_MLP_FC_W: l.fc_w = mat; break;
+    case WGML_GPT2_MLP_PROJ_W: l.mlp_proj_w = mat; break;
+    }
+    return WGML_OK;
+}
+
+int wgml_gpt2_set_vector(wgml_gpt2 *m, int which, uint32_t layer, const float *host,
+                         uint32_t len) {
+    WGML_REQUIRE(m && host, "wgml_gpt2_set_vector: null argument");
+    const wgml_gpt2_params &p = m->p;
+    uint32_t expect = p.n_embd;
+    float **slot = nullptr;
+    if (which == WGML_GPT2_LN_F_G) slot = &m->ln_f_g;
+    else if (which == WGML_GPT2_LN_F_B) slot = &m->ln_f_b;
+    else {
+        WGML_REQUIRE(layer < p.n_layer, "wgml_gpt2_set_vector: layer %u of %u", layer, p.n_layer);
+        Gpt2Layer &l = m->layers[layer];
+        switch (which) {
+        case WGML_GPT2_LN_1_G: slot = &l.ln_1_g; break;
+        case WGML_GPT2_LN_1_B: slot = &l.ln_1_b; break;
+        case WGML_GPT2_LN_2_G: slot = &l.ln_2_g; break;
+        case WGML_GPT2_LN_2_B: slot = &l.ln_2_b; break;
+        case WGML_GPT2_ATTN_B: slot = &l.attn_b; expect = p.attn_b; break;
+        case WGML_GPT2_ATTN_PROJ_B: slot = &l.proj_b; break;
+        case WGML_GPT2_MLP_FC_B: slot = &l.fc_b; expect = p.ff_len; break;
+        case WGML_GPT2_MLP_PROJ_B: slot = &l.mlp_proj_b; break;
+        default: return set_error(WGML_E_INVALID, "wgml_gpt2_set_vector: unknown vector %d", which);
+        }
+    }
+    WGML_REQUIRE(len == expect, "wgml_gpt2_set_vector: vector %d has %u elements, expected %u",
+                 which, len, expect);
+    if (!*slot) WGML_TRY(dev_alloc(m, slot, len, false));
+    WGML_CHECK_HIP(hipMemcpyAsync(*slot, host, (size_t)len * 4, hipMemcpyHostToDevice,
+                                  m->ctx->stream));
+    WGML_CHECK_HIP(hipStreamSynchronize(m->ctx->stream));
+    return WGML_OK;
+}
+
+int wgml_gpt2_set_embeddings(wgml_gpt2 *m, const float *wte, const float *wpe) {
+    WGML_REQUIRE(m && wte && wpe, "wgml_gpt2_set_embeddings: null argument");
+    const uint64_t nt = (uint64_t)m->p.n_embd * m->p.n_vocab, np = (uint64_t)m->p.n_embd * m->p.n_seq;
+    if (!m->wte) WGML_TRY(dev_alloc(m, &m->wte, nt, false));
+    if (!m->wpe) WGML_TRY(dev_alloc(m, &m->wpe, np, false));
+    WGML_CHECK_HIP(hipMemcpyAsync(m->wte, wte, nt * 4, hipMemcpyHostToDevice, m->ctx->stream));
+    WGML_CHECK_HIP(hipMemcpyAsync(m->wpe, wpe, np * 4, hipMemcpyHostToDevice, m->ctx->stream));
+    WGML_CHECK_HIP(hipStreamSynchronize(m->ctx->stream));
+    return WGML_OK;
+}
+
+// Gpt2::dispatch (models/gpt2/transformer.rs:265-477).  The reference's
+// mul_assign/add_assign after each layernorm and the add_assign after each
+// matmul are folded into the producing launch (affine layernorm, GEMV bias and
+// accumulate epilogues); the copies of q/k/v out of the fused qkv vector
+// (:329-353) are avoided by letting the attention read q in place and by
+// copying only k and v into their cache columns.
+int wgml_gpt2_forward(wgml_gpt2 *m, uint32_t token, uint32_t pos) {
+    WGML_REQUIRE(m != nullptr, "wgml_gpt2_forward: null model");
+    WGML_TRY(check_ready(m));
+    const wgml_gpt2_params &p = m->p;
+    WGML_REQUIRE(token < p.n_vocab, "wgml_gpt2_forward: token %u outside vocabulary %u", token,
+                 p.n_vocab);
+    WGML_REQUIRE(pos < p.n_seq, "wgml_gpt2_forward: pos %u outside n_seq %u", pos, p.n_seq);
+    wgml_ctx *ctx = m->ctx;
+    const uint32_t n = p.n_embd;
+    const DynPos dpos{nullptr, pos};
+    const wgml_attn_params ap{p.n_seq, n, 1u, p.n_head, n / p.n_head, pos};
+
+    // layer_input = wte[:, token] + wpe[:, pos]   (:277-290)
+    WGML_CHECK_HIP(hipMemcpyAsync(m->layer_input, m->wte + (size_t)token * n, (size_t)n * 4,
+                                  hipMemcpyDeviceToDevice, ctx->stream));
+    WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, m->layer_input, m->wpe + (size_t)pos * n, n));
+
+    for (uint32_t l = 0; l < p.n_layer; ++l) {
+        const Gpt2Layer &w = m->layers[l];
+        WGML_TRY(launch_layernorm(ctx, m->curr_768, m->layer_input, w.ln_1_g, w.ln_1_b, n));
+        WGML_TRY(launch_gemv_quant(ctx, m->curr_2304, w.attn_w, m->curr_768,
+                                   GemvEpilogue{w.attn_b, 0}));
+        // k -> key_cache[:, pos], v -> value_cache[:, pos]; contiguous so one copy each
+        WGML_CHECK_HIP(hipMemcpyAsync(w.key_cache + (size_t)pos * n, m->curr_2304 + n,
+                                      (size_t)n * 4, hipMemcpyDeviceToDevice, ctx->stream));
+        WGML_CHECK_HIP(hipMemcpyAsync(w.value_cache + (size_t)pos * n, m->curr_2304 + 2 * n,
+                                      (size_t)n * 4, hipMemcpyDeviceToDevice, ctx->stream));
+        WGML_TRY(launch_attention_planned(ctx, ap, dpos, pos + 1, m->curr_2304, w.key_cache,
+                                          w.value_cache, nullptr, m->curr_768));
+        // layer_input += proj_w * attn + proj_b   (:372-395)
+        WGML_TRY(launch_gemv_quant(ctx, m->layer_input, w.proj_w, m->curr_768,
+                                   GemvEpilogue{w.proj_b, 1}));
+        WGML_TRY(launch_layernorm(ctx, m->curr_768, m->layer_input, w.ln_2_g, w.ln_2_b, n));
+        WGML_TRY(launch_gemv_quant(ctx, m->curr_3072, w.fc_w, m->curr_768,
+                                   GemvEpilogue{w.fc_b, 0}));
+        WGML_TRY(launch_unary(ctx, WGML_UNARY_GELU, m->curr_3072, p.ff_len, nullptr));
+        // layer_input += mlp_proj_w * h + mlp_proj_b   (:433-452)
+        WGML_TRY(launch_gemv_quant(ctx, m->layer_input, w.mlp_proj_w, m->curr_3072,
+                                   GemvEpilogue{w.mlp_proj_b, 1}));
+    }
+    WGML_TRY(launch_layernorm(ctx, m->curr_768, m->layer_input, m->ln_f_g, m->ln_f_b, n));
+    WGML_TRY(launch_gemv_quant(ctx, m->curr_vocab, m->lm_head, m->curr_768, GemvEpilogue{}));
+    return WGML_OK;
+}
+
+int wgml_gpt2_read_logits(wgml_gpt2 *m, float *host_out) {
+    WGML_REQUIRE(m && host_out, "wgml_gpt2_read_logits: null argument");
+    WGML_CHECK_HIP(hipMemcpyAsync(host_out, m->curr_vocab, (size_t)m->p.n_vocab * 4,
+                                  hipMemcpyDeviceToHost, m->ctx->stream));
+    WGML_CHECK_HIP(hipStreamSynchronize(m->ctx->stream));
+    return WGML_OK;
+}
+
+int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_prompt,
+                              uint32_t n_total, uint32_t *out_tokens) {
+    WGML_REQUIRE(m && prompt && out_tokens, "wgml_gpt2_generate_greedy: null argument");
+    WGML_REQUIRE(n_prompt >= 1, "wgml_gpt2_generate_greedy: empty prompt");
+    WGML_REQUIRE(n_total <= m->p.n_seq, "wgml_gpt2_generate_greedy: %u positions exceed n_seq %u",
+                 n_total, m->p.n_seq);
+    wgml_ctx *ctx = m->ctx;
+    uint32_t token = prompt[0];
+    for (uint32_t pos = 0; pos < n_total; ++pos) {
+        WGML_TRY(wgml_gpt2_forward(m, token, pos));
+        WGML_TRY(launch_argmax(ctx, m->curr_vocab, m->p.n_vocab, ctx->d_scalar));
+        WGML_CHECK_HIP(hipMemcpyAsync(ctx->h_scalar, ctx->d_scalar, 4, hipMemcpyDeviceToHost,
+                                      ctx->stream));
+        WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+        const uint32_t best = ctx->h_scalar[0];
+        out_tokens[pos] = best;
+        token = (pos + 1 < n_prompt) ? prompt[pos + 1] : best;
+    }
+    return WGML_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,319 @@
+// Quantized matrices on the device: GGUF block layouts (quantization.rs:29-42,
+// 204-244, 322-389 of the reference), their re-layout into aligned planes, and
+// the bit-exact dequantization kernels.
+//
+// This file must be compiled with -ffp-contract=off: the reference's CPU
+// dequantizers round every product and difference separately
+// (quantization.rs:233-236, 366, 370) and the kernels below must match them bit
+// for bit.
+#include "common.h"
+#include "device_utils.h"
+
+using namespace wgml;
+
+namespace {
+
+constexpr uint32_t QK8_0 = 32, QK_K = 256;
+constexpr uint32_t Q8_0_BYTES = 34, Q4_K_BYTES = 144, Q6_K_BYTES = 210;
+
+inline uint64_t align256(uint64_t v) { return (v + 255) & ~uint64_t(255); }
+
+// ---- re-layout kernels (run once per matrix at load) ------------------------
+
+// raw: nblocks x {u16 d; i8 qs[32]} (2-byte aligned) -> qs plane + d plane.
+__global__ void repack_q8_0(const uint16_t *__restrict__ raw, uint32_t *__restrict__ qs,
+                            uint16_t *__restrict__ d, uint64_t nblocks) {
+    uint64_t b = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const uint16_t *src = raw + b * 17;
+    d[b] = src[0];
+    uint32_t *dst = qs + b * 8;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) dst[k] = (uint32_t)src[1 + 2 * k] | ((uint32_t)src[2 + 2 * k] << 16);
+}
+
+// raw: nblocks x {u8 ql[128]; u8 qh[64]; i8 scales[16]; u16 d} (2-byte aligned).
+__global__ void repack_q6_k(const uint16_t *__restrict__ raw, uint16_t *__restrict__ ql,
+                            uint16_t *__restrict__ qh, uint16_t *__restrict__ sc,
+                            uint16_t *__restrict__ d, uint64_t nblocks) {
+    // One wave-quarter (16 lanes) would be enough; keep it simple: 105 halfwords
+    // per block, one thread per halfword.
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t b = i / 105;
+    uint32_t h = (uint32_t)(i % 105);
+    if (b >= nblocks) return;
+    uint16_t v = raw[b * 105 + h];
+    if (h < 64) ql[b * 64 + h] = v;
+    else if (h < 96) qh[b * 32 + (h - 64)] = v;
+    else if (h < 104) sc[b * 8 + (h - 96)] = v;
+    else d[b] = v;
+}
+
+// ---- dequantization kernels ---------------------------------------------------
+
+// quantization.rs:38-41
+__global__ void dequant_q8_0(const int8_t *__restrict__ qs, const uint16_t *__restrict__ d,
+                             float *__restrict__ out, uint64_t n) {
+    uint64_t e = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    float scale = f16_bits_to_f32(d[e / QK8_0]);
+    out[e] = (float)qs[e] * scale;
+}
+
+// quantization.rs:347-389; one thread per byte of qs (two outputs).
+__global__ void dequant_q4_k(const uint8_t *__restrict__ blocks, float *__restrict__ out,
+                             uint64_t nblocks) {
+    uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t b = t / 128;
+    uint32_t l = (uint32_t)(t % 128);  // byte index in qs
+    if (b >= nblocks) return;
+    const uint8_t *blk = blocks + b * Q4_K_BYTES;
+    float d = f16_bits_to_f32(*(const uint16_t *)(blk + 0));
+    float dmin = f16_bits_to_f32(*(const uint16_t *)(blk + 2));
+    const uint8_t *scales = blk + 4;
+    uint32_t j = l / 32;  // 64-element group
+    uint8_t sc1, m1, sc2, m2;
+    get_scale_min_k4(2 * j, scales, sc1, m1);
+    get_scale_min_k4(2 * j + 1, scales, sc2, m2);
+    float d1 = d * (float)sc1, mm1 = dmin * (float)m1;
+    float d2 = d * (float)sc2, mm2 = dmin * (float)m2;
+    uint8_t q = blk[16 + l];
+    float *o = out + b * QK_K + j * 64 + (l % 32);
+    o[0] = d1 * (float)(q & 0xF) - mm1;
+    o[32] = d2 * (float)(q >> 4) - mm2;
+}
+
+// quantization.rs:214-243; one thread per (block, half i, l): four outputs.
+__global__ void dequant_q6_k(const uint8_t *__restrict__ ql, const uint8_t *__restrict__ qh,
+                             const int8_t *__restrict__ sc, const uint16_t *__restrict__ dd,
+                             float *__restrict__ out, uint64_t nblocks) {
+    uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t b = t / 64;
+    uint32_t i = (uint32_t)(t % 64) / 32, l = (uint32_t)(t % 32);
+    if (b >= nblocks) return;
+    float d = f16_bits_to_f32(dd[b]);
+    uint32_t is = l / 16;
+    uint8_t ql0 = ql[b * 128 + i * 64 + l], ql32 = ql[b * 128 + i * 64 + l + 32];
+    uint8_t h = qh[b * 64 + i * 32 + l];
+    int q1 = (int)((ql0 & 0xF) | (((h >> 0) & 3) << 4)) - 32;
+    int q2 = (int)((ql32 & 0xF) | (((h >> 2) & 3) << 4)) - 32;
+    int q3 = (int)((ql0 >> 4) | (((h >> 4) & 3) << 4)) - 32;
+    int q4 = (int)((ql32 >> 4) | (((h >> 6) & 3) << 4)) - 32;
+    const int8_t *s = sc + b * 16 + i * 8 + is;
+    float *o = out + b * QK_K + i * 128 + l;
+    o[0] = d * (float)s[0] * (float)q1;
+    o[32] = d * (float)s[2] * (float)q2;
+    o[64] = d * (float)s[4] * (float)q3;
+    o[96] = d * (float)s[6] * (float)q4;
+}
+
+// quantization.rs:16-24
+__global__ void f16_to_f32_kernel(const uint16_t *__restrict__ in, float *__restrict__ out,
+                                  uint32_t n) {
+    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = f16_bits_to_f32(in[i]);
+}
+
+uint32_t block_elems(int type) {
+    switch (type) {
+    case WGML_F32: return 1;
+    case WGML_Q8_0: return QK8_0;
+    case WGML_Q4_K: return QK_K;
+    case WGML_Q6_K: return QK_K;
+    default: return 0;
+    }
+}
+
+uint32_t block_bytes(int type) {
+    switch (type) {
+    case WGML_F32: return 4;
+    case WGML_Q8_0: return Q8_0_BYTES;
+    case WGML_Q4_K: return Q4_K_BYTES;
+    case WGML_Q6_K: return Q6_K_BYTES;
+    default: return 0;
+    }
+}
+
+}  // namespace
+
+namespace wgml {
+
+int launch_dequantize(wgml_ctx *ctx, float *out, const wgml_qmat *m) {
+    uint64_t n = (uint64_t)m->nrows * m->ncols;
+    const int T = 256;
+    switch (m->type) {
+    case WGML_F32:
+        WGML_CHECK_HIP(hipMemcpyAsync(out, m->p0, n * 4, hipMemcpyDeviceToDevice, ctx->stream));
+        break;
+    case WGML_Q8_0:
+        dequant_q8_0<<<dim3((unsigned)((n + T - 1) / T)), dim3(T), 0, ctx->stream>>>(
+            (const int8_t *)m->p0, (const uint16_t *)m->p1, out, n);
+        break;
+    case WGML_Q4_K: {
+        uint64_t nb = n / QK_K, nt = nb * 128;
+        dequant_q4_k<<<dim3((unsigned)((nt + T - 1) / T)), dim3(T), 0, ctx->stream>>>(m->p0, out,
+                                                                                      nb);
+        break;
+    }
+    case WGML_Q6_K: {
+        uint64_t nb = n / QK_K, nt = nb * 64;
+        dequant_q6_k<<<dim3((unsigned)((nt + T - 1) / T)), dim3(T), 0, ctx->stream>>>(
+            m->p0, m->p1, (const int8_t *)m->p2, (const uint16_t *)m->p3, out, nb);
+        break;
+    }
+    default: return set_error(WGML_E_UNSUPPORTED, "dequantize: unsupported type %d", m->type);
+    }
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
+}  // namespace wgml
+
+extern "C" {
+
+uint32_t wgml_quant_block_elems(int type) { return block_elems(type); }
+
+uint64_t wgml_quant_bytes(int type, uint64_t nelems) {
+    uint32_t be = block_elems(type);
+    if (!be || nelems % be) return 0;
+    return nelems / be * block_bytes(type);
+}
+
+int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t ncols,
+                             const void *gguf_bytes, wgml_qmat **out) {
+    WGML_REQUIRE(ctx && out && gguf_bytes, "wgml_quant_matrix_create: null argument");
+    *out = nullptr;
+    uint32_t be = block_elems(type);
+    if (!be)
+        return set_error(WGML_E_UNSUPPORTED,
+                         "wgml_quant_matrix_create: quantization type %d is not supported "
+                         "(supported: F32, Q8_0, Q4_K, Q6_K)",
+                         type);
+    WGML_REQUIRE(nrows > 0 && ncols > 0, "wgml_quant_matrix_create: empty matrix %ux%u", nrows,
+                 ncols);
+    WGML_REQUIRE(ncols % be == 0,
+                 "wgml_quant_matrix_create: ncols %u is not a multiple of the block length %u",
+                 ncols, be);
+    // x is staged as float4; every quantized block length is a multiple of 4, f32 needs it too.
+    WGML_REQUIRE(ncols % 4 == 0, "wgml_quant_matrix_create: ncols %u must be a multiple of 4",
+                 ncols);
+    uint64_t nelem = (uint64_t)nrows * ncols;
+    uint64_t nblocks = nelem / be;
+    uint64_t gguf = nblocks * block_bytes(type);
+
+    wgml_qmat *m = new wgml_qmat();
+    m->ctx = ctx;
+    m->type = type;
+    m->nrows = nrows;
+    m->ncols = ncols;
+    m->gguf_bytes = gguf;
+
+    uint64_t o1 = 0, o2 = 0, o3 = 0, total = 0;
+    switch (type) {
+    case WGML_F32:
+    case WGML_Q4_K: total = align256(gguf); break;
+    case WGML_Q8_0:
+        o1 = align256(nblocks * 32);
+        total = o1 + align256(nblocks * 2);
+        break;
+    case WGML_Q6_K:
+        o1 = align256(nblocks * 128);
+        o2 = o1 + align256(nblocks * 64);
+        o3 = o2 + align256(nblocks * 16);
+        total = o3 + align256(nblocks * 2);
+        break;
+    }
+    // 256 spare bytes so that whole-wave 16-byte loads of a partly filled last
+    // tile never leave the allocation.
+    total += 256;
+    hipError_t e = hipMalloc((void **)&m->base, total);
+    if (e != hipSuccess) {
+        delete m;
+        return set_error(WGML_E_OOM, "wgml_quant_matrix_create: hipMalloc(%llu) failed: %s",
+                         (unsigned long long)total, hipGetErrorString(e));
+    }
+    m->alloc_bytes = total;
+    m->p0 = m->base;
+    m->p1 = m->base + o1;
+    m->p2 = m->base + o2;
+    m->p3 = m->base + o3;
+
+    auto fail = [&](hipError_t err, const char *what) {
+        (void)hipFree(m->base);
+        delete m;
+        return set_error(WGML_E_HIP, "wgml_quant_matrix_create: %s: %s", what,
+                         hipGetErrorString(err));
+    };
+
+    if (type == WGML_F32 || type == WGML_Q4_K) {
+        e = hipMemcpyAsync(m->base, gguf_bytes, gguf, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) return fail(e, "upload");
+    } else {
+        uint8_t *raw = nullptr;
+        e = hipMalloc((void **)&raw, gguf);
+        if (e != hipSuccess) return fail(e, "staging hipMalloc");
+        e = hipMemcpyAsync(raw, gguf_bytes, gguf, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) {
+            const int T = 256;
+            if (type == WGML_Q8_0) {
+                repack_q8_0<<<dim3((unsigned)((nblocks + T - 1) / T)), dim3(T), 0, ctx->stream>>>(
+                    (const uint16_t *)raw, (uint32_t *)m->p0, (uint16_t *)m->p1, nblocks);
+            } else {
+                uint64_t nt = nblocks * 105;
+                repack_q6_k<<<dim3((unsigned)((nt + T - 1) / T)), dim3(T), 0, ctx->stream>>>(
+                    (const uint16_t *)raw, (uint16_t *)m->p0, (uint16_t *)m->p1,
+                    (uint16_t *)m->p2, (uint16_t *)m->p3, nblocks);
+            }
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        (void)hipFree(raw);
+        if (e != hipSuccess) return fail(e, "re-layout");
+    }
+    *out = m;
+    return WGML_OK;
+}
+
+int wgml_quant_matrix_destroy(wgml_qmat *m) {
+    if (!m) return WGML_OK;
+    if (m->ctx && m->ctx->stream) (void)hipStreamSynchronize(m->ctx->stream);
+    if (m->base) (void)hipFree(m->base);
+    delete m;
+    return WGML_OK;
+}
+
+int wgml_quant_matrix_shape(const wgml_qmat *m, int *type, uint32_t *nrows, uint32_t *ncols) {
+    WGML_REQUIRE(m != nullptr, "wgml_quant_matrix_shape: null matrix");
+    if (type) *type = m->type;
+    if (nrows) *nrows = m->nrows;
+    if (ncols) *ncols = m->ncols;
+    return WGML_OK;
+}
+
+uint64_t wgml_quant_matrix_gguf_bytes(const wgml_qmat *m) { return m ? m->gguf_bytes : 0; }
+
+int wgml_dequantize(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m) {
+    WGML_REQUIRE(ctx && m, "wgml_dequantize: null argument");
+    WGML_TRY(check_view(out, "wgml_dequantize: out"));
+    WGML_REQUIRE((uint64_t)out.len == (uint64_t)m->nrows * m->ncols,
+                 "wgml_dequantize: out has %u elements, matrix has %llu", out.len,
+                 (unsigned long long)m->nrows * m->ncols);
+    return launch_dequantize(ctx, view_ptr(out), m);
+}
+
+int wgml_f16_to_f32(wgml_ctx *ctx, wgml_view out, const wgml_buf *in, uint64_t in_offset_bytes) {
+    WGML_REQUIRE(ctx && in, "wgml_f16_to_f32: null argument");
+    WGML_TRY(check_view(out, "wgml_f16_to_f32: out"));
+    WGML_REQUIRE(in_offset_bytes % 2 == 0 && in_offset_bytes + 2ull * out.len <= in->bytes,
+                 "wgml_f16_to_f32: input range exceeds buffer");
+    if (out.len == 0) return WGML_OK;
+    f16_to_f32_kernel<<<dim3((out.len + 255) / 256), dim3(256), 0, ctx->stream>>>(
+        (const uint16_t *)((const char *)in->ptr + in_offset_bytes), view_ptr(out), out.len);
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
+}  // extern "C"
