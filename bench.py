@@ -1,0 +1,209 @@
+#!/usr/bin/env python3
+"""Benchmark of the batch-1 token-decode path on one MI355X.
+
+Workload (default): Llama-2-7B shape (dim 4096, 32 layers, 32 heads, FFN 11008,
+vocab 32000), weights seeded N(0, 0.02) quantized with the ggml reference
+quantizers in a Q4_K_M-style mix (Q4_K; Q6_K for attn_v, output and the
+ffn_down layers picked by use_more_bits), embedding f32, activations and KV
+cache f32.  `--warmup` prompt tokens are pushed through the decoder one at a
+time (untimed), then exactly `--steps` greedy decode steps are timed: one step =
+one token = one pass over every weight.
+
+Prints ONE JSON line: decode tok/s, the HBM roofline of the dominant kernel
+(the Q4_K GEMV of the 11008x4096 gate/up projections) measured with HIP events
+on the library's own stream, a GEMV sweep at 4096x11008 for the three formats,
+and the CPU baseline (the single-threaded C restatement of the reference's CPU
+transformer) timed on this host on a bounded sample.
+
+    python bench.py [--gpus 1] [--steps 256] [--warmup 128] [--model 7b|tiny]
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def gemv_bytes(qtype_bytes_per_matrix: int, nrows: int, ncols: int) -> int:
+    """Algorithmic bytes of one GEMV: GGUF bytes of W + x (f32) + y (f32)."""
+    return qtype_bytes_per_matrix + 4 * ncols + 4 * nrows
+
+
+def time_gemv(W, gpu, mats, nrows, ncols, iters):
+    """Average GPU duration (us) of out = M x over `iters` graph-recorded launches
+    rotating through `mats` (distinct device copies, so nothing stays cached)."""
+    from wgml_amd._lib import call
+
+    out = W.GpuVector.uninit(gpu, nrows)
+    x = W.GpuVector.init(gpu, W.rng_normal(99, ncols))
+    arr = (C.c_void_p * len(mats))(*[m.handle for m in mats])
+    ms = C.c_float()
+    best = None
+    for _ in range(3):
+        call("wgml_bench_gemv_quant", gpu.handle, arr, len(mats), out.view(), x.view(), iters, 1,
+             C.byref(ms))
+        us = ms.value * 1e3 / iters
+        best = us if best is None else min(best, us)
+    return best
+
+
+def gemv_sweep(W, gpu, nrows, ncols, min_total_bytes=640 << 20):
+    """4096x11008 (ffn_down shape) for Q8_0 / Q4_K / Q6_K: GB/s and fraction of HBM peak."""
+    res = {}
+    vals = W.rng_normal(4242, nrows * ncols, 0.0, 0.02)
+    for qtype, name in ((W.Q8_0, "q8_0"), (W.Q4_K, "q4_k"), (W.Q6_K, "q6_k")):
+        raw = W.quantize(qtype, vals)
+        n_copies = max(2, -(-min_total_bytes // raw.nbytes))
+        mats = [W.GpuQuantMatrix(gpu, qtype, nrows, ncols, raw) for _ in range(n_copies)]
+        us = time_gemv(W, gpu, mats, nrows, ncols, iters=4 * n_copies)
+        b = gemv_bytes(raw.nbytes, nrows, ncols)
+        gbs = b / us * 1e-3
+        res[name] = {"us": round(us, 3), "GB/s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+                     "bytes": b, "copies": n_copies}
+        log(f"  gemv {name} {nrows}x{ncols}: {us:.2f} us  {gbs:.0f} GB/s  "
+            f"({100 * gbs / HBM_PEAK_GBS:.1f}% of HBM peak)")
+        del mats
+    return res
+
+
+def cpu_baseline(weights, prompt, n_steps):
+    """Times the CPU oracle (port of the reference's single-threaded CPU
+    transformer, weights expanded to f32 at load as the reference does) on the
+    first `n_steps` positions of the same model and prompt."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle as orc
+
+    t0 = time.perf_counter()
+    m = orc.Llama2(weights, predequantize=True)
+    t_load = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    for pos in range(n_steps):
+        m.forward(int(prompt[pos]), pos)
+    dt = time.perf_counter() - t0
+    log(f"  cpu oracle: load (dequantize) {t_load:.1f}s, {n_steps} steps in {dt:.1f}s")
+    return {"value": round(n_steps / dt, 4), "unit": "tok/s", "cores": 1, "kind": "port",
+            "sample": f"{n_steps} decode steps (positions 0..{n_steps - 1}) of the same model, "
+                      f"f32 weights dequantized at load, single thread"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=128)
+    ap.add_argument("--model", default="7b", choices=["7b", "tiny"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--cpu-steps", type=int, default=0, help="CPU baseline steps (0 = auto)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (every kernel uses a single device; "
+                 "no collectives are built). Use --gpus 1.")
+
+    import numpy as np
+
+    import wgml_amd as W
+    from wgml_amd.models import LLAMA2_7B, TINY_LLAMA, Llama2, synth_llama
+
+    gpu = W.GpuInstance(0)
+    name, n_cu = gpu.info()
+    log(f"device: {name}, {n_cu} CUs")
+
+    if args.model == "7b":
+        cfg, scheme, label = LLAMA2_7B, "q4_k_m", "llama2-7b-shape q4_k_m"
+    else:
+        cfg, scheme, label = TINY_LLAMA, "q8_0", "tiny-llama2 q8_0"
+    assert args.warmup >= 1 and args.warmup + args.steps <= cfg.seq_len, "positions exceed seq_len"
+
+    t0 = time.perf_counter()
+    weights = synth_llama(cfg, seed=4, scheme=scheme,
+                          progress=lambda l: log(f"  built layer {l + 1}/{cfg.n_layers} "
+                                                 f"({time.perf_counter() - t0:.0f}s)")
+                          if (l + 1) % 8 == 0 else None)
+    log(f"weights built in {time.perf_counter() - t0:.0f}s "
+        f"({weights.weight_bytes_per_token() / 1e9:.3f} GB per token)")
+    model = Llama2(gpu, cfg).load(weights)
+    prompt = W.prompt_tokens(4, args.warmup, cfg.vocab_size)
+
+    # warm-up: the prompt, one token at a time (the reference has no batched prefill)
+    out = model.generate_greedy(prompt, args.warmup)
+    gpu.synchronize()
+    first = int(out[-1])
+
+    # timed region: exactly `steps` greedy decode steps, host round trip per token included
+    gpu.synchronize()
+    t0 = time.perf_counter()
+    toks = model.decode_greedy(first, args.warmup, args.steps)
+    gpu.synchronize()
+    dt = time.perf_counter() - t0
+    tok_s = args.steps / dt
+    wbytes = weights.weight_bytes_per_token()
+    kv_bytes_mid = 2 * cfg.n_layers * cfg.kv_dim * 4 * (args.warmup + args.steps // 2)
+    roof_tok_s = HBM_PEAK_GBS * 1e9 / wbytes
+    log(f"decode: {args.steps} steps in {dt * 1e3:.1f} ms -> {tok_s:.1f} tok/s "
+        f"({100 * tok_s / roof_tok_s:.1f}% of the weight-bytes roofline {roof_tok_s:.0f} tok/s); "
+        f"{model.launches_per_token()} launches/token")
+
+    # dominant kernel: Q4_K GEMV of the gate/up projections, timed live over the model's own
+    # per-layer matrices (distinct memory, > last-level cache in total)
+    roofline = None
+    if args.model == "7b":
+        gate = [W.GpuQuantMatrix(gpu, W.Q4_K, cfg.hidden_dim, cfg.dim, l["ffn_gate"].data)
+                for l in weights.layers[:24]]
+        us = time_gemv(W, gpu, gate, cfg.hidden_dim, cfg.dim, iters=4 * len(gate))
+        b = gemv_bytes(gate[0].gguf_bytes(), cfg.hidden_dim, cfg.dim)
+        gbs = b / us * 1e-3
+        traffic = None
+        tpath = os.path.join(ROOT, "profiles", "traffic.json")
+        if os.path.exists(tpath):
+            traffic = json.load(open(tpath)).get("gemv_q4_k_11008x4096_bytes_per_launch")
+        roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                    "kernel": "gemv_quant_kernel<FmtQ4K,4> 11008x4096", "bytes_per_launch": b,
+                    "us_per_launch": round(us, 3)}
+        log(f"dominant kernel Q4_K gemv 11008x4096: {us:.2f} us, {gbs:.0f} GB/s")
+        del gate
+
+    sweep = None
+    if not args.no_sweep and args.model == "7b":
+        sweep = gemv_sweep(W, gpu, 4096, 11008)
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        n = args.cpu_steps or (2 if args.model == "7b" else 32)
+        cpu = cpu_baseline(weights, prompt, min(n, args.warmup))
+
+    line = {
+        "metric": "decode tok/s bs1 Llama-2-7B-shape Q4_K" if args.model == "7b"
+        else "decode tok/s bs1 tiny Llama-2 Q8_0",
+        "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(dt * 1e3 / args.steps, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{label} bs1 greedy decode: {args.warmup}-token prompt "
+                               f"(one token per step), then {args.steps} timed steps",
+                   "weights": "seeded N(0,0.02), ggml reference quantizers; embedding/activations/KV f32",
+                   "weight_bytes_per_token": wbytes, "kv_bytes_per_token_mid_run": kv_bytes_mid,
+                   "roofline_tok_s_at_8TBs": round(roof_tok_s, 1),
+                   "frac_of_weight_roofline": round(tok_s / roof_tok_s, 4),
+                   "launches_per_token": model.launches_per_token(),
+                   "last_token": int(toks[-1])},
+        "roofline": roofline, "cpu_baseline": cpu, "gemv_sweep_4096x11008": sweep,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

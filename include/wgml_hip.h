@@ -105,7 +105,7 @@ WGML_API int wgml_buf_zero(wgml_buf *buf);
  * the reference there is no pairing rule (ncols % 64 / % 512) and no silent
  * fall-back to f32: any ncols that is a multiple of the block length stays
  * quantized.  The bytes are re-laid out on the device (see the layout notes
- * in csrc/quant.hip); the values are unchanged. */
+ * in csrc/common.h); the values are unchanged. */
 WGML_API int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t ncols,
                                       const void *gguf_bytes, wgml_qmat **out);
 WGML_API int wgml_quant_matrix_destroy(wgml_qmat *m);
@@ -297,6 +297,16 @@ WGML_API int wgml_gpt2_read_logits(wgml_gpt2 *m, float *host_out);
 /* ChatGpt2::forward's loop with greedy sampling (wgml-chat/src/chat_gpt2.rs:43-151). */
 WGML_API int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_prompt,
                                        uint32_t n_total, uint32_t *out_tokens);
+
+/* ---- measurement: wgml-bench's bench_gemv (wgml-bench/src/main.rs:187-250) ---- *
+ * Enqueues out = mats[i % n_mats] * v for i in 0..iters back to back between two
+ * GPU timestamps and returns the elapsed milliseconds.  Rotating over several
+ * matrices keeps the weights out of the last-level cache.  use_graph != 0
+ * records the launches into a HIP graph first, so host launch time is not
+ * part of the measurement. */
+WGML_API int wgml_bench_gemv_quant(wgml_ctx *ctx, const wgml_qmat *const *mats, uint32_t n_mats,
+                                   wgml_view out, wgml_view v, uint32_t iters, int use_graph,
+                                   float *total_ms);
 
 /* ---- host-side input makers (no device needed) ---------------------------- *
  * The reference only de-quantizes; its inputs come from GGUF files written by

@@ -127,6 +127,7 @@ PROTOTYPES = {
     "wgml_gpt2_forward": (_i, [_P, _u32, _u32]),
     "wgml_gpt2_read_logits": (_i, [_P, _P]),
     "wgml_gpt2_generate_greedy": (_i, [_P, _P, _u32, _u32, _P]),
+    "wgml_bench_gemv_quant": (_i, [_P, _PP, _u32, View, View, _u32, _i, _fp]),
     "wgml_quantize": (_i, [_i, _P, _P, _u64, _i]),
     "wgml_rng_normal": (_i, [_u64, _P, _u64, _f, _f, _i]),
     "wgml_rng_uniform_u32": (_i, [_u64, _P, _u64, _u32]),

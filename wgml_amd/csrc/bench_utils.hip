@@ -1,0 +1,67 @@
+// GPU-timed back-to-back GEMV launches: the measuring loop of wgml-bench's
+// bench_gemv (crates/wgml-bench/src/main.rs:187-250 of the reference: N
+// dispatches between two GPU timestamps), with the launches recorded into a HIP
+// graph so that host launch overhead does not sit between the kernels.
+#include "common.h"
+
+using namespace wgml;
+
+extern "C" {
+
+int wgml_bench_gemv_quant(wgml_ctx *ctx, const wgml_qmat *const *mats, uint32_t n_mats,
+                          wgml_view out, wgml_view v, uint32_t iters, int use_graph,
+                          float *total_ms) {
+    WGML_REQUIRE(ctx && mats && total_ms && n_mats > 0 && iters > 0,
+                 "wgml_bench_gemv_quant: bad argument");
+    WGML_TRY(check_view(out, "wgml_bench_gemv_quant: out"));
+    WGML_TRY(check_view(v, "wgml_bench_gemv_quant: v"));
+    for (uint32_t i = 0; i < n_mats; ++i) {
+        WGML_REQUIRE(mats[i] != nullptr, "wgml_bench_gemv_quant: null matrix %u", i);
+        WGML_REQUIRE(mats[i]->ncols == v.len && mats[i]->nrows == out.len,
+                     "wgml_bench_gemv_quant: matrix %u does not match the vectors", i);
+    }
+    float *po = view_ptr(out);
+    const float *pv = view_ptr(v);
+    if (!use_graph) {
+        WGML_CHECK_HIP(hipEventRecord(ctx->ev_start, ctx->stream));
+        for (uint32_t i = 0; i < iters; ++i)
+            WGML_TRY(launch_gemv_quant(ctx, po, mats[i % n_mats], pv, GemvEpilogue{}));
+        WGML_CHECK_HIP(hipEventRecord(ctx->ev_stop, ctx->stream));
+        WGML_CHECK_HIP(hipEventSynchronize(ctx->ev_stop));
+        WGML_CHECK_HIP(hipEventElapsedTime(total_ms, ctx->ev_start, ctx->ev_stop));
+        return WGML_OK;
+    }
+    // one untimed launch per matrix first: opt-in attributes and lazy module
+    // loading must not happen during capture
+    for (uint32_t i = 0; i < n_mats && i < iters; ++i)
+        WGML_TRY(launch_gemv_quant(ctx, po, mats[i], pv, GemvEpilogue{}));
+    WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    int rc = WGML_OK;
+    for (uint32_t i = 0; i < iters && rc == WGML_OK; ++i)
+        rc = launch_gemv_quant(ctx, po, mats[i % n_mats], pv, GemvEpilogue{});
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    if (rc != WGML_OK) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc;
+    }
+    if (e != hipSuccess)
+        return set_error(WGML_E_HIP, "wgml_bench_gemv_quant: end capture: %s", hipGetErrorString(e));
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e == hipSuccess) e = hipGraphLaunch(exec, ctx->stream);  // warm replay, untimed
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess) e = hipEventRecord(ctx->ev_start, ctx->stream);
+    if (e == hipSuccess) e = hipGraphLaunch(exec, ctx->stream);
+    if (e == hipSuccess) e = hipEventRecord(ctx->ev_stop, ctx->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(ctx->ev_stop);
+    if (e == hipSuccess) e = hipEventElapsedTime(total_ms, ctx->ev_start, ctx->ev_stop);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    if (e != hipSuccess)
+        return set_error(WGML_E_HIP, "wgml_bench_gemv_quant: %s", hipGetErrorString(e));
+    return WGML_OK;
+}
+
+}  // extern "C"

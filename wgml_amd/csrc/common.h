@@ -55,6 +55,10 @@ struct wgml_ctx {
     float *attn_ws = nullptr;
     size_t attn_ws_bytes = 0;
     uint64_t launches = 0;  // kernels enqueued so far (diagnostics)
+    // Buffers, matrices and models keep their context alive: the device objects
+    // are torn down when the last reference goes, whatever order handles are
+    // destroyed in.
+    int refs = 1;
 };
 
 struct wgml_buf {
@@ -87,6 +91,9 @@ namespace wgml {
 inline float *view_ptr(const wgml_view &v) {
     return reinterpret_cast<float *>(v.buf->ptr) + v.offset;
 }
+
+void ctx_retain(wgml_ctx *ctx);
+void ctx_release(wgml_ctx *ctx);
 
 // Validates that a view lies inside its buffer.
 int check_view(const wgml_view &v, const char *what);

@@ -76,6 +76,7 @@ int wgml_gpt2_create(wgml_ctx *ctx, const wgml_gpt2_params *p, wgml_gpt2 **out) 
     WGML_REQUIRE(p->n_embd / p->n_head <= 256, "wgml_gpt2_create: head size above 256");
     wgml_gpt2 *m = new wgml_gpt2();
     m->ctx = ctx;
+    ctx_retain(ctx);
     m->p = *p;
     m->layers.resize(p->n_layer);
     int rc = WGML_OK;
@@ -106,6 +107,7 @@ int wgml_gpt2_destroy(wgml_gpt2 *m) {
     if (!m) return WGML_OK;
     if (m->ctx && m->ctx->stream) (void)hipStreamSynchronize(m->ctx->stream);
     for (void *p : m->allocs) (void)hipFree(p);
+    ctx_release(m->ctx);
     delete m;
     return WGML_OK;
 }

@@ -83,6 +83,7 @@ int wgml_llama2_create(wgml_ctx *ctx, const wgml_llama2_config *cfg, int model_t
                  "wgml_llama2_create: dim and hidden_dim must be multiples of 4");
     wgml_llama2 *m = new wgml_llama2();
     m->ctx = ctx;
+    ctx_retain(ctx);
     m->cfg = *cfg;
     m->model_type = model_type;
     // Llama2Config::derived_configs (models/llama2/cpu.rs:111-141)
@@ -90,6 +91,7 @@ int wgml_llama2_create(wgml_ctx *ctx, const wgml_llama2_config *cfg, int model_t
     m->head_size = cfg->dim / cfg->n_q_heads;
     m->kv_mul = cfg->n_q_heads / cfg->n_kv_heads;
     if (m->head_size % 2 != 0 || m->head_size > 256) {
+        ctx_release(ctx);
         delete m;
         return set_error(WGML_E_UNSUPPORTED, "wgml_llama2_create: head_size %u unsupported",
                          cfg->dim / cfg->n_q_heads);
@@ -124,6 +126,7 @@ int wgml_llama2_destroy(wgml_llama2 *m) {
     if (!m) return WGML_OK;
     if (m->ctx && m->ctx->stream) (void)hipStreamSynchronize(m->ctx->stream);
     for (void *p : m->allocs) (void)hipFree(p);
+    ctx_release(m->ctx);
     delete m;
     return WGML_OK;
 }

@@ -204,6 +204,7 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
 
     wgml_qmat *m = new wgml_qmat();
     m->ctx = ctx;
+    ctx_retain(ctx);
     m->type = type;
     m->nrows = nrows;
     m->ncols = ncols;
@@ -229,6 +230,7 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
     total += 256;
     hipError_t e = hipMalloc((void **)&m->base, total);
     if (e != hipSuccess) {
+        ctx_release(ctx);
         delete m;
         return set_error(WGML_E_OOM, "wgml_quant_matrix_create: hipMalloc(%llu) failed: %s",
                          (unsigned long long)total, hipGetErrorString(e));
@@ -241,6 +243,7 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
 
     auto fail = [&](hipError_t err, const char *what) {
         (void)hipFree(m->base);
+        ctx_release(ctx);
         delete m;
         return set_error(WGML_E_HIP, "wgml_quant_matrix_create: %s: %s", what,
                          hipGetErrorString(err));
@@ -280,6 +283,7 @@ int wgml_quant_matrix_destroy(wgml_qmat *m) {
     if (!m) return WGML_OK;
     if (m->ctx && m->ctx->stream) (void)hipStreamSynchronize(m->ctx->stream);
     if (m->base) (void)hipFree(m->base);
+    ctx_release(m->ctx);
     delete m;
     return WGML_OK;
 }

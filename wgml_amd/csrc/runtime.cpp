@@ -23,6 +23,23 @@ int check_view(const wgml_view &v, const char *what) {
     return WGML_OK;
 }
 
+void ctx_retain(wgml_ctx *ctx) {
+    if (ctx) ++ctx->refs;
+}
+
+void ctx_release(wgml_ctx *ctx) {
+    if (!ctx || --ctx->refs > 0) return;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->attn_ws) (void)hipFree(ctx->attn_ws);
+    if (ctx->d_scalar) (void)hipFree(ctx->d_scalar);
+    if (ctx->h_scalar) (void)hipHostFree(ctx->h_scalar);
+    if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
+    if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
 }  // namespace wgml
 
 using namespace wgml;
@@ -68,15 +85,8 @@ int wgml_ctx_create(int device, wgml_ctx **out) {
 
 int wgml_ctx_destroy(wgml_ctx *ctx) {
     if (!ctx) return WGML_OK;
-    (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
-    if (ctx->attn_ws) (void)hipFree(ctx->attn_ws);
-    if (ctx->d_scalar) (void)hipFree(ctx->d_scalar);
-    if (ctx->h_scalar) (void)hipHostFree(ctx->h_scalar);
-    if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
-    if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
-    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
-    delete ctx;
+    ctx_release(ctx);
     return WGML_OK;
 }
 
@@ -118,6 +128,7 @@ int wgml_buf_create(wgml_ctx *ctx, uint64_t bytes, wgml_buf **out) {
                          (unsigned long long)bytes, hipGetErrorString(e));
     wgml_buf *b = new wgml_buf();
     b->ctx = ctx;
+    ctx_retain(ctx);
     b->ptr = p;
     b->bytes = bytes;
     *out = b;
@@ -128,6 +139,7 @@ int wgml_buf_destroy(wgml_buf *buf) {
     if (!buf) return WGML_OK;
     if (buf->ctx && buf->ctx->stream) (void)hipStreamSynchronize(buf->ctx->stream);
     if (buf->ptr) (void)hipFree(buf->ptr);
+    ctx_release(buf->ctx);
     delete buf;
     return WGML_OK;
 }
