@@ -29,7 +29,7 @@ def test_every_declared_symbol_is_exported():
 
 def test_binding_covers_the_header():
     declared = set(header_symbols())
-    bound = set(_lib.PROTOTYPES) - {"wgml_debug_set_gemv_rows_per_wave"}
+    bound = {n for n in _lib.PROTOTYPES if not n.startswith("wgml_debug_")}
     assert declared == bound, declared ^ bound
 
 

@@ -16,6 +16,18 @@ import wgml_amd as W
 pytestmark = pytest.mark.gpu
 QT = [W.Q8_0, W.Q4_K, W.Q6_K]
 
+# Two GEMV implementations sit behind the same entry point: the default integer-dot path
+# (activations staged as 16-bit block fixed point, rounding <= 2^-16 of a block's maximum) and
+# the fp32-activation path.  Observed error / rms(ref): ~3e-5 and ~1e-6 respectively.
+MODES = {"int_dot": 5e-4, "f32_act": 1e-4}
+
+
+@pytest.fixture(params=list(MODES))
+def mode(request):
+    W._lib.lib.wgml_debug_set_gemv_f32_activations(1 if request.param == "f32_act" else 0)
+    yield request.param
+    W._lib.lib.wgml_debug_set_gemv_f32_activations(0)
+
 
 def close(got, ref):
     ref = np.asarray(ref, dtype=np.float64)
@@ -40,17 +52,17 @@ def weights(qtype, nrows, ncols, seed):
 @pytest.mark.parametrize("qtype", QT)
 @pytest.mark.parametrize("nrows,ncols", [(4, 256), (8, 512), (1, 256), (5, 768), (13, 2304),
                                          (33, 4096), (260, 11008), (7, 14336)])
-def test_gemv_small_and_ragged(gpu, qtype, nrows, ncols):
+def test_gemv_small_and_ragged(gpu, mode, qtype, nrows, ncols):
     raw = weights(qtype, nrows, ncols, 100 + nrows)
     x = W.rng_normal(200 + ncols, ncols)
     _, ref = orc.gemv_quant(qtype, raw, nrows, ncols, x)
     ok, e = close(gemv(gpu, qtype, raw, nrows, ncols, x), ref)
     assert ok, e
-    assert e < 1e-4
+    assert e < MODES[mode], e
 
 
 @pytest.mark.parametrize("ncols", [32, 288, 96])
-def test_gemv_q8_0_unpaired_block_counts(gpu, ncols):
+def test_gemv_q8_0_unpaired_block_counts(gpu, mode, ncols):
     # the reference needs ncols % 64 == 0 (% 128 in its kernel) and otherwise falls back to f32
     # (gguf.rs:146-159); the tiny Llama has 288 columns = 9 blocks
     nrows = 50
@@ -62,8 +74,8 @@ def test_gemv_q8_0_unpaired_block_counts(gpu, ncols):
 
 
 @pytest.mark.parametrize("qtype", QT)
-@pytest.mark.parametrize("r", [1, 2, 4])
-def test_gemv_rows_per_wave_variants(gpu, qtype, r):
+@pytest.mark.parametrize("r", [1, 2])
+def test_gemv_rows_per_wave_variants(gpu, mode, qtype, r):
     nrows, ncols = 1030, 1024  # not a multiple of rows-per-workgroup
     raw = weights(qtype, nrows, ncols, 8)
     x = W.rng_normal(9, ncols)
@@ -77,7 +89,7 @@ def test_gemv_rows_per_wave_variants(gpu, qtype, r):
 
 
 @pytest.mark.parametrize("qtype", QT)
-def test_gemv_one_hot_gives_dequantized_column(gpu, qtype):
+def test_gemv_one_hot_gives_dequantized_column(gpu, mode, qtype):
     nrows, ncols = 16, 512
     be = npref.BLOCK_ELEMS[qtype]
     raw = npref.random_blocks(qtype, nrows * ncols // be, seed=5)
@@ -86,12 +98,13 @@ def test_gemv_one_hot_gives_dequantized_column(gpu, qtype):
         x = np.zeros(ncols, dtype=np.float32)
         x[j] = 1.0
         got = gemv(gpu, qtype, raw, nrows, ncols, x)
-        # same value up to the rounding of the regrouped scale arithmetic
-        np.testing.assert_allclose(got, deq[:, j], rtol=2e-6, atol=1e-30)
+        # same value up to the rounding of the regrouped scale arithmetic (and, on the
+        # integer-dot path, of 1.0 in 16-bit block fixed point: 32512/32512 exactly)
+        np.testing.assert_allclose(got, deq[:, j], rtol=4e-6, atol=1e-6 * np.abs(deq[:, j]).max())
 
 
 @pytest.mark.parametrize("qtype", QT)
-def test_gemv_random_block_bits(gpu, qtype):
+def test_gemv_random_block_bits(gpu, mode, qtype):
     # wgml-bench feeds random raw bits (gemv_quant.rs:83-101): every scale/min pattern occurs
     nrows, ncols = 64, 1024
     raw = npref.random_blocks(qtype, nrows * ncols // npref.BLOCK_ELEMS[qtype], seed=21)
@@ -104,7 +117,7 @@ def test_gemv_random_block_bits(gpu, qtype):
 @pytest.mark.parametrize("qtype", QT)
 @pytest.mark.parametrize("nrows,ncols", [(4096, 4096), (11008, 4096), (4096, 11008),
                                          (32000, 4096)])
-def test_gemv_benchmark_shapes(gpu, qtype, nrows, ncols):
+def test_gemv_benchmark_shapes(gpu, mode, qtype, nrows, ncols):
     raw = weights(qtype, nrows, ncols, 1000 + qtype)
     x = W.rng_normal(31, ncols)
     m = W.GpuQuantMatrix(gpu, qtype, nrows, ncols, raw)

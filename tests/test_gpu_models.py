@@ -50,10 +50,10 @@ def test_llama_micro_logits_and_kv(gpu, scheme, model_type, fusion):
         ok, e = logits_close(got, want)
         assert ok, (pos, e)
     for layer in range(MICRO.n_layers):
-        np.testing.assert_allclose(m.kv_download(layer, 0, 0, len(toks)),
-                                   ref.key_cache(layer)[:len(toks)], atol=1e-4)
-        np.testing.assert_allclose(m.kv_download(layer, 1, 0, len(toks)),
-                                   ref.value_cache(layer)[:len(toks)], atol=1e-4)
+        for which, ref_c in ((0, ref.key_cache(layer)), (1, ref.value_cache(layer))):
+            want_c = ref_c[:len(toks)]
+            np.testing.assert_allclose(m.kv_download(layer, which, 0, len(toks)), want_c,
+                                       rtol=0, atol=1e-3 * np.abs(want_c).max())
 
 
 def test_tiny_llama_greedy_tokens_identical(gpu):

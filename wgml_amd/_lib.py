@@ -133,6 +133,8 @@ PROTOTYPES = {
     "wgml_rng_uniform_u32": (_i, [_u64, _P, _u64, _u32]),
     # debug knob, not part of the reference surface
     "wgml_debug_set_gemv_rows_per_wave": (_i, [_i]),
+    "wgml_debug_set_gemv_config": (_i, [_i, _i, _i, _i]),
+    "wgml_debug_set_gemv_f32_activations": (_i, [_i]),
 }
 
 # calls whose return value is not a status code

@@ -38,7 +38,16 @@ struct GemvParams {
     const float *bias;
     uint32_t nrows, ncols;
     int accumulate;
+    int debug;  // experiments: bit0 skip x staging, bit1 skip the dot products
 };
+
+// Hides a value from the optimizer (no instruction is emitted).  Used on masked
+// 32-bit words so that the four bytes are converted with v_cvt_f32_ubyte0..3 of
+// the *shared* masked word instead of one bit-field extract per element.
+__device__ __forceinline__ uint32_t opaque(uint32_t v) {
+    asm("" : "+v"(v));
+    return v;
+}
 
 // ------------------------------------------------------------------ Q4_K ----
 struct FmtQ4K {
@@ -59,8 +68,6 @@ struct FmtQ4K {
         tile = g >> 4;
         chunk = g & 15;
     }
-    // which sum a chunk contributes to
-    __device__ static uint32_t sum_of_chunk(uint32_t chunk) { return chunk >> 3; }
     __device__ static void load(Row &w, const RowBase &rb, uint32_t tile) {
         const uint8_t *blk = rb.blocks + (size_t)(tile >> 2) * 144;
         w.hdr = *reinterpret_cast<const uint4 *>(blk);
@@ -68,44 +75,56 @@ struct FmtQ4K {
         w.qa = q[0];
         w.qb = q[1];
     }
-    __device__ static float dot(const Row &w, const float4 (&x)[CHUNKS], const float (&s)[NSUM],
-                                uint32_t tile) {
+    // acc[r] += dot(row r tile, x tile).  xl points at this lane's slot of chunk 0
+    // (chunk c is xl[c * 64]); s = the two half-tile sums of x.
+    template <int R>
+    __device__ static void accumulate(const Row (&w)[R], const float4 *xl, const float *s,
+                                      uint32_t tile, float (&acc)[R]) {
         const uint32_t j = tile & 3;
-        const float d = f16_bits_to_f32((uint16_t)(w.hdr.x & 0xffffu));
-        const float dmin = f16_bits_to_f32((uint16_t)(w.hdr.x >> 16));
-        // 6-bit scale/min pairs of sub-blocks 2j and 2j+1 (get_scale_min_k4).
         const uint32_t sh = (j & 1u) * 16u;
-        const uint32_t a = (w.hdr.y >> sh) & 0xffffu, b = (w.hdr.z >> sh) & 0xffffu,
-                       c = (w.hdr.w >> sh) & 0xffffu;
-        uint32_t sc2, m2;
-        if (j < 2) {
-            sc2 = a & 0x3f3fu;
-            m2 = b & 0x3f3fu;
-        } else {
-            sc2 = (c & 0x0f0fu) | ((a >> 2) & 0x3030u);
-            m2 = ((c >> 4) & 0x0f0fu) | ((b >> 2) & 0x3030u);
-        }
-        const float sc_lo = ub0(sc2), sc_hi = ub1(sc2), m_lo = ub0(m2), m_hi = ub1(m2);
-        const uint32_t q[8] = {w.qa.x, w.qa.y, w.qa.z, w.qa.w, w.qb.x, w.qb.y, w.qb.z, w.qb.w};
-        float dlo = 0.f, dhi = 0.f;
+        float dlo[R], dhi[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) dlo[r] = dhi[r] = 0.f;
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            const uint32_t lo = q[k] & 0x0f0f0f0fu;
-            const uint32_t hi = q[k] & 0xf0f0f0f0u;  // 16 * nibble per byte
-            const float4 xl = x[k], xh = x[8 + k];
-            dlo = fmaf(ub0(lo), xl.x, dlo);
-            dlo = fmaf(ub1(lo), xl.y, dlo);
-            dlo = fmaf(ub2(lo), xl.z, dlo);
-            dlo = fmaf(ub3(lo), xl.w, dlo);
-            dhi = fmaf(ub0(hi), xh.x, dhi);
-            dhi = fmaf(ub1(hi), xh.y, dhi);
-            dhi = fmaf(ub2(hi), xh.z, dhi);
-            dhi = fmaf(ub3(hi), xh.w, dhi);
+            const float4 xa = xl[k * 64], xb = xl[(8 + k) * 64];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const uint32_t q = k < 4 ? (&w[r].qa.x)[k] : (&w[r].qb.x)[k - 4];
+                const uint32_t lo = opaque(q & 0x0f0f0f0fu);
+                const uint32_t hi = opaque(q & 0xf0f0f0f0u);  // 16 * nibble per byte
+                dlo[r] = fmaf(ub0(lo), xa.x, dlo[r]);
+                dlo[r] = fmaf(ub1(lo), xa.y, dlo[r]);
+                dlo[r] = fmaf(ub2(lo), xa.z, dlo[r]);
+                dlo[r] = fmaf(ub3(lo), xa.w, dlo[r]);
+                dhi[r] = fmaf(ub0(hi), xb.x, dhi[r]);
+                dhi[r] = fmaf(ub1(hi), xb.y, dhi[r]);
+                dhi[r] = fmaf(ub2(hi), xb.z, dhi[r]);
+                dhi[r] = fmaf(ub3(hi), xb.w, dhi[r]);
+            }
         }
-        float r = (d * sc_lo) * dlo;
-        r = fmaf((d * sc_hi) * 0.0625f, dhi, r);
-        r = fmaf(-dmin, fmaf(m_lo, s[0], m_hi * s[1]), r);
-        return r;
+        const float s0 = s[0], s1 = s[1];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float d = f16_bits_to_f32((uint16_t)(w[r].hdr.x & 0xffffu));
+            const float dmin = f16_bits_to_f32((uint16_t)(w[r].hdr.x >> 16));
+            // 6-bit scale/min pairs of sub-blocks 2j and 2j+1 (get_scale_min_k4).
+            const uint32_t a = (w[r].hdr.y >> sh) & 0xffffu, b = (w[r].hdr.z >> sh) & 0xffffu,
+                           c = (w[r].hdr.w >> sh) & 0xffffu;
+            uint32_t sc2, m2;
+            if (j < 2) {
+                sc2 = a & 0x3f3fu;
+                m2 = b & 0x3f3fu;
+            } else {
+                sc2 = (c & 0x0f0fu) | ((a >> 2) & 0x3030u);
+                m2 = ((c >> 4) & 0x0f0fu) | ((b >> 2) & 0x3030u);
+            }
+            const float sc_lo = ub0(sc2), sc_hi = ub1(sc2), m_lo = ub0(m2), m_hi = ub1(m2);
+            float v = (d * sc_lo) * dlo[r];
+            v = fmaf((d * sc_hi) * 0.0625f, dhi[r], v);
+            v = fmaf(-dmin, fmaf(m_lo, s0, m_hi * s1), v);
+            acc[r] += v;
+        }
     }
 };
 
@@ -133,7 +152,6 @@ struct FmtQ6K {
         tile = blk * 4 + i * 2 + s;
         chunk = quarter * 4 + k4;
     }
-    __device__ static uint32_t sum_of_chunk(uint32_t chunk) { return chunk >> 2; }
     __device__ static void load(Row &w, const RowBase &rb, uint32_t tile) {
         const size_t blk = tile >> 2;
         const uint32_t i = (tile >> 1) & 1, s = tile & 1;
@@ -144,46 +162,54 @@ struct FmtQ6K {
         w.sc = *reinterpret_cast<const uint2 *>(rb.sc + blk * 16 + i * 8);
         w.d = *reinterpret_cast<const uint16_t *>(rb.d + blk * 2);
     }
-    __device__ static float dot(const Row &w, const float4 (&x)[CHUNKS], const float (&s)[NSUM],
-                                uint32_t tile) {
-        const uint32_t sb = (tile & 1u) * 8u;  // bit offset of scales[is], is = tile & 1
-        const float sc1 = sb0(w.sc.x >> sb), sc2 = sb0(w.sc.x >> (sb + 16)),
-                    sc3 = sb0(w.sc.y >> sb), sc4 = sb0(w.sc.y >> (sb + 16));
-        const uint32_t l0[4] = {w.l0.x, w.l0.y, w.l0.z, w.l0.w};
-        const uint32_t l1[4] = {w.l1.x, w.l1.y, w.l1.z, w.l1.w};
-        const uint32_t hh[4] = {w.h.x, w.h.y, w.h.z, w.h.w};
-        float d1 = 0.f, d2 = 0.f, d3 = 0.f, d4 = 0.f;
+    template <int R>
+    __device__ static void accumulate(const Row (&w)[R], const float4 *xl, const float *s,
+                                      uint32_t tile, float (&acc)[R]) {
+        float d1[R], d2[R], d3[R], d4[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) d1[r] = d2[r] = d3[r] = d4[r] = 0.f;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const uint32_t H = hh[k];
-            const uint32_t q1 = (l0[k] & 0x0f0f0f0fu) | ((H << 4) & 0x30303030u);
-            const uint32_t q2 = (l1[k] & 0x0f0f0f0fu) | ((H << 2) & 0x30303030u);
-            const uint32_t q3 = ((l0[k] >> 4) & 0x0f0f0f0fu) | (H & 0x30303030u);
-            const uint32_t q4 = ((l1[k] >> 4) & 0x0f0f0f0fu) | ((H >> 2) & 0x30303030u);
-            const float4 x1 = x[k], x2 = x[4 + k], x3 = x[8 + k], x4 = x[12 + k];
-            d1 = fmaf(ub0(q1), x1.x, d1);
-            d1 = fmaf(ub1(q1), x1.y, d1);
-            d1 = fmaf(ub2(q1), x1.z, d1);
-            d1 = fmaf(ub3(q1), x1.w, d1);
-            d2 = fmaf(ub0(q2), x2.x, d2);
-            d2 = fmaf(ub1(q2), x2.y, d2);
-            d2 = fmaf(ub2(q2), x2.z, d2);
-            d2 = fmaf(ub3(q2), x2.w, d2);
-            d3 = fmaf(ub0(q3), x3.x, d3);
-            d3 = fmaf(ub1(q3), x3.y, d3);
-            d3 = fmaf(ub2(q3), x3.z, d3);
-            d3 = fmaf(ub3(q3), x3.w, d3);
-            d4 = fmaf(ub0(q4), x4.x, d4);
-            d4 = fmaf(ub1(q4), x4.y, d4);
-            d4 = fmaf(ub2(q4), x4.z, d4);
-            d4 = fmaf(ub3(q4), x4.w, d4);
+            const float4 x1 = xl[k * 64], x2 = xl[(4 + k) * 64], x3 = xl[(8 + k) * 64],
+                         x4 = xl[(12 + k) * 64];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const uint32_t L0 = (&w[r].l0.x)[k], L1 = (&w[r].l1.x)[k], H = (&w[r].h.x)[k];
+                const uint32_t q1 = opaque((L0 & 0x0f0f0f0fu) | ((H << 4) & 0x30303030u));
+                const uint32_t q2 = opaque((L1 & 0x0f0f0f0fu) | ((H << 2) & 0x30303030u));
+                const uint32_t q3 = opaque(((L0 >> 4) & 0x0f0f0f0fu) | (H & 0x30303030u));
+                const uint32_t q4 = opaque(((L1 >> 4) & 0x0f0f0f0fu) | ((H >> 2) & 0x30303030u));
+                d1[r] = fmaf(ub0(q1), x1.x, d1[r]);
+                d1[r] = fmaf(ub1(q1), x1.y, d1[r]);
+                d1[r] = fmaf(ub2(q1), x1.z, d1[r]);
+                d1[r] = fmaf(ub3(q1), x1.w, d1[r]);
+                d2[r] = fmaf(ub0(q2), x2.x, d2[r]);
+                d2[r] = fmaf(ub1(q2), x2.y, d2[r]);
+                d2[r] = fmaf(ub2(q2), x2.z, d2[r]);
+                d2[r] = fmaf(ub3(q2), x2.w, d2[r]);
+                d3[r] = fmaf(ub0(q3), x3.x, d3[r]);
+                d3[r] = fmaf(ub1(q3), x3.y, d3[r]);
+                d3[r] = fmaf(ub2(q3), x3.z, d3[r]);
+                d3[r] = fmaf(ub3(q3), x3.w, d3[r]);
+                d4[r] = fmaf(ub0(q4), x4.x, d4[r]);
+                d4[r] = fmaf(ub1(q4), x4.y, d4[r]);
+                d4[r] = fmaf(ub2(q4), x4.z, d4[r]);
+                d4[r] = fmaf(ub3(q4), x4.w, d4[r]);
+            }
         }
-        // q - 32 folded in through the sub-block sums of x.
-        float r = sc1 * fmaf(-32.f, s[0], d1);
-        r = fmaf(sc2, fmaf(-32.f, s[1], d2), r);
-        r = fmaf(sc3, fmaf(-32.f, s[2], d3), r);
-        r = fmaf(sc4, fmaf(-32.f, s[3], d4), r);
-        return f16_bits_to_f32(w.d) * r;
+        const uint32_t sb = (tile & 1u) * 8u;  // bit offset of scales[is], is = tile & 1
+        const float s0 = s[0], s1 = s[1], s2 = s[2], s3 = s[3];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float sc1 = sb0(w[r].sc.x >> sb), sc2 = sb0(w[r].sc.x >> (sb + 16)),
+                        sc3 = sb0(w[r].sc.y >> sb), sc4 = sb0(w[r].sc.y >> (sb + 16));
+            // q - 32 folded in through the sub-block sums of x.
+            float v = sc1 * fmaf(-32.f, s0, d1[r]);
+            v = fmaf(sc2, fmaf(-32.f, s1, d2[r]), v);
+            v = fmaf(sc3, fmaf(-32.f, s2, d3[r]), v);
+            v = fmaf(sc4, fmaf(-32.f, s3, d4[r]), v);
+            acc[r] = fmaf(f16_bits_to_f32(w[r].d), v, acc[r]);
+        }
     }
 };
 
@@ -191,7 +217,7 @@ struct FmtQ6K {
 struct FmtQ8_0 {
     static constexpr int TILE = 32;
     static constexpr int CHUNKS = 8;
-    static constexpr int NSUM = 0;
+    static constexpr int NSUM = 1;  // sum of the tile's x: quants are used as q + 128
     struct Row {
         uint4 a, b;
         uint16_t d;
@@ -206,26 +232,35 @@ struct FmtQ8_0 {
         tile = g >> 3;
         chunk = g & 7;
     }
-    __device__ static uint32_t sum_of_chunk(uint32_t) { return 0; }
     __device__ static void load(Row &w, const RowBase &rb, uint32_t tile) {
         const uint4 *q = reinterpret_cast<const uint4 *>(rb.qs + (size_t)tile * 32);
         w.a = q[0];
         w.b = q[1];
         w.d = *reinterpret_cast<const uint16_t *>(rb.d + (size_t)tile * 2);
     }
-    __device__ static float dot(const Row &w, const float4 (&x)[CHUNKS], const float (&)[1],
-                                uint32_t) {
-        const uint32_t q[8] = {w.a.x, w.a.y, w.a.z, w.a.w, w.b.x, w.b.y, w.b.z, w.b.w};
-        float acc = 0.f;
+    template <int R>
+    __device__ static void accumulate(const Row (&w)[R], const float4 *xl, const float *s,
+                                      uint32_t, float (&acc)[R]) {
+        float dt[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) dt[r] = 0.f;
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            const float4 xv = x[k];
-            acc = fmaf(sb0(q[k]), xv.x, acc);
-            acc = fmaf(sb1(q[k]), xv.y, acc);
-            acc = fmaf(sb2(q[k]), xv.z, acc);
-            acc = fmaf(sb3(q[k]), xv.w, acc);
+            const float4 xv = xl[k * 64];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const uint32_t q = k < 4 ? (&w[r].a.x)[k] : (&w[r].b.x)[k - 4];
+                const uint32_t u = opaque(q ^ 0x80808080u);  // q + 128 per byte, unsigned
+                dt[r] = fmaf(ub0(u), xv.x, dt[r]);
+                dt[r] = fmaf(ub1(u), xv.y, dt[r]);
+                dt[r] = fmaf(ub2(u), xv.z, dt[r]);
+                dt[r] = fmaf(ub3(u), xv.w, dt[r]);
+            }
         }
-        return f16_bits_to_f32(w.d) * acc;
+        const float s0 = s[0];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            acc[r] = fmaf(f16_bits_to_f32(w[r].d), fmaf(-128.f, s0, dt[r]), acc[r]);
     }
 };
 
@@ -235,10 +270,41 @@ __device__ __forceinline__ uint32_t lds_slot(uint32_t tile, uint32_t chunk) {
     return ((tile >> 6) * F::CHUNKS + chunk) * 64 + (tile & 63);
 }
 
+// Loads the tiles of the R rows of row-group `g` for tile index `tile`.
 template <class F, int R>
-__global__ __launch_bounds__(256) void gemv_quant_kernel(const GemvParams p) {
+__device__ __forceinline__ void load_group(typename F::Row (&w)[R], const GemvParams &p,
+                                           uint32_t g, uint32_t tile) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t row = min(g * R + r, p.nrows - 1);
+        F::load(w[r], F::row_base(p, row), tile);
+    }
+}
+
+template <int R>
+__device__ __forceinline__ void reduce_and_store(const GemvParams &p, uint32_t g,
+                                                 const float (&acc)[R], uint32_t lane) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float total = wave_sum(acc[r]);
+        const uint32_t row = g * R + r;
+        if (lane == 0 && row < p.nrows) {
+            float v = total;
+            if (p.bias) v += p.bias[row];
+            if (p.accumulate) v += p.out[row];
+            p.out[row] = v;
+        }
+    }
+}
+
+// Persistent kernel: the grid is sized to the machine, every wave walks over
+// row-groups (R consecutive rows) with stride = total waves.  The (group, step)
+// pairs of a wave form one sequence that is software-pipelined D deep: D
+// register sets hold weights in flight (a ring, unrolled so that no register
+// copies are needed), so D-1 loads stay outstanding while one set is consumed.
+template <class F, int R, int D, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_quant_kernel(const GemvParams p) {
     extern __shared__ float4 smem[];
-    constexpr int NS = F::NSUM > 0 ? F::NSUM : 1;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t nwaves = blockDim.x >> 6;
     const uint32_t ntiles = p.ncols / F::TILE;
@@ -246,85 +312,379 @@ __global__ __launch_bounds__(256) void gemv_quant_kernel(const GemvParams p) {
     const uint32_t ntiles_pad = nsteps << 6;
     float *sums = reinterpret_cast<float *>(smem + (size_t)ntiles_pad * F::CHUNKS);
 
-    const uint32_t row0 = (blockIdx.x * nwaves + wave) * R;
+    const uint32_t gw = blockIdx.x * nwaves + wave, GW = gridDim.x * nwaves;
+    const uint32_t ngroups = (p.nrows + R - 1) / R;
+    // this wave's sequence: groups gw, gw+GW, ... ; nsteps steps each
+    const uint32_t my_groups = gw < ngroups ? (ngroups - gw + GW - 1) / GW : 0;
+    const uint32_t n_it = my_groups * nsteps;
 
-    // First step's weights are requested before x is staged: they do not depend on it.
-    typename F::RowBase rb[R];
-    typename F::Row w[R];
+    // Requests for the first D (group, step) pairs go out before x is staged:
+    // they do not depend on it.
+    typename F::Row w[D][R];
+    uint32_t lg = gw, ls = 0;  // (group, step) of the next load
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const uint32_t row = min(row0 + r, p.nrows - 1);
-        rb[r] = F::row_base(p, row);
-    }
-    if (lane < ntiles) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) F::load(w[r], rb[r], lane);
+    for (int d = 0; d < D; ++d) {
+        if ((uint32_t)d < n_it) {
+            const uint32_t tile = ls * 64 + lane;
+            if (tile < ntiles) load_group<F, R>(w[d], p, lg, tile);
+            if (++ls == nsteps) {
+                ls = 0;
+                lg += GW;
+            }
+        }
     }
 
-    // Stage x.
+    // Stage x (lane-transposed) and the per-tile sums of x.
     const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
     const uint32_t n4 = p.ncols >> 2;
-    for (uint32_t g = tid; g < n4; g += blockDim.x) {
+    for (uint32_t g4 = tid; g4 < n4; g4 += blockDim.x) {
         uint32_t tile, chunk;
-        F::map(g, tile, chunk);
-        smem[lds_slot<F>(tile, chunk)] = x4[g];
+        F::map(g4, tile, chunk);
+        smem[lds_slot<F>(tile, chunk)] = x4[g4];
     }
     __syncthreads();
-    if (F::NSUM > 0) {
-        constexpr int CPS = F::CHUNKS / NS;  // chunks per sum
-        for (uint32_t t = tid; t < ntiles * NS; t += blockDim.x) {
+    {
+        constexpr int CPS = F::CHUNKS / F::NSUM;  // chunks per sum
+        for (uint32_t t = tid; t < ntiles * F::NSUM; t += blockDim.x) {
             const uint32_t tile = t % ntiles, si = t / ntiles;
-            float acc = 0.f;
+            float a = 0.f;
 #pragma unroll
             for (int c = 0; c < CPS; ++c) {
                 const float4 v = smem[lds_slot<F>(tile, si * CPS + c)];
-                acc += (v.x + v.y) + (v.z + v.w);
+                a += (v.x + v.y) + (v.z + v.w);
             }
-            sums[si * ntiles_pad + tile] = acc;
+            sums[tile * F::NSUM + si] = a;
         }
         __syncthreads();
     }
+    if (n_it == 0) return;
 
+    uint32_t g = gw, step = 0;  // (group, step) being computed
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    for (uint32_t base = 0; base < n_it; base += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const uint32_t it = base + d;
+            if (it < n_it) {
+                const uint32_t tile = step * 64 + lane;
+                if (tile < ntiles)
+                    F::template accumulate<R>(w[d], smem + (size_t)step * F::CHUNKS * 64 + lane,
+                                              sums + (size_t)tile * F::NSUM, tile, acc);
+                if (++step == nsteps) {
+                    reduce_and_store<R>(p, g, acc, lane);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+                    step = 0;
+                    g += GW;
+                }
+                // refill this register set with the pair D positions ahead
+                if (it + D < n_it) {
+                    const uint32_t tile_n = ls * 64 + lane;
+                    if (tile_n < ntiles) load_group<F, R>(w[d], p, lg, tile_n);
+                    if (++ls == nsteps) {
+                        ls = 0;
+                        lg += GW;
+                    }
+                }
+            }
+        }
+    }
+}
 
-    for (uint32_t step = 0; step < nsteps; ++step) {
-        const uint32_t tile = step * 64 + lane;
-        const bool active = tile < ntiles;
-        // Prefetch the next step's weights while this step is computed.
-        typename F::Row wn[R];
-        const uint32_t tile_n = tile + 64;
-        const bool active_n = (step + 1 < nsteps) && tile_n < ntiles;
-        if (active_n) {
+// =========================================================================
+// Integer-dot path (default).  The fp32 path above spends ~3 VALU operations
+// per weight element (convert, multiply-add, unpack), which makes the 4-bit
+// formats issue-bound on the four SIMD16 units of a CU well below HBM speed.
+// Here the activation vector is staged once per workgroup as 16-bit block
+// fixed point: per block of XB elements a scale s = max|x| / 32512 and
+// X = round(x / s), stored as two int8 planes X = 256*hi + lo (hi in
+// [-127,127], lo in [-128,127]).  Weights are unpacked to bytes and multiplied
+// with v_dot4c_i32_i8 (four exact integer MACs per lane-operation); the two
+// int32 partial sums are recombined as 256*hi + lo and scaled once per
+// sub-block in fp32.  The rounding of x is at most 2^-16 of the block maximum
+// per element (about 3e-5 of a block's RMS), i.e. ~30x inside the 1e-3
+// tolerance of the GEMV.  The result is the product of the exactly dequantized
+// weights with the rounded activation vector: the block sums used for the
+// minima / offsets are sums of the rounded values too.  Everything after the
+// sub-block dot product is fp32.
+// =========================================================================
+
+__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float v) {
+    return fmaxf(v, dpp_f32<CTRL>(v));
+}
+
+// --- formats: TILE elements per lane, XB elements per activation block ------
+struct IFmtQ4K {
+    using W = FmtQ4K;
+    static constexpr int TILE = 64, XB = 32, NXB = 2, NSUM = 2;
+    // element index e of x -> tile, element within tile, block within tile
+    __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
+        tile = e >> 6;
+        local = e & 63;
+        xb = local >> 5;
+    }
+    template <int R>
+    __device__ static void accumulate(const W::Row (&w)[R], const uint4 *xq, const float *meta,
+                                      uint32_t tile, float (&acc)[R]) {
+        // xq: this lane's slot of chunk 0 of the hi plane; chunk c at xq[c*64], lo plane 4 chunks on
+        uint4 xh[4], xl[4];
 #pragma unroll
-            for (int r = 0; r < R; ++r) F::load(wn[r], rb[r], tile_n);
+        for (int c = 0; c < 4; ++c) {
+            xh[c] = xq[c * 64];
+            xl[c] = xq[(4 + c) * 64];
         }
-        if (active) {
-            float4 xr[F::CHUNKS];
+        const float4 mt = *reinterpret_cast<const float4 *>(meta);  // s0, s1, S0, S1
+        const uint32_t j = tile & 3;
+        const uint32_t sh = (j & 1u) * 16u;
 #pragma unroll
-            for (int c = 0; c < F::CHUNKS; ++c) xr[c] = smem[(step * F::CHUNKS + c) * 64 + lane];
-            float s[NS];
+        for (int r = 0; r < R; ++r) {
+            int hlo = 0, llo = 0, hhi = 0, lhi = 0;
 #pragma unroll
-            for (int k = 0; k < NS; ++k) s[k] = F::NSUM > 0 ? sums[k * ntiles_pad + tile] : 0.f;
-#pragma unroll
-            for (int r = 0; r < R; ++r) acc[r] += F::dot(w[r], xr, s, tile);
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t q = k < 4 ? (&w[r].qa.x)[k] : (&w[r].qb.x)[k - 4];
+                const uint32_t lo = q & 0x0f0f0f0fu, hi = (q >> 4) & 0x0f0f0f0fu;
+                hlo = sdot4(lo, (&xh[k >> 2].x)[k & 3], hlo);
+                llo = sdot4(lo, (&xl[k >> 2].x)[k & 3], llo);
+                hhi = sdot4(hi, (&xh[2 + (k >> 2)].x)[k & 3], hhi);
+                lhi = sdot4(hi, (&xl[2 + (k >> 2)].x)[k & 3], lhi);
+            }
+            const float flo = (float)((hlo << 8) + llo) * mt.x;
+            const float fhi = (float)((hhi << 8) + lhi) * mt.y;
+            const float d = f16_bits_to_f32((uint16_t)(w[r].hdr.x & 0xffffu));
+            const float dmin = f16_bits_to_f32((uint16_t)(w[r].hdr.x >> 16));
+            const uint32_t a = (w[r].hdr.y >> sh) & 0xffffu, b = (w[r].hdr.z >> sh) & 0xffffu,
+                           c = (w[r].hdr.w >> sh) & 0xffffu;
+            uint32_t sc2, m2;
+            if (j < 2) {
+                sc2 = a & 0x3f3fu;
+                m2 = b & 0x3f3fu;
+            } else {
+                sc2 = (c & 0x0f0fu) | ((a >> 2) & 0x3030u);
+                m2 = ((c >> 4) & 0x0f0fu) | ((b >> 2) & 0x3030u);
+            }
+            float v = (d * ub0(sc2)) * flo;
+            v = fmaf(d * ub1(sc2), fhi, v);
+            v = fmaf(-dmin, fmaf(ub0(m2), mt.z, ub1(m2) * mt.w), v);
+            acc[r] += v;
         }
-        if (active_n) {
+    }
+};
+
+struct IFmtQ6K {
+    using W = FmtQ6K;
+    static constexpr int TILE = 64, XB = 16, NXB = 4, NSUM = 4;
+    __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
+        const uint32_t blk = e >> 8, i = (e >> 7) & 1, quarter = (e >> 5) & 3, s = (e >> 4) & 1;
+        tile = blk * 4 + i * 2 + s;
+        xb = quarter;
+        local = quarter * 16 + (e & 15);
+    }
+    template <int R>
+    __device__ static void accumulate(const W::Row (&w)[R], const uint4 *xq, const float *meta,
+                                      uint32_t tile, float (&acc)[R]) {
+        uint4 xh[4], xl[4];  // chunk = quarter
 #pragma unroll
-            for (int r = 0; r < R; ++r) w[r] = wn[r];
+        for (int c = 0; c < 4; ++c) {
+            xh[c] = xq[c * 64];
+            xl[c] = xq[(4 + c) * 64];
+        }
+        const float4 ms = *reinterpret_cast<const float4 *>(meta);      // s of the 4 quarters
+        const float4 mS = *reinterpret_cast<const float4 *>(meta + 4);  // exact sums
+        const uint32_t sb = (tile & 1u) * 8u;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int h1 = 0, l1 = 0, h2 = 0, l2 = 0, h3 = 0, l3 = 0, h4 = 0, l4 = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t L0 = (&w[r].l0.x)[k], L1 = (&w[r].l1.x)[k], H = (&w[r].h.x)[k];
+                const uint32_t q1 = (L0 & 0x0f0f0f0fu) | ((H << 4) & 0x30303030u);
+                const uint32_t q2 = (L1 & 0x0f0f0f0fu) | ((H << 2) & 0x30303030u);
+                const uint32_t q3 = ((L0 >> 4) & 0x0f0f0f0fu) | (H & 0x30303030u);
+                const uint32_t q4 = ((L1 >> 4) & 0x0f0f0f0fu) | ((H >> 2) & 0x30303030u);
+                h1 = sdot4(q1, (&xh[0].x)[k], h1);
+                l1 = sdot4(q1, (&xl[0].x)[k], l1);
+                h2 = sdot4(q2, (&xh[1].x)[k], h2);
+                l2 = sdot4(q2, (&xl[1].x)[k], l2);
+                h3 = sdot4(q3, (&xh[2].x)[k], h3);
+                l3 = sdot4(q3, (&xl[2].x)[k], l3);
+                h4 = sdot4(q4, (&xh[3].x)[k], h4);
+                l4 = sdot4(q4, (&xl[3].x)[k], l4);
+            }
+            const float f1 = fmaf((float)((h1 << 8) + l1), ms.x, -32.f * mS.x);
+            const float f2 = fmaf((float)((h2 << 8) + l2), ms.y, -32.f * mS.y);
+            const float f3 = fmaf((float)((h3 << 8) + l3), ms.z, -32.f * mS.z);
+            const float f4 = fmaf((float)((h4 << 8) + l4), ms.w, -32.f * mS.w);
+            const float sc1 = sb0(w[r].sc.x >> sb), sc2 = sb0(w[r].sc.x >> (sb + 16)),
+                        sc3 = sb0(w[r].sc.y >> sb), sc4 = sb0(w[r].sc.y >> (sb + 16));
+            float v = sc1 * f1;
+            v = fmaf(sc2, f2, v);
+            v = fmaf(sc3, f3, v);
+            v = fmaf(sc4, f4, v);
+            acc[r] = fmaf(f16_bits_to_f32(w[r].d), v, acc[r]);
+        }
+    }
+};
+
+struct IFmtQ8_0 {
+    using W = FmtQ8_0;
+    static constexpr int TILE = 32, XB = 32, NXB = 1, NSUM = 0;
+    __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
+        tile = e >> 5;
+        local = e & 31;
+        xb = 0;
+    }
+    template <int R>
+    __device__ static void accumulate(const W::Row (&w)[R], const uint4 *xq, const float *meta,
+                                      uint32_t, float (&acc)[R]) {
+        uint4 xh[2], xl[2];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            xh[c] = xq[c * 64];
+            xl[c] = xq[(2 + c) * 64];
+        }
+        const float s0 = meta[0];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int h = 0, l = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t q = k < 4 ? (&w[r].a.x)[k] : (&w[r].b.x)[k - 4];
+                h = sdot4(q, (&xh[k >> 2].x)[k & 3], h);
+                l = sdot4(q, (&xl[k >> 2].x)[k & 3], l);
+            }
+            acc[r] = fmaf(f16_bits_to_f32(w[r].d) * s0, (float)((h << 8) + l), acc[r]);
+        }
+    }
+};
+
+// LDS: uint4 xq[step][plane(2)][chunk(PCH)][lane(64)], then float meta[tile][MF].
+template <class F, int R, int D, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p) {
+    using WF = typename F::W;
+    constexpr int PCH = F::TILE / 16;         // 16-byte chunks per plane per tile
+    constexpr int MF = F::NXB + F::NSUM;      // floats of meta per tile
+    constexpr int LPB = F::XB / 4;            // lanes (float4) per activation block
+    extern __shared__ float4 smem4[];
+    uint4 *xq = reinterpret_cast<uint4 *>(smem4);
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t nwaves = blockDim.x >> 6;
+    const uint32_t ntiles = p.ncols / F::TILE;
+    const uint32_t nsteps = (ntiles + 63) >> 6;
+    const uint32_t ntiles_pad = nsteps << 6;
+    float *meta = reinterpret_cast<float *>(xq + (size_t)ntiles_pad * 2 * PCH);
+
+    const uint32_t gw = blockIdx.x * nwaves + wave, GW = gridDim.x * nwaves;
+    const uint32_t ngroups = (p.nrows + R - 1) / R;
+    const uint32_t my_groups = gw < ngroups ? (ngroups - gw + GW - 1) / GW : 0;
+    const uint32_t n_it = my_groups * nsteps;
+
+    typename WF::Row w[D][R];
+    uint32_t lg = gw, ls = 0;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        if ((uint32_t)d < n_it) {
+            const uint32_t tile = ls * 64 + lane;
+            if (tile < ntiles) load_group<WF, R>(w[d], p, lg, tile);
+            if (++ls == nsteps) {
+                ls = 0;
+                lg += GW;
+            }
         }
     }
 
+    // Stage x as 16-bit block fixed point (two int8 planes) + per-block scale and sum.
+    if (!(p.debug & 1)) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
+        const uint32_t n4 = p.ncols >> 2;
+        uint32_t *xq32 = reinterpret_cast<uint32_t *>(xq);
+        for (uint32_t g4 = tid; g4 < n4; g4 += blockDim.x) {
+            const float4 v = x4[g4];
+            float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+            float sum;
+            amax = dpp_max<0xB1>(amax);
+            amax = dpp_max<0x4E>(amax);
+            if (LPB == 8) amax = dpp_max<0x141>(amax);
+            const float inv = amax > 0.f ? 32512.f / amax : 0.f;
+            const int X0 = __float2int_rn(v.x * inv), X1 = __float2int_rn(v.y * inv),
+                      X2 = __float2int_rn(v.z * inv), X3 = __float2int_rn(v.w * inv);
+            // block sum of the *rounded* activations, so that the minima / offset terms
+            // see exactly the same vector as the dot products (exact in fp32: |sum| < 2^21)
+            sum = (float)((X0 + X1) + (X2 + X3));
+            sum += dpp_f32<0xB1>(sum);
+            sum += dpp_f32<0x4E>(sum);
+            if (LPB == 8) sum += dpp_f32<0x141>(sum);
+            sum *= amax * (1.0f / 32512.f);
+            const int l0 = ((X0 + 128) & 255) - 128, l1 = ((X1 + 128) & 255) - 128,
+                      l2 = ((X2 + 128) & 255) - 128, l3 = ((X3 + 128) & 255) - 128;
+            const int h0 = (X0 - l0) >> 8, h1 = (X1 - l1) >> 8, h2 = (X2 - l2) >> 8,
+                      h3 = (X3 - l3) >> 8;
+            const uint32_t hi = (uint32_t)(h0 & 255) | ((uint32_t)(h1 & 255) << 8) |
+                                ((uint32_t)(h2 & 255) << 16) | ((uint32_t)(h3 & 255) << 24);
+            const uint32_t lo = (uint32_t)(l0 & 255) | ((uint32_t)(l1 & 255) << 8) |
+                                ((uint32_t)(l2 & 255) << 16) | ((uint32_t)(l3 & 255) << 24);
+            uint32_t tile, local, xb;
+            F::locate(g4 * 4, tile, local, xb);
+            const uint32_t dl = local >> 2, chunk = dl >> 2, sub = dl & 3;
+            const uint32_t slot = ((tile >> 6) * 2 * PCH + chunk) * 64 + (tile & 63);
+            xq32[(size_t)slot * 4 + sub] = hi;
+            xq32[(size_t)(slot + PCH * 64) * 4 + sub] = lo;
+            if ((g4 & (LPB - 1)) == 0) {
+                meta[tile * MF + xb] = amax * (1.0f / 32512.f);
+                if (F::NSUM > 0) meta[tile * MF + F::NXB + xb] = sum;
+            }
+        }
+        __syncthreads();
+    }
+    if (n_it == 0) return;
+
+    uint32_t g = gw, step = 0;
+    float acc[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const float total = wave_sum(acc[r]);
-        const uint32_t row = row0 + r;
-        if (lane == 0 && row < p.nrows) {
-            float v = total;
-            if (p.bias) v += p.bias[row];
-            if (p.accumulate) v += p.out[row];
-            p.out[row] = v;
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    for (uint32_t base = 0; base < n_it; base += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const uint32_t it = base + d;
+            if (it < n_it) {
+                const uint32_t tile = step * 64 + lane;
+                if (tile < ntiles) {
+                    if (p.debug & 2) {
+#pragma unroll
+                        for (int r = 0; r < R; ++r) {
+                            const uint32_t *ww = reinterpret_cast<const uint32_t *>(&w[d][r]);
+                            uint32_t xx = 0;
+#pragma unroll
+                            for (int q = 0; q < (int)(sizeof(typename WF::Row) / 4); ++q) xx ^= ww[q];
+                            acc[r] += __uint_as_float(xx & 0x3fffffffu);
+                        }
+                    } else {
+                        F::template accumulate<R>(w[d], xq + (size_t)step * 2 * PCH * 64 + lane,
+                                                  meta + (size_t)tile * MF, tile, acc);
+                    }
+                }
+                if (++step == nsteps) {
+                    reduce_and_store<R>(p, g, acc, lane);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+                    step = 0;
+                    g += GW;
+                }
+                if (it + D < n_it) {
+                    const uint32_t tile_n = ls * 64 + lane;
+                    if (tile_n < ntiles) load_group<WF, R>(w[d], p, lg, tile_n);
+                    if (++ls == nsteps) {
+                        ls = 0;
+                        lg += GW;
+                    }
+                }
+            }
         }
     }
 }
@@ -381,8 +741,114 @@ __global__ __launch_bounds__(256) void gemv_tr_f32_kernel(const float *__restric
     out[j] = acc;
 }
 
-int g_force_r = 0;  // 0 = heuristic
+int g_force_r = 0;      // rows per wave, 0 = heuristic
+int g_force_waves = 0;  // waves per workgroup, 0 = heuristic
+int g_force_depth = 0;  // pipeline depth, 0 = heuristic
+int g_force_wg_per_cu = 0;
+int g_debug_flags = 0;
+int g_f32_activations = 0;  // 1: fp32-activation kernels instead of the integer-dot path
 constexpr size_t kMaxLds = 128 * 1024;
+
+template <class KF, int R, int D, int MAXT>
+int launch_kernel(wgml_ctx *ctx, const GemvParams &p, size_t lds, const void *fn,
+                  void (*kern)(const GemvParams), bool &opted_in, size_t &cached_lds,
+                  int &cached_blocks) {
+    if (lds > 64 * 1024 && !opted_in) {
+        // gfx950 has 160 KB of LDS per CU; above 64 KB a kernel must opt in once.
+        WGML_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)kMaxLds));
+        opted_in = true;
+    }
+    if (cached_lds != lds) {  // workgroups resident per CU for this variant and LDS size
+        int nb = 0;
+        WGML_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fn, MAXT, lds));
+        cached_blocks = nb > 0 ? nb : 1;
+        cached_lds = lds;
+    }
+    int per_cu = cached_blocks;
+    if (g_force_wg_per_cu > 0 && g_force_wg_per_cu < per_cu) per_cu = g_force_wg_per_cu;
+    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
+    const uint32_t nwaves = MAXT / 64;
+    const uint32_t ngroups = (p.nrows + R - 1) / R;
+    // Balanced persistent grid: every wave gets k or k-1 groups, k minimal such
+    // that the grid fits the machine.
+    const uint32_t resident_waves = cu * (uint32_t)per_cu * nwaves;
+    const uint32_t k = (ngroups + resident_waves - 1) / resident_waves;
+    const uint32_t grid = (ngroups + nwaves * k - 1) / (nwaves * k);
+    kern<<<dim3(grid), dim3(MAXT), lds, ctx->stream>>>(p);
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
+template <class F, int R, int D, int MAXT>
+int launch_variant(wgml_ctx *ctx, const GemvParams &p, size_t lds) {
+    static bool opted_in = false;
+    static size_t cached_lds = ~size_t(0);
+    static int cached_blocks = 0;
+    return launch_kernel<F, R, D, MAXT>(ctx, p, lds,
+                                        (const void *)gemv_quant_kernel<F, R, D, MAXT>,
+                                        gemv_quant_kernel<F, R, D, MAXT>, opted_in, cached_lds,
+                                        cached_blocks);
+}
+
+template <class F, int R, int D, int MAXT>
+int launch_variant_i8(wgml_ctx *ctx, const GemvParams &p, size_t lds) {
+    static bool opted_in = false;
+    static size_t cached_lds = ~size_t(0);
+    static int cached_blocks = 0;
+    return launch_kernel<F, R, D, MAXT>(ctx, p, lds,
+                                        (const void *)gemv_quant_i8_kernel<F, R, D, MAXT>,
+                                        gemv_quant_i8_kernel<F, R, D, MAXT>, opted_in, cached_lds,
+                                        cached_blocks);
+}
+
+template <class F, int R, int D>
+int launch_rd_i8(wgml_ctx *ctx, const GemvParams &p, size_t lds, int waves) {
+    switch (waves) {
+    case 16: return launch_variant_i8<F, R, D, 1024>(ctx, p, lds);
+    case 8: return launch_variant_i8<F, R, D, 512>(ctx, p, lds);
+    default: return launch_variant_i8<F, R, D, 256>(ctx, p, lds);
+    }
+}
+
+template <class F>
+int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
+    constexpr int PCH = F::TILE / 16, MF = F::NXB + F::NSUM;
+    const uint32_t ntiles = p.ncols / F::TILE;
+    const uint32_t ntiles_pad = ((ntiles + 63) / 64) * 64;
+    const size_t lds = (size_t)ntiles_pad * 2 * PCH * 16 + (size_t)ntiles_pad * MF * 4;
+    if (lds > kMaxLds)
+        return set_error(WGML_E_UNSUPPORTED,
+                         "gemv_quant: %u columns need %zu bytes of LDS (limit %zu)", p.ncols, lds,
+                         kMaxLds);
+    // Defaults from a sweep over the Llama-2-7B shapes on MI355X: one row per
+    // wave and 16-wave workgroups (x is staged once per 16 rows in flight);
+    // Q8_0 rows span more steps, so long rows get a deeper pipeline.
+    int R = g_force_r, waves = g_force_waves, depth = g_force_depth;
+    const bool q8 = F::TILE == 32;
+    if (!R) R = 1;
+    if (!waves) waves = (q8 && p.ncols <= 8192) ? 8 : 16;
+    if (!depth) depth = (q8 && p.ncols > 8192) ? 4 : 2;
+    if (R == 2) {
+        if (depth >= 3) return launch_rd_i8<F, 2, 3>(ctx, p, lds, waves);
+        return launch_rd_i8<F, 2, 2>(ctx, p, lds, waves);
+    }
+    if (depth >= 4) return launch_rd_i8<F, 1, 4>(ctx, p, lds, waves);
+    if (depth == 3) return launch_rd_i8<F, 1, 3>(ctx, p, lds, waves);
+    return launch_rd_i8<F, 1, 2>(ctx, p, lds, waves);
+}
+
+// fp32-activation path: one configuration per format
+template <class F, int R, int D>
+int launch_rd(wgml_ctx *ctx, const GemvParams &p, size_t lds, int) {
+    return launch_variant<F, R, D, 512>(ctx, p, lds);
+}
+
+template <class F, int R>
+int launch_r(wgml_ctx *ctx, const GemvParams &p, size_t lds, int waves, int) {
+    return launch_rd<F, R, 2>(ctx, p, lds, waves);
+}
 
 template <class F>
 int launch_fmt(wgml_ctx *ctx, const GemvParams &p) {
@@ -394,42 +860,12 @@ int launch_fmt(wgml_ctx *ctx, const GemvParams &p) {
         return set_error(WGML_E_UNSUPPORTED,
                          "gemv_quant: %u columns need %zu bytes of LDS (limit %zu)", p.ncols, lds,
                          kMaxLds);
-    if (lds > 64 * 1024) {
-        // gfx950 has 160 KB of LDS per CU; above 64 KB a kernel must opt in once.
-        static bool opted_in = false;
-        if (!opted_in) {
-            WGML_CHECK_HIP(hipFuncSetAttribute((const void *)gemv_quant_kernel<F, 1>,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               (int)kMaxLds));
-            WGML_CHECK_HIP(hipFuncSetAttribute((const void *)gemv_quant_kernel<F, 2>,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               (int)kMaxLds));
-            WGML_CHECK_HIP(hipFuncSetAttribute((const void *)gemv_quant_kernel<F, 4>,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               (int)kMaxLds));
-            opted_in = true;
-        }
-    }
-    const int waves = 4;
-    // Rows per wave: more rows amortise the LDS reads of x, fewer rows give more
-    // waves to hide HBM latency when the matrix has few rows.
-    int R = g_force_r;
-    if (!R) {
-        const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
-        if (p.nrows >= cu * 8 * 4) R = 4;
-        else if (p.nrows >= cu * 8 * 2) R = 2;
-        else R = 1;
-    }
-    const uint32_t rows_per_wg = waves * R;
-    const dim3 grid((p.nrows + rows_per_wg - 1) / rows_per_wg), block(waves * 64);
-    switch (R) {
-    case 4: gemv_quant_kernel<F, 4><<<grid, block, lds, ctx->stream>>>(p); break;
-    case 2: gemv_quant_kernel<F, 2><<<grid, block, lds, ctx->stream>>>(p); break;
-    default: gemv_quant_kernel<F, 1><<<grid, block, lds, ctx->stream>>>(p); break;
-    }
-    WGML_CHECK_LAUNCH();
-    ctx->launches++;
-    return WGML_OK;
+    int R = g_force_r, waves = g_force_waves, depth = g_force_depth;
+    if (!R) R = 1;
+    if (!waves) waves = 8;
+    if (!depth) depth = 2;
+    (void)R;
+    return launch_r<F, 1>(ctx, p, lds, waves, depth);
 }
 
 }  // namespace
@@ -480,6 +916,15 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
     p.nrows = m->nrows;
     p.ncols = m->ncols;
     p.accumulate = ep.accumulate;
+    p.debug = g_debug_flags;
+    if (!g_f32_activations) {
+        switch (m->type) {
+        case WGML_Q4_K: return launch_fmt_i8<IFmtQ4K>(ctx, p);
+        case WGML_Q6_K: return launch_fmt_i8<IFmtQ6K>(ctx, p);
+        case WGML_Q8_0: return launch_fmt_i8<IFmtQ8_0>(ctx, p);
+        default: break;
+        }
+    }
     switch (m->type) {
     case WGML_Q4_K: return launch_fmt<FmtQ4K>(ctx, p);
     case WGML_Q6_K: return launch_fmt<FmtQ6K>(ctx, p);
@@ -492,11 +937,36 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
 
 extern "C" {
 
-// Debug knob for kernel sweeps: rows per wave of the quantized GEMV (0 = heuristic).
+// Debug knobs for kernel sweeps (0 = heuristic): rows per wave, waves per
+// workgroup and a cap on resident workgroups per CU of the quantized GEMV.
 WGML_API int wgml_debug_set_gemv_rows_per_wave(int r) {
-    WGML_REQUIRE(r == 0 || r == 1 || r == 2 || r == 4,
-                 "wgml_debug_set_gemv_rows_per_wave: %d not in {0,1,2,4}", r);
+    WGML_REQUIRE(r == 0 || r == 1 || r == 2,
+                 "wgml_debug_set_gemv_rows_per_wave: %d not in {0,1,2}", r);
     g_force_r = r;
+    return WGML_OK;
+}
+WGML_API int wgml_debug_set_gemv_flags(int f) {
+    g_debug_flags = f;
+    return WGML_OK;
+}
+// 1 selects the fp32-activation GEMV kernels, 0 (default) the integer-dot path.
+WGML_API int wgml_debug_set_gemv_f32_activations(int on) {
+    g_f32_activations = on ? 1 : 0;
+    return WGML_OK;
+}
+WGML_API int wgml_debug_set_gemv_config(int rows_per_wave, int waves_per_wg, int wg_per_cu,
+                                        int depth) {
+    WGML_REQUIRE(rows_per_wave == 0 || rows_per_wave == 1 || rows_per_wave == 2,
+                 "wgml_debug_set_gemv_config: rows_per_wave %d not in {0,1,2}", rows_per_wave);
+    WGML_REQUIRE(depth == 0 || (depth >= 2 && depth <= 4),
+                 "wgml_debug_set_gemv_config: depth %d not in {0,2,3,4}", depth);
+    g_force_depth = depth;
+    WGML_REQUIRE(waves_per_wg == 0 || waves_per_wg == 4 || waves_per_wg == 8 || waves_per_wg == 16,
+                 "wgml_debug_set_gemv_config: waves_per_wg %d not in {0,4,8,16}", waves_per_wg);
+    WGML_REQUIRE(wg_per_cu >= 0, "wgml_debug_set_gemv_config: negative wg_per_cu");
+    g_force_r = rows_per_wave;
+    g_force_waves = waves_per_wg;
+    g_force_wg_per_cu = wg_per_cu;
     return WGML_OK;
 }
 
