@@ -244,8 +244,9 @@ WGML_API int wgml_llama2_read_logits(wgml_llama2 *m, float *host_out);
  * (chat_llama2.rs:51-153, wgml-chat/src/sampler.rs:91-111): positions
  * 0..n_total-1; position p consumes prompt[p] while p < n_prompt, else the
  * arg-max of the previous step.  out_tokens[p] receives the arg-max after
- * position p (n_total entries).  The arg-max runs on the device; only the
- * 4-byte index crosses to the host. */
+ * position p (n_total entries).  Sampling and the loop bookkeeping run on the
+ * device: one recorded step (a HIP graph) is replayed per token and the host
+ * synchronises once, at the end. */
 WGML_API int wgml_llama2_generate_greedy(wgml_llama2 *m, const uint32_t *prompt,
                                          uint32_t n_prompt, uint32_t n_total,
                                          uint32_t *out_tokens);
@@ -253,6 +254,11 @@ WGML_API int wgml_llama2_generate_greedy(wgml_llama2 *m, const uint32_t *prompt,
  * for positions < start_pos; first consumed token is `first_token`. */
 WGML_API int wgml_llama2_decode_greedy(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos,
                                        uint32_t n_steps, uint32_t *out_tokens);
+/* The same loop with a blocking read-back of the sampled token after every
+ * step, as the reference's chat loop does (chat_llama2.rs:205-220). */
+WGML_API int wgml_llama2_decode_greedy_sync(wgml_llama2 *m, uint32_t first_token,
+                                            uint32_t start_pos, uint32_t n_steps,
+                                            uint32_t *out_tokens);
 /* Direct KV-cache access (tests; pre-filled long-context runs). which: 0 = key,
  * 1 = value; `n_pos` positions starting at `first_pos`, kv_dim floats each. */
 WGML_API int wgml_llama2_kv_upload(wgml_llama2 *m, uint32_t layer, int which, uint32_t first_pos,
@@ -262,7 +268,9 @@ WGML_API int wgml_llama2_kv_download(wgml_llama2 *m, uint32_t layer, int which,
 /* Number of kernel launches one forward enqueues (diagnostics). */
 WGML_API int wgml_llama2_launches_per_token(const wgml_llama2 *m);
 /* 0: one launch per reference op (mirrors Llama2::dispatch one to one);
- * 1 (default): fused kernels.  Both give the same results to fp32 rounding. */
+ * 1: bias and residual adds folded into the GEMV epilogues; 2 (default): also
+ * every RMSNorm folded into the GEMVs that consume it.  All levels give the
+ * same results to fp32 rounding. */
 WGML_API int wgml_llama2_set_fusion(wgml_llama2 *m, int level);
 
 /* ---- GPT-2: Gpt2 / Gpt2State / Gpt2Weights -------------------------------- */

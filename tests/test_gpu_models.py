@@ -36,7 +36,7 @@ def spice(w, cfg, seed, biases):
 
 @pytest.mark.parametrize("scheme", ["q8_0", "q4_k", "q6_k", "q4_k_m", "f32"])
 @pytest.mark.parametrize("model_type", [LlamaModelType.Llama, LlamaModelType.Qwen2])
-@pytest.mark.parametrize("fusion", [0, 1])
+@pytest.mark.parametrize("fusion", [0, 1, 2, 3])
 def test_llama_micro_logits_and_kv(gpu, scheme, model_type, fusion):
     w = synth_llama(MICRO, seed=21, scheme=scheme)
     spice(w, MICRO, 5, biases=model_type == LlamaModelType.Qwen2)
@@ -68,10 +68,30 @@ def test_tiny_llama_greedy_tokens_identical(gpu):
     print(f"top-2 logit margin: min {margins.min():.3e}, median {np.median(margins):.3e}; "
           f"{m.launches_per_token()} launches/token")
     assert np.array_equal(got, want)
-    # and once more without the fused epilogues
+    # and once more without any fusion (one launch per reference op)
     m2 = Llama2(gpu, cfg).load(w)
     m2.set_fusion(0)
     assert np.array_equal(m2.generate_greedy(prompt, n_total), want)
+    # the recorded loop (device-side sampling, no host round trip) and the loop that reads
+    # every token back must agree, from any start position, and be repeatable
+    a = m.decode_greedy(int(want[15]), 16, 64)
+    b = m.decode_greedy_sync(int(want[15]), 16, 64)
+    assert np.array_equal(a, want[16:80]) and np.array_equal(b, want[16:80])
+    assert np.array_equal(m.decode_greedy(int(want[15]), 16, 64), a)
+
+
+@pytest.mark.parametrize("model_type", [LlamaModelType.Llama, LlamaModelType.Qwen2])
+def test_llama_recorded_loop_matches_oracle(gpu, model_type):
+    # grouped-query micro model with biases: the recorded step must handle the
+    # position-dependent KV-cache column, RoPE variant and forced prompt tokens
+    w = synth_llama(MICRO, seed=31, scheme="q4_k_m")
+    spice(w, MICRO, 6, biases=model_type == LlamaModelType.Qwen2)
+    prompt = W.prompt_tokens(31, 5, MICRO.vocab_size)
+    want, _ = orc.Llama2(w, rope_variant=model_type).generate_greedy(prompt, MICRO.seq_len)
+    for fusion in (0, 1, 2, 3):
+        m = Llama2(gpu, MICRO, model_type).load(w)
+        m.set_fusion(fusion)
+        assert np.array_equal(m.generate_greedy(prompt, MICRO.seq_len), want), fusion
 
 
 def test_llama_decode_from_uploaded_kv(gpu):

@@ -180,8 +180,9 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnArgs a, uint3
 
 int ensure_ws(wgml_ctx *ctx, size_t bytes) {
     if (bytes <= ctx->attn_ws_bytes) return WGML_OK;
-    WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
-    if (ctx->attn_ws) WGML_CHECK_HIP(hipFree(ctx->attn_ws));
+    // The old buffer is kept until the context goes: recorded launches (HIP graphs)
+    // may still point at it, and it is large enough for the plans they were made for.
+    if (ctx->attn_ws) ctx->retired.push_back(ctx->attn_ws);
     ctx->attn_ws = nullptr;
     ctx->attn_ws_bytes = 0;
     hipError_t e = hipMalloc((void **)&ctx->attn_ws, bytes);
@@ -212,24 +213,50 @@ namespace wgml {
 
 // `plan_positions`: the number of positions the grid is sized for (pos+1 for a
 // one-off launch, seq_len when the launch is replayed for growing positions).
-int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
-                             uint32_t plan_positions, const float *q, const float *kc,
-                             const float *vc, float *att, float *xb) {
+struct AttnPlan {
+    int nv, km;
+    uint32_t groups, chunk, n_wg_y, hsp;
+};
+
+static int make_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions,
+                     AttnPlan &pl) {
     const uint32_t hs = p.head_size;
     if (hs == 0 || hs > 256)
         return set_error(WGML_E_UNSUPPORTED, "attention: head_size %u not in 1..256", hs);
-    const int nv = (int)((hs + 63) / 64);
-    int km = 1;
-    if (p.kv_mul == 2 || p.kv_mul == 4 || p.kv_mul == 8) km = (int)p.kv_mul;
+    pl.nv = (int)((hs + 63) / 64);
+    pl.km = 1;
+    if (p.kv_mul == 2 || p.kv_mul == 4 || p.kv_mul == 8) pl.km = (int)p.kv_mul;
     // LDS: WAVES*km*(nv*64+2) floats; keep it modest for large heads
-    while (km > 1 && (size_t)WAVES * km * (nv * 64 + 2) * 4 > 48 * 1024) km >>= 1;
-    const uint32_t groups = p.n_heads / km;
+    while (pl.km > 1 && (size_t)WAVES * pl.km * (pl.nv * 64 + 2) * 4 > 48 * 1024) pl.km >>= 1;
+    pl.groups = p.n_heads / pl.km;
     const uint32_t target_waves = 8u * (ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u);
-    uint32_t chunk = (uint32_t)(((uint64_t)plan_positions * groups + target_waves - 1) / target_waves);
+    uint32_t chunk =
+        (uint32_t)(((uint64_t)plan_positions * pl.groups + target_waves - 1) / target_waves);
     chunk = ((chunk + 7) / 8) * 8;
     if (chunk < 16) chunk = 16;
+    pl.chunk = chunk;
     const uint32_t n_chunks = (plan_positions + chunk - 1) / chunk;
-    const uint32_t n_wg_y = (n_chunks + WAVES - 1) / WAVES;
+    pl.n_wg_y = (n_chunks + WAVES - 1) / WAVES;
+    pl.hsp = (uint32_t)pl.nv * 64;
+    return WGML_OK;
+}
+
+// Sizes the partials workspace for a launch planned for `plan_positions`
+// (so that no allocation happens while launches are being recorded).
+int reserve_attention_workspace(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions) {
+    AttnPlan pl;
+    WGML_TRY(make_plan(ctx, p, plan_positions, pl));
+    return ensure_ws(ctx, (size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4);
+}
+
+int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
+                             uint32_t plan_positions, const float *q, const float *kc,
+                             const float *vc, float *att, float *xb) {
+    AttnPlan pl;
+    WGML_TRY(make_plan(ctx, p, plan_positions, pl));
+    const uint32_t hs = p.head_size;
+    const int nv = pl.nv, km = pl.km;
+    const uint32_t groups = pl.groups, chunk = pl.chunk, n_wg_y = pl.n_wg_y;
 
     AttnArgs a;
     a.q = q;
@@ -247,7 +274,7 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
     a.n_wg_y = n_wg_y;
     a.direct = (n_wg_y == 1 && att == nullptr) ? 1 : 0;
     a.ws = nullptr;
-    const uint32_t hsp = (uint32_t)nv * 64;
+    const uint32_t hsp = pl.hsp;
     if (!a.direct) {
         WGML_TRY(ensure_ws(ctx, (size_t)p.n_heads * n_wg_y * (2 + hsp) * 4));
         a.ws = ctx->attn_ws;

@@ -22,7 +22,7 @@ int wgml_bench_gemv_quant(wgml_ctx *ctx, const wgml_qmat *const *mats, uint32_t 
     }
     float *po = view_ptr(out);
     const float *pv = view_ptr(v);
-    if (!use_graph) {
+    if (!use_graph || graphs_disabled()) {
         WGML_CHECK_HIP(hipEventRecord(ctx->ev_start, ctx->stream));
         for (uint32_t i = 0; i < iters; ++i)
             WGML_TRY(launch_gemv_quant(ctx, po, mats[i % n_mats], pv, GemvEpilogue{}));

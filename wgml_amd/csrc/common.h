@@ -54,6 +54,7 @@ struct wgml_ctx {
     // scratch for split attention partials, grown on demand
     float *attn_ws = nullptr;
     size_t attn_ws_bytes = 0;
+    std::vector<void *> retired;  // outgrown workspaces, freed with the context
     uint64_t launches = 0;  // kernels enqueued so far (diagnostics)
     // Buffers, matrices and models keep their context alive: the device objects
     // are torn down when the last reference goes, whatever order handles are
@@ -92,6 +93,11 @@ inline float *view_ptr(const wgml_view &v) {
     return reinterpret_cast<float *>(v.buf->ptr) + v.offset;
 }
 
+// True when the environment variable WGML_DISABLE_GRAPHS is set to a non-zero
+// value: recorded launch sequences are then enqueued launch by launch instead of
+// being replayed as HIP graphs (same kernels, same order; useful under profilers
+// that cannot trace graph launches).
+bool graphs_disabled();
 void ctx_retain(wgml_ctx *ctx);
 void ctx_release(wgml_ctx *ctx);
 
@@ -111,7 +117,39 @@ struct GemvEpilogue {
     // out[r] = acc (+ bias[r]) (+ out[r] if accumulate)
     const float *bias = nullptr;
     int accumulate = 0;
+    // out is displaced by (*dyn_pos) * out_pos_stride floats: lets a recorded launch
+    // write "the KV-cache column of the current position"
+    const uint32_t *dyn_pos = nullptr;
+    uint32_t out_pos_stride = 0;
+    // if norm_w != null the input is RMS-normalised first: v <- (v * rsqrt(mean(v^2) + eps)) * norm_w
+    const float *norm_w = nullptr;
+    float norm_eps = 0.f;
 };
+
+// One launch for up to three quantized matrices that consume the same vector
+// (Q8_0 / Q4_K / Q6_K, formats may differ between the matrices).
+enum { FUSED_PLAIN = 0, FUSED_ROPE = 1, FUSED_SILU = 2 };
+struct FusedGemvJob {
+    const wgml_qmat *a = nullptr;  // the matrix (SILU: the gate matrix)
+    const wgml_qmat *b = nullptr;  // SILU only: the up matrix
+    float *out = nullptr;
+    const float *bias = nullptr;
+    int mode = FUSED_PLAIN;  // ROPE: adjacent-pair rotation of the output rows by pos
+    int accumulate = 0;
+    uint32_t out_pos_stride = 0;  // out += pos * out_pos_stride
+};
+struct FusedGemv {
+    FusedGemvJob jobs[3];
+    int njobs = 0;
+    const float *x = nullptr;
+    const float *norm_w = nullptr;  // optional fused RMSNorm of x
+    float norm_eps = 0.f;
+    DynPos pos{nullptr, 0};
+    uint32_t head_size = 0;
+    float rope_base = 10000.f;
+};
+bool gemv_fused_supported(const wgml_qmat *m);
+int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f);
 
 int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float *v,
                       const GemvEpilogue &ep);
@@ -130,6 +168,13 @@ int launch_silu(wgml_ctx *ctx, float *h1, const float *h2, uint32_t n);
 int launch_unary(wgml_ctx *ctx, int op, float *x, uint32_t n, const float *args4);
 int launch_op_assign(wgml_ctx *ctx, int op, float *a, const float *b, uint32_t n);
 int launch_argmax(wgml_ctx *ctx, const float *v, uint32_t n, uint32_t *d_out);
+// Token-loop state on the device: {pos, token, n_generated, n_prompt}.
+struct DynState {
+    uint32_t pos, token, count, n_prompt;
+};
+int launch_embed(wgml_ctx *ctx, float *x, const float *table, uint32_t dim, DynPos token);
+int launch_argmax_next(wgml_ctx *ctx, const float *v, uint32_t n, DynState *dyn,
+                       const uint32_t *prompt, uint32_t *tokens_out);
 int launch_dequantize(wgml_ctx *ctx, float *out, const wgml_qmat *m);
 
 }  // namespace wgml

@@ -39,6 +39,10 @@ struct GemvParams {
     uint32_t nrows, ncols;
     int accumulate;
     int debug;  // experiments: bit0 skip x staging, bit1 skip the dot products
+    const uint32_t *dyn_pos;  // out += *dyn_pos * out_pos_stride
+    uint32_t out_pos_stride;
+    const float *norm_w;  // optional fused RMSNorm of x
+    float norm_eps;
 };
 
 // Hides a value from the optimizer (no instruction is emitted).  Used on masked
@@ -270,6 +274,31 @@ __device__ __forceinline__ uint32_t lds_slot(uint32_t tile, uint32_t chunk) {
     return ((tile >> 6) * F::CHUNKS + chunk) * 64 + (tile & 63);
 }
 
+// rsqrt(mean(x^2) + eps) over the whole vector, computed by the workgroup
+// (ops/rms_norm.wgsl:36-60 of the reference).  Contains barriers.
+__device__ __forceinline__ float block_rms_scale(const GemvParams &p, float *red) {
+    const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
+    const uint32_t n4 = p.ncols >> 2;
+    float ss = 0.f;
+    for (uint32_t g4 = threadIdx.x; g4 < n4; g4 += blockDim.x) {
+        const float4 v = x4[g4];
+        ss = fmaf(v.x, v.x, ss);
+        ss = fmaf(v.y, v.y, ss);
+        ss = fmaf(v.z, v.z, ss);
+        ss = fmaf(v.w, v.w, ss);
+    }
+    const float total = block_sum(ss, red);
+    return 1.0f / sqrtf(total / (float)p.ncols + p.norm_eps);
+}
+
+__device__ __forceinline__ float4 apply_norm(float4 v, float rms, const float4 w) {
+    v.x = (v.x * rms) * w.x;
+    v.y = (v.y * rms) * w.y;
+    v.z = (v.z * rms) * w.z;
+    v.w = (v.w * rms) * w.w;
+    return v;
+}
+
 // Loads the tiles of the R rows of row-group `g` for tile index `tile`.
 template <class F, int R>
 __device__ __forceinline__ void load_group(typename F::Row (&w)[R], const GemvParams &p,
@@ -289,10 +318,12 @@ __device__ __forceinline__ void reduce_and_store(const GemvParams &p, uint32_t g
         const float total = wave_sum(acc[r]);
         const uint32_t row = g * R + r;
         if (lane == 0 && row < p.nrows) {
+            float *out = p.out;
+            if (p.dyn_pos) out += (size_t)(*p.dyn_pos) * p.out_pos_stride;
             float v = total;
             if (p.bias) v += p.bias[row];
-            if (p.accumulate) v += p.out[row];
-            p.out[row] = v;
+            if (p.accumulate) v += out[row];
+            out[row] = v;
         }
     }
 }
@@ -335,12 +366,18 @@ __global__ __launch_bounds__(MAXT) void gemv_quant_kernel(const GemvParams p) {
     }
 
     // Stage x (lane-transposed) and the per-tile sums of x.
+    __shared__ float red[16];
+    float rms = 1.f;
+    if (p.norm_w) rms = block_rms_scale(p, red);
     const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
+    const float4 *nw4 = reinterpret_cast<const float4 *>(p.norm_w);
     const uint32_t n4 = p.ncols >> 2;
     for (uint32_t g4 = tid; g4 < n4; g4 += blockDim.x) {
         uint32_t tile, chunk;
         F::map(g4, tile, chunk);
-        smem[lds_slot<F>(tile, chunk)] = x4[g4];
+        float4 v = x4[g4];
+        if (p.norm_w) v = apply_norm(v, rms, nw4[g4]);
+        smem[lds_slot<F>(tile, chunk)] = v;
     }
     __syncthreads();
     {
@@ -564,9 +601,31 @@ struct IFmtQ8_0 {
     }
 };
 
+// Row source / sink of a plain single-matrix GEMV: group g = rows g*R .. g*R+R-1.
+struct PlainPolicy {
+    const GemvParams &p;
+    __device__ uint32_t nrows() const { return p.nrows; }
+    template <int R>
+    __device__ uint32_t ngroups() const {
+        return (p.nrows + R - 1) / R;
+    }
+    template <class WF, int R>
+    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t tile) const {
+        load_group<WF, R>(w, p, g, tile);
+    }
+    template <int R>
+    __device__ void store(uint32_t g, const float (&acc)[R], uint32_t lane) const {
+        reduce_and_store<R>(p, g, acc, lane);
+    }
+};
+
+// The body shared by the single-matrix and the fused multi-matrix kernels.  `p`
+// supplies x, ncols, the optional RMSNorm and the debug flags; `pol` the rows.
+// The workgroup is number `wg` of `nwg` working on this matrix.
 // LDS: uint4 xq[step][plane(2)][chunk(PCH)][lane(64)], then float meta[tile][MF].
-template <class F, int R, int D, int MAXT>
-__global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p) {
+template <class F, int R, int D, class Policy>
+__device__ __forceinline__ void gemv_i8_body(const GemvParams &p, const Policy &pol, uint32_t wg,
+                                             uint32_t nwg) {
     using WF = typename F::W;
     constexpr int PCH = F::TILE / 16;         // 16-byte chunks per plane per tile
     constexpr int MF = F::NXB + F::NSUM;      // floats of meta per tile
@@ -580,8 +639,8 @@ __global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p)
     const uint32_t ntiles_pad = nsteps << 6;
     float *meta = reinterpret_cast<float *>(xq + (size_t)ntiles_pad * 2 * PCH);
 
-    const uint32_t gw = blockIdx.x * nwaves + wave, GW = gridDim.x * nwaves;
-    const uint32_t ngroups = (p.nrows + R - 1) / R;
+    const uint32_t gw = wg * nwaves + wave, GW = nwg * nwaves;
+    const uint32_t ngroups = pol.template ngroups<R>();
     const uint32_t my_groups = gw < ngroups ? (ngroups - gw + GW - 1) / GW : 0;
     const uint32_t n_it = my_groups * nsteps;
 
@@ -591,7 +650,7 @@ __global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p)
     for (int d = 0; d < D; ++d) {
         if ((uint32_t)d < n_it) {
             const uint32_t tile = ls * 64 + lane;
-            if (tile < ntiles) load_group<WF, R>(w[d], p, lg, tile);
+            if (tile < ntiles) pol.template load<WF, R>(w[d], lg, tile);
             if (++ls == nsteps) {
                 ls = 0;
                 lg += GW;
@@ -601,11 +660,16 @@ __global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p)
 
     // Stage x as 16-bit block fixed point (two int8 planes) + per-block scale and sum.
     if (!(p.debug & 1)) {
+        __shared__ float red[16];
+        float rms = 1.f;
+        if (p.norm_w) rms = block_rms_scale(p, red);
         const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
+        const float4 *nw4 = reinterpret_cast<const float4 *>(p.norm_w);
         const uint32_t n4 = p.ncols >> 2;
         uint32_t *xq32 = reinterpret_cast<uint32_t *>(xq);
         for (uint32_t g4 = tid; g4 < n4; g4 += blockDim.x) {
-            const float4 v = x4[g4];
+            float4 v = x4[g4];
+            if (p.norm_w) v = apply_norm(v, rms, nw4[g4]);
             float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
             float sum;
             amax = dpp_max<0xB1>(amax);
@@ -670,7 +734,7 @@ __global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p)
                     }
                 }
                 if (++step == nsteps) {
-                    reduce_and_store<R>(p, g, acc, lane);
+                    pol.template store<R>(g, acc, lane);
 #pragma unroll
                     for (int r = 0; r < R; ++r) acc[r] = 0.f;
                     step = 0;
@@ -678,7 +742,7 @@ __global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p)
                 }
                 if (it + D < n_it) {
                     const uint32_t tile_n = ls * 64 + lane;
-                    if (tile_n < ntiles) load_group<WF, R>(w[d], p, lg, tile_n);
+                    if (tile_n < ntiles) pol.template load<WF, R>(w[d], lg, tile_n);
                     if (++ls == nsteps) {
                         ls = 0;
                         lg += GW;
@@ -689,22 +753,143 @@ __global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p)
     }
 }
 
+template <class F, int R, int D, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p) {
+    gemv_i8_body<F, R, D>(p, PlainPolicy{p}, blockIdx.x, gridDim.x);
+}
+
+// ------------------------------------------------------------------------
+// Fused multi-matrix launch.  Up to three matrices that consume the same input
+// vector share one launch (Q, K and V; gate and up): each workgroup works on one
+// of them (so mixed quantization formats are fine: the format decides the
+// workgroup's staging layout and inner loop), and the row pairs of a wave get an
+// epilogue:
+//   PLAIN  out[row] = dot (+ bias) (+ out)
+//   ROPE   the pair (2g, 2g+1) is rotated by the RoPE angle of pair g before it
+//          is stored (ops/rope.wgsl:35-58, adjacent-pair variant)
+//   SILU   the wave holds row g of the gate matrix and row g of the up matrix and
+//          stores up * gate / (1 + exp(-gate))   (ops/silu.wgsl:13-27)
+// Outputs may be displaced by pos * out_pos_stride (KV-cache column of the
+// current position).
+enum { JOB_PLAIN = 0, JOB_ROPE = 1, JOB_SILU = 2 };
+
+struct GemvJob {
+    const uint8_t *a0, *a1, *a2, *a3;  // matrix planes
+    const uint8_t *b0, *b1, *b2, *b3;  // second matrix (SILU: a = gate, b = up)
+    float *out;
+    const float *bias;
+    uint32_t nrows;
+    int type, mode, accumulate;
+    uint32_t out_pos_stride;
+    uint32_t wg_begin, wg_count;  // workgroups assigned to this matrix
+};
+
+struct FusedParams {
+    GemvJob jobs[3];
+    int njobs;
+    const float *x;
+    uint32_t ncols;
+    const float *norm_w;
+    float norm_eps;
+    DynPos pos;
+    uint32_t head_size;
+    float rope_base;
+};
+
+struct JobPolicy {
+    const GemvJob &j;
+    const GemvParams &pa, &pb;  // plane views of the two matrices
+    uint32_t pos, head_size;
+    float rope_base;
+    __device__ uint32_t nrows() const { return j.nrows; }
+    template <int R>
+    __device__ uint32_t ngroups() const {
+        static_assert(R == 2, "fused launches work on row pairs");
+        return j.mode == JOB_SILU ? j.nrows : (j.nrows + 1) / 2;
+    }
+    template <class WF, int R>
+    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t tile) const {
+        if (j.mode == JOB_SILU) {
+            WF::load(w[0], WF::row_base(pa, g), tile);
+            WF::load(w[1], WF::row_base(pb, g), tile);
+        } else {
+            WF::load(w[0], WF::row_base(pa, min(2 * g, j.nrows - 1)), tile);
+            WF::load(w[1], WF::row_base(pa, min(2 * g + 1, j.nrows - 1)), tile);
+        }
+    }
+    template <int R>
+    __device__ void store(uint32_t g, const float (&acc)[R], uint32_t lane) const {
+        float t0 = wave_sum(acc[0]), t1 = wave_sum(acc[1]);
+        float *out = j.out + (size_t)pos * j.out_pos_stride;
+        if (j.mode == JOB_SILU) {
+            if (lane == 0) out[g] = t1 * (t0 / (1.0f + expf(-t0)));
+            return;
+        }
+        const uint32_t r0 = 2 * g, r1 = r0 + 1;
+        if (j.bias) {
+            t0 += j.bias[min(r0, j.nrows - 1)];
+            t1 += j.bias[min(r1, j.nrows - 1)];
+        }
+        if (j.mode == JOB_ROPE) {
+            const float head_dim = (float)(r0 % head_size);
+            const float theta = powf(rope_base, -head_dim / (float)head_size);
+            float sn, cs;
+            sincosf((float)pos * theta, &sn, &cs);
+            const float x = t0, y = t1;
+            t0 = cs * x - sn * y;
+            t1 = sn * x + cs * y;
+        }
+        if (lane == 0) {
+            if (r0 < j.nrows) out[r0] = j.accumulate ? out[r0] + t0 : t0;
+            if (r1 < j.nrows) out[r1] = j.accumulate ? out[r1] + t1 : t1;
+        }
+    }
+};
+
+template <class F, int D>
+__device__ __forceinline__ void fused_job_body(const FusedParams &P, const GemvJob &j) {
+    GemvParams xp{};
+    xp.x = P.x;
+    xp.ncols = P.ncols;
+    xp.norm_w = P.norm_w;
+    xp.norm_eps = P.norm_eps;
+    xp.nrows = j.nrows;
+    GemvParams pa = xp, pb = xp;
+    pa.p0 = j.a0; pa.p1 = j.a1; pa.p2 = j.a2; pa.p3 = j.a3;
+    pb.p0 = j.b0; pb.p1 = j.b1; pb.p2 = j.b2; pb.p3 = j.b3;
+    const JobPolicy pol{j, pa, pb, dyn_pos(P.pos), P.head_size, P.rope_base};
+    gemv_i8_body<F, 2, D>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count);
+}
+
+template <int D, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_fused_kernel(const FusedParams P) {
+    int ji = 0;
+    if (P.njobs > 1 && blockIdx.x >= P.jobs[1].wg_begin) ji = 1;
+    if (P.njobs > 2 && blockIdx.x >= P.jobs[2].wg_begin) ji = 2;
+    const GemvJob &j = P.jobs[ji];
+    switch (j.type) {
+    case WGML_Q4_K: fused_job_body<IFmtQ4K, D>(P, j); break;
+    case WGML_Q6_K: fused_job_body<IFmtQ6K, D>(P, j); break;
+    default: fused_job_body<IFmtQ8_0, D>(P, j); break;
+    }
+}
+
 // ------------------------------------------------------------- dense f32 ----
-// out = A v, A row-major.  One wave per row, float4 loads, x from LDS.
-__global__ __launch_bounds__(256) void gemv_f32_kernel(const float *__restrict__ a,
-                                                       const float *__restrict__ x,
-                                                       float *__restrict__ out,
-                                                       const float *__restrict__ bias,
-                                                       uint32_t nrows, uint32_t ncols,
-                                                       int accumulate, int vec4) {
+// out = A v, A row-major f32 (p.p0).  One wave per row, float4 loads, x from LDS.
+__global__ __launch_bounds__(256) void gemv_f32_kernel(const GemvParams p, int vec4) {
     extern __shared__ float4 smem[];
+    __shared__ float red[16];
     float *xs = reinterpret_cast<float *>(smem);
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
-    for (uint32_t i = tid; i < ncols; i += blockDim.x) xs[i] = x[i];
+    const uint32_t nrows = p.nrows, ncols = p.ncols;
+    float rms = 1.f;
+    if (p.norm_w) rms = block_rms_scale(p, red);  // needs ncols % 4 == 0 and aligned x
+    for (uint32_t i = tid; i < ncols; i += blockDim.x)
+        xs[i] = p.norm_w ? (p.x[i] * rms) * p.norm_w[i] : p.x[i];
     __syncthreads();
     const uint32_t row = blockIdx.x * nwaves + wave;
     if (row >= nrows) return;
-    const float *ar = a + (size_t)row * ncols;
+    const float *ar = reinterpret_cast<const float *>(p.p0) + (size_t)row * ncols;
     float acc = 0.f;
     if (vec4) {
         const float4 *a4 = reinterpret_cast<const float4 *>(ar);
@@ -722,9 +907,11 @@ __global__ __launch_bounds__(256) void gemv_f32_kernel(const float *__restrict__
     }
     const float total = wave_sum(acc);
     if (lane == 0) {
+        float *out = p.out;
+        if (p.dyn_pos) out += (size_t)(*p.dyn_pos) * p.out_pos_stride;
         float v = total;
-        if (bias) v += bias[row];
-        if (accumulate) v += out[row];
+        if (p.bias) v += p.bias[row];
+        if (p.accumulate) v += out[row];
         out[row] = v;
     }
 }
@@ -882,8 +1069,13 @@ int launch_gemv_f32(wgml_ctx *ctx, float *out, const float *a, uint32_t nrows, u
         if (lds > 64 * 1024)
             return set_error(WGML_E_UNSUPPORTED, "gemv_f32: %u columns exceed the LDS limit", ncols);
         const int vec4 = (ncols % 4 == 0) && ((uintptr_t)a % 16 == 0);
-        gemv_f32_kernel<<<dim3((nrows + 3) / 4), dim3(256), lds, ctx->stream>>>(
-            a, v, out, nullptr, nrows, ncols, 0, vec4);
+        GemvParams p{};
+        p.p0 = reinterpret_cast<const uint8_t *>(a);
+        p.x = v;
+        p.out = out;
+        p.nrows = nrows;
+        p.ncols = ncols;
+        gemv_f32_kernel<<<dim3((nrows + 3) / 4), dim3(256), lds, ctx->stream>>>(p, vec4);
     }
     WGML_CHECK_LAUNCH();
     ctx->launches++;
@@ -894,17 +1086,6 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
                       const GemvEpilogue &ep) {
     if ((uintptr_t)v % 16 != 0)
         return set_error(WGML_E_INVALID, "gemv_quant: the input vector must be 16-byte aligned");
-    if (m->type == WGML_F32) {
-        const size_t lds = (size_t)m->ncols * 4;
-        if (lds > 64 * 1024)
-            return set_error(WGML_E_UNSUPPORTED, "gemv_f32: %u columns exceed the LDS limit",
-                             m->ncols);
-        gemv_f32_kernel<<<dim3((m->nrows + 3) / 4), dim3(256), lds, ctx->stream>>>(
-            (const float *)m->p0, v, out, ep.bias, m->nrows, m->ncols, ep.accumulate, 1);
-        WGML_CHECK_LAUNCH();
-        ctx->launches++;
-        return WGML_OK;
-    }
     GemvParams p;
     p.p0 = m->p0;
     p.p1 = m->p1;
@@ -917,6 +1098,20 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
     p.ncols = m->ncols;
     p.accumulate = ep.accumulate;
     p.debug = g_debug_flags;
+    p.dyn_pos = ep.dyn_pos;
+    p.out_pos_stride = ep.out_pos_stride;
+    p.norm_w = ep.norm_w;
+    p.norm_eps = ep.norm_eps;
+    if (m->type == WGML_F32) {
+        const size_t lds = (size_t)m->ncols * 4;
+        if (lds > 64 * 1024)
+            return set_error(WGML_E_UNSUPPORTED, "gemv_f32: %u columns exceed the LDS limit",
+                             m->ncols);
+        gemv_f32_kernel<<<dim3((m->nrows + 3) / 4), dim3(256), lds, ctx->stream>>>(p, 1);
+        WGML_CHECK_LAUNCH();
+        ctx->launches++;
+        return WGML_OK;
+    }
     if (!g_f32_activations) {
         switch (m->type) {
         case WGML_Q4_K: return launch_fmt_i8<IFmtQ4K>(ctx, p);
@@ -931,6 +1126,111 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
     case WGML_Q8_0: return launch_fmt<FmtQ8_0>(ctx, p);
     default: return set_error(WGML_E_UNSUPPORTED, "gemv_quant: unsupported type %d", m->type);
     }
+}
+
+static size_t lds_bytes_i8(int type, uint32_t ncols) {
+    uint32_t tile, pch, mf;
+    switch (type) {
+    case WGML_Q4_K: tile = 64; pch = 4; mf = IFmtQ4K::NXB + IFmtQ4K::NSUM; break;
+    case WGML_Q6_K: tile = 64; pch = 4; mf = IFmtQ6K::NXB + IFmtQ6K::NSUM; break;
+    default: tile = 32; pch = 2; mf = IFmtQ8_0::NXB + IFmtQ8_0::NSUM; break;
+    }
+    const uint32_t ntiles = ncols / tile;
+    const uint32_t ntiles_pad = ((ntiles + 63) / 64) * 64;
+    return (size_t)ntiles_pad * 2 * pch * 16 + (size_t)ntiles_pad * mf * 4;
+}
+
+bool gemv_fused_supported(const wgml_qmat *m) {
+    return m && (m->type == WGML_Q4_K || m->type == WGML_Q6_K || m->type == WGML_Q8_0);
+}
+
+int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
+    constexpr int MAXT = 512, D = 2;
+    constexpr uint32_t nwaves = MAXT / 64;
+    if (f.njobs < 1 || f.njobs > 3)
+        return set_error(WGML_E_INVALID, "gemv_fused: %d jobs", f.njobs);
+    if ((uintptr_t)f.x % 16 != 0)
+        return set_error(WGML_E_INVALID, "gemv_fused: the input vector must be 16-byte aligned");
+    FusedParams P{};
+    P.njobs = f.njobs;
+    P.x = f.x;
+    P.norm_w = f.norm_w;
+    P.norm_eps = f.norm_eps;
+    P.pos = f.pos;
+    P.head_size = f.head_size ? f.head_size : 2;
+    P.rope_base = f.rope_base;
+    const uint32_t ncols = f.jobs[0].a->ncols;
+    P.ncols = ncols;
+    size_t lds = 0;
+    uint64_t bytes[3] = {0, 0, 0}, total_bytes = 0;
+    uint32_t ngroups[3];
+    for (int i = 0; i < f.njobs; ++i) {
+        const FusedGemvJob &s = f.jobs[i];
+        if (!gemv_fused_supported(s.a) || s.a->ncols != ncols)
+            return set_error(WGML_E_INVALID, "gemv_fused: job %d has an unsupported matrix", i);
+        GemvJob &j = P.jobs[i];
+        j.a0 = s.a->p0; j.a1 = s.a->p1; j.a2 = s.a->p2; j.a3 = s.a->p3;
+        j.out = s.out;
+        j.bias = s.bias;
+        j.nrows = s.a->nrows;
+        j.type = s.a->type;
+        j.mode = s.mode;
+        j.accumulate = s.accumulate;
+        j.out_pos_stride = s.out_pos_stride;
+        bytes[i] = s.a->gguf_bytes;
+        if (s.mode == JOB_SILU) {
+            if (!s.b || s.b->type != s.a->type || s.b->nrows != s.a->nrows || s.b->ncols != ncols)
+                return set_error(WGML_E_INVALID, "gemv_fused: job %d: gate/up matrices differ", i);
+            j.b0 = s.b->p0; j.b1 = s.b->p1; j.b2 = s.b->p2; j.b3 = s.b->p3;
+            bytes[i] += s.b->gguf_bytes;
+            ngroups[i] = j.nrows;
+        } else {
+            if (s.mode == JOB_ROPE && (j.nrows % 2 != 0 || P.head_size % 2 != 0))
+                return set_error(WGML_E_INVALID, "gemv_fused: RoPE needs even row counts");
+            ngroups[i] = (j.nrows + 1) / 2;
+        }
+        total_bytes += bytes[i];
+        const size_t l = lds_bytes_i8(j.type, ncols);
+        if (l > lds) lds = l;
+    }
+    if (lds > kMaxLds)
+        return set_error(WGML_E_UNSUPPORTED, "gemv_fused: %u columns need %zu bytes of LDS", ncols,
+                         lds);
+    const void *fn = (const void *)gemv_fused_kernel<D, MAXT>;
+    static bool opted_in = false;
+    if (lds > 64 * 1024 && !opted_in) {
+        WGML_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)kMaxLds));
+        opted_in = true;
+    }
+    static size_t cached_lds = ~size_t(0);
+    static int cached_blocks = 0;
+    if (cached_lds != lds) {
+        int nb = 0;
+        WGML_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fn, MAXT, lds));
+        cached_blocks = nb > 0 ? nb : 1;
+        cached_lds = lds;
+    }
+    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
+    const uint32_t resident = cu * (uint32_t)cached_blocks;
+    // Workgroups are shared out in proportion to the bytes each matrix streams, then
+    // trimmed so that every wave of a matrix gets the same number of row pairs.
+    uint32_t begin = 0;
+    for (int i = 0; i < f.njobs; ++i) {
+        uint32_t share = (uint32_t)((double)resident * (double)bytes[i] / (double)total_bytes);
+        if (share < 1) share = 1;
+        const uint32_t max_wg = (ngroups[i] + nwaves - 1) / nwaves;
+        if (share > max_wg) share = max_wg;
+        const uint32_t k = (ngroups[i] + share * nwaves - 1) / (share * nwaves);
+        const uint32_t wgs = (ngroups[i] + nwaves * k - 1) / (nwaves * k);
+        P.jobs[i].wg_begin = begin;
+        P.jobs[i].wg_count = wgs;
+        begin += wgs;
+    }
+    gemv_fused_kernel<D, MAXT><<<dim3(begin), dim3(MAXT), lds, ctx->stream>>>(P);
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
 }
 
 }  // namespace wgml

@@ -2,6 +2,13 @@
 // Mirrors Llama2State / Llama2Weights / Llama2::dispatch
 // (models/llama2/transformer.rs:17-476 of the reference) and the token loop of
 // ChatLlama2 (wgml-chat/src/chat_llama2.rs:51-228).
+//
+// One decode step is a fixed sequence of launches.  It exists in two forms:
+//   * eager: token and position are host values (wgml_llama2_forward);
+//   * recorded: token and position live in a small device struct that the
+//     kernels read, the arg-max kernel writes the next token and advances the
+//     position, and the whole step is a HIP graph replayed once per token with
+//     no host round trip in between (the greedy loops).
 #include "common.h"
 
 using namespace wgml;
@@ -10,7 +17,8 @@ namespace wgml {
 int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
                              uint32_t plan_positions, const float *q, const float *kc,
                              const float *vc, float *att, float *xb);
-}
+int reserve_attention_workspace(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions);
+}  // namespace wgml
 
 struct LlamaLayer {
     const wgml_qmat *attn_q = nullptr, *attn_k = nullptr, *attn_v = nullptr, *attn_output = nullptr,
@@ -24,7 +32,7 @@ struct wgml_llama2 {
     wgml_ctx *ctx = nullptr;
     wgml_llama2_config cfg{};
     int model_type = WGML_MODEL_LLAMA;
-    int fusion = 1;
+    int fusion = 3;
     uint32_t kv_dim = 0, head_size = 0, kv_mul = 0;
     std::vector<LlamaLayer> layers;
     const wgml_qmat *output = nullptr;
@@ -33,22 +41,32 @@ struct wgml_llama2 {
     // Llama2State (models/llama2/transformer.rs:17-45)
     float *x = nullptr, *xb = nullptr, *xb2 = nullptr, *hb = nullptr, *hb2 = nullptr, *q = nullptr,
           *logits = nullptr;
+    // token-loop state on the device
+    DynState *dyn = nullptr;
+    uint32_t *d_prompt = nullptr, *d_tokens = nullptr;  // seq_len entries each
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    int graph_fusion = -1;
     std::vector<void *> allocs;
     uint64_t launches_last = 0;
 };
 
 namespace {
 
-int dev_alloc(wgml_llama2 *m, float **p, uint64_t n_floats, bool zero) {
+int dev_alloc_bytes(wgml_llama2 *m, void **p, uint64_t bytes, bool zero) {
     void *d = nullptr;
-    hipError_t e = hipMalloc(&d, n_floats * 4);
+    hipError_t e = hipMalloc(&d, bytes);
     if (e != hipSuccess)
         return set_error(WGML_E_OOM, "wgml_llama2: hipMalloc(%llu) failed: %s",
-                         (unsigned long long)(n_floats * 4), hipGetErrorString(e));
+                         (unsigned long long)bytes, hipGetErrorString(e));
     m->allocs.push_back(d);
-    if (zero) WGML_CHECK_HIP(hipMemsetAsync(d, 0, n_floats * 4, m->ctx->stream));
-    *p = (float *)d;
+    if (zero) WGML_CHECK_HIP(hipMemsetAsync(d, 0, bytes, m->ctx->stream));
+    *p = d;
     return WGML_OK;
+}
+
+int dev_alloc(wgml_llama2 *m, float **p, uint64_t n_floats, bool zero) {
+    return dev_alloc_bytes(m, (void **)p, n_floats * 4, zero);
 }
 
 int check_ready(const wgml_llama2 *m) {
@@ -60,6 +78,268 @@ int check_ready(const wgml_llama2 *m) {
     }
     WGML_REQUIRE(m->output && m->output_norm && m->token_embd,
                  "wgml_llama2: output / output_norm / token_embd not set");
+    return WGML_OK;
+}
+
+void drop_graph(wgml_llama2 *m) {
+    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+    if (m->graph) (void)hipGraphDestroy(m->graph);
+    m->graph_exec = nullptr;
+    m->graph = nullptr;
+    m->graph_fusion = -1;
+}
+
+// Enqueues one decode step (Llama2::dispatch, models/llama2/transformer.rs:298-431,
+// preceded by the embedding copy of chat_llama2.rs:185-187).
+//   dynamic == false: token/pos are the given host values;
+//   dynamic == true : they are read from m->dyn on the device, the attention
+//                     grid is planned for seq_len positions.
+// fusion 0: one launch per reference op.  1: bias and residual adds folded into
+// the GEMV epilogues.  2: additionally every RMSNorm folded into the staging of
+// the GEMVs that consume it.
+int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos) {
+    const wgml_llama2_config &c = m->cfg;
+    wgml_ctx *ctx = m->ctx;
+    const uint32_t dim = c.dim, kv_dim = m->kv_dim;
+    const DynPos dpos{dynamic ? &m->dyn->pos : nullptr, pos};
+    const DynPos dtok{dynamic ? &m->dyn->token : nullptr, token};
+    const int variant = m->model_type == WGML_MODEL_QWEN2 ? WGML_ROPE_NEOX : WGML_ROPE_ORIGINAL;
+    const wgml_attn_params ap{c.seq_len, kv_dim, m->kv_mul, c.n_q_heads, m->head_size, pos};
+    const int fusion = m->fusion;
+    const uint32_t plan = dynamic ? c.seq_len : pos + 1;
+
+    WGML_TRY(launch_embed(ctx, m->x, m->token_embd, dim, dtok));
+
+    for (uint32_t l = 0; l < c.n_layers; ++l) {
+        const LlamaLayer &w = m->layers[l];
+        if (fusion >= 3 && gemv_fused_supported(w.attn_q) && gemv_fused_supported(w.attn_k) &&
+            gemv_fused_supported(w.attn_v) && gemv_fused_supported(w.ffn_gate) &&
+            gemv_fused_supported(w.ffn_up) && w.ffn_gate->type == w.ffn_up->type) {
+            // 5 launches per layer: [norm + Q,K,V + bias + RoPE + KV-cache write],
+            // attention (+ merge), [Wo + residual], [norm + gate,up + SiLU], [down + residual]
+            const bool rope_fused = variant == WGML_ROPE_ORIGINAL;
+            FusedGemv f;
+            f.njobs = 3;
+            f.x = m->x;
+            f.norm_w = w.attn_norm;
+            f.norm_eps = c.rms_norm_eps;
+            f.pos = dpos;
+            f.head_size = m->head_size;
+            f.rope_base = c.rope_base_freq;
+            f.jobs[0].a = w.attn_q;
+            f.jobs[0].out = m->q;
+            f.jobs[0].bias = w.bq;
+            f.jobs[0].mode = rope_fused ? FUSED_ROPE : FUSED_PLAIN;
+            f.jobs[1].a = w.attn_k;
+            f.jobs[1].out = w.key_cache;
+            f.jobs[1].bias = w.bk;
+            f.jobs[1].mode = rope_fused ? FUSED_ROPE : FUSED_PLAIN;
+            f.jobs[1].out_pos_stride = kv_dim;
+            f.jobs[2].a = w.attn_v;
+            f.jobs[2].out = w.value_cache;
+            f.jobs[2].bias = w.bv;
+            f.jobs[2].out_pos_stride = kv_dim;
+            WGML_TRY(launch_gemv_fused(ctx, f));
+            if (!rope_fused)
+                WGML_TRY(launch_rope(ctx, variant, m->head_size, kv_dim, dpos, c.rope_base_freq,
+                                     m->q, dim, w.key_cache, kv_dim));
+            WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, m->q, w.key_cache,
+                                              w.value_cache, nullptr, m->xb));
+            GemvEpilogue eacc;
+            eacc.accumulate = 1;
+            WGML_TRY(launch_gemv_quant(ctx, m->x, w.attn_output, m->xb, eacc));
+            FusedGemv g;
+            g.njobs = 1;
+            g.x = m->x;
+            g.norm_w = w.ffn_norm;
+            g.norm_eps = c.rms_norm_eps;
+            g.jobs[0].a = w.ffn_gate;
+            g.jobs[0].b = w.ffn_up;
+            g.jobs[0].out = m->hb;
+            g.jobs[0].mode = FUSED_SILU;
+            WGML_TRY(launch_gemv_fused(ctx, g));
+            WGML_TRY(launch_gemv_quant(ctx, m->x, w.ffn_down, m->hb, eacc));
+            continue;
+        }
+        // the KV-cache column of this position
+        float *k_cache = w.key_cache, *v_cache = w.value_cache;
+        GemvEpilogue eq, ek, ev;
+        if (dynamic) {
+            ek.dyn_pos = ev.dyn_pos = &m->dyn->pos;
+            ek.out_pos_stride = ev.out_pos_stride = kv_dim;
+        } else {
+            k_cache += (size_t)pos * kv_dim;
+            v_cache += (size_t)pos * kv_dim;
+        }
+        const float *qkv_in = m->xb;
+        if (fusion >= 2) {
+            qkv_in = m->x;
+            eq.norm_w = ek.norm_w = ev.norm_w = w.attn_norm;
+            eq.norm_eps = ek.norm_eps = ev.norm_eps = c.rms_norm_eps;
+        } else {
+            WGML_TRY(launch_rms_norm(ctx, c.rms_norm_eps, m->xb, m->x, w.attn_norm, dim));
+        }
+        // recorded steps always add the biases in the epilogue: a separate add would
+        // need the position-dependent cache column as its destination
+        const bool bias_in_epilogue = fusion >= 1 || dynamic;
+        if (bias_in_epilogue) {
+            eq.bias = w.bq;
+            ek.bias = w.bk;
+            ev.bias = w.bv;
+        }
+        WGML_TRY(launch_gemv_quant(ctx, m->q, w.attn_q, qkv_in, eq));
+        WGML_TRY(launch_gemv_quant(ctx, k_cache, w.attn_k, qkv_in, ek));
+        WGML_TRY(launch_gemv_quant(ctx, v_cache, w.attn_v, qkv_in, ev));
+        if (!bias_in_epilogue) {
+            if (w.bq) WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, m->q, w.bq, dim));
+            if (w.bk) WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, k_cache, w.bk, kv_dim));
+            if (w.bv) WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, v_cache, w.bv, kv_dim));
+        }
+        WGML_TRY(launch_rope(ctx, variant, m->head_size, kv_dim, dpos, c.rope_base_freq, m->q, dim,
+                             dynamic ? w.key_cache : k_cache, dynamic ? kv_dim : 0));
+        WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, m->q, w.key_cache, w.value_cache,
+                                          nullptr, m->xb));
+        if (fusion >= 1) {
+            // x += Wo * xb in the GEMV epilogue
+            GemvEpilogue e;
+            e.accumulate = 1;
+            WGML_TRY(launch_gemv_quant(ctx, m->x, w.attn_output, m->xb, e));
+        } else {
+            WGML_TRY(launch_gemv_quant(ctx, m->xb2, w.attn_output, m->xb, GemvEpilogue{}));
+            WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, m->x, m->xb2, dim));
+        }
+        GemvEpilogue eg;
+        const float *ffn_in = m->xb;
+        if (fusion >= 2) {
+            ffn_in = m->x;
+            eg.norm_w = w.ffn_norm;
+            eg.norm_eps = c.rms_norm_eps;
+        } else {
+            WGML_TRY(launch_rms_norm(ctx, c.rms_norm_eps, m->xb, m->x, w.ffn_norm, dim));
+        }
+        WGML_TRY(launch_gemv_quant(ctx, m->hb, w.ffn_gate, ffn_in, eg));
+        WGML_TRY(launch_gemv_quant(ctx, m->hb2, w.ffn_up, ffn_in, eg));
+        WGML_TRY(launch_silu(ctx, m->hb, m->hb2, c.hidden_dim));
+        if (fusion >= 1) {
+            GemvEpilogue e;
+            e.accumulate = 1;
+            WGML_TRY(launch_gemv_quant(ctx, m->x, w.ffn_down, m->hb, e));
+        } else {
+            WGML_TRY(launch_gemv_quant(ctx, m->xb2, w.ffn_down, m->hb, GemvEpilogue{}));
+            WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, m->x, m->xb2, dim));
+        }
+    }
+    GemvEpilogue eo;
+    const float *out_in = m->xb;
+    if (fusion >= 2) {
+        out_in = m->x;
+        eo.norm_w = m->output_norm;
+        eo.norm_eps = c.rms_norm_eps;
+    } else {
+        WGML_TRY(launch_rms_norm(ctx, c.rms_norm_eps, m->xb, m->x, m->output_norm, dim));
+    }
+    WGML_TRY(launch_gemv_quant(ctx, m->logits, m->output, out_in, eo));
+    return WGML_OK;
+}
+
+// Records one step (+ greedy sampling and bookkeeping) into a HIP graph.
+int build_graph(wgml_llama2 *m) {
+    if (m->graph_exec && m->graph_fusion == m->fusion) return WGML_OK;
+    drop_graph(m);
+    wgml_ctx *ctx = m->ctx;
+    const wgml_llama2_config &c = m->cfg;
+    // Everything that allocates or sets function attributes happens before capture:
+    // the attention workspace for the largest plan, and one eager step.
+    const wgml_attn_params ap{c.seq_len, m->kv_dim, m->kv_mul, c.n_q_heads, m->head_size, 0};
+    WGML_TRY(reserve_attention_workspace(ctx, ap, c.seq_len));
+    // The eager step runs at position 0 and would overwrite that column of every KV
+    // cache (the caller may have filled it): keep a copy and put it back.
+    const size_t col = (size_t)m->kv_dim * 4;
+    void *saved = nullptr;
+    WGML_CHECK_HIP(hipMalloc(&saved, col * 2 * c.n_layers));
+    for (uint32_t l = 0; l < c.n_layers; ++l) {
+        (void)hipMemcpyAsync((char *)saved + col * (2 * l), m->layers[l].key_cache, col,
+                             hipMemcpyDeviceToDevice, ctx->stream);
+        (void)hipMemcpyAsync((char *)saved + col * (2 * l + 1), m->layers[l].value_cache, col,
+                             hipMemcpyDeviceToDevice, ctx->stream);
+    }
+    const DynState init{0, 0, 0, 0};
+    hipError_t ew = hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream);
+    int rcw = ew == hipSuccess ? enqueue_step(m, true, 0, 0) : WGML_E_HIP;
+    if (rcw == WGML_OK)
+        rcw = launch_argmax_next(ctx, m->logits, c.vocab_size, m->dyn, m->d_prompt, m->d_tokens);
+    for (uint32_t l = 0; l < c.n_layers; ++l) {
+        (void)hipMemcpyAsync(m->layers[l].key_cache, (char *)saved + col * (2 * l), col,
+                             hipMemcpyDeviceToDevice, ctx->stream);
+        (void)hipMemcpyAsync(m->layers[l].value_cache, (char *)saved + col * (2 * l + 1), col,
+                             hipMemcpyDeviceToDevice, ctx->stream);
+    }
+    ew = hipStreamSynchronize(ctx->stream);
+    (void)hipFree(saved);
+    if (rcw != WGML_OK) return rcw;
+    if (ew != hipSuccess)
+        return set_error(WGML_E_HIP, "wgml_llama2: warm-up step failed: %s", hipGetErrorString(ew));
+
+    WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    const uint64_t launches0 = ctx->launches;
+    int rc = enqueue_step(m, true, 0, 0);
+    if (rc == WGML_OK)
+        rc = launch_argmax_next(ctx, m->logits, c.vocab_size, m->dyn, m->d_prompt, m->d_tokens);
+    m->launches_last = ctx->launches - launches0;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &m->graph);
+    if (rc != WGML_OK) {
+        drop_graph(m);
+        return rc;
+    }
+    if (e != hipSuccess) {
+        drop_graph(m);
+        return set_error(WGML_E_HIP, "wgml_llama2: graph capture failed: %s", hipGetErrorString(e));
+    }
+    e = hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        drop_graph(m);
+        return set_error(WGML_E_HIP, "wgml_llama2: graph instantiate failed: %s",
+                         hipGetErrorString(e));
+    }
+    m->graph_fusion = m->fusion;
+    return WGML_OK;
+}
+
+// Runs n_steps recorded steps from (first_token, start_pos); prompt tokens (if
+// any) are forced.  One synchronisation at the end.
+int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint32_t n_steps,
+                 const uint32_t *prompt, uint32_t n_prompt, uint32_t *out_tokens) {
+    wgml_ctx *ctx = m->ctx;
+    WGML_TRY(check_ready(m));
+    const bool use_graph = !graphs_disabled();
+    if (use_graph) {
+        WGML_TRY(build_graph(m));
+    } else {
+        const wgml_attn_params ap{m->cfg.seq_len, m->kv_dim, m->kv_mul, m->cfg.n_q_heads,
+                                  m->head_size, 0};
+        WGML_TRY(reserve_attention_workspace(ctx, ap, m->cfg.seq_len));
+    }
+    if (n_prompt)
+        WGML_CHECK_HIP(hipMemcpyAsync(m->d_prompt, prompt, (size_t)n_prompt * 4,
+                                      hipMemcpyHostToDevice, ctx->stream));
+    const DynState init{start_pos, first_token, 0, n_prompt};
+    WGML_CHECK_HIP(hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream));
+    WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));  // `init` is a stack object
+    for (uint32_t i = 0; i < n_steps; ++i) {
+        if (use_graph) {
+            WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec, ctx->stream));
+        } else {
+            // the same launches, enqueued one by one (no host synchronisation either)
+            const uint64_t launches0 = ctx->launches;
+            WGML_TRY(enqueue_step(m, true, 0, 0));
+            WGML_TRY(launch_argmax_next(ctx, m->logits, m->cfg.vocab_size, m->dyn, m->d_prompt,
+                                        m->d_tokens));
+            m->launches_last = ctx->launches - launches0;
+        }
+    }
+    WGML_CHECK_HIP(hipMemcpyAsync(out_tokens, m->d_tokens, (size_t)n_steps * 4,
+                                  hipMemcpyDeviceToHost, ctx->stream));
+    WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
     return WGML_OK;
 }
 
@@ -81,6 +361,10 @@ int wgml_llama2_create(wgml_ctx *ctx, const wgml_llama2_config *cfg, int model_t
                  cfg->n_q_heads, cfg->n_kv_heads);
     WGML_REQUIRE(cfg->dim % 4 == 0 && cfg->hidden_dim % 4 == 0,
                  "wgml_llama2_create: dim and hidden_dim must be multiples of 4");
+    const uint32_t head_size = cfg->dim / cfg->n_q_heads;
+    if (head_size % 2 != 0 || head_size > 256)
+        return set_error(WGML_E_UNSUPPORTED, "wgml_llama2_create: head_size %u unsupported",
+                         head_size);
     wgml_llama2 *m = new wgml_llama2();
     m->ctx = ctx;
     ctx_retain(ctx);
@@ -88,14 +372,8 @@ int wgml_llama2_create(wgml_ctx *ctx, const wgml_llama2_config *cfg, int model_t
     m->model_type = model_type;
     // Llama2Config::derived_configs (models/llama2/cpu.rs:111-141)
     m->kv_dim = cfg->dim * cfg->n_kv_heads / cfg->n_q_heads;
-    m->head_size = cfg->dim / cfg->n_q_heads;
+    m->head_size = head_size;
     m->kv_mul = cfg->n_q_heads / cfg->n_kv_heads;
-    if (m->head_size % 2 != 0 || m->head_size > 256) {
-        ctx_release(ctx);
-        delete m;
-        return set_error(WGML_E_UNSUPPORTED, "wgml_llama2_create: head_size %u unsupported",
-                         cfg->dim / cfg->n_q_heads);
-    }
     m->layers.resize(cfg->n_layers);
     int rc = WGML_OK;
     auto A = [&](float **p, uint64_t n, bool z) {
@@ -112,6 +390,9 @@ int wgml_llama2_create(wgml_ctx *ctx, const wgml_llama2_config *cfg, int model_t
         A(&l.key_cache, (uint64_t)m->kv_dim * cfg->seq_len, true);
         A(&l.value_cache, (uint64_t)m->kv_dim * cfg->seq_len, true);
     }
+    if (rc == WGML_OK) rc = dev_alloc_bytes(m, (void **)&m->dyn, 256, true);
+    if (rc == WGML_OK) rc = dev_alloc_bytes(m, (void **)&m->d_prompt, (uint64_t)cfg->seq_len * 4, true);
+    if (rc == WGML_OK) rc = dev_alloc_bytes(m, (void **)&m->d_tokens, (uint64_t)cfg->seq_len * 4, true);
     if (rc == WGML_OK && hipStreamSynchronize(ctx->stream) != hipSuccess)
         rc = set_error(WGML_E_HIP, "wgml_llama2_create: synchronize failed");
     if (rc != WGML_OK) {
@@ -125,6 +406,7 @@ int wgml_llama2_create(wgml_ctx *ctx, const wgml_llama2_config *cfg, int model_t
 int wgml_llama2_destroy(wgml_llama2 *m) {
     if (!m) return WGML_OK;
     if (m->ctx && m->ctx->stream) (void)hipStreamSynchronize(m->ctx->stream);
+    drop_graph(m);
     for (void *p : m->allocs) (void)hipFree(p);
     ctx_release(m->ctx);
     delete m;
@@ -149,6 +431,7 @@ int wgml_llama2_set_matrix(wgml_llama2 *m, int which, uint32_t layer, const wgml
     WGML_REQUIRE(mat->nrows == er && mat->ncols == ec,
                  "wgml_llama2_set_matrix: matrix %d is %ux%u, expected %ux%u", which, mat->nrows,
                  mat->ncols, er, ec);
+    drop_graph(m);  // recorded launches hold the old pointers
     if (which == WGML_LLAMA2_OUTPUT) {
         m->output = mat;
         return WGML_OK;
@@ -192,7 +475,10 @@ int wgml_llama2_set_vector(wgml_llama2 *m, int which, uint32_t layer, const floa
     }
     WGML_REQUIRE(len == expect, "wgml_llama2_set_vector: vector %d has %u elements, expected %u",
                  which, len, expect);
-    if (!*slot) WGML_TRY(dev_alloc(m, slot, len, false));
+    if (!*slot) {
+        WGML_TRY(dev_alloc(m, slot, len, false));
+        drop_graph(m);
+    }
     WGML_CHECK_HIP(hipMemcpyAsync(*slot, host, (size_t)len * 4, hipMemcpyHostToDevice,
                                   m->ctx->stream));
     WGML_CHECK_HIP(hipStreamSynchronize(m->ctx->stream));
@@ -202,7 +488,10 @@ int wgml_llama2_set_vector(wgml_llama2 *m, int which, uint32_t layer, const floa
 int wgml_llama2_set_token_embd(wgml_llama2 *m, const float *host) {
     WGML_REQUIRE(m && host, "wgml_llama2_set_token_embd: null argument");
     const uint64_t n = (uint64_t)m->cfg.dim * m->cfg.vocab_size;
-    if (!m->token_embd) WGML_TRY(dev_alloc(m, &m->token_embd, n, false));
+    if (!m->token_embd) {
+        WGML_TRY(dev_alloc(m, &m->token_embd, n, false));
+        drop_graph(m);
+    }
     WGML_CHECK_HIP(hipMemcpyAsync(m->token_embd, host, n * 4, hipMemcpyHostToDevice,
                                   m->ctx->stream));
     WGML_CHECK_HIP(hipStreamSynchronize(m->ctx->stream));
@@ -211,7 +500,7 @@ int wgml_llama2_set_token_embd(wgml_llama2 *m, const float *host) {
 
 int wgml_llama2_set_fusion(wgml_llama2 *m, int level) {
     WGML_REQUIRE(m != nullptr, "wgml_llama2_set_fusion: null model");
-    WGML_REQUIRE(level == 0 || level == 1, "wgml_llama2_set_fusion: level %d not in {0,1}", level);
+    WGML_REQUIRE(level >= 0 && level <= 3, "wgml_llama2_set_fusion: level %d not in 0..3", level);
     m->fusion = level;
     return WGML_OK;
 }
@@ -227,61 +516,9 @@ int wgml_llama2_forward(wgml_llama2 *m, uint32_t token, uint32_t pos) {
     WGML_REQUIRE(token < c.vocab_size, "wgml_llama2_forward: token %u outside vocabulary %u", token,
                  c.vocab_size);
     WGML_REQUIRE(pos < c.seq_len, "wgml_llama2_forward: pos %u outside seq_len %u", pos, c.seq_len);
-    wgml_ctx *ctx = m->ctx;
-    const uint64_t launches0 = ctx->launches;
-    const uint32_t dim = c.dim, kv_dim = m->kv_dim;
-    const DynPos dpos{nullptr, pos};
-    const int variant = m->model_type == WGML_MODEL_QWEN2 ? WGML_ROPE_NEOX : WGML_ROPE_ORIGINAL;
-    const wgml_attn_params ap{c.seq_len, kv_dim, m->kv_mul, c.n_q_heads, m->head_size, pos};
-    const bool fused = m->fusion >= 1;
-
-    // state.x.copy_from_view(token_embd.column(token))  (chat_llama2.rs:185-187)
-    WGML_CHECK_HIP(hipMemcpyAsync(m->x, m->token_embd + (size_t)token * dim, (size_t)dim * 4,
-                                  hipMemcpyDeviceToDevice, ctx->stream));
-
-    for (uint32_t l = 0; l < c.n_layers; ++l) {
-        const LlamaLayer &w = m->layers[l];
-        float *k_cache = w.key_cache + (size_t)pos * kv_dim;
-        float *v_cache = w.value_cache + (size_t)pos * kv_dim;
-
-        WGML_TRY(launch_rms_norm(ctx, c.rms_norm_eps, m->xb, m->x, w.attn_norm, dim));
-        if (fused) {
-            WGML_TRY(launch_gemv_quant(ctx, m->q, w.attn_q, m->xb, GemvEpilogue{w.bq, 0}));
-            WGML_TRY(launch_gemv_quant(ctx, k_cache, w.attn_k, m->xb, GemvEpilogue{w.bk, 0}));
-            WGML_TRY(launch_gemv_quant(ctx, v_cache, w.attn_v, m->xb, GemvEpilogue{w.bv, 0}));
-        } else {
-            WGML_TRY(launch_gemv_quant(ctx, m->q, w.attn_q, m->xb, GemvEpilogue{}));
-            WGML_TRY(launch_gemv_quant(ctx, k_cache, w.attn_k, m->xb, GemvEpilogue{}));
-            WGML_TRY(launch_gemv_quant(ctx, v_cache, w.attn_v, m->xb, GemvEpilogue{}));
-            if (w.bq) WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, m->q, w.bq, dim));
-            if (w.bk) WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, k_cache, w.bk, kv_dim));
-            if (w.bv) WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, v_cache, w.bv, kv_dim));
-        }
-        WGML_TRY(launch_rope(ctx, variant, m->head_size, kv_dim, dpos, c.rope_base_freq, m->q, dim,
-                             k_cache, 0));
-        WGML_TRY(launch_attention_planned(ctx, ap, dpos, pos + 1, m->q, w.key_cache,
-                                          w.value_cache, nullptr, m->xb));
-        if (fused) {
-            // x += Wo * xb in the GEMV epilogue
-            WGML_TRY(launch_gemv_quant(ctx, m->x, w.attn_output, m->xb, GemvEpilogue{nullptr, 1}));
-        } else {
-            WGML_TRY(launch_gemv_quant(ctx, m->xb2, w.attn_output, m->xb, GemvEpilogue{}));
-            WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, m->x, m->xb2, dim));
-        }
-        WGML_TRY(launch_rms_norm(ctx, c.rms_norm_eps, m->xb, m->x, w.ffn_norm, dim));
-        WGML_TRY(launch_gemv_quant(ctx, m->hb, w.ffn_gate, m->xb, GemvEpilogue{}));
-        WGML_TRY(launch_gemv_quant(ctx, m->hb2, w.ffn_up, m->xb, GemvEpilogue{}));
-        WGML_TRY(launch_silu(ctx, m->hb, m->hb2, c.hidden_dim));
-        if (fused) {
-            WGML_TRY(launch_gemv_quant(ctx, m->x, w.ffn_down, m->hb, GemvEpilogue{nullptr, 1}));
-        } else {
-            WGML_TRY(launch_gemv_quant(ctx, m->xb2, w.ffn_down, m->hb, GemvEpilogue{}));
-            WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, m->x, m->xb2, dim));
-        }
-    }
-    WGML_TRY(launch_rms_norm(ctx, c.rms_norm_eps, m->xb, m->x, m->output_norm, dim));
-    WGML_TRY(launch_gemv_quant(ctx, m->logits, m->output, m->xb, GemvEpilogue{}));
-    m->launches_last = ctx->launches - launches0;
+    const uint64_t launches0 = m->ctx->launches;
+    WGML_TRY(enqueue_step(m, false, token, pos));
+    m->launches_last = m->ctx->launches - launches0;
     return WGML_OK;
 }
 
@@ -299,6 +536,33 @@ int wgml_llama2_decode_greedy(wgml_llama2 *m, uint32_t first_token, uint32_t sta
     WGML_REQUIRE((uint64_t)start_pos + n_steps <= m->cfg.seq_len,
                  "wgml_llama2_decode_greedy: %u steps from %u exceed seq_len %u", n_steps, start_pos,
                  m->cfg.seq_len);
+    WGML_REQUIRE(first_token < m->cfg.vocab_size, "wgml_llama2_decode_greedy: token outside vocabulary");
+    if (n_steps == 0) return WGML_OK;
+    return run_recorded(m, first_token, start_pos, n_steps, nullptr, 0, out_tokens);
+}
+
+int wgml_llama2_generate_greedy(wgml_llama2 *m, const uint32_t *prompt, uint32_t n_prompt,
+                                uint32_t n_total, uint32_t *out_tokens) {
+    WGML_REQUIRE(m && prompt && out_tokens, "wgml_llama2_generate_greedy: null argument");
+    WGML_REQUIRE(n_prompt >= 1, "wgml_llama2_generate_greedy: empty prompt");
+    WGML_REQUIRE(n_total <= m->cfg.seq_len && n_prompt <= m->cfg.seq_len,
+                 "wgml_llama2_generate_greedy: %u positions exceed seq_len %u", n_total,
+                 m->cfg.seq_len);
+    for (uint32_t i = 0; i < n_prompt; ++i)
+        WGML_REQUIRE(prompt[i] < m->cfg.vocab_size,
+                     "wgml_llama2_generate_greedy: prompt token %u outside vocabulary", prompt[i]);
+    if (n_total == 0) return WGML_OK;
+    return run_recorded(m, prompt[0], 0, n_total, prompt, n_prompt, out_tokens);
+}
+
+// The same loop with a host round trip per token, as the reference's chat loop
+// does it (read back after every step): for comparison and for callers that
+// stream tokens out as they appear.
+int wgml_llama2_decode_greedy_sync(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos,
+                                   uint32_t n_steps, uint32_t *out_tokens) {
+    WGML_REQUIRE(m && out_tokens, "wgml_llama2_decode_greedy_sync: null argument");
+    WGML_REQUIRE((uint64_t)start_pos + n_steps <= m->cfg.seq_len,
+                 "wgml_llama2_decode_greedy_sync: steps exceed seq_len");
     wgml_ctx *ctx = m->ctx;
     uint32_t token = first_token;
     for (uint32_t i = 0; i < n_steps; ++i) {
@@ -309,29 +573,6 @@ int wgml_llama2_decode_greedy(wgml_llama2 *m, uint32_t first_token, uint32_t sta
         WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
         token = ctx->h_scalar[0];
         out_tokens[i] = token;
-    }
-    return WGML_OK;
-}
-
-int wgml_llama2_generate_greedy(wgml_llama2 *m, const uint32_t *prompt, uint32_t n_prompt,
-                                uint32_t n_total, uint32_t *out_tokens) {
-    WGML_REQUIRE(m && prompt && out_tokens, "wgml_llama2_generate_greedy: null argument");
-    WGML_REQUIRE(n_prompt >= 1, "wgml_llama2_generate_greedy: empty prompt");
-    WGML_REQUIRE(n_total <= m->cfg.seq_len,
-                 "wgml_llama2_generate_greedy: %u positions exceed seq_len %u", n_total,
-                 m->cfg.seq_len);
-    wgml_ctx *ctx = m->ctx;
-    uint32_t token = prompt[0];
-    for (uint32_t pos = 0; pos < n_total; ++pos) {
-        WGML_TRY(wgml_llama2_forward(m, token, pos));
-        WGML_TRY(launch_argmax(ctx, m->logits, m->cfg.vocab_size, ctx->d_scalar));
-        WGML_CHECK_HIP(hipMemcpyAsync(ctx->h_scalar, ctx->d_scalar, 4, hipMemcpyDeviceToHost,
-                                      ctx->stream));
-        WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
-        const uint32_t best = ctx->h_scalar[0];
-        out_tokens[pos] = best;
-        // forced prompt tokens win over the sample (wgml-chat/src/sampler.rs:102-107)
-        token = (pos + 1 < n_prompt) ? prompt[pos + 1] : best;
     }
     return WGML_OK;
 }

@@ -158,9 +158,8 @@ __global__ void op_assign_kernel(float *__restrict__ a, const float *__restrict_
 
 // models/sampler.rs:54-56: first index of the maximum.  One workgroup; ties go
 // to the lower index.  NaN never wins (comparisons with NaN are false), as with
-// nalgebra's imax on well-formed logits.
-__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ v, uint32_t n,
-                                                      uint32_t *__restrict__ out) {
+// nalgebra's imax on well-formed logits.  The result is valid in thread 0.
+__device__ __forceinline__ uint32_t block_argmax(const float *__restrict__ v, uint32_t n) {
     __shared__ float bv[16];
     __shared__ uint32_t bi[16];
     float best = -INFINITY;
@@ -193,8 +192,41 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
                 best = bv[w];
                 idx = bi[w];
             }
-        out[0] = idx;
     }
+    return idx;
+}
+
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ v, uint32_t n,
+                                                      uint32_t *__restrict__ out) {
+    const uint32_t idx = block_argmax(v, n);
+    if (threadIdx.x == 0) out[0] = idx;
+}
+
+// Greedy sampling + the token loop's bookkeeping on the device
+// (ChatLlama2::forward / sample_next_token with temperature 0,
+// wgml-chat/src/chat_llama2.rs:51-153, wgml-chat/src/sampler.rs:91-111): records
+// the arg-max, picks the next input token (a forced prompt token wins over the
+// sample) and advances the position, so that the next step can be enqueued
+// without a host round trip.
+__global__ __launch_bounds__(1024) void argmax_next_kernel(const float *__restrict__ v, uint32_t n,
+                                                           DynState *dyn,
+                                                           const uint32_t *__restrict__ prompt,
+                                                           uint32_t *__restrict__ tokens_out) {
+    const uint32_t idx = block_argmax(v, n);
+    if (threadIdx.x == 0) {
+        const uint32_t pos = dyn->pos, cnt = dyn->count;
+        tokens_out[cnt] = idx;
+        dyn->token = (pos + 1 < dyn->n_prompt) ? prompt[pos + 1] : idx;
+        dyn->pos = pos + 1;
+        dyn->count = cnt + 1;
+    }
+}
+
+// state.x.copy_from_view(token_embd.column(token)) (wgml-chat/src/chat_llama2.rs:185-187)
+__global__ void embed_kernel(float *__restrict__ x, const float *__restrict__ table, uint32_t dim,
+                             DynPos token) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < dim) x[i] = table[(size_t)dyn_pos(token) * dim + i];
 }
 
 inline dim3 grid1(uint32_t n, uint32_t t = 256) { return dim3((n + t - 1) / t); }
@@ -262,6 +294,21 @@ int launch_op_assign(wgml_ctx *ctx, int op, float *a, const float *b, uint32_t n
 
 int launch_argmax(wgml_ctx *ctx, const float *v, uint32_t n, uint32_t *d_out) {
     argmax_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(v, n, d_out);
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
+int launch_embed(wgml_ctx *ctx, float *x, const float *table, uint32_t dim, DynPos token) {
+    embed_kernel<<<grid1(dim), dim3(256), 0, ctx->stream>>>(x, table, dim, token);
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
+int launch_argmax_next(wgml_ctx *ctx, const float *v, uint32_t n, DynState *dyn,
+                       const uint32_t *prompt, uint32_t *tokens_out) {
+    argmax_next_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(v, n, dyn, prompt, tokens_out);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;

@@ -23,6 +23,11 @@ int check_view(const wgml_view &v, const char *what) {
     return WGML_OK;
 }
 
+bool graphs_disabled() {
+    const char *v = getenv("WGML_DISABLE_GRAPHS");
+    return v && *v && strcmp(v, "0") != 0;
+}
+
 void ctx_retain(wgml_ctx *ctx) {
     if (ctx) ++ctx->refs;
 }
@@ -32,6 +37,7 @@ void ctx_release(wgml_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->attn_ws) (void)hipFree(ctx->attn_ws);
+    for (void *p : ctx->retired) (void)hipFree(p);
     if (ctx->d_scalar) (void)hipFree(ctx->d_scalar);
     if (ctx->h_scalar) (void)hipHostFree(ctx->h_scalar);
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);

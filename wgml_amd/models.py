@@ -171,6 +171,12 @@ class Llama2:
         call("wgml_llama2_decode_greedy", self._h, first_token, start_pos, n_steps, _ptr(out))
         return out
 
+    def decode_greedy_sync(self, first_token: int, start_pos: int, n_steps: int) -> np.ndarray:
+        """Same as decode_greedy with a host read-back of every token."""
+        out = np.empty(n_steps, dtype=np.uint32)
+        call("wgml_llama2_decode_greedy_sync", self._h, first_token, start_pos, n_steps, _ptr(out))
+        return out
+
     def kv_upload(self, layer: int, which: int, first_pos: int, data: np.ndarray) -> None:
         a = np.ascontiguousarray(data, dtype=np.float32)
         n_pos = a.size // self.config.kv_dim
