@@ -147,6 +147,9 @@ struct FusedGemv {
     DynPos pos{nullptr, 0};
     uint32_t head_size = 0;
     float rope_base = 10000.f;
+    // optional table of (cos, sin) pairs for the current position, one per rotated
+    // pair of a head (head_size / 2 entries); computed in-kernel when null
+    const float *rope_cs = nullptr;
 };
 bool gemv_fused_supported(const wgml_qmat *m);
 int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f);
@@ -172,7 +175,8 @@ int launch_argmax(wgml_ctx *ctx, const float *v, uint32_t n, uint32_t *d_out);
 struct DynState {
     uint32_t pos, token, count, n_prompt;
 };
-int launch_embed(wgml_ctx *ctx, float *x, const float *table, uint32_t dim, DynPos token);
+int launch_embed(wgml_ctx *ctx, float *x, const float *table, uint32_t dim, DynPos token,
+                 float *rope_cs, uint32_t head_size, float rope_base, DynPos pos);
 int launch_argmax_next(wgml_ctx *ctx, const float *v, uint32_t n, DynState *dyn,
                        const uint32_t *prompt, uint32_t *tokens_out);
 int launch_dequantize(wgml_ctx *ctx, float *out, const wgml_qmat *m);

@@ -659,17 +659,31 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, const Policy &
     }
 
     // Stage x as 16-bit block fixed point (two int8 planes) + per-block scale and sum.
+    // A fused RMSNorm costs no extra pass and no extra barrier: the normalisation
+    // factor rsqrt(mean(x^2) + eps) is one scalar for the whole vector, so x * w is
+    // staged, the sum of squares is gathered on the way and the factor multiplies
+    // the finished dot products instead.
+    __shared__ float red[16];
+    float out_scale = 1.f;
     if (!(p.debug & 1)) {
-        __shared__ float red[16];
-        float rms = 1.f;
-        if (p.norm_w) rms = block_rms_scale(p, red);
         const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
         const float4 *nw4 = reinterpret_cast<const float4 *>(p.norm_w);
         const uint32_t n4 = p.ncols >> 2;
         uint32_t *xq32 = reinterpret_cast<uint32_t *>(xq);
+        float ss = 0.f;
         for (uint32_t g4 = tid; g4 < n4; g4 += blockDim.x) {
             float4 v = x4[g4];
-            if (p.norm_w) v = apply_norm(v, rms, nw4[g4]);
+            if (p.norm_w) {
+                ss = fmaf(v.x, v.x, ss);
+                ss = fmaf(v.y, v.y, ss);
+                ss = fmaf(v.z, v.z, ss);
+                ss = fmaf(v.w, v.w, ss);
+                const float4 nw = nw4[g4];
+                v.x *= nw.x;
+                v.y *= nw.y;
+                v.z *= nw.z;
+                v.w *= nw.w;
+            }
             float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
             float sum;
             amax = dpp_max<0xB1>(amax);
@@ -704,7 +718,16 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, const Policy &
                 if (F::NSUM > 0) meta[tile * MF + F::NXB + xb] = sum;
             }
         }
+        if (p.norm_w) {
+            ss = wave_sum(ss);
+            if (lane == 0) red[wave] = ss;
+        }
         __syncthreads();
+        if (p.norm_w) {
+            float total = 0.f;
+            for (uint32_t k = 0; k < nwaves; ++k) total += red[k];
+            out_scale = 1.0f / sqrtf(total / (float)p.ncols + p.norm_eps);
+        }
     }
     if (n_it == 0) return;
 
@@ -734,6 +757,8 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, const Policy &
                     }
                 }
                 if (++step == nsteps) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) acc[r] *= out_scale;
                     pol.template store<R>(g, acc, lane);
 #pragma unroll
                     for (int r = 0; r < R; ++r) acc[r] = 0.f;
@@ -794,6 +819,7 @@ struct FusedParams {
     DynPos pos;
     uint32_t head_size;
     float rope_base;
+    const float2 *rope_cs;  // optional: (cos, sin) of the current position per pair of a head
 };
 
 struct JobPolicy {
@@ -801,6 +827,7 @@ struct JobPolicy {
     const GemvParams &pa, &pb;  // plane views of the two matrices
     uint32_t pos, head_size;
     float rope_base;
+    const float2 *rope_cs;
     __device__ uint32_t nrows() const { return j.nrows; }
     template <int R>
     __device__ uint32_t ngroups() const {
@@ -831,10 +858,16 @@ struct JobPolicy {
             t1 += j.bias[min(r1, j.nrows - 1)];
         }
         if (j.mode == JOB_ROPE) {
-            const float head_dim = (float)(r0 % head_size);
-            const float theta = powf(rope_base, -head_dim / (float)head_size);
             float sn, cs;
-            sincosf((float)pos * theta, &sn, &cs);
+            if (rope_cs) {
+                const float2 t = rope_cs[(r0 % head_size) >> 1];
+                cs = t.x;
+                sn = t.y;
+            } else {
+                const float head_dim = (float)(r0 % head_size);
+                const float theta = powf(rope_base, -head_dim / (float)head_size);
+                sincosf((float)pos * theta, &sn, &cs);
+            }
             const float x = t0, y = t1;
             t0 = cs * x - sn * y;
             t1 = sn * x + cs * y;
@@ -857,12 +890,13 @@ __device__ __forceinline__ void fused_job_body(const FusedParams &P, const GemvJ
     GemvParams pa = xp, pb = xp;
     pa.p0 = j.a0; pa.p1 = j.a1; pa.p2 = j.a2; pa.p3 = j.a3;
     pb.p0 = j.b0; pb.p1 = j.b1; pb.p2 = j.b2; pb.p3 = j.b3;
-    const JobPolicy pol{j, pa, pb, dyn_pos(P.pos), P.head_size, P.rope_base};
+    const JobPolicy pol{j, pa, pb, dyn_pos(P.pos), P.head_size, P.rope_base, P.rope_cs};
     gemv_i8_body<F, 2, D>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count);
 }
 
+// Register budget: 4 waves per SIMD, so that two 8-wave workgroups share a CU.
 template <int D, int MAXT>
-__global__ __launch_bounds__(MAXT) void gemv_fused_kernel(const FusedParams P) {
+__global__ __launch_bounds__(MAXT, 4) void gemv_fused_kernel(const FusedParams P) {
     int ji = 0;
     if (P.njobs > 1 && blockIdx.x >= P.jobs[1].wg_begin) ji = 1;
     if (P.njobs > 2 && blockIdx.x >= P.jobs[2].wg_begin) ji = 2;
@@ -961,7 +995,11 @@ int launch_kernel(wgml_ctx *ctx, const GemvParams &p, size_t lds, const void *fn
     // that the grid fits the machine.
     const uint32_t resident_waves = cu * (uint32_t)per_cu * nwaves;
     const uint32_t k = (ngroups + resident_waves - 1) / resident_waves;
-    const uint32_t grid = (ngroups + nwaves * k - 1) / (nwaves * k);
+    uint32_t grid = (ngroups + nwaves * k - 1) / (nwaves * k);
+    if (p.debug & 4) {  // experiment: fill the machine, waves differ by one group
+        grid = (ngroups + nwaves - 1) / nwaves;
+        if (grid > cu * (uint32_t)per_cu) grid = cu * (uint32_t)per_cu;
+    }
     kern<<<dim3(grid), dim3(MAXT), lds, ctx->stream>>>(p);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
@@ -1159,6 +1197,7 @@ int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
     P.pos = f.pos;
     P.head_size = f.head_size ? f.head_size : 2;
     P.rope_base = f.rope_base;
+    P.rope_cs = reinterpret_cast<const float2 *>(f.rope_cs);
     const uint32_t ncols = f.jobs[0].a->ncols;
     P.ncols = ncols;
     size_t lds = 0;

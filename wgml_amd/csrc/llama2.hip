@@ -41,6 +41,7 @@ struct wgml_llama2 {
     // Llama2State (models/llama2/transformer.rs:17-45)
     float *x = nullptr, *xb = nullptr, *xb2 = nullptr, *hb = nullptr, *hb2 = nullptr, *q = nullptr,
           *logits = nullptr;
+    float *rope_cs = nullptr;  // (cos, sin) of the current position, head_size/2 pairs
     // token-loop state on the device
     DynState *dyn = nullptr;
     uint32_t *d_prompt = nullptr, *d_tokens = nullptr;  // seq_len entries each
@@ -108,7 +109,9 @@ int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos) {
     const int fusion = m->fusion;
     const uint32_t plan = dynamic ? c.seq_len : pos + 1;
 
-    WGML_TRY(launch_embed(ctx, m->x, m->token_embd, dim, dtok));
+    // dim >= head_size / 2, so the embedding launch also covers the RoPE table
+    WGML_TRY(launch_embed(ctx, m->x, m->token_embd, dim, dtok, m->rope_cs, m->head_size,
+                          c.rope_base_freq, dpos));
 
     for (uint32_t l = 0; l < c.n_layers; ++l) {
         const LlamaLayer &w = m->layers[l];
@@ -126,6 +129,7 @@ int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos) {
             f.pos = dpos;
             f.head_size = m->head_size;
             f.rope_base = c.rope_base_freq;
+            f.rope_cs = m->rope_cs;
             f.jobs[0].a = w.attn_q;
             f.jobs[0].out = m->q;
             f.jobs[0].bias = w.bq;
@@ -386,6 +390,7 @@ int wgml_llama2_create(wgml_ctx *ctx, const wgml_llama2_config *cfg, int model_t
     A(&m->hb2, cfg->hidden_dim, true);
     A(&m->q, cfg->dim, true);
     A(&m->logits, cfg->vocab_size, true);
+    A(&m->rope_cs, head_size, true);
     for (auto &l : m->layers) {
         A(&l.key_cache, (uint64_t)m->kv_dim * cfg->seq_len, true);
         A(&l.value_cache, (uint64_t)m->kv_dim * cfg->seq_len, true);

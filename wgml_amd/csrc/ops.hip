@@ -223,10 +223,20 @@ __global__ __launch_bounds__(1024) void argmax_next_kernel(const float *__restri
 }
 
 // state.x.copy_from_view(token_embd.column(token)) (wgml-chat/src/chat_llama2.rs:185-187)
+// Also fills the step's RoPE table (if given): (cos, sin) of pos * theta_i for the
+// head_size/2 pairs of a head, with the angle formed exactly as ops/rope.wgsl:38-41.
 __global__ void embed_kernel(float *__restrict__ x, const float *__restrict__ table, uint32_t dim,
-                             DynPos token) {
+                             DynPos token, float2 *__restrict__ rope_cs, uint32_t head_size,
+                             float rope_base, DynPos pos) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < dim) x[i] = table[(size_t)dyn_pos(token) * dim + i];
+    if (rope_cs && i < head_size / 2) {
+        const float head_dim = (float)(2 * i);
+        const float theta = powf(rope_base, -head_dim / (float)head_size);
+        float sn, cs;
+        sincosf((float)dyn_pos(pos) * theta, &sn, &cs);
+        rope_cs[i] = make_float2(cs, sn);
+    }
 }
 
 inline dim3 grid1(uint32_t n, uint32_t t = 256) { return dim3((n + t - 1) / t); }
@@ -299,8 +309,10 @@ int launch_argmax(wgml_ctx *ctx, const float *v, uint32_t n, uint32_t *d_out) {
     return WGML_OK;
 }
 
-int launch_embed(wgml_ctx *ctx, float *x, const float *table, uint32_t dim, DynPos token) {
-    embed_kernel<<<grid1(dim), dim3(256), 0, ctx->stream>>>(x, table, dim, token);
+int launch_embed(wgml_ctx *ctx, float *x, const float *table, uint32_t dim, DynPos token,
+                 float *rope_cs, uint32_t head_size, float rope_base, DynPos pos) {
+    embed_kernel<<<grid1(dim), dim3(256), 0, ctx->stream>>>(
+        x, table, dim, token, reinterpret_cast<float2 *>(rope_cs), head_size, rope_base, pos);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
