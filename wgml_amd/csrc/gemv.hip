@@ -43,6 +43,9 @@ struct GemvParams {
     uint32_t out_pos_stride;
     const float *norm_w;  // optional fused RMSNorm of x
     float norm_eps;
+    // integer-dot kernels: the first `active_waves` waves of every workgroup walk
+    // the row-groups with stride gridDim.x * active_waves
+    uint32_t active_waves;
 };
 
 // Hides a value from the optimizer (no instruction is emitted).  Used on masked
@@ -603,30 +606,42 @@ struct IFmtQ8_0 {
 
 // Row source / sink of a plain single-matrix GEMV: group g = rows g*R .. g*R+R-1.
 struct PlainPolicy {
+    static constexpr int S = 1;  // passes per group
     const GemvParams &p;
-    __device__ uint32_t nrows() const { return p.nrows; }
-    template <int R>
-    __device__ uint32_t ngroups() const {
-        return (p.nrows + R - 1) / R;
-    }
     template <class WF, int R>
-    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t tile) const {
+    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t, uint32_t tile) const {
         load_group<WF, R>(w, p, g, tile);
     }
+    // Lane n holds finished result n of the segment that starts at group g0:
+    // result n belongs to row (g0 + (n / R) * GW) * R + n % R.
     template <int R>
-    __device__ void store(uint32_t g, const float (&acc)[R], uint32_t lane) const {
-        reduce_and_store<R>(p, g, acc, lane);
+    __device__ void finish(float mine, uint32_t n, uint32_t g0, uint32_t GW, uint32_t lane) {
+        const uint32_t row = (g0 + (lane / R) * GW) * R + lane % R;
+        if (lane < n && row < p.nrows) {
+            float *out = p.out;
+            if (p.dyn_pos) out += (size_t)(*p.dyn_pos) * p.out_pos_stride;
+            float v = mine;
+            if (p.bias) v += p.bias[row];
+            if (p.accumulate) v += out[row];
+            out[row] = v;
+        }
     }
 };
 
 // The body shared by the single-matrix and the fused multi-matrix kernels.  `p`
 // supplies x, ncols, the optional RMSNorm and the debug flags; `pol` the rows.
-// The workgroup is number `wg` of `nwg` working on this matrix.
+// The workgroup is number `wg` of the `nwg` that share the matrix; its waves
+// w < nw take the row-groups (wg * nw + w) + i * (nwg * nw) < ngroups, so that at
+// any time the machine reads one contiguous window of the matrix.  A group is
+// Policy::S passes over R rows each (a fused pair is two single-row passes of
+// the same wave).  The (group, pass, step) triples
+// of a wave form one sequence that is software-pipelined D deep.
 // LDS: uint4 xq[step][plane(2)][chunk(PCH)][lane(64)], then float meta[tile][MF].
 template <class F, int R, int D, class Policy>
-__device__ __forceinline__ void gemv_i8_body(const GemvParams &p, const Policy &pol, uint32_t wg,
-                                             uint32_t nwg) {
+__device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, uint32_t wg,
+                                             uint32_t nwg, uint32_t nw, uint32_t ngroups) {
     using WF = typename F::W;
+    constexpr int S = Policy::S;
     constexpr int PCH = F::TILE / 16;         // 16-byte chunks per plane per tile
     constexpr int MF = F::NXB + F::NSUM;      // floats of meta per tile
     constexpr int LPB = F::XB / 4;            // lanes (float4) per activation block
@@ -639,21 +654,43 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, const Policy &
     const uint32_t ntiles_pad = nsteps << 6;
     float *meta = reinterpret_cast<float *>(xq + (size_t)ntiles_pad * 2 * PCH);
 
-    const uint32_t gw = wg * nwaves + wave, GW = nwg * nwaves;
-    const uint32_t ngroups = pol.template ngroups<R>();
-    const uint32_t my_groups = gw < ngroups ? (ngroups - gw + GW - 1) / GW : 0;
-    const uint32_t n_it = my_groups * nsteps;
+    const uint32_t first = wg * nw + wave, GW = nwg * nw;
+    const uint32_t my_groups = (wave < nw && first < ngroups) ? (ngroups - first + GW - 1) / GW : 0;
+    const uint32_t n_it = my_groups * S * nsteps;
+
+    // The requests for x go out first, the first D weight requests after them: a
+    // wave's loads return in order, so x, a cache hit, is not held up behind the
+    // weights and is staged while they are in flight.
+    constexpr int XP = 3;  // float4 of x per thread requested up front
+    const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
+    const float4 *nw4 = reinterpret_cast<const float4 *>(p.norm_w);
+    const uint32_t n4 = p.ncols >> 2;
+    const bool stage = !(p.debug & 1);
+    float4 xv[XP], nv[XP];
+#pragma unroll
+    for (int i = 0; i < XP; ++i) {
+        const uint32_t g4 = tid + i * blockDim.x;
+        xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        nv[i] = make_float4(1.f, 1.f, 1.f, 1.f);
+        if (stage && g4 < n4) {
+            xv[i] = x4[g4];
+            if (p.norm_w) nv[i] = nw4[g4];
+        }
+    }
 
     typename WF::Row w[D][R];
-    uint32_t lg = gw, ls = 0;
+    uint32_t lg = first, lsub = 0, ls = 0;  // (group, pass, step) of the next load
 #pragma unroll
     for (int d = 0; d < D; ++d) {
         if ((uint32_t)d < n_it) {
             const uint32_t tile = ls * 64 + lane;
-            if (tile < ntiles) pol.template load<WF, R>(w[d], lg, tile);
+            if (tile < ntiles) pol.template load<WF, R>(w[d], lg, lsub, tile);
             if (++ls == nsteps) {
                 ls = 0;
-                lg += GW;
+                if (++lsub == S) {
+                    lsub = 0;
+                    lg += GW;
+                }
             }
         }
     }
@@ -665,20 +702,15 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, const Policy &
     // the finished dot products instead.
     __shared__ float red[16];
     float out_scale = 1.f;
-    if (!(p.debug & 1)) {
-        const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
-        const float4 *nw4 = reinterpret_cast<const float4 *>(p.norm_w);
-        const uint32_t n4 = p.ncols >> 2;
+    if (stage) {
         uint32_t *xq32 = reinterpret_cast<uint32_t *>(xq);
         float ss = 0.f;
-        for (uint32_t g4 = tid; g4 < n4; g4 += blockDim.x) {
-            float4 v = x4[g4];
+        auto stage_one = [&](uint32_t g4, float4 v, const float4 nw) {
             if (p.norm_w) {
                 ss = fmaf(v.x, v.x, ss);
                 ss = fmaf(v.y, v.y, ss);
                 ss = fmaf(v.z, v.z, ss);
                 ss = fmaf(v.w, v.w, ss);
-                const float4 nw = nw4[g4];
                 v.x *= nw.x;
                 v.y *= nw.y;
                 v.z *= nw.z;
@@ -717,21 +749,38 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, const Policy &
                 meta[tile * MF + xb] = amax * (1.0f / 32512.f);
                 if (F::NSUM > 0) meta[tile * MF + F::NXB + xb] = sum;
             }
+        };
+        // ncols is a multiple of the tile size, so the LPB lanes of a block are
+        // active together in every one of these branches
+#pragma unroll
+        for (int i = 0; i < XP; ++i) {
+            const uint32_t g4 = tid + i * blockDim.x;
+            if (g4 < n4) stage_one(g4, xv[i], nv[i]);
         }
+        for (uint32_t g4 = tid + XP * blockDim.x; g4 < n4; g4 += blockDim.x)
+            stage_one(g4, x4[g4], p.norm_w ? nw4[g4] : make_float4(1.f, 1.f, 1.f, 1.f));
         if (p.norm_w) {
             ss = wave_sum(ss);
             if (lane == 0) red[wave] = ss;
         }
         __syncthreads();
         if (p.norm_w) {
-            float total = 0.f;
-            for (uint32_t k = 0; k < nwaves; ++k) total += red[k];
+            // one LDS read per lane and a 16-lane DPP sum instead of a chain of
+            // dependent reads (a workgroup has at most 16 waves)
+            const float part = lane < nwaves ? red[lane] : 0.f;
+            const float total = readlane_f32(row16_sum(part), 0);
             out_scale = 1.0f / sqrtf(total / (float)p.ncols + p.norm_eps);
         }
     }
     if (n_it == 0) return;
 
-    uint32_t g = gw, step = 0;
+    // Finished row sums are parked one per lane (result n in lane n) and handed
+    // to the policy 64 at a time: the epilogue's loads and stores (bias, RoPE table,
+    // accumulate) would otherwise sit between the weight loads in flight, and a
+    // wave waits for its memory operations in order.
+    uint32_t g = first, sub = 0, step = 0;  // (group, pass, step) being computed
+    uint32_t nres = 0, gseg = first;
+    float mine = 0.f;
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
@@ -758,29 +807,45 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, const Policy &
                 }
                 if (++step == nsteps) {
 #pragma unroll
-                    for (int r = 0; r < R; ++r) acc[r] *= out_scale;
-                    pol.template store<R>(g, acc, lane);
-#pragma unroll
-                    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+                    for (int r = 0; r < R; ++r) {
+                        const float t = wave_sum(acc[r]) * out_scale;
+                        mine = lane == nres ? t : mine;
+                        ++nres;
+                        acc[r] = 0.f;
+                    }
                     step = 0;
-                    g += GW;
+                    if (++sub == S) {
+                        sub = 0;
+                        g += GW;
+                        if (nres + S * R > 64) {
+                            pol.template finish<R>(mine, nres, gseg, GW, lane);
+                            nres = 0;
+                            gseg = g;
+                        }
+                    }
                 }
+                // refill this register set with the triple D positions ahead
                 if (it + D < n_it) {
                     const uint32_t tile_n = ls * 64 + lane;
-                    if (tile_n < ntiles) pol.template load<WF, R>(w[d], lg, tile_n);
+                    if (tile_n < ntiles) pol.template load<WF, R>(w[d], lg, lsub, tile_n);
                     if (++ls == nsteps) {
                         ls = 0;
-                        lg += GW;
+                        if (++lsub == S) {
+                            lsub = 0;
+                            lg += GW;
+                        }
                     }
                 }
             }
         }
     }
+    if (nres) pol.template finish<R>(mine, nres, gseg, GW, lane);
 }
 
 template <class F, int R, int D, int MAXT>
 __global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p) {
-    gemv_i8_body<F, R, D>(p, PlainPolicy{p}, blockIdx.x, gridDim.x);
+    PlainPolicy pol{p};
+    gemv_i8_body<F, R, D>(p, pol, blockIdx.x, gridDim.x, p.active_waves, (p.nrows + R - 1) / R);
 }
 
 // ------------------------------------------------------------------------
@@ -807,6 +872,7 @@ struct GemvJob {
     int type, mode, accumulate;
     uint32_t out_pos_stride;
     uint32_t wg_begin, wg_count;  // workgroups assigned to this matrix
+    uint32_t active_waves;        // waves of a workgroup that walk its row pairs
 };
 
 struct FusedParams {
@@ -820,62 +886,67 @@ struct FusedParams {
     uint32_t head_size;
     float rope_base;
     const float2 *rope_cs;  // optional: (cos, sin) of the current position per pair of a head
+    int debug;
 };
 
+// A group is a pair of rows, done as two single-row passes of one wave:
+//   PLAIN / ROPE  rows 2g and 2g+1 of the matrix
+//   SILU          row g of the gate matrix, then row g of the up matrix
 struct JobPolicy {
+    static constexpr int S = 2;
     const GemvJob &j;
     const GemvParams &pa, &pb;  // plane views of the two matrices
     uint32_t pos, head_size;
     float rope_base;
     const float2 *rope_cs;
-    __device__ uint32_t nrows() const { return j.nrows; }
-    template <int R>
-    __device__ uint32_t ngroups() const {
-        static_assert(R == 2, "fused launches work on row pairs");
-        return j.mode == JOB_SILU ? j.nrows : (j.nrows + 1) / 2;
-    }
     template <class WF, int R>
-    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t tile) const {
-        if (j.mode == JOB_SILU) {
-            WF::load(w[0], WF::row_base(pa, g), tile);
-            WF::load(w[1], WF::row_base(pb, g), tile);
-        } else {
-            WF::load(w[0], WF::row_base(pa, min(2 * g, j.nrows - 1)), tile);
-            WF::load(w[1], WF::row_base(pa, min(2 * g + 1, j.nrows - 1)), tile);
-        }
+    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t sub, uint32_t tile) const {
+        static_assert(R == 1, "fused launches make single-row passes");
+        // plane pointers are picked one by one (wave-uniform selects): choosing between
+        // the two parameter blocks by reference would force them into memory
+        const bool second = j.mode == JOB_SILU && sub;
+        GemvParams q{};
+        q.p0 = second ? pb.p0 : pa.p0;
+        q.p1 = second ? pb.p1 : pa.p1;
+        q.p2 = second ? pb.p2 : pa.p2;
+        q.p3 = second ? pb.p3 : pa.p3;
+        q.ncols = pa.ncols;
+        const uint32_t row = j.mode == JOB_SILU ? g : min(2 * g + sub, j.nrows - 1);
+        WF::load(w[0], WF::row_base(q, row), tile);
     }
+    // Lanes 2i and 2i+1 hold the two pass results of group g0 + i * GW.
     template <int R>
-    __device__ void store(uint32_t g, const float (&acc)[R], uint32_t lane) const {
-        float t0 = wave_sum(acc[0]), t1 = wave_sum(acc[1]);
+    __device__ void finish(float mine, uint32_t n, uint32_t g0, uint32_t GW, uint32_t lane) {
+        const uint32_t g = g0 + (lane >> 1) * GW, sub = lane & 1;
+        const bool valid = lane < n;
         float *out = j.out + (size_t)pos * j.out_pos_stride;
         if (j.mode == JOB_SILU) {
-            if (lane == 0) out[g] = t1 * (t0 / (1.0f + expf(-t0)));
+            const float up = dpp_f32<0xB1>(mine);  // the neighbouring lane's value
+            if (valid && sub == 0) out[g] = up * (mine / (1.0f + expf(-mine)));
             return;
         }
-        const uint32_t r0 = 2 * g, r1 = r0 + 1;
-        if (j.bias) {
-            t0 += j.bias[min(r0, j.nrows - 1)];
-            t1 += j.bias[min(r1, j.nrows - 1)];
-        }
-        if (j.mode == JOB_ROPE) {
-            float sn, cs;
-            if (rope_cs) {
-                const float2 t = rope_cs[(r0 % head_size) >> 1];
-                cs = t.x;
-                sn = t.y;
-            } else {
-                const float head_dim = (float)(r0 % head_size);
-                const float theta = powf(rope_base, -head_dim / (float)head_size);
-                sincosf((float)pos * theta, &sn, &cs);
+        const uint32_t row = 2 * g + sub;
+        const bool store = valid && row < j.nrows;
+        float t = mine;
+        if (j.bias && store) t += j.bias[row];
+        if (j.mode == JOB_ROPE) {  // ROPE matrices have an even number of rows
+            const float other = dpp_f32<0xB1>(t);
+            float sn = 0.f, cs = 1.f;
+            if (store) {
+                if (rope_cs) {
+                    const float2 c = rope_cs[((row & ~1u) % head_size) >> 1];
+                    cs = c.x;
+                    sn = c.y;
+                } else {
+                    const float head_dim = (float)((row & ~1u) % head_size);
+                    const float theta = powf(rope_base, -head_dim / (float)head_size);
+                    sincosf((float)pos * theta, &sn, &cs);
+                }
             }
-            const float x = t0, y = t1;
-            t0 = cs * x - sn * y;
-            t1 = sn * x + cs * y;
+            // (x, y) = (even row, odd row):  x' = cs x - sn y,  y' = sn x + cs y
+            t = sub ? sn * other + cs * t : cs * t - sn * other;
         }
-        if (lane == 0) {
-            if (r0 < j.nrows) out[r0] = j.accumulate ? out[r0] + t0 : t0;
-            if (r1 < j.nrows) out[r1] = j.accumulate ? out[r1] + t1 : t1;
-        }
+        if (store) out[row] = j.accumulate ? out[row] + t : t;
     }
 };
 
@@ -887,16 +958,18 @@ __device__ __forceinline__ void fused_job_body(const FusedParams &P, const GemvJ
     xp.norm_w = P.norm_w;
     xp.norm_eps = P.norm_eps;
     xp.nrows = j.nrows;
+    xp.debug = P.debug;
     GemvParams pa = xp, pb = xp;
     pa.p0 = j.a0; pa.p1 = j.a1; pa.p2 = j.a2; pa.p3 = j.a3;
     pb.p0 = j.b0; pb.p1 = j.b1; pb.p2 = j.b2; pb.p3 = j.b3;
-    const JobPolicy pol{j, pa, pb, dyn_pos(P.pos), P.head_size, P.rope_base, P.rope_cs};
-    gemv_i8_body<F, 2, D>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count);
+    JobPolicy pol{j, pa, pb, dyn_pos(P.pos), P.head_size, P.rope_base, P.rope_cs};
+    const uint32_t ngroups = j.mode == JOB_SILU ? j.nrows : (j.nrows + 1) / 2;
+    gemv_i8_body<F, 1, D>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves, ngroups);
 }
 
-// Register budget: 4 waves per SIMD, so that two 8-wave workgroups share a CU.
-template <int D, int MAXT>
-__global__ __launch_bounds__(MAXT, 4) void gemv_fused_kernel(const FusedParams P) {
+// MINW: waves per SIMD the register budget must allow.
+template <int D, int MAXT, int MINW>
+__global__ __launch_bounds__(MAXT, MINW) void gemv_fused_kernel(const FusedParams P) {
     int ji = 0;
     if (P.njobs > 1 && blockIdx.x >= P.jobs[1].wg_begin) ji = 1;
     if (P.njobs > 2 && blockIdx.x >= P.jobs[2].wg_begin) ji = 2;
@@ -967,6 +1040,8 @@ int g_force_waves = 0;  // waves per workgroup, 0 = heuristic
 int g_force_depth = 0;  // pipeline depth, 0 = heuristic
 int g_force_wg_per_cu = 0;
 int g_debug_flags = 0;
+int g_fused_variant = 0;
+int g_force_active_waves = 0;
 int g_f32_activations = 0;  // 1: fp32-activation kernels instead of the integer-dot path
 constexpr size_t kMaxLds = 128 * 1024;
 
@@ -996,10 +1071,6 @@ int launch_kernel(wgml_ctx *ctx, const GemvParams &p, size_t lds, const void *fn
     const uint32_t resident_waves = cu * (uint32_t)per_cu * nwaves;
     const uint32_t k = (ngroups + resident_waves - 1) / resident_waves;
     uint32_t grid = (ngroups + nwaves * k - 1) / (nwaves * k);
-    if (p.debug & 4) {  // experiment: fill the machine, waves differ by one group
-        grid = (ngroups + nwaves - 1) / nwaves;
-        if (grid > cu * (uint32_t)per_cu) grid = cu * (uint32_t)per_cu;
-    }
     kern<<<dim3(grid), dim3(MAXT), lds, ctx->stream>>>(p);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
@@ -1017,15 +1088,58 @@ int launch_variant(wgml_ctx *ctx, const GemvParams &p, size_t lds) {
                                         cached_blocks);
 }
 
+// Shares `ngroups` row-groups out over at most `max_wgs` workgroups of up to
+// `max_waves` waves: every workgroup gets the same count c (the last one the
+// remainder), and the fewest waves are active that still give every wave at most
+// ceil(c / max_waves) groups, so that the waves of a workgroup finish together.
+struct WgPlan {
+    uint32_t groups_per_wg, active_waves, wgs;
+};
+WgPlan plan_groups(uint32_t ngroups, uint32_t max_wgs, uint32_t max_waves, uint32_t min_c = 1) {
+    if (ngroups == 0) return {1, 1, 1};
+    if (max_wgs < 1) max_wgs = 1;
+    uint32_t c = (ngroups + max_wgs - 1) / max_wgs;
+    // small matrices: a few groups per workgroup rather than one wave per workgroup
+    const uint32_t floor_c = max_waves < 4 ? max_waves : 4;
+    if (c < floor_c) c = floor_c;
+    if (c < min_c) c = min_c;
+    if (c > ngroups) c = ngroups;
+    const uint32_t wgs = (ngroups + c - 1) / c;
+    c = (ngroups + wgs - 1) / wgs;
+    const uint32_t k = (c + max_waves - 1) / max_waves;
+    uint32_t nw = (c + k - 1) / k;
+    if (g_force_active_waves > 0 && (uint32_t)g_force_active_waves <= max_waves)
+        nw = (uint32_t)g_force_active_waves;
+    return {c, nw, wgs};
+}
+
 template <class F, int R, int D, int MAXT>
-int launch_variant_i8(wgml_ctx *ctx, const GemvParams &p, size_t lds) {
+int launch_variant_i8(wgml_ctx *ctx, const GemvParams &p0, size_t lds) {
     static bool opted_in = false;
     static size_t cached_lds = ~size_t(0);
     static int cached_blocks = 0;
-    return launch_kernel<F, R, D, MAXT>(ctx, p, lds,
-                                        (const void *)gemv_quant_i8_kernel<F, R, D, MAXT>,
-                                        gemv_quant_i8_kernel<F, R, D, MAXT>, opted_in, cached_lds,
-                                        cached_blocks);
+    const void *fn = (const void *)gemv_quant_i8_kernel<F, R, D, MAXT>;
+    if (lds > 64 * 1024 && !opted_in) {
+        WGML_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)kMaxLds));
+        opted_in = true;
+    }
+    if (cached_lds != lds) {
+        int nb = 0;
+        WGML_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fn, MAXT, lds));
+        cached_blocks = nb > 0 ? nb : 1;
+        cached_lds = lds;
+    }
+    int per_cu = cached_blocks;
+    if (g_force_wg_per_cu > 0 && g_force_wg_per_cu < per_cu) per_cu = g_force_wg_per_cu;
+    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
+    const WgPlan plan = plan_groups((p0.nrows + R - 1) / R, cu * (uint32_t)per_cu, MAXT / 64);
+    GemvParams p = p0;
+    p.active_waves = plan.active_waves;
+    gemv_quant_i8_kernel<F, R, D, MAXT><<<dim3(plan.wgs), dim3(MAXT), lds, ctx->stream>>>(p);
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
 }
 
 template <class F, int R, int D>
@@ -1124,7 +1238,7 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
                       const GemvEpilogue &ep) {
     if ((uintptr_t)v % 16 != 0)
         return set_error(WGML_E_INVALID, "gemv_quant: the input vector must be 16-byte aligned");
-    GemvParams p;
+    GemvParams p{};
     p.p0 = m->p0;
     p.p1 = m->p1;
     p.p2 = m->p2;
@@ -1182,8 +1296,8 @@ bool gemv_fused_supported(const wgml_qmat *m) {
     return m && (m->type == WGML_Q4_K || m->type == WGML_Q6_K || m->type == WGML_Q8_0);
 }
 
-int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
-    constexpr int MAXT = 512, D = 2;
+template <int D, int MAXT, int MINW>
+static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
     constexpr uint32_t nwaves = MAXT / 64;
     if (f.njobs < 1 || f.njobs > 3)
         return set_error(WGML_E_INVALID, "gemv_fused: %d jobs", f.njobs);
@@ -1198,6 +1312,7 @@ int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
     P.head_size = f.head_size ? f.head_size : 2;
     P.rope_base = f.rope_base;
     P.rope_cs = reinterpret_cast<const float2 *>(f.rope_cs);
+    P.debug = g_debug_flags;
     const uint32_t ncols = f.jobs[0].a->ncols;
     P.ncols = ncols;
     size_t lds = 0;
@@ -1235,7 +1350,7 @@ int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
     if (lds > kMaxLds)
         return set_error(WGML_E_UNSUPPORTED, "gemv_fused: %u columns need %zu bytes of LDS", ncols,
                          lds);
-    const void *fn = (const void *)gemv_fused_kernel<D, MAXT>;
+    const void *fn = (const void *)gemv_fused_kernel<D, MAXT, MINW>;
     static bool opted_in = false;
     if (lds > 64 * 1024 && !opted_in) {
         WGML_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1252,24 +1367,52 @@ int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
     }
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
     const uint32_t resident = cu * (uint32_t)cached_blocks;
-    // Workgroups are shared out in proportion to the bytes each matrix streams, then
-    // trimmed so that every wave of a matrix gets the same number of row pairs.
-    uint32_t begin = 0;
+    // Every workgroup streams about the same number of bytes: the smallest per-
+    // workgroup budget T is searched for which the matrices together need no more
+    // workgroups than the machine holds at once.
+    double bpg[3], lo = 0.0, hi = 0.0;
     for (int i = 0; i < f.njobs; ++i) {
-        uint32_t share = (uint32_t)((double)resident * (double)bytes[i] / (double)total_bytes);
-        if (share < 1) share = 1;
-        const uint32_t max_wg = (ngroups[i] + nwaves - 1) / nwaves;
-        if (share > max_wg) share = max_wg;
-        const uint32_t k = (ngroups[i] + share * nwaves - 1) / (share * nwaves);
-        const uint32_t wgs = (ngroups[i] + nwaves * k - 1) / (nwaves * k);
-        P.jobs[i].wg_begin = begin;
-        P.jobs[i].wg_count = wgs;
-        begin += wgs;
+        bpg[i] = (double)bytes[i] / (double)ngroups[i];
+        hi += (double)bytes[i];
     }
-    gemv_fused_kernel<D, MAXT><<<dim3(begin), dim3(MAXT), lds, ctx->stream>>>(P);
+    auto wgs_needed = [&](double T) {
+        uint64_t n = 0;
+        for (int i = 0; i < f.njobs; ++i) {
+            uint64_t c = (uint64_t)(T / bpg[i]);
+            if (c < 1) c = 1;
+            n += (ngroups[i] + c - 1) / c;
+        }
+        return n;
+    };
+    for (int it = 0; it < 50; ++it) {
+        const double mid = 0.5 * (lo + hi);
+        if (wgs_needed(mid) <= resident) hi = mid; else lo = mid;
+    }
+    uint32_t begin = 0, max_nw = 1;
+    for (int i = 0; i < f.njobs; ++i) {
+        uint32_t c = (uint32_t)(hi / bpg[i]);
+        if (c < 1) c = 1;
+        const WgPlan plan = plan_groups(ngroups[i], (ngroups[i] + c - 1) / c, nwaves);
+        P.jobs[i].wg_begin = begin;
+        P.jobs[i].wg_count = plan.wgs;
+        P.jobs[i].active_waves = plan.active_waves;
+        if (plan.active_waves > max_nw) max_nw = plan.active_waves;
+        begin += plan.wgs;
+    }
+    (void)max_nw;
+    gemv_fused_kernel<D, MAXT, MINW><<<dim3(begin), dim3(MAXT), lds, ctx->stream>>>(P);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
+}
+
+int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
+    switch (g_fused_variant) {
+    case 1: return launch_gemv_fused_variant<2, 512, 2>(ctx, f);
+    case 2: return launch_gemv_fused_variant<3, 1024, 1>(ctx, f);
+    case 3: return launch_gemv_fused_variant<2, 512, 4>(ctx, f);
+    default: return launch_gemv_fused_variant<2, 1024, 1>(ctx, f);
+    }
 }
 
 }  // namespace wgml
@@ -1282,6 +1425,14 @@ WGML_API int wgml_debug_set_gemv_rows_per_wave(int r) {
     WGML_REQUIRE(r == 0 || r == 1 || r == 2,
                  "wgml_debug_set_gemv_rows_per_wave: %d not in {0,1,2}", r);
     g_force_r = r;
+    return WGML_OK;
+}
+WGML_API int wgml_debug_set_gemv_active_waves(int v) {
+    g_force_active_waves = v;
+    return WGML_OK;
+}
+WGML_API int wgml_debug_set_gemv_fused_variant(int v) {
+    g_fused_variant = v;
     return WGML_OK;
 }
 WGML_API int wgml_debug_set_gemv_flags(int f) {
