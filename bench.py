@@ -10,8 +10,10 @@ time (untimed), then exactly `--steps` greedy decode steps are timed: one step =
 one token = one pass over every weight.
 
 Prints ONE JSON line: decode tok/s, the HBM roofline of the dominant kernel
-(the Q4_K GEMV of the 11008x4096 gate/up projections) measured with HIP events
-on the library's own stream, a GEMV sweep at 4096x11008 for the three formats,
+(gemv_fused_kernel as launched for the gate/up projections: two Q4_K 11008x4096
+matrices, RMSNorm folded into the staging of x, SiLU gating in the epilogue)
+measured with HIP events on the library's own stream over the model's 32
+layers, a GEMV sweep at 4096x11008 for the three formats,
 and the CPU baseline (the single-threaded C restatement of the reference's CPU
 transformer) timed on this host on a bounded sample.
 
@@ -57,6 +59,37 @@ def time_gemv(W, gpu, mats, nrows, ncols, iters):
         us = ms.value * 1e3 / iters
         best = us if best is None else min(best, us)
     return best
+
+
+def time_gate_up(W, gpu, cfg, weights):
+    """Average GPU duration (us) of the decoder's fused gate/up launch, back to back over
+    every layer's own matrices (distinct memory, 1.6 GB in total), and its algorithmic bytes."""
+    from wgml_amd._lib import View, call
+
+    layers = weights.layers
+    gate = [W.GpuQuantMatrix(gpu, l["ffn_gate"].qtype, cfg.hidden_dim, cfg.dim, l["ffn_gate"].data)
+            for l in layers]
+    up = [W.GpuQuantMatrix(gpu, l["ffn_up"].qtype, cfg.hidden_dim, cfg.dim, l["ffn_up"].data)
+          for l in layers]
+    n = len(layers)
+    a = (C.c_void_p * n)(*[m.handle for m in gate])
+    b = (C.c_void_p * n)(*[m.handle for m in up])
+    modes = (C.c_int * 1)(2)
+    out = W.GpuVector.uninit(gpu, cfg.hidden_dim)
+    x = W.GpuVector.init(gpu, W.rng_normal(99, cfg.dim))
+    nw = W.GpuVector.init(gpu, layers[0]["ffn_norm"])
+    nwv = nw.view()
+    ms = C.c_float()
+    best = None
+    iters = 4 * n
+    for _ in range(3):
+        call("wgml_bench_gemv_fused", gpu.handle, a, b, modes, 1, n, out.view(), cfg.hidden_dim,
+             x.view(), C.byref(nwv), iters, C.byref(ms))
+        us = ms.value * 1e3 / iters
+        best = us if best is None else min(best, us)
+    # W_gate + W_up (GGUF bytes) + x + norm weights (f32) in, hidden_dim f32 out
+    nbytes = gate[0].gguf_bytes() + up[0].gguf_bytes() + 4 * cfg.dim * 2 + 4 * cfg.hidden_dim
+    return best, nbytes
 
 
 def gemv_sweep(W, gpu, nrows, ncols, min_total_bytes=640 << 20):
@@ -107,6 +140,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--cpu-steps", type=int, default=0, help="CPU baseline steps (0 = auto)")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="only the dominant-kernel measurement (for profiler runs): the fused "
+                         "gate/up launches, then three plain copies of 256 MiB (op_assign Copy) "
+                         "as the known-size kernel that calibrates the HBM byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every kernel uses a single device; "
@@ -134,6 +171,19 @@ def main():
                           if (l + 1) % 8 == 0 else None)
     log(f"weights built in {time.perf_counter() - t0:.0f}s "
         f"({weights.weight_bytes_per_token() / 1e9:.3f} GB per token)")
+    if args.roofline_only:
+        us, b = time_gate_up(W, gpu, cfg, weights)
+        n = 64 << 20
+        src = W.GpuVector.init(gpu, np.zeros(n, np.float32))
+        dst = W.GpuVector.uninit(gpu, n)
+        for _ in range(3):
+            W.OpAssign(gpu, W.OpAssignVariant.Copy).dispatch(dst, src)
+        gpu.synchronize()
+        print(json.dumps({"kernel": "gemv_fused_kernel gate+up", "us_per_launch": round(us, 3),
+                          "bytes_per_launch": b, "GB/s": round(b / us * 1e-3, 1),
+                          "calibration": "op_assign Copy of 67108864 f32: 268435456 B read, "
+                                         "268435456 B written per launch"}), flush=True)
+        return
     model = Llama2(gpu, cfg).load(weights)
     prompt = W.prompt_tokens(4, args.warmup, cfg.vocab_size)
 
@@ -170,25 +220,31 @@ def main():
         f"{model.launches_per_token()} launches/token; with a host read-back per token: "
         f"{tok_s_sync:.1f} tok/s")
 
-    # dominant kernel: Q4_K GEMV of the gate/up projections, timed live over the model's own
-    # per-layer matrices (distinct memory, > last-level cache in total)
+    # dominant kernel: the fused gate/up launch (27% of a step), timed live over the model's
+    # own per-layer matrices; the plain single-matrix Q4_K GEMV of the same shape beside it
     roofline = None
     if args.model == "7b":
-        gate = [W.GpuQuantMatrix(gpu, W.Q4_K, cfg.hidden_dim, cfg.dim, l["ffn_gate"].data)
-                for l in weights.layers[:24]]
-        us = time_gemv(W, gpu, gate, cfg.hidden_dim, cfg.dim, iters=4 * len(gate))
-        b = gemv_bytes(gate[0].gguf_bytes(), cfg.hidden_dim, cfg.dim)
+        us, b = time_gate_up(W, gpu, cfg, weights)
         gbs = b / us * 1e-3
         traffic = None
         tpath = os.path.join(ROOT, "profiles", "traffic.json")
         if os.path.exists(tpath):
-            traffic = json.load(open(tpath)).get("gemv_q4_k_11008x4096_bytes_per_launch")
+            traffic = json.load(open(tpath)).get("gemv_fused_gate_up_bytes_per_launch")
+        gate = [W.GpuQuantMatrix(gpu, W.Q4_K, cfg.hidden_dim, cfg.dim, l["ffn_gate"].data)
+                for l in weights.layers[:24]]
+        us1 = time_gemv(W, gpu, gate, cfg.hidden_dim, cfg.dim, iters=4 * len(gate))
+        b1 = gemv_bytes(gate[0].gguf_bytes(), cfg.hidden_dim, cfg.dim)
+        del gate
         roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                    "kernel": "gemv_quant_kernel<FmtQ4K,4> 11008x4096", "bytes_per_launch": b,
-                    "us_per_launch": round(us, 3)}
-        log(f"dominant kernel Q4_K gemv 11008x4096: {us:.2f} us, {gbs:.0f} GB/s")
-        del gate
+                    "kernel": "gemv_fused_kernel, gate+up launch: 2 x Q4_K 11008x4096, RMSNorm "
+                              "folded into staging, SiLU epilogue",
+                    "bytes_per_launch": b, "us_per_launch": round(us, 3),
+                    "plain_gemv_q4_k_11008x4096": {"us_per_launch": round(us1, 3),
+                                                   "bytes_per_launch": b1,
+                                                   "GB/s": round(b1 / us1 * 1e-3, 1)}}
+        log(f"dominant kernel gemv_fused_kernel gate+up: {us:.2f} us, {gbs:.0f} GB/s; "
+            f"plain Q4_K gemv 11008x4096: {us1:.2f} us, {b1 / us1 * 1e-3:.0f} GB/s")
 
     sweep = None
     if not args.no_sweep and args.model == "7b":

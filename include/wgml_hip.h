@@ -268,9 +268,11 @@ WGML_API int wgml_llama2_kv_download(wgml_llama2 *m, uint32_t layer, int which,
 /* Number of kernel launches one forward enqueues (diagnostics). */
 WGML_API int wgml_llama2_launches_per_token(const wgml_llama2 *m);
 /* 0: one launch per reference op (mirrors Llama2::dispatch one to one);
- * 1: bias and residual adds folded into the GEMV epilogues; 2 (default): also
- * every RMSNorm folded into the GEMVs that consume it.  All levels give the
- * same results to fp32 rounding. */
+ * 1: bias and residual adds folded into the GEMV epilogues; 2: also every
+ * RMSNorm folded into the GEMVs that consume it; 3 (default): also Q, K and V
+ * (with bias, RoPE and the KV-cache write) in one launch and gate and up (with
+ * the SiLU gating) in one launch.  All levels give the same results to fp32
+ * rounding. */
 WGML_API int wgml_llama2_set_fusion(wgml_llama2 *m, int level);
 
 /* ---- GPT-2: Gpt2 / Gpt2State / Gpt2Weights -------------------------------- */
@@ -315,6 +317,19 @@ WGML_API int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uin
 WGML_API int wgml_bench_gemv_quant(wgml_ctx *ctx, const wgml_qmat *const *mats, uint32_t n_mats,
                                    wgml_view out, wgml_view v, uint32_t iters, int use_graph,
                                    float *total_ms);
+
+/* The same loop for the fused launches of the decoder: launch i covers the
+ * `njobs` (1..3) matrices a[(i % nsets) * njobs + j], all consuming `v` (RMS-
+ * normalised with `norm_w` first when norm_w->buf is non-null), job j writing
+ * out[j * stride ..].  modes[j]: 0 plain rows, 1 adjacent row pairs rotated as by
+ * RoPE at position 0 with head size 128, 2 SiLU-gated: b[...] holds the `up`
+ * matrix that goes with the `gate` matrix in a[...] (null entries otherwise).
+ * These are the launches Llama2::dispatch's Q/K/V and gate/up GEMVs
+ * (models/llama2/transformer.rs:261-374) are folded into. */
+WGML_API int wgml_bench_gemv_fused(wgml_ctx *ctx, const wgml_qmat *const *a,
+                                   const wgml_qmat *const *b, const int *modes, uint32_t njobs,
+                                   uint32_t nsets, wgml_view out, uint32_t stride, wgml_view v,
+                                   const wgml_view *norm_w, uint32_t iters, float *total_ms);
 
 /* ---- host-side input makers (no device needed) ---------------------------- *
  * The reference only de-quantizes; its inputs come from GGUF files written by

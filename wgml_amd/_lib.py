@@ -129,6 +129,8 @@ PROTOTYPES = {
     "wgml_gpt2_read_logits": (_i, [_P, _P]),
     "wgml_gpt2_generate_greedy": (_i, [_P, _P, _u32, _u32, _P]),
     "wgml_bench_gemv_quant": (_i, [_P, _PP, _u32, View, View, _u32, _i, _fp]),
+    "wgml_bench_gemv_fused": (_i, [_P, _PP, _PP, C.POINTER(C.c_int), _u32, _u32, View, _u32, View,
+                                   C.POINTER(View), _u32, _fp]),
     "wgml_quantize": (_i, [_i, _P, _P, _u64, _i]),
     "wgml_rng_normal": (_i, [_u64, _P, _u64, _f, _f, _i]),
     "wgml_rng_uniform_u32": (_i, [_u64, _P, _u64, _u32]),
@@ -136,6 +138,9 @@ PROTOTYPES = {
     "wgml_debug_set_gemv_rows_per_wave": (_i, [_i]),
     "wgml_debug_set_gemv_config": (_i, [_i, _i, _i, _i]),
     "wgml_debug_set_gemv_f32_activations": (_i, [_i]),
+    "wgml_debug_set_gemv_flags": (_i, [_i]),
+    "wgml_debug_set_gemv_fused_variant": (_i, [_i]),
+    "wgml_debug_set_gemv_active_waves": (_i, [_i]),
 }
 
 # calls whose return value is not a status code

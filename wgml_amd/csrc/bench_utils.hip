@@ -64,26 +64,22 @@ int wgml_bench_gemv_quant(wgml_ctx *ctx, const wgml_qmat *const *mats, uint32_t 
     return WGML_OK;
 }
 
-// Back-to-back fused launches (debug / tuning aid): `nsets` sets of `njobs`
-// matrices; job j of a set writes out[j * stride ..].  b[] holds the second matrix
-// of SILU jobs (null otherwise).
-WGML_API int wgml_debug_bench_gemv_fused(wgml_ctx *ctx, const wgml_qmat *const *a,
-                                         const wgml_qmat *const *b, const int *modes,
-                                         uint32_t njobs, uint32_t nsets, wgml_view out,
-                                         uint32_t stride, wgml_view v, const wgml_view *norm_w,
-                                         uint32_t iters, float *total_ms) {
+int wgml_bench_gemv_fused(wgml_ctx *ctx, const wgml_qmat *const *a,
+                          const wgml_qmat *const *b, const int *modes, uint32_t njobs,
+                          uint32_t nsets, wgml_view out, uint32_t stride, wgml_view v,
+                          const wgml_view *norm_w, uint32_t iters, float *total_ms) {
     WGML_REQUIRE(ctx && a && modes && total_ms && njobs >= 1 && njobs <= 3 && nsets > 0 && iters > 0,
-                 "wgml_debug_bench_gemv_fused: bad argument");
-    WGML_TRY(check_view(out, "wgml_debug_bench_gemv_fused: out"));
-    WGML_TRY(check_view(v, "wgml_debug_bench_gemv_fused: v"));
-    WGML_REQUIRE((uint64_t)stride * njobs <= out.len, "wgml_debug_bench_gemv_fused: out too small");
+                 "wgml_bench_gemv_fused: bad argument");
+    WGML_TRY(check_view(out, "wgml_bench_gemv_fused: out"));
+    WGML_TRY(check_view(v, "wgml_bench_gemv_fused: v"));
+    WGML_REQUIRE((uint64_t)stride * njobs <= out.len, "wgml_bench_gemv_fused: out too small");
     std::vector<FusedGemv> sets(nsets);
     for (uint32_t s = 0; s < nsets; ++s) {
         FusedGemv &f = sets[s];
         f.njobs = (int)njobs;
         f.x = view_ptr(v);
         if (norm_w && norm_w->buf) {
-            WGML_TRY(check_view(*norm_w, "wgml_debug_bench_gemv_fused: norm_w"));
+            WGML_TRY(check_view(*norm_w, "wgml_bench_gemv_fused: norm_w"));
             f.norm_w = view_ptr(*norm_w);
             f.norm_eps = 1e-5f;
         }
@@ -91,7 +87,7 @@ WGML_API int wgml_debug_bench_gemv_fused(wgml_ctx *ctx, const wgml_qmat *const *
         for (uint32_t j = 0; j < njobs; ++j) {
             const wgml_qmat *m = a[s * njobs + j];
             WGML_REQUIRE(m && m->ncols == v.len && m->nrows <= stride,
-                         "wgml_debug_bench_gemv_fused: matrix %u/%u does not fit", s, j);
+                         "wgml_bench_gemv_fused: matrix %u/%u does not fit", s, j);
             f.jobs[j].a = m;
             f.jobs[j].b = b ? b[s * njobs + j] : nullptr;
             f.jobs[j].mode = modes[j];
@@ -100,6 +96,14 @@ WGML_API int wgml_debug_bench_gemv_fused(wgml_ctx *ctx, const wgml_qmat *const *
     }
     for (uint32_t s = 0; s < nsets && s < iters; ++s) WGML_TRY(launch_gemv_fused(ctx, sets[s]));
     WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    if (graphs_disabled()) {
+        WGML_CHECK_HIP(hipEventRecord(ctx->ev_start, ctx->stream));
+        for (uint32_t i = 0; i < iters; ++i) WGML_TRY(launch_gemv_fused(ctx, sets[i % nsets]));
+        WGML_CHECK_HIP(hipEventRecord(ctx->ev_stop, ctx->stream));
+        WGML_CHECK_HIP(hipEventSynchronize(ctx->ev_stop));
+        WGML_CHECK_HIP(hipEventElapsedTime(total_ms, ctx->ev_start, ctx->ev_stop));
+        return WGML_OK;
+    }
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
@@ -121,7 +125,7 @@ WGML_API int wgml_debug_bench_gemv_fused(wgml_ctx *ctx, const wgml_qmat *const *
     if (exec) (void)hipGraphExecDestroy(exec);
     if (graph) (void)hipGraphDestroy(graph);
     if (e != hipSuccess)
-        return set_error(WGML_E_HIP, "wgml_debug_bench_gemv_fused: %s", hipGetErrorString(e));
+        return set_error(WGML_E_HIP, "wgml_bench_gemv_fused: %s", hipGetErrorString(e));
     return WGML_OK;
 }
 
