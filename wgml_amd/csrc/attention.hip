@@ -12,8 +12,18 @@
 // workspace and a second, tiny kernel.  With few positions a single workgroup
 // per head group writes the result directly.
 //
-// Lane layout: lane L holds dimensions L, L+64, L+128, ... of a head
-// (coalesced 256-byte loads per K/V row segment).
+// Lane layout of the general kernel: lane L holds dimensions L, L+64, L+128, ...
+// of a head (coalesced 256-byte loads per K/V row segment).
+//
+// Fast kernel (no score output wanted, head size a multiple of 4, 16-byte aligned
+// operands): 16 lanes share a position (float4 loads, 16-lane DPP reductions), a
+// wave works on 4 positions at a time and keeps 16 positions in flight; the chunk
+// per wave is derived from the current position on the device, so every wave of
+// a recorded launch has work at any position.  Up to 128 positions one 16-wave
+// workgroup per head group does everything and writes the result (one launch, no
+// workspace); beyond that 4-wave workgroups write partials for the merge kernel.
+// (Merging in the workgroup that arrives last was tried and dropped: every
+// device-scope fence is an L2 write-back here, 20 us per launch.)
 #include "common.h"
 #include "device_utils.h"
 
@@ -29,6 +39,7 @@ struct AttnArgs {
     uint32_t seq_len, kv_dim, kv_mul, n_heads, head_size;
     DynPos pos;
     uint32_t chunk;  // positions per wave
+    uint32_t spec_rows;  // rows of the caches that exist (may be read before pos is known)
     uint32_t n_wg_y;
     int direct;  // 1: grid.y == 1 and the workgroup writes xb itself
 };
@@ -146,35 +157,251 @@ __global__ __launch_bounds__(WAVES * 64) void attn_split_kernel(const AttnArgs a
     }
 }
 
+// Fast kernel: positions are dealt out in quads (4 consecutive positions, one per
+// 16-lane row of a wave); quad Q belongs to wave Q % (n_wg_y * nw) of the head
+// group, counted over the workgroups.  The assignment does not depend on the
+// current position, so the loads for a wave's first quads can be requested before
+// the position is known.
+__device__ __forceinline__ uint32_t fast_n_used(uint32_t pos, uint32_t n_wg_y, uint32_t nw) {
+    const uint32_t nq = pos / 4 + 1;  // quads that hold a position <= pos
+    return min(n_wg_y, (nq + nw - 1) / nw);
+}
+
 // Merges the per-workgroup partials of one head; optionally normalises `att`.
+// All partials are requested at once (a loop of dependent loads would cost one
+// memory round trip per partial).
+constexpr int MERGE_MAX_Y = 64;
 __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnArgs a, uint32_t hsp) {
+    __shared__ float sm_w[MERGE_MAX_Y];
+    __shared__ float sm_ML[2];
     const uint32_t h = blockIdx.x;
     const uint32_t pos = dyn_pos(a.pos);
     const uint32_t stride = 2 + hsp;
     const float *base = a.ws + (size_t)h * a.n_wg_y * stride;
-    // workgroups whose chunks start beyond pos hold empty partials
-    const uint32_t per_wg = a.chunk * WAVES;
-    const uint32_t n_used = min(a.n_wg_y, pos / per_wg + 1);
-    float M = -INFINITY;
-    for (uint32_t y = 0; y < n_used; ++y) M = fmaxf(M, base[(size_t)y * stride]);
-    float L = 0.f;
-    for (uint32_t y = 0; y < n_used; ++y) {
-        const float my = base[(size_t)y * stride];
-        const float wgt = my == -INFINITY ? 0.f : __expf(my - M);
-        L = fmaf(base[(size_t)y * stride + 1], wgt, L);
-    }
-    for (uint32_t d = threadIdx.x; d < a.head_size; d += blockDim.x) {
-        float o = 0.f;
+    // workgroups whose positions start beyond pos hold no partial
+    // (chunk == 0: partials of the fast kernel)
+    const uint32_t n_used = a.chunk ? min(a.n_wg_y, pos / (a.chunk * WAVES) + 1)
+                                    : fast_n_used(pos, a.n_wg_y, WAVES);
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    float M, L;
+    if (n_used <= MERGE_MAX_Y) {
+        if (tid < 64) {  // wave 0: one partial per lane
+            const float my = lane < n_used ? base[(size_t)lane * stride] : -INFINITY;
+            const float ly = lane < n_used ? base[(size_t)lane * stride + 1] : 0.f;
+            const float mm = wave_max(my);
+            const float wgt = my == -INFINITY ? 0.f : __expf(my - mm);
+            const float ll = wave_sum(ly * wgt);
+            sm_w[lane] = wgt;
+            if (lane == 0) {
+                sm_ML[0] = mm;
+                sm_ML[1] = ll;
+            }
+        }
+        __syncthreads();
+        M = sm_ML[0];
+        L = sm_ML[1];
+        for (uint32_t d = tid; d < a.head_size; d += blockDim.x) {
+            float o = 0.f;
+            for (uint32_t y0 = 0; y0 < n_used; y0 += 8) {
+                float v[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    v[k] = y0 + k < n_used ? base[(size_t)(y0 + k) * stride + 2 + d] : 0.f;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) o = fmaf(v[k], y0 + k < n_used ? sm_w[y0 + k] : 0.f, o);
+            }
+            a.xb[(size_t)h * a.head_size + d] = o / L;
+        }
+    } else {
+        M = -INFINITY;
+        for (uint32_t y = 0; y < n_used; ++y) M = fmaxf(M, base[(size_t)y * stride]);
+        L = 0.f;
         for (uint32_t y = 0; y < n_used; ++y) {
             const float my = base[(size_t)y * stride];
             const float wgt = my == -INFINITY ? 0.f : __expf(my - M);
-            o = fmaf(base[(size_t)y * stride + 2 + d], wgt, o);
+            L = fmaf(base[(size_t)y * stride + 1], wgt, L);
         }
-        a.xb[(size_t)h * a.head_size + d] = o / L;
+        for (uint32_t d = tid; d < a.head_size; d += blockDim.x) {
+            float o = 0.f;
+            for (uint32_t y = 0; y < n_used; ++y) {
+                const float my = base[(size_t)y * stride];
+                const float wgt = my == -INFINITY ? 0.f : __expf(my - M);
+                o = fmaf(base[(size_t)y * stride + 2 + d], wgt, o);
+            }
+            a.xb[(size_t)h * a.head_size + d] = o / L;
+        }
     }
     if (a.att) {
         float *att = a.att + (size_t)h * a.seq_len;
-        for (uint32_t t = threadIdx.x; t <= pos; t += blockDim.x) att[t] = expf(att[t] - M) / L;
+        for (uint32_t t = tid; t <= pos; t += blockDim.x) att[t] = expf(att[t] - M) / L;
+    }
+}
+
+// ---------------------------------------------------------------- fast kernel
+__device__ __forceinline__ float dot4(const float4 a, const float4 b, float acc) {
+    acc = fmaf(a.x, b.x, acc);
+    acc = fmaf(a.y, b.y, acc);
+    acc = fmaf(a.z, b.z, acc);
+    return fmaf(a.w, b.w, acc);
+}
+__device__ __forceinline__ float4 axpby4(const float4 a, float sa, const float4 b, float sb) {
+    return make_float4(fmaf(a.x, sa, b.x * sb), fmaf(a.y, sa, b.y * sb), fmaf(a.z, sa, b.z * sb),
+                       fmaf(a.w, sa, b.w * sb));
+}
+__device__ __forceinline__ float shfl_xor_f32(float v, int mask) { return __shfl_xor(v, mask, 64); }
+
+template <int NV4, int KM, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
+    constexpr int HSP = NV4 * 64;  // dimension capacity: 16 lanes x 4 x NV4
+    __shared__ float sm_m[NW][KM], sm_l[NW][KM];
+    __shared__ float sm_acc[NW][KM][HSP];
+
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t sub = lane & 15, quarter = lane >> 4;
+    const uint32_t hs = a.head_size;
+    const uint32_t h0 = blockIdx.x * KM;
+    const uint32_t kvh = h0 / a.kv_mul;
+    const uint32_t gid = blockIdx.y * NW + wave, total = a.n_wg_y * NW;
+    const float inv_sqrt_hs = 1.0f / sqrtf((float)hs);
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float *kb = a.kc + (size_t)kvh * hs;
+    const float *vb = a.vc + (size_t)kvh * hs;
+    bool dv[NV4];  // this lane's float4 number v lies inside the head
+#pragma unroll
+    for (int v = 0; v < NV4; ++v) dv[v] = (sub + 16 * v) * 4 < hs;
+
+    // This wave's quads are gid, gid + total, ...; a batch is four of them.  The
+    // first quad is requested before the position is known (`spec_rows` rows of the
+    // caches may be read; rows beyond the position are masked out below), the
+    // others once it is, and only those that hold a position <= pos.
+    float4 kr[4][NV4], vr[4][NV4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+#pragma unroll
+        for (int v = 0; v < NV4; ++v) kr[u][v] = vr[u][v] = zero4;
+    }
+    auto request = [&](uint32_t i0, uint32_t last, int u_begin, uint32_t nq_limit) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t quad = (i0 + u) * total + gid;
+            if (u >= u_begin && quad < nq_limit) {  // uniform over the wave
+                const uint32_t tt = min(quad * 4 + quarter, last);
+                const float4 *kp = reinterpret_cast<const float4 *>(kb + (size_t)tt * a.kv_dim);
+                const float4 *vp = reinterpret_cast<const float4 *>(vb + (size_t)tt * a.kv_dim);
+#pragma unroll
+                for (int v = 0; v < NV4; ++v) kr[u][v] = dv[v] ? kp[sub + 16 * v] : zero4;
+#pragma unroll
+                for (int v = 0; v < NV4; ++v) vr[u][v] = dv[v] ? vp[sub + 16 * v] : zero4;
+            }
+        }
+    };
+    const bool spec = gid * 4 < a.spec_rows;
+    if (spec) request(0, a.spec_rows - 1, 0, gid + 1);
+
+    float4 q[KM][NV4], acc[KM][NV4];
+    float mx[KM], l[KM];
+#pragma unroll
+    for (int m = 0; m < KM; ++m) {
+        mx[m] = -INFINITY;
+        l[m] = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV4; ++v) {
+            q[m][v] = dv[v] ? reinterpret_cast<const float4 *>(a.q + (size_t)(h0 + m) * hs)[sub + 16 * v]
+                            : zero4;
+            acc[m][v] = zero4;
+        }
+    }
+
+    const uint32_t pos = dyn_pos(a.pos);
+    const uint32_t n_used = fast_n_used(pos, a.n_wg_y, NW);  // workgroups with work
+    if (blockIdx.y >= n_used) return;
+    const uint32_t nq = pos / 4 + 1;
+    for (uint32_t i0 = 0; i0 * total + gid < nq; i0 += 4) {
+        if (i0 == 0)
+            request(0, pos, spec ? 1 : 0, nq);
+        else
+            request(i0, pos, 0, nq);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            // uniform within each 16-lane row, so the row reductions below see whole rows
+            if (((i0 + u) * total + gid) * 4 + quarter <= pos) {
+#pragma unroll
+                for (int m = 0; m < KM; ++m) {
+                    float part = 0.f;
+#pragma unroll
+                    for (int v = 0; v < NV4; ++v) part = dot4(q[m][v], kr[u][v], part);
+                    const float s = row16_sum(part) * inv_sqrt_hs;
+                    const float mn = fmaxf(mx[m], s);
+                    const float sc = __expf(mx[m] - mn);
+                    const float p = __expf(s - mn);
+                    l[m] = fmaf(l[m], sc, p);
+#pragma unroll
+                    for (int v = 0; v < NV4; ++v) acc[m][v] = axpby4(acc[m][v], sc, vr[u][v], p);
+                    mx[m] = mn;
+                }
+            }
+        }
+    }
+
+    // merge the four quarters of the wave (every lane ends up with the merged state)
+#pragma unroll
+    for (int step = 16; step <= 32; step <<= 1) {
+#pragma unroll
+        for (int m = 0; m < KM; ++m) {
+            const float om = shfl_xor_f32(mx[m], step), ol = shfl_xor_f32(l[m], step);
+            const float M = fmaxf(mx[m], om);
+            const float sa = mx[m] == -INFINITY ? 0.f : __expf(mx[m] - M);
+            const float sb = om == -INFINITY ? 0.f : __expf(om - M);
+            l[m] = fmaf(l[m], sa, ol * sb);
+#pragma unroll
+            for (int v = 0; v < NV4; ++v) {
+                float4 o;
+                o.x = shfl_xor_f32(acc[m][v].x, step);
+                o.y = shfl_xor_f32(acc[m][v].y, step);
+                o.z = shfl_xor_f32(acc[m][v].z, step);
+                o.w = shfl_xor_f32(acc[m][v].w, step);
+                acc[m][v] = axpby4(acc[m][v], sa, o, sb);
+            }
+            mx[m] = M;
+        }
+    }
+    // merge the waves of this workgroup
+#pragma unroll
+    for (int m = 0; m < KM; ++m) {
+        if (lane == 0) {
+            sm_m[wave][m] = mx[m];
+            sm_l[wave][m] = l[m];
+        }
+        if (quarter == 0) {
+#pragma unroll
+            for (int v = 0; v < NV4; ++v)
+                reinterpret_cast<float4 *>(&sm_acc[wave][m][0])[sub + 16 * v] = acc[m][v];
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < KM * HSP; i += blockDim.x) {
+        const uint32_t m = i / HSP, d = i % HSP;
+        float M = sm_m[0][m];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) M = fmaxf(M, sm_m[w][m]);
+        float L = 0.f, o = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const float mw = sm_m[w][m];
+            const float wgt = mw == -INFINITY ? 0.f : __expf(mw - M);
+            L = fmaf(sm_l[w][m], wgt, L);
+            o = fmaf(sm_acc[w][m][d], wgt, o);
+        }
+        if (a.n_wg_y == 1) {
+            if (d < hs) a.xb[(size_t)(h0 + m) * hs + d] = o / L;
+        } else {
+            float *p = a.ws + ((size_t)(h0 + m) * a.n_wg_y + blockIdx.y) * (2 + HSP);
+            if (d == 0) {
+                p[0] = M;
+                p[1] = L;
+            }
+            p[2 + d] = o;
+        }
     }
 }
 
@@ -207,6 +434,40 @@ int launch_nv(wgml_ctx *ctx, const AttnArgs &a, int km, dim3 grid) {
     return WGML_OK;
 }
 
+template <int NV4, int NW>
+int launch_fast_nv(wgml_ctx *ctx, const AttnArgs &a, int km, dim3 grid) {
+    const dim3 block(NW * 64);
+    // the planner keeps km * NV4 within the register budget of the variant
+    constexpr int kMaxKmNv = NW == 16 ? 4 : 8;
+    if (km * NV4 > kMaxKmNv)
+        return set_error(WGML_E_INVALID, "attention: no kernel for km %d, %d float4 per lane", km,
+                         NV4);
+    if constexpr (4 * NV4 <= kMaxKmNv) {
+        if (km == 4) attn_fast_kernel<NV4, 4, NW><<<grid, block, 0, ctx->stream>>>(a);
+    }
+    if constexpr (2 * NV4 <= kMaxKmNv) {
+        if (km == 2) attn_fast_kernel<NV4, 2, NW><<<grid, block, 0, ctx->stream>>>(a);
+    }
+    if (km == 1) attn_fast_kernel<NV4, 1, NW><<<grid, block, 0, ctx->stream>>>(a);
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
+template <int NW>
+int launch_fast(wgml_ctx *ctx, const AttnArgs &a, int nv, int km, dim3 grid) {
+    switch (nv) {
+    case 1: return launch_fast_nv<1, NW>(ctx, a, km, grid);
+    case 2: return launch_fast_nv<2, NW>(ctx, a, km, grid);
+    default: break;
+    }
+    if constexpr (NW != 16) {  // large heads: only the 4-wave variant has the registers
+        if (nv == 3) return launch_fast_nv<3, NW>(ctx, a, km, grid);
+        return launch_fast_nv<4, NW>(ctx, a, km, grid);
+    }
+    return set_error(WGML_E_INVALID, "attention: no 16-wave kernel for %d float4 per lane", nv);
+}
+
 }  // namespace
 
 namespace wgml {
@@ -216,7 +477,46 @@ namespace wgml {
 struct AttnPlan {
     int nv, km;
     uint32_t groups, chunk, n_wg_y, hsp;
+    int wide;  // fast plan: one 16-wave workgroup per head group, no partials
 };
+
+// The fast kernel needs float4-addressable heads; `aligned` says that q and the
+// cache views start on 16-byte boundaries.
+static bool fast_ok(const wgml_attn_params &p, bool aligned, bool wants_scores) {
+    return !wants_scores && aligned && p.head_size % 4 == 0 && p.kv_dim % 4 == 0 &&
+           p.head_size <= 256;
+}
+
+constexpr uint32_t kWidePositions = 128;  // up to here one workgroup per head group
+
+static int make_fast_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions,
+                          AttnPlan &pl) {
+    const uint32_t hs = p.head_size;
+    pl.nv = (int)((hs + 63) / 64);  // float4 per lane: 16 lanes x 4 floats x nv
+    pl.wide = (plan_positions <= kWidePositions && pl.nv <= 2) ? 1 : 0;
+    pl.km = 1;
+    if (p.kv_mul == 2 || p.kv_mul == 4) pl.km = (int)p.kv_mul;
+    if (p.kv_mul == 8) pl.km = 4;
+    // register budget (q and acc are km * nv float4 each): 128 VGPRs for the
+    // 16-wave variant, 256 for the 4-wave one
+    const int max_kmnv = pl.wide ? 4 : 8;
+    while (pl.km > 1 && pl.km * pl.nv > max_kmnv) pl.km >>= 1;
+    pl.groups = p.n_heads / pl.km;
+    pl.chunk = 0;  // derived from the position on the device
+    pl.hsp = (uint32_t)pl.nv * 64;
+    if (pl.wide) {
+        pl.n_wg_y = 1;
+        return WGML_OK;
+    }
+    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
+    // about two workgroups per CU, each with at least 16 positions at full length
+    uint32_t n_wg_y = (2 * cu + pl.groups - 1) / pl.groups;
+    const uint32_t max_y = (plan_positions + 4 * WAVES - 1) / (4 * WAVES);
+    if (n_wg_y > max_y) n_wg_y = max_y;
+    if (n_wg_y < 2) n_wg_y = 2;
+    pl.n_wg_y = n_wg_y;
+    return WGML_OK;
+}
 
 static int make_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions,
                      AttnPlan &pl) {
@@ -246,19 +546,51 @@ static int make_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_pos
 int reserve_attention_workspace(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions) {
     AttnPlan pl;
     WGML_TRY(make_plan(ctx, p, plan_positions, pl));
-    return ensure_ws(ctx, (size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4);
+    size_t bytes = (size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4;
+    if (fast_ok(p, true, false)) {
+        WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl));
+        const size_t fast = (size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4;
+        if (fast > bytes) bytes = fast;
+    }
+    return ensure_ws(ctx, bytes);
 }
 
 int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
-                             uint32_t plan_positions, const float *q, const float *kc,
-                             const float *vc, float *att, float *xb) {
+                             uint32_t plan_positions, uint32_t cache_rows, const float *q,
+                             const float *kc, const float *vc, float *att, float *xb) {
     AttnPlan pl;
+    const bool aligned = (((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) & 15u) == 0;
+    if (fast_ok(p, aligned, att != nullptr)) {
+        WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl));
+        AttnArgs a{};
+        a.q = q;
+        a.kc = kc;
+        a.vc = vc;
+        a.xb = xb;
+        a.seq_len = p.seq_len;
+        a.kv_dim = p.kv_dim;
+        a.kv_mul = p.kv_mul;
+        a.n_heads = p.n_heads;
+        a.head_size = p.head_size;
+        a.pos = pos;
+        a.n_wg_y = pl.n_wg_y;
+        a.spec_rows = cache_rows;
+        const dim3 grid(pl.groups, pl.n_wg_y);
+        if (pl.wide) return launch_fast<16>(ctx, a, pl.nv, pl.km, grid);
+        WGML_TRY(ensure_ws(ctx, (size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4));
+        a.ws = ctx->attn_ws;
+        WGML_TRY(launch_fast<WAVES>(ctx, a, pl.nv, pl.km, grid));
+        attn_merge_kernel<<<dim3(p.n_heads), dim3(256), 0, ctx->stream>>>(a, pl.hsp);
+        WGML_CHECK_LAUNCH();
+        ctx->launches++;
+        return WGML_OK;
+    }
     WGML_TRY(make_plan(ctx, p, plan_positions, pl));
     const uint32_t hs = p.head_size;
     const int nv = pl.nv, km = pl.km;
     const uint32_t groups = pl.groups, chunk = pl.chunk, n_wg_y = pl.n_wg_y;
 
-    AttnArgs a;
+    AttnArgs a{};
     a.q = q;
     a.kc = kc;
     a.vc = vc;
@@ -294,10 +626,11 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
     return WGML_OK;
 }
 
-int launch_attention(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos, const float *q,
-                     const float *kc, const float *vc, float *att, float *xb) {
-    return launch_attention_planned(ctx, p, pos, pos.ptr ? p.seq_len : pos.val + 1, q, kc, vc, att,
-                                    xb);
+// `cache_rows`: positions the cache views hold (at least pos + 1).
+int launch_attention(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos, uint32_t cache_rows,
+                     const float *q, const float *kc, const float *vc, float *att, float *xb) {
+    return launch_attention_planned(ctx, p, pos, pos.ptr ? p.seq_len : pos.val + 1, cache_rows, q,
+                                    kc, vc, att, xb);
 }
 
 }  // namespace wgml
@@ -333,8 +666,11 @@ int wgml_attention(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q, wgml_v
         att_ptr = view_ptr(att);
     }
     DynPos pos{nullptr, p->pos};
-    return launch_attention(ctx, *p, pos, view_ptr(q), view_ptr(key_cache),
-                            view_ptr(value_cache), att_ptr, view_ptr(xb));
+    const uint64_t rows = (key_cache.len < value_cache.len ? key_cache.len : value_cache.len) /
+                          p->kv_dim;
+    return launch_attention(ctx, *p, pos, (uint32_t)(rows < p->seq_len ? rows : p->seq_len),
+                            view_ptr(q), view_ptr(key_cache), view_ptr(value_cache), att_ptr,
+                            view_ptr(xb));
 }
 
 }  // extern "C"

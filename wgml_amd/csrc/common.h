@@ -165,8 +165,8 @@ int launch_layernorm(wgml_ctx *ctx, float *out, const float *x, const float *gam
 int launch_rope(wgml_ctx *ctx, int variant, uint32_t head_size, uint32_t kv_dim, DynPos pos,
                 float base_freq, float *q, uint32_t q_len, float *k, uint64_t k_pos_stride);
 int launch_softmax(wgml_ctx *ctx, float *mat, uint32_t nrows, uint32_t ncols, uint32_t col_stride);
-int launch_attention(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos, const float *q,
-                     const float *kc, const float *vc, float *att, float *xb);
+int launch_attention(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos, uint32_t cache_rows,
+                     const float *q, const float *kc, const float *vc, float *att, float *xb);
 int launch_silu(wgml_ctx *ctx, float *h1, const float *h2, uint32_t n);
 int launch_unary(wgml_ctx *ctx, int op, float *x, uint32_t n, const float *args4);
 int launch_op_assign(wgml_ctx *ctx, int op, float *a, const float *b, uint32_t n);

@@ -470,17 +470,26 @@ struct IFmtQ4K {
         local = e & 63;
         xb = local >> 5;
     }
-    template <int R>
-    __device__ static void accumulate(const W::Row (&w)[R], const uint4 *xq, const float *meta,
-                                      uint32_t tile, float (&acc)[R]) {
-        // xq: this lane's slot of chunk 0 of the hi plane; chunk c at xq[c*64], lo plane 4 chunks on
+    // A lane's tile of the staged activations.
+    struct X {
         uint4 xh[4], xl[4];
+        float4 mt;  // s0, s1, S0, S1
+    };
+    // xq: this lane's slot of chunk 0 of the hi plane; chunk c at xq[c*64], lo plane 4 chunks on
+    __device__ static void load_x(X &x, const uint4 *xq, const float *meta) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            xh[c] = xq[c * 64];
-            xl[c] = xq[(4 + c) * 64];
+            x.xh[c] = xq[c * 64];
+            x.xl[c] = xq[(4 + c) * 64];
         }
-        const float4 mt = *reinterpret_cast<const float4 *>(meta);  // s0, s1, S0, S1
+        x.mt = *reinterpret_cast<const float4 *>(meta);
+    }
+    template <int R>
+    __device__ static void accumulate(const W::Row (&w)[R], const X &x, uint32_t tile,
+                                      float (&acc)[R]) {
+        const uint4(&xh)[4] = x.xh;
+        const uint4(&xl)[4] = x.xl;
+        const float4 mt = x.mt;
         const uint32_t j = tile & 3;
         const uint32_t sh = (j & 1u) * 16u;
 #pragma unroll
@@ -526,17 +535,25 @@ struct IFmtQ6K {
         xb = quarter;
         local = quarter * 16 + (e & 15);
     }
-    template <int R>
-    __device__ static void accumulate(const W::Row (&w)[R], const uint4 *xq, const float *meta,
-                                      uint32_t tile, float (&acc)[R]) {
+    struct X {
         uint4 xh[4], xl[4];  // chunk = quarter
+        float4 ms, mS;       // scales of the 4 quarters, sums of the rounded values
+    };
+    __device__ static void load_x(X &x, const uint4 *xq, const float *meta) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            xh[c] = xq[c * 64];
-            xl[c] = xq[(4 + c) * 64];
+            x.xh[c] = xq[c * 64];
+            x.xl[c] = xq[(4 + c) * 64];
         }
-        const float4 ms = *reinterpret_cast<const float4 *>(meta);      // s of the 4 quarters
-        const float4 mS = *reinterpret_cast<const float4 *>(meta + 4);  // exact sums
+        x.ms = *reinterpret_cast<const float4 *>(meta);
+        x.mS = *reinterpret_cast<const float4 *>(meta + 4);
+    }
+    template <int R>
+    __device__ static void accumulate(const W::Row (&w)[R], const X &x, uint32_t tile,
+                                      float (&acc)[R]) {
+        const uint4(&xh)[4] = x.xh;
+        const uint4(&xl)[4] = x.xl;
+        const float4 ms = x.ms, mS = x.mS;
         const uint32_t sb = (tile & 1u) * 8u;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -580,16 +597,24 @@ struct IFmtQ8_0 {
         local = e & 31;
         xb = 0;
     }
-    template <int R>
-    __device__ static void accumulate(const W::Row (&w)[R], const uint4 *xq, const float *meta,
-                                      uint32_t, float (&acc)[R]) {
+    struct X {
         uint4 xh[2], xl[2];
+        float s0;
+    };
+    __device__ static void load_x(X &x, const uint4 *xq, const float *meta) {
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
-            xh[c] = xq[c * 64];
-            xl[c] = xq[(2 + c) * 64];
+            x.xh[c] = xq[c * 64];
+            x.xl[c] = xq[(2 + c) * 64];
         }
-        const float s0 = meta[0];
+        x.s0 = meta[0];
+    }
+    template <int R>
+    __device__ static void accumulate(const W::Row (&w)[R], const X &x, uint32_t,
+                                      float (&acc)[R]) {
+        const uint4(&xh)[2] = x.xh;
+        const uint4(&xl)[2] = x.xl;
+        const float s0 = x.s0;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             int h = 0, l = 0;
@@ -613,16 +638,35 @@ struct PlainPolicy {
         load_group<WF, R>(w, p, g, tile);
     }
     // Lane n holds finished result n of the segment that starts at group g0:
-    // result n belongs to row (g0 + (n / R) * GW) * R + n % R.
+    // result n belongs to row (g0 + (n / R) * GW) * R + n % R.  The operands the
+    // epilogue of the first segment needs are fetched by prefetch() at kernel start:
+    // fetched at the end they would add a memory round trip to every wave's tail.
+    float *out;
+    float pre_bias, pre_out;
     template <int R>
-    __device__ void finish(float mine, uint32_t n, uint32_t g0, uint32_t GW, uint32_t lane) {
+    __device__ void prefetch(uint32_t g0, uint32_t GW, uint32_t my_groups, uint32_t lane) {
+        out = p.out;
+        if (p.dyn_pos) out += (size_t)(*p.dyn_pos) * p.out_pos_stride;
+        pre_bias = pre_out = 0.f;
+        const uint32_t row = (g0 + (lane / R) * GW) * R + lane % R;
+        if (lane < my_groups * R && row < p.nrows) {
+            if (p.bias) pre_bias = p.bias[row];
+            if (p.accumulate) pre_out = out[row];
+        }
+    }
+    template <int R>
+    __device__ void finish(float mine, uint32_t n, uint32_t g0, uint32_t GW, uint32_t lane,
+                           bool first_segment) {
         const uint32_t row = (g0 + (lane / R) * GW) * R + lane % R;
         if (lane < n && row < p.nrows) {
-            float *out = p.out;
-            if (p.dyn_pos) out += (size_t)(*p.dyn_pos) * p.out_pos_stride;
             float v = mine;
-            if (p.bias) v += p.bias[row];
-            if (p.accumulate) v += out[row];
+            if (first_segment) {
+                v += pre_bias;
+                v += pre_out;
+            } else {
+                if (p.bias) v += p.bias[row];
+                if (p.accumulate) v += out[row];
+            }
             out[row] = v;
         }
     }
@@ -637,7 +681,9 @@ struct PlainPolicy {
 // the same wave).  The (group, pass, step) triples
 // of a wave form one sequence that is software-pipelined D deep.
 // LDS: uint4 xq[step][plane(2)][chunk(PCH)][lane(64)], then float meta[tile][MF].
-template <class F, int R, int D, class Policy>
+// XREG: rows fit one step (ncols <= 64 tiles), so a lane's tile of x is the same
+// for every row and is read from LDS once instead of once per row.
+template <class F, int R, int D, bool XREG, class Policy>
 __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, uint32_t wg,
                                              uint32_t nwg, uint32_t nw, uint32_t ngroups) {
     using WF = typename F::W;
@@ -657,6 +703,8 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     const uint32_t first = wg * nw + wave, GW = nwg * nw;
     const uint32_t my_groups = (wave < nw && first < ngroups) ? (ngroups - first + GW - 1) / GW : 0;
     const uint32_t n_it = my_groups * S * nsteps;
+
+    pol.template prefetch<R>(first, GW, my_groups, lane);
 
     // The requests for x go out first, the first D weight requests after them: a
     // wave's loads return in order, so x, a cache hit, is not held up behind the
@@ -778,6 +826,8 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     // to the policy 64 at a time: the epilogue's loads and stores (bias, RoPE table,
     // accumulate) would otherwise sit between the weight loads in flight, and a
     // wave waits for its memory operations in order.
+    typename F::X xr;
+    if (XREG && lane < ntiles) F::load_x(xr, xq + lane, meta + (size_t)lane * MF);
     uint32_t g = first, sub = 0, step = 0;  // (group, pass, step) being computed
     uint32_t nres = 0, gseg = first;
     float mine = 0.f;
@@ -800,9 +850,13 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
                             for (int q = 0; q < (int)(sizeof(typename WF::Row) / 4); ++q) xx ^= ww[q];
                             acc[r] += __uint_as_float(xx & 0x3fffffffu);
                         }
+                    } else if (XREG) {
+                        F::template accumulate<R>(w[d], xr, tile, acc);
                     } else {
-                        F::template accumulate<R>(w[d], xq + (size_t)step * 2 * PCH * 64 + lane,
-                                                  meta + (size_t)tile * MF, tile, acc);
+                        typename F::X xt;
+                        F::load_x(xt, xq + (size_t)step * 2 * PCH * 64 + lane,
+                                  meta + (size_t)tile * MF);
+                        F::template accumulate<R>(w[d], xt, tile, acc);
                     }
                 }
                 if (++step == nsteps) {
@@ -818,7 +872,7 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
                         sub = 0;
                         g += GW;
                         if (nres + S * R > 64) {
-                            pol.template finish<R>(mine, nres, gseg, GW, lane);
+                            pol.template finish<R>(mine, nres, gseg, GW, lane, gseg == first);
                             nres = 0;
                             gseg = g;
                         }
@@ -839,13 +893,17 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
             }
         }
     }
-    if (nres) pol.template finish<R>(mine, nres, gseg, GW, lane);
+    if (nres) pol.template finish<R>(mine, nres, gseg, GW, lane, gseg == first);
 }
 
 template <class F, int R, int D, int MAXT>
 __global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p) {
-    PlainPolicy pol{p};
-    gemv_i8_body<F, R, D>(p, pol, blockIdx.x, gridDim.x, p.active_waves, (p.nrows + R - 1) / R);
+    PlainPolicy pol{p, nullptr, 0.f, 0.f};
+    const uint32_t ngroups = (p.nrows + R - 1) / R;
+    if (p.ncols <= 64 * F::TILE)
+        gemv_i8_body<F, R, D, true>(p, pol, blockIdx.x, gridDim.x, p.active_waves, ngroups);
+    else
+        gemv_i8_body<F, R, D, false>(p, pol, blockIdx.x, gridDim.x, p.active_waves, ngroups);
 }
 
 // ------------------------------------------------------------------------
@@ -914,9 +972,34 @@ struct JobPolicy {
         const uint32_t row = j.mode == JOB_SILU ? g : min(2 * g + sub, j.nrows - 1);
         WF::load(w[0], WF::row_base(q, row), tile);
     }
-    // Lanes 2i and 2i+1 hold the two pass results of group g0 + i * GW.
+    // Lanes 2i and 2i+1 hold the two pass results of group g0 + i * GW.  prefetch()
+    // fetches what the epilogue of the first segment needs at kernel start.
+    float pre_bias, pre_out;
+    float2 pre_cs;
+    __device__ float2 rope_entry(uint32_t row) const {
+        if (rope_cs) return rope_cs[((row & ~1u) % head_size) >> 1];
+        const float head_dim = (float)((row & ~1u) % head_size);
+        const float theta = powf(rope_base, -head_dim / (float)head_size);
+        float sn, cs;
+        sincosf((float)pos * theta, &sn, &cs);
+        return make_float2(cs, sn);
+    }
     template <int R>
-    __device__ void finish(float mine, uint32_t n, uint32_t g0, uint32_t GW, uint32_t lane) {
+    __device__ void prefetch(uint32_t g0, uint32_t GW, uint32_t my_groups, uint32_t lane) {
+        pre_bias = pre_out = 0.f;
+        pre_cs = make_float2(1.f, 0.f);
+        if (j.mode == JOB_SILU) return;
+        const uint32_t row = 2 * (g0 + (lane >> 1) * GW) + (lane & 1);
+        if (lane < 2 * my_groups && row < j.nrows) {
+            const float *out = j.out + (size_t)pos * j.out_pos_stride;
+            if (j.bias) pre_bias = j.bias[row];
+            if (j.accumulate) pre_out = out[row];
+            if (j.mode == JOB_ROPE) pre_cs = rope_entry(row);
+        }
+    }
+    template <int R>
+    __device__ void finish(float mine, uint32_t n, uint32_t g0, uint32_t GW, uint32_t lane,
+                           bool first_segment) {
         const uint32_t g = g0 + (lane >> 1) * GW, sub = lane & 1;
         const bool valid = lane < n;
         float *out = j.out + (size_t)pos * j.out_pos_stride;
@@ -927,26 +1010,22 @@ struct JobPolicy {
         }
         const uint32_t row = 2 * g + sub;
         const bool store = valid && row < j.nrows;
-        float t = mine;
-        if (j.bias && store) t += j.bias[row];
+        float t = mine, prev = 0.f;
+        float2 c = pre_cs;
+        if (first_segment) {
+            t += pre_bias;
+            prev = pre_out;
+        } else if (store) {
+            if (j.bias) t += j.bias[row];
+            if (j.accumulate) prev = out[row];
+            if (j.mode == JOB_ROPE) c = rope_entry(row);
+        }
         if (j.mode == JOB_ROPE) {  // ROPE matrices have an even number of rows
             const float other = dpp_f32<0xB1>(t);
-            float sn = 0.f, cs = 1.f;
-            if (store) {
-                if (rope_cs) {
-                    const float2 c = rope_cs[((row & ~1u) % head_size) >> 1];
-                    cs = c.x;
-                    sn = c.y;
-                } else {
-                    const float head_dim = (float)((row & ~1u) % head_size);
-                    const float theta = powf(rope_base, -head_dim / (float)head_size);
-                    sincosf((float)pos * theta, &sn, &cs);
-                }
-            }
             // (x, y) = (even row, odd row):  x' = cs x - sn y,  y' = sn x + cs y
-            t = sub ? sn * other + cs * t : cs * t - sn * other;
+            t = sub ? c.y * other + c.x * t : c.x * t - c.y * other;
         }
-        if (store) out[row] = j.accumulate ? out[row] + t : t;
+        if (store) out[row] = j.accumulate ? prev + t : t;
     }
 };
 
@@ -962,9 +1041,14 @@ __device__ __forceinline__ void fused_job_body(const FusedParams &P, const GemvJ
     GemvParams pa = xp, pb = xp;
     pa.p0 = j.a0; pa.p1 = j.a1; pa.p2 = j.a2; pa.p3 = j.a3;
     pb.p0 = j.b0; pb.p1 = j.b1; pb.p2 = j.b2; pb.p3 = j.b3;
-    JobPolicy pol{j, pa, pb, dyn_pos(P.pos), P.head_size, P.rope_base, P.rope_cs};
+    JobPolicy pol{j, pa, pb, dyn_pos(P.pos), P.head_size, P.rope_base, P.rope_cs, 0.f, 0.f, make_float2(1.f, 0.f)};
     const uint32_t ngroups = j.mode == JOB_SILU ? j.nrows : (j.nrows + 1) / 2;
-    gemv_i8_body<F, 1, D>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves, ngroups);
+    if (P.ncols <= 64 * F::TILE)
+        gemv_i8_body<F, 1, D, true>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves,
+                                    ngroups);
+    else
+        gemv_i8_body<F, 1, D, false>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves,
+                                     ngroups);
 }
 
 // MINW: waves per SIMD the register budget must allow.

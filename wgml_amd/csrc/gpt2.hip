@@ -10,8 +10,8 @@ using namespace wgml;
 
 namespace wgml {
 int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
-                             uint32_t plan_positions, const float *q, const float *kc,
-                             const float *vc, float *att, float *xb);
+                             uint32_t plan_positions, uint32_t cache_rows, const float *q,
+                             const float *kc, const float *vc, float *att, float *xb);
 }
 
 struct Gpt2Layer {
@@ -218,7 +218,7 @@ int wgml_gpt2_forward(wgml_gpt2 *m, uint32_t token, uint32_t pos) {
                                       (size_t)n * 4, hipMemcpyDeviceToDevice, ctx->stream));
         WGML_CHECK_HIP(hipMemcpyAsync(w.value_cache + (size_t)pos * n, m->curr_2304 + 2 * n,
                                       (size_t)n * 4, hipMemcpyDeviceToDevice, ctx->stream));
-        WGML_TRY(launch_attention_planned(ctx, ap, dpos, pos + 1, m->curr_2304, w.key_cache,
+        WGML_TRY(launch_attention_planned(ctx, ap, dpos, pos + 1, ap.seq_len, m->curr_2304, w.key_cache,
                                           w.value_cache, nullptr, m->curr_768));
         // layer_input += proj_w * attn + proj_b   (:372-395)
         WGML_TRY(launch_gemv_quant(ctx, m->layer_input, w.proj_w, m->curr_768,

@@ -15,8 +15,8 @@ using namespace wgml;
 
 namespace wgml {
 int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
-                             uint32_t plan_positions, const float *q, const float *kc,
-                             const float *vc, float *att, float *xb);
+                             uint32_t plan_positions, uint32_t cache_rows, const float *q,
+                             const float *kc, const float *vc, float *att, float *xb);
 int reserve_attention_workspace(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions);
 }  // namespace wgml
 
@@ -147,7 +147,7 @@ int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos) {
             if (!rope_fused)
                 WGML_TRY(launch_rope(ctx, variant, m->head_size, kv_dim, dpos, c.rope_base_freq,
                                      m->q, dim, w.key_cache, kv_dim));
-            WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, m->q, w.key_cache,
+            WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, ap.seq_len, m->q, w.key_cache,
                                               w.value_cache, nullptr, m->xb));
             GemvEpilogue eacc;
             eacc.accumulate = 1;
@@ -201,7 +201,7 @@ int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos) {
         }
         WGML_TRY(launch_rope(ctx, variant, m->head_size, kv_dim, dpos, c.rope_base_freq, m->q, dim,
                              dynamic ? w.key_cache : k_cache, dynamic ? kv_dim : 0));
-        WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, m->q, w.key_cache, w.value_cache,
+        WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, ap.seq_len, m->q, w.key_cache, w.value_cache,
                                           nullptr, m->xb));
         if (fusion >= 1) {
             // x += Wo * xb in the GEMV epilogue
