@@ -1051,17 +1051,27 @@ __device__ __forceinline__ void fused_job_body(const FusedParams &P, const GemvJ
                                      ngroups);
 }
 
-// MINW: waves per SIMD the register budget must allow.
-template <int D, int MAXT, int MINW>
+// MINW: waves per SIMD the register budget must allow.  FMT: 0 = the matrices of
+// a launch may differ in format (decided per workgroup), else the one format all
+// of them have (smaller code, registers of that format only).
+template <int D, int MAXT, int MINW, int FMT>
 __global__ __launch_bounds__(MAXT, MINW) void gemv_fused_kernel(const FusedParams P) {
     int ji = 0;
     if (P.njobs > 1 && blockIdx.x >= P.jobs[1].wg_begin) ji = 1;
     if (P.njobs > 2 && blockIdx.x >= P.jobs[2].wg_begin) ji = 2;
-    const GemvJob &j = P.jobs[ji];
-    switch (j.type) {
-    case WGML_Q4_K: fused_job_body<IFmtQ4K, D>(P, j); break;
-    case WGML_Q6_K: fused_job_body<IFmtQ6K, D>(P, j); break;
-    default: fused_job_body<IFmtQ8_0, D>(P, j); break;
+    const GemvJob j = P.jobs[ji];  // a copy: fields stay in registers, not re-read in the loop
+    if (FMT == WGML_Q4_K) {
+        fused_job_body<IFmtQ4K, D>(P, j);
+    } else if (FMT == WGML_Q6_K) {
+        fused_job_body<IFmtQ6K, D>(P, j);
+    } else if (FMT == WGML_Q8_0) {
+        fused_job_body<IFmtQ8_0, D>(P, j);
+    } else {
+        switch (j.type) {
+        case WGML_Q4_K: fused_job_body<IFmtQ4K, D>(P, j); break;
+        case WGML_Q6_K: fused_job_body<IFmtQ6K, D>(P, j); break;
+        default: fused_job_body<IFmtQ8_0, D>(P, j); break;
+        }
     }
 }
 
@@ -1434,21 +1444,33 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
     if (lds > kMaxLds)
         return set_error(WGML_E_UNSUPPORTED, "gemv_fused: %u columns need %zu bytes of LDS", ncols,
                          lds);
-    const void *fn = (const void *)gemv_fused_kernel<D, MAXT, MINW>;
-    static bool opted_in = false;
-    if (lds > 64 * 1024 && !opted_in) {
+    // one kernel per format when all matrices share it, else the mixed one
+    int fmt = P.jobs[0].type, slot = 0;
+    for (int i = 1; i < f.njobs; ++i)
+        if (P.jobs[i].type != fmt) fmt = 0;
+    void (*kern)(const FusedParams) = gemv_fused_kernel<D, MAXT, MINW, 0>;
+    switch (fmt) {
+    case WGML_Q4_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q4_K>; slot = 1; break;
+    case WGML_Q6_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q6_K>; slot = 2; break;
+    case WGML_Q8_0: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q8_0>; slot = 3; break;
+    default: break;
+    }
+    const void *fn = (const void *)kern;
+    static bool opted_in[4] = {false, false, false, false};
+    if (lds > 64 * 1024 && !opted_in[slot]) {
         WGML_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)kMaxLds));
-        opted_in = true;
+        opted_in[slot] = true;
     }
-    static size_t cached_lds = ~size_t(0);
-    static int cached_blocks = 0;
-    if (cached_lds != lds) {
+    static size_t cached_lds_s[4] = {~size_t(0), ~size_t(0), ~size_t(0), ~size_t(0)};
+    static int cached_blocks_s[4] = {0, 0, 0, 0};
+    if (cached_lds_s[slot] != lds) {
         int nb = 0;
         WGML_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fn, MAXT, lds));
-        cached_blocks = nb > 0 ? nb : 1;
-        cached_lds = lds;
+        cached_blocks_s[slot] = nb > 0 ? nb : 1;
+        cached_lds_s[slot] = lds;
     }
+    const int cached_blocks = cached_blocks_s[slot];
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
     const uint32_t resident = cu * (uint32_t)cached_blocks;
     // Every workgroup streams about the same number of bytes: the smallest per-
@@ -1484,7 +1506,7 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
         begin += plan.wgs;
     }
     (void)max_nw;
-    gemv_fused_kernel<D, MAXT, MINW><<<dim3(begin), dim3(MAXT), lds, ctx->stream>>>(P);
+    kern<<<dim3(begin), dim3(MAXT), lds, ctx->stream>>>(P);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
@@ -1492,9 +1514,7 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
 
 int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
     switch (g_fused_variant) {
-    case 1: return launch_gemv_fused_variant<2, 512, 2>(ctx, f);
-    case 2: return launch_gemv_fused_variant<3, 1024, 1>(ctx, f);
-    case 3: return launch_gemv_fused_variant<2, 512, 4>(ctx, f);
+    case 1: return launch_gemv_fused_variant<3, 1024, 1>(ctx, f);
     default: return launch_gemv_fused_variant<2, 1024, 1>(ctx, f);
     }
 }
