@@ -270,33 +270,36 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
 #pragma unroll
     for (int v = 0; v < NV4; ++v) dv[v] = (sub + 16 * v) * 4 < hs;
 
-    // This wave's quads are gid, gid + total, ...; a batch is four of them.  The
-    // first quad is requested before the position is known (`spec_rows` rows of the
-    // caches may be read; rows beyond the position are masked out below), the
-    // others once it is, and only those that hold a position <= pos.
-    float4 kr[4][NV4], vr[4][NV4];
+    // This wave's quads are gid, gid + total, ...  Two register sets of two quads
+    // each take turns: while one is consumed the other's loads are in flight.  The
+    // very first quad is requested before the position is known (`spec_rows` rows
+    // of the caches may be read; rows beyond the position are masked out below),
+    // the others once it is, and only those that hold a position <= pos.
+    float4 kA[2][NV4], vA[2][NV4], kB[2][NV4], vB[2][NV4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < 2; ++u) {
 #pragma unroll
-        for (int v = 0; v < NV4; ++v) kr[u][v] = vr[u][v] = zero4;
+        for (int v = 0; v < NV4; ++v) kA[u][v] = vA[u][v] = kB[u][v] = vB[u][v] = zero4;
     }
-    auto request = [&](uint32_t i0, uint32_t last, int u_begin, uint32_t nq_limit) {
+    // requests quads number i0 + u (u_begin <= u < 2) of this wave into a set
+    auto request = [&](float4(&kk)[2][NV4], float4(&vv)[2][NV4], uint32_t i0, uint32_t last,
+                       int u_begin, uint32_t nq_limit) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < 2; ++u) {
             const uint32_t quad = (i0 + u) * total + gid;
             if (u >= u_begin && quad < nq_limit) {  // uniform over the wave
                 const uint32_t tt = min(quad * 4 + quarter, last);
                 const float4 *kp = reinterpret_cast<const float4 *>(kb + (size_t)tt * a.kv_dim);
                 const float4 *vp = reinterpret_cast<const float4 *>(vb + (size_t)tt * a.kv_dim);
 #pragma unroll
-                for (int v = 0; v < NV4; ++v) kr[u][v] = dv[v] ? kp[sub + 16 * v] : zero4;
+                for (int v = 0; v < NV4; ++v) kk[u][v] = dv[v] ? kp[sub + 16 * v] : zero4;
 #pragma unroll
-                for (int v = 0; v < NV4; ++v) vr[u][v] = dv[v] ? vp[sub + 16 * v] : zero4;
+                for (int v = 0; v < NV4; ++v) vv[u][v] = dv[v] ? vp[sub + 16 * v] : zero4;
             }
         }
     };
     const bool spec = gid * 4 < a.spec_rows;
-    if (spec) request(0, a.spec_rows - 1, 0, gid + 1);
+    if (spec) request(kA, vA, 0, a.spec_rows - 1, 0, gid + 1);
 
     float4 q[KM][NV4], acc[KM][NV4];
     float mx[KM], l[KM];
@@ -316,31 +319,36 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
     const uint32_t n_used = fast_n_used(pos, a.n_wg_y, NW);  // workgroups with work
     if (blockIdx.y >= n_used) return;
     const uint32_t nq = pos / 4 + 1;
-    for (uint32_t i0 = 0; i0 * total + gid < nq; i0 += 4) {
-        if (i0 == 0)
-            request(0, pos, spec ? 1 : 0, nq);
-        else
-            request(i0, pos, 0, nq);
+    // online-softmax update with the two quads of a set
+    auto consume = [&](const float4(&kk)[2][NV4], const float4(&vv)[2][NV4], uint32_t i0) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < 2; ++u) {
             // uniform within each 16-lane row, so the row reductions below see whole rows
             if (((i0 + u) * total + gid) * 4 + quarter <= pos) {
 #pragma unroll
                 for (int m = 0; m < KM; ++m) {
                     float part = 0.f;
 #pragma unroll
-                    for (int v = 0; v < NV4; ++v) part = dot4(q[m][v], kr[u][v], part);
+                    for (int v = 0; v < NV4; ++v) part = dot4(q[m][v], kk[u][v], part);
                     const float s = row16_sum(part) * inv_sqrt_hs;
                     const float mn = fmaxf(mx[m], s);
                     const float sc = __expf(mx[m] - mn);
                     const float p = __expf(s - mn);
                     l[m] = fmaf(l[m], sc, p);
 #pragma unroll
-                    for (int v = 0; v < NV4; ++v) acc[m][v] = axpby4(acc[m][v], sc, vr[u][v], p);
+                    for (int v = 0; v < NV4; ++v) acc[m][v] = axpby4(acc[m][v], sc, vv[u][v], p);
                     mx[m] = mn;
                 }
             }
         }
+    };
+    request(kA, vA, 0, pos, spec ? 1 : 0, nq);
+    request(kB, vB, 2, pos, 0, nq);
+    for (uint32_t i0 = 0; i0 * total + gid < nq; i0 += 4) {
+        consume(kA, vA, i0);
+        request(kA, vA, i0 + 4, pos, 0, nq);
+        consume(kB, vB, i0 + 2);
+        request(kB, vB, i0 + 6, pos, 0, nq);
     }
 
     // merge the four quarters of the wave (every lane ends up with the merged state)
@@ -513,6 +521,7 @@ static int make_fast_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pla
     uint32_t n_wg_y = (2 * cu + pl.groups - 1) / pl.groups;
     const uint32_t max_y = (plan_positions + 4 * WAVES - 1) / (4 * WAVES);
     if (n_wg_y > max_y) n_wg_y = max_y;
+    if (n_wg_y > (uint32_t)MERGE_MAX_Y) n_wg_y = MERGE_MAX_Y;  // what the merge takes in one go
     if (n_wg_y < 2) n_wg_y = 2;
     pl.n_wg_y = n_wg_y;
     return WGML_OK;

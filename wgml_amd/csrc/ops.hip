@@ -164,11 +164,23 @@ __device__ __forceinline__ uint32_t block_argmax(const float *__restrict__ v, ui
     __shared__ uint32_t bi[16];
     float best = -INFINITY;
     uint32_t idx = 0xffffffffu;
-    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
-        const float x = v[i];
-        if (idx == 0xffffffffu || x > best) {
-            best = x;
-            idx = i;
+    // 16 independent loads per round: the scan of a thread is a chain of memory
+    // round trips otherwise (125 of them for a 128k vocabulary)
+    constexpr int U = 16;
+    for (uint32_t i0 = threadIdx.x; i0 < n; i0 += U * blockDim.x) {
+        float x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t i = i0 + u * blockDim.x;
+            x[u] = i < n ? v[i] : -INFINITY;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t i = i0 + u * blockDim.x;
+            if (i < n && (idx == 0xffffffffu || x[u] > best)) {
+                best = x[u];
+                idx = i;
+            }
         }
     }
     // wave reduce (value, index) with xor-shuffles
