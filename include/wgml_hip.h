@@ -331,12 +331,58 @@ WGML_API int wgml_bench_gemv_fused(wgml_ctx *ctx, const wgml_qmat *const *a,
                                    uint32_t nsets, wgml_view out, uint32_t stride, wgml_view v,
                                    const wgml_view *norm_w, uint32_t iters, float *total_ms);
 
+/* ---- GGUF container: Gguf::from_bytes (gguf.rs:450-607), host only -------- *
+ * The file is memory-mapped (or the caller's bytes are used in place); the
+ * pointers handed out below point into it and stay valid until close.
+ * Metadata value types: 0 u8, 1 i8, 2 u16, 3 i16, 4 u32, 5 i32, 6 f32, 7 bool,
+ * 8 string, 9 array, 10 u64, 11 i64, 12 f64 (gguf.rs:330-361).  Tensor types are
+ * the WGML_* tags above (gguf.rs:70-103). */
+typedef struct wgml_gguf wgml_gguf;
+typedef struct {
+    const char *key;
+    int type;           /* metadata value type */
+    int array_type;     /* element type when type == 9 */
+    uint64_t array_len; /* element count when type == 9 */
+    const void *data;   /* scalar: its bytes; string: its bytes (not terminated);
+                           array of scalars: the elements; array of strings: null */
+    uint64_t nbytes;    /* bytes at `data` */
+} wgml_gguf_kv;
+typedef struct {
+    const char *name;
+    int type;
+    uint32_t ndims;
+    uint64_t dims[4]; /* dims[0] is the contiguous one (GGML order); unused ones are 1 */
+    uint64_t offset;  /* from the start of the file */
+    uint64_t nbytes;  /* 0 for tensor types whose block size is not known here */
+    const void *data;
+} wgml_gguf_tensor_info;
+WGML_API int wgml_gguf_open(const char *path, wgml_gguf **out);
+WGML_API int wgml_gguf_open_bytes(const void *bytes, uint64_t size, wgml_gguf **out);
+WGML_API int wgml_gguf_close(wgml_gguf *g);
+WGML_API uint32_t wgml_gguf_version(const wgml_gguf *g);
+WGML_API uint32_t wgml_gguf_alignment(const wgml_gguf *g); /* general.alignment, default 32 */
+WGML_API uint64_t wgml_gguf_n_metadata(const wgml_gguf *g);
+WGML_API uint64_t wgml_gguf_n_tensors(const wgml_gguf *g);
+/* Index of a key / tensor name, -1 if absent (Gguf::metadata / Gguf::tensors lookups). */
+WGML_API int64_t wgml_gguf_find_metadata(const wgml_gguf *g, const char *key);
+WGML_API int64_t wgml_gguf_find_tensor(const wgml_gguf *g, const char *name);
+WGML_API int wgml_gguf_metadata(const wgml_gguf *g, uint64_t i, wgml_gguf_kv *out);
+/* Element k of a string array. */
+WGML_API int wgml_gguf_metadata_string(const wgml_gguf *g, uint64_t i, uint64_t k, const char **s,
+                                       uint64_t *len);
+WGML_API int wgml_gguf_tensor(const wgml_gguf *g, uint64_t i, wgml_gguf_tensor_info *out);
+
 /* ---- host-side input makers (no device needed) ---------------------------- *
  * The reference only de-quantizes; its inputs come from GGUF files written by
  * ggml.  These restate ggml's reference quantizers (quantize_row_q8_0_ref,
  * quantize_row_q4_K_ref, quantize_row_q6_K_ref) so that synthetic weights can
  * be produced in-process.  nthreads <= 0 picks the available cores. */
 WGML_API int wgml_quantize(int type, const float *src, void *dst, uint64_t nelems, int nthreads);
+/* Block*::dequantize on the host (quantization.rs:16-42, 204-244, 322-389) for
+ * F32, F16, Q8_0, Q4_K, Q6_K: what the reference does at load for tensors it
+ * keeps in f32 (token_embd, models/llama2/transformer.rs:239-242). */
+WGML_API int wgml_dequantize_host(int type, const void *src, float *dst, uint64_t nelems,
+                                  int nthreads);
 /* Counter-based generator: element i depends only on (seed, i).
  * normal: mean + std * N(0,1) by Box-Muller in f32. */
 WGML_API int wgml_rng_normal(uint64_t seed, float *out, uint64_t n, float mean, float std,

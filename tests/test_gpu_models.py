@@ -117,6 +117,23 @@ def test_llama_decode_from_uploaded_kv(gpu):
     assert list(got) == want
 
 
+def test_llama_from_gguf_file(gpu, tmp_path):
+    # weights written to a GGUF file under the reference's tensor / key names, loaded back
+    # through the GGUF reader: same greedy tokens as the oracle on the original weights
+    import gguf_writer as gw
+
+    w = synth_llama(MICRO, seed=41, scheme="q4_k_m")
+    spice(w, MICRO, 8, biases=True)
+    path = tmp_path / "micro.gguf"
+    gw.llama_to_gguf(path, w, model_name="qwen2")
+    prompt = W.prompt_tokens(41, 4, MICRO.vocab_size)
+    want, _ = orc.Llama2(w, rope_variant=LlamaModelType.Qwen2).generate_greedy(prompt, 24)
+    g = W.Gguf(path)
+    m = Llama2.from_gguf(gpu, g, LlamaModelType.Qwen2)
+    assert m.config.dim == MICRO.dim and m.config.vocab_size == MICRO.vocab_size
+    assert np.array_equal(m.generate_greedy(prompt, 24), want)
+
+
 def test_llama_argument_checks(gpu):
     m = Llama2(gpu, MICRO)
     with pytest.raises(W.WgmlError, match="unset weights"):

@@ -9,3 +9,4 @@ from ._lib import (F32, Q4_K, Q6_K, Q8_0, LIB_PATH, WgmlError, lib)  # noqa: F40
 from .ops import *  # noqa: F401,F403
 from .models import *  # noqa: F401,F403
 from .models import prompt_tokens  # noqa: F401
+from .gguf import Gguf, GgufTensor, llama2_config_from_gguf, llama2_weights_from_gguf  # noqa: F401

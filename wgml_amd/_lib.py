@@ -64,6 +64,21 @@ class Gpt2ParamsC(C.Structure):
                 ("attn_b", C.c_uint32)]
 
 
+class GgufKv(C.Structure):
+    """wgml_gguf_kv"""
+
+    _fields_ = [("key", C.c_char_p), ("type", C.c_int), ("array_type", C.c_int),
+                ("array_len", C.c_uint64), ("data", C.c_void_p), ("nbytes", C.c_uint64)]
+
+
+class GgufTensorInfo(C.Structure):
+    """wgml_gguf_tensor_info"""
+
+    _fields_ = [("name", C.c_char_p), ("type", C.c_int), ("ndims", C.c_uint32),
+                ("dims", C.c_uint64 * 4), ("offset", C.c_uint64), ("nbytes", C.c_uint64),
+                ("data", C.c_void_p)]
+
+
 _P = C.c_void_p
 _PP = C.POINTER(C.c_void_p)
 _u32, _u64, _i, _f = C.c_uint32, C.c_uint64, C.c_int, C.c_float
@@ -131,7 +146,20 @@ PROTOTYPES = {
     "wgml_bench_gemv_quant": (_i, [_P, _PP, _u32, View, View, _u32, _i, _fp]),
     "wgml_bench_gemv_fused": (_i, [_P, _PP, _PP, C.POINTER(C.c_int), _u32, _u32, View, _u32, View,
                                    C.POINTER(View), _u32, _fp]),
+    "wgml_gguf_open": (_i, [C.c_char_p, _PP]),
+    "wgml_gguf_open_bytes": (_i, [_P, _u64, _PP]),
+    "wgml_gguf_close": (_i, [_P]),
+    "wgml_gguf_version": (_u32, [_P]),
+    "wgml_gguf_alignment": (_u32, [_P]),
+    "wgml_gguf_n_metadata": (_u64, [_P]),
+    "wgml_gguf_n_tensors": (_u64, [_P]),
+    "wgml_gguf_find_metadata": (C.c_int64, [_P, C.c_char_p]),
+    "wgml_gguf_find_tensor": (C.c_int64, [_P, C.c_char_p]),
+    "wgml_gguf_metadata": (_i, [_P, _u64, C.POINTER(GgufKv)]),
+    "wgml_gguf_metadata_string": (_i, [_P, _u64, _u64, C.POINTER(C.c_char_p), C.POINTER(_u64)]),
+    "wgml_gguf_tensor": (_i, [_P, _u64, C.POINTER(GgufTensorInfo)]),
     "wgml_quantize": (_i, [_i, _P, _P, _u64, _i]),
+    "wgml_dequantize_host": (_i, [_i, _P, _P, _u64, _i]),
     "wgml_rng_normal": (_i, [_u64, _P, _u64, _f, _f, _i]),
     "wgml_rng_uniform_u32": (_i, [_u64, _P, _u64, _u32]),
     # debug knob, not part of the reference surface
@@ -145,7 +173,9 @@ PROTOTYPES = {
 
 # calls whose return value is not a status code
 _NON_STATUS = {"wgml_last_error", "wgml_version", "wgml_buf_size", "wgml_quant_matrix_gguf_bytes",
-               "wgml_quant_bytes", "wgml_quant_block_elems", "wgml_llama2_launches_per_token"}
+               "wgml_quant_bytes", "wgml_quant_block_elems", "wgml_llama2_launches_per_token",
+               "wgml_gguf_version", "wgml_gguf_alignment", "wgml_gguf_n_metadata",
+               "wgml_gguf_n_tensors", "wgml_gguf_find_metadata", "wgml_gguf_find_tensor"}
 
 
 def _load() -> C.CDLL:

@@ -1410,7 +1410,7 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
     const uint32_t ncols = f.jobs[0].a->ncols;
     P.ncols = ncols;
     size_t lds = 0;
-    uint64_t bytes[3] = {0, 0, 0}, total_bytes = 0;
+    uint64_t bytes[3] = {0, 0, 0};
     uint32_t ngroups[3];
     for (int i = 0; i < f.njobs; ++i) {
         const FusedGemvJob &s = f.jobs[i];
@@ -1437,7 +1437,6 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
                 return set_error(WGML_E_INVALID, "gemv_fused: RoPE needs even row counts");
             ngroups[i] = (j.nrows + 1) / 2;
         }
-        total_bytes += bytes[i];
         const size_t l = lds_bytes_i8(j.type, ncols);
         if (l > lds) lds = l;
     }

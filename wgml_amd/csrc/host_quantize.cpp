@@ -400,6 +400,80 @@ int wgml_quantize(int type, const float *src, void *dst, uint64_t nelems, int nt
     return WGML_OK;
 }
 
+// Block*::dequantize of the reference (quantization.rs:16-42, 204-244, 322-389),
+// on the host: used where the reference expands a tensor at load
+// (token_embd, models/llama2/transformer.rs:239-242).
+int wgml_dequantize_host(int type, const void *src, float *dst, uint64_t nelems, int nthreads) {
+    WGML_REQUIRE(src && dst, "wgml_dequantize_host: null argument");
+    if (type == WGML_F32) {
+        memcpy(dst, src, nelems * 4);
+        return WGML_OK;
+    }
+    if (type == WGML_F16) {
+        const uint16_t *h = (const uint16_t *)src;
+        parallel_for(nelems, nthreads, [=](uint64_t b, uint64_t e) {
+            for (uint64_t i = b; i < e; ++i) dst[i] = f16_to_f32(h[i]);
+        });
+        return WGML_OK;
+    }
+    const uint32_t be = wgml_quant_block_elems(type);
+    if (!be || (type != WGML_Q8_0 && type != WGML_Q4_K && type != WGML_Q6_K))
+        return set_error(WGML_E_UNSUPPORTED, "wgml_dequantize_host: unsupported type %d", type);
+    WGML_REQUIRE(nelems % be == 0,
+                 "wgml_dequantize_host: %llu elements is not a whole number of blocks",
+                 (unsigned long long)nelems);
+    parallel_for(nelems / be, nthreads, [=](uint64_t b0, uint64_t b1) {
+        for (uint64_t b = b0; b < b1; ++b) {
+            float *y = dst + b * be;
+            if (type == WGML_Q8_0) {
+                const block_q8_0 &k = ((const block_q8_0 *)src)[b];
+                const float d = f16_to_f32(k.d);
+                for (int j = 0; j < QK8_0; ++j) y[j] = (float)k.qs[j] * d;
+            } else if (type == WGML_Q4_K) {
+                const block_q4_K &k = ((const block_q4_K *)src)[b];
+                const float d = f16_to_f32(k.d), dmin = f16_to_f32(k.dmin);
+                const uint8_t *q = k.qs;
+                for (int j = 0, is = 0; j < 4; ++j, is += 2, q += 32) {
+                    uint8_t sc[2], m[2];
+                    for (int t = 0; t < 2; ++t) {  // get_scale_min_k4
+                        const int jj = is + t;
+                        if (jj < 4) {
+                            sc[t] = k.scales[jj] & 63;
+                            m[t] = k.scales[jj + 4] & 63;
+                        } else {
+                            sc[t] = (uint8_t)((k.scales[jj + 4] & 0xF) | ((k.scales[jj - 4] >> 6) << 4));
+                            m[t] = (uint8_t)((k.scales[jj + 4] >> 4) | ((k.scales[jj] >> 6) << 4));
+                        }
+                    }
+                    const float d1 = d * (float)sc[0], m1 = dmin * (float)m[0];
+                    const float d2 = d * (float)sc[1], m2 = dmin * (float)m[1];
+                    for (int l = 0; l < 32; ++l) y[64 * j + l] = d1 * (float)(q[l] & 0xF) - m1;
+                    for (int l = 0; l < 32; ++l) y[64 * j + 32 + l] = d2 * (float)(q[l] >> 4) - m2;
+                }
+            } else {
+                const block_q6_K &k = ((const block_q6_K *)src)[b];
+                const float d = f16_to_f32(k.d);
+                for (int i = 0; i < 2; ++i) {
+                    const uint8_t *ql = k.ql + 64 * i, *qh = k.qh + 32 * i;
+                    const int8_t *sc = k.scales + 8 * i;
+                    for (int l = 0; l < 32; ++l) {
+                        const int is = l / 16;
+                        const int q1 = (int)((ql[l] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+                        const int q2 = (int)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+                        const int q3 = (int)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+                        const int q4 = (int)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+                        y[128 * i + l] = d * (float)sc[is] * (float)q1;
+                        y[128 * i + l + 32] = d * (float)sc[is + 2] * (float)q2;
+                        y[128 * i + l + 64] = d * (float)sc[is + 4] * (float)q3;
+                        y[128 * i + l + 96] = d * (float)sc[is + 6] * (float)q4;
+                    }
+                }
+            }
+        }
+    });
+    return WGML_OK;
+}
+
 int wgml_rng_normal(uint64_t seed, float *out, uint64_t n, float mean, float std_, int nthreads) {
     WGML_REQUIRE(out != nullptr || n == 0, "wgml_rng_normal: null output");
     parallel_for((n + 1) / 2, nthreads, [=](uint64_t b, uint64_t e) {

@@ -144,6 +144,15 @@ class Llama2:
         call("wgml_llama2_set_token_embd", self._h, _ptr(te))
         return self
 
+    @classmethod
+    def from_gguf(cls, gpu: GpuInstance, gguf, model_type: int = LlamaModelType.Llama) -> "Llama2":
+        """Llama2Config::from_gguf + Llama2Weights::from_gguf (models/llama2/cpu.rs:75-109,
+        models/llama2/transformer.rs:137-268) from a `wgml_amd.Gguf`."""
+        from .gguf import llama2_config_from_gguf, llama2_weights_from_gguf
+
+        config = llama2_config_from_gguf(gguf, model_type)
+        return cls(gpu, config, model_type).load(llama2_weights_from_gguf(gguf, config))
+
     def set_fusion(self, level: int) -> None:
         call("wgml_llama2_set_fusion", self._h, level)
 

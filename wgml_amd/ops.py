@@ -366,6 +366,15 @@ def quant_bytes(qtype: int, nelems: int) -> int:
     return _lib.lib.wgml_quant_bytes(qtype, nelems)
 
 
+def dequantize_host(qtype: int, data: np.ndarray, nelems: int, nthreads: int = 0) -> np.ndarray:
+    """GGUF bytes (F32 / F16 / Q8_0 / Q4_K / Q6_K) -> f32 values, on the host."""
+    src = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+    out = np.empty(nelems, dtype=np.float32)
+    call("wgml_dequantize_host", qtype, src.ctypes.data_as(C.c_void_p),
+         out.ctypes.data_as(C.c_void_p), nelems, nthreads)
+    return out
+
+
 def quantize(qtype: int, values: np.ndarray, nthreads: int = 0) -> np.ndarray:
     """ggml reference quantizer (Q8_0 / Q4_K / Q6_K) -> GGUF bytes (uint8)."""
     a = np.ascontiguousarray(values, dtype=np.float32).reshape(-1)
