@@ -307,6 +307,15 @@ WGML_API int wgml_gpt2_read_logits(wgml_gpt2 *m, float *host_out);
 /* ChatGpt2::forward's loop with greedy sampling (wgml-chat/src/chat_gpt2.rs:43-151). */
 WGML_API int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_prompt,
                                        uint32_t n_total, uint32_t *out_tokens);
+/* 0: layernorm, GELU and the q/k/v copies are launches of their own and the token
+ * loop reads every token back (mirrors Gpt2::dispatch and chat_gpt2.rs one to
+ * one); 1 (default): LayerNorm folded into the GEMV that consumes it, bias /
+ * residual / GELU into GEMV epilogues, k and v written straight into their cache
+ * columns, and the token loop replays one recorded step per token.  Same results
+ * to fp32 rounding. */
+WGML_API int wgml_gpt2_set_fusion(wgml_gpt2 *m, int level);
+/* Number of kernel launches of one decode step (diagnostics). */
+WGML_API int wgml_gpt2_launches_per_token(const wgml_gpt2 *m);
 
 /* ---- measurement: wgml-bench's bench_gemv (wgml-bench/src/main.rs:187-250) ---- *
  * Enqueues out = mats[i % n_mats] * v for i in 0..iters back to back between two

@@ -149,7 +149,8 @@ def test_llama_argument_checks(gpu):
         m.forward(0, MICRO.seq_len)
 
 
-def test_gpt2_micro_logits(gpu):
+@pytest.mark.parametrize("fusion", [0, 1])
+def test_gpt2_micro_logits(gpu, fusion):
     p = Gpt2Params(n_vocab=300, n_seq=32, n_embd=64, n_head=4, n_layer=2, ff_len=256, attn_b=192)
     w = synth_gpt2(p, seed=5)
     rng = np.random.default_rng(4)
@@ -160,6 +161,7 @@ def test_gpt2_micro_logits(gpu):
             l[b] = (0.1 * rng.standard_normal(p.n_embd)).astype(np.float32)
     ref = orc.Gpt2(w)
     m = Gpt2(gpu, p).load(w)
+    m.set_fusion(fusion)
     for pos, t in enumerate([1, 250, 33, 7, 7, 100]):
         want = ref.forward(t, pos)
         m.forward(t, pos)
@@ -175,6 +177,30 @@ def test_gpt2_124m_greedy_prefix(gpu):
     prompt = W.prompt_tokens(3, 32, p.n_vocab)
     n_total = 32 + 24
     want, margins = orc.Gpt2(w, predequantize=True).generate_greedy(prompt, n_total)
-    got = Gpt2(gpu, p).load(w).generate_greedy(prompt, n_total)
-    print(f"gpt2 top-2 logit margin: min {margins.min():.3e}")
+    m = Gpt2(gpu, p).load(w)
+    got = m.generate_greedy(prompt, n_total)  # recorded step, folded launches
+    print(f"gpt2 top-2 logit margin: min {margins.min():.3e}; {m.launches_per_token()} launches/token")
     assert np.array_equal(got, want)
+    assert np.array_equal(m.generate_greedy(prompt, n_total), want)  # replayable
+    m.set_fusion(0)  # one launch per op group, host round trip per token
+    assert np.array_equal(m.generate_greedy(prompt, n_total), want)
+
+
+def test_gpt2_micro_greedy_with_norm_affine(gpu):
+    # non-trivial LayerNorm gains / shifts and biases through the folded, recorded loop
+    p = Gpt2Params(n_vocab=300, n_seq=48, n_embd=128, n_head=4, n_layer=3, ff_len=512, attn_b=384)
+    w = synth_gpt2(p, seed=9)
+    rng = np.random.default_rng(2)
+    for l in w.layers:
+        for g in ("ln_1_g", "ln_2_g"):
+            l[g] = (1 + 0.2 * rng.standard_normal(p.n_embd)).astype(np.float32)
+        for b in ("ln_1_b", "ln_2_b"):
+            l[b] = (0.2 * rng.standard_normal(p.n_embd)).astype(np.float32)
+    w.ln_f_g = (1 + 0.2 * rng.standard_normal(p.n_embd)).astype(np.float32)
+    w.ln_f_b = (0.2 * rng.standard_normal(p.n_embd)).astype(np.float32)
+    prompt = W.prompt_tokens(9, 6, p.n_vocab)
+    want, _ = orc.Gpt2(w).generate_greedy(prompt, p.n_seq)
+    m = Gpt2(gpu, p).load(w)
+    assert np.array_equal(m.generate_greedy(prompt, p.n_seq), want)
+    m.set_fusion(0)
+    assert np.array_equal(m.generate_greedy(prompt, p.n_seq), want)

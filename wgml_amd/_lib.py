@@ -143,6 +143,8 @@ PROTOTYPES = {
     "wgml_gpt2_forward": (_i, [_P, _u32, _u32]),
     "wgml_gpt2_read_logits": (_i, [_P, _P]),
     "wgml_gpt2_generate_greedy": (_i, [_P, _P, _u32, _u32, _P]),
+    "wgml_gpt2_set_fusion": (_i, [_P, _i]),
+    "wgml_gpt2_launches_per_token": (_i, [_P]),
     "wgml_bench_gemv_quant": (_i, [_P, _PP, _u32, View, View, _u32, _i, _fp]),
     "wgml_bench_gemv_fused": (_i, [_P, _PP, _PP, C.POINTER(C.c_int), _u32, _u32, View, _u32, View,
                                    C.POINTER(View), _u32, _fp]),
@@ -174,6 +176,7 @@ PROTOTYPES = {
 # calls whose return value is not a status code
 _NON_STATUS = {"wgml_last_error", "wgml_version", "wgml_buf_size", "wgml_quant_matrix_gguf_bytes",
                "wgml_quant_bytes", "wgml_quant_block_elems", "wgml_llama2_launches_per_token",
+               "wgml_gpt2_launches_per_token",
                "wgml_gguf_version", "wgml_gguf_alignment", "wgml_gguf_n_metadata",
                "wgml_gguf_n_tensors", "wgml_gguf_find_metadata", "wgml_gguf_find_tensor"}
 

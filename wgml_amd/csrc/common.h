@@ -124,6 +124,12 @@ struct GemvEpilogue {
     // if norm_w != null the input is RMS-normalised first: v <- (v * rsqrt(mean(v^2) + eps)) * norm_w
     const float *norm_w = nullptr;
     float norm_eps = 0.f;
+    // if ln_gamma != null the input goes through LayerNorm first (eps 1e-5, as
+    // ops/layernorm.rs:46-53): v <- (v - mean) / sqrt(var + 1e-5) * ln_gamma + ln_beta
+    const float *ln_gamma = nullptr, *ln_beta = nullptr;
+    // activation applied to acc + bias before it is stored: 0 none, 1 GELU (tanh form,
+    // ops/unary.rs:106-110)
+    int act = 0;
 };
 
 // One launch for up to three quantized matrices that consume the same vector
@@ -137,6 +143,9 @@ struct FusedGemvJob {
     int mode = FUSED_PLAIN;  // ROPE: adjacent-pair rotation of the output rows by pos
     int accumulate = 0;
     uint32_t out_pos_stride = 0;  // out += pos * out_pos_stride
+    // the job covers rows [row0, row0 + nrows) of `a` (nrows 0: all of them); `bias`
+    // and `out` are indexed from the job's first row
+    uint32_t row0 = 0, nrows = 0;
 };
 struct FusedGemv {
     FusedGemvJob jobs[3];
@@ -144,6 +153,7 @@ struct FusedGemv {
     const float *x = nullptr;
     const float *norm_w = nullptr;  // optional fused RMSNorm of x
     float norm_eps = 0.f;
+    const float *ln_gamma = nullptr, *ln_beta = nullptr;  // optional fused LayerNorm of x
     DynPos pos{nullptr, 0};
     uint32_t head_size = 0;
     float rope_base = 10000.f;
@@ -176,7 +186,8 @@ struct DynState {
     uint32_t pos, token, count, n_prompt;
 };
 int launch_embed(wgml_ctx *ctx, float *x, const float *table, uint32_t dim, DynPos token,
-                 float *rope_cs, uint32_t head_size, float rope_base, DynPos pos);
+                 float *rope_cs, uint32_t head_size, float rope_base, DynPos pos,
+                 const float *pos_table = nullptr);
 int launch_argmax_next(wgml_ctx *ctx, const float *v, uint32_t n, DynState *dyn,
                        const uint32_t *prompt, uint32_t *tokens_out);
 int launch_dequantize(wgml_ctx *ctx, float *out, const wgml_qmat *m);

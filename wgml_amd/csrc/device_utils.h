@@ -95,6 +95,11 @@ __device__ __forceinline__ float block_max(float v, float *red) {
     return t;
 }
 
+// GELU, tanh form (UnaryOp::Gelu, ops/unary.rs:106-110).
+__device__ __forceinline__ float gelu_tanh(float x) {
+    return 0.5f * x * (1.0f + tanhf(0.79788456080286535588f * x * (1.0f + 0.044715f * x * x)));
+}
+
 // Unsigned byte k of a 32-bit word as float (v_cvt_f32_ubyteK).
 __device__ __forceinline__ float ub0(uint32_t w) { return (float)(w & 0xffu); }
 __device__ __forceinline__ float ub1(uint32_t w) { return (float)((w >> 8) & 0xffu); }

@@ -43,6 +43,8 @@ struct GemvParams {
     uint32_t out_pos_stride;
     const float *norm_w;  // optional fused RMSNorm of x
     float norm_eps;
+    const float *ln_g, *ln_b;  // optional fused LayerNorm of x (integer-dot kernels)
+    int act;                   // 1: GELU on acc + bias before the store
     // integer-dot kernels: the first `active_waves` waves of every workgroup walk
     // the row-groups with stride gridDim.x * active_waves
     uint32_t active_waves;
@@ -660,13 +662,9 @@ struct PlainPolicy {
         const uint32_t row = (g0 + (lane / R) * GW) * R + lane % R;
         if (lane < n && row < p.nrows) {
             float v = mine;
-            if (first_segment) {
-                v += pre_bias;
-                v += pre_out;
-            } else {
-                if (p.bias) v += p.bias[row];
-                if (p.accumulate) v += out[row];
-            }
+            v += first_segment ? pre_bias : (p.bias ? p.bias[row] : 0.f);
+            if (p.act == 1) v = gelu_tanh(v);
+            v += first_segment ? pre_out : (p.accumulate ? out[row] : 0.f);
             out[row] = v;
         }
     }
@@ -753,6 +751,53 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     if (stage) {
         uint32_t *xq32 = reinterpret_cast<uint32_t *>(xq);
         float ss = 0.f;
+        if (p.ln_g) {
+            // LayerNorm folded in (host guarantees that the XP float4 per thread cover
+            // x): mean, then variance about the mean (two exact passes over registers,
+            // ops/layernorm.rs:46-53), then x <- (x - mean) * rstd * gamma + beta.
+            __shared__ float red_a[16], red_b[16];
+            auto block_total = [&](float v, float *buf) {
+                v = wave_sum(v);
+                if (lane == 0) buf[wave] = v;
+                __syncthreads();
+                const float part = lane < nwaves ? buf[lane] : 0.f;
+                return readlane_f32(row16_sum(part), 0);
+            };
+            float s1 = 0.f;
+#pragma unroll
+            for (int i = 0; i < XP; ++i)
+                if (tid + i * blockDim.x < n4) s1 += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
+            const float mean = block_total(s1, red_a) / (float)p.ncols;
+            float s2 = 0.f;
+#pragma unroll
+            for (int i = 0; i < XP; ++i) {
+                if (tid + i * blockDim.x < n4) {
+                    xv[i].x -= mean;
+                    xv[i].y -= mean;
+                    xv[i].z -= mean;
+                    xv[i].w -= mean;
+                    s2 = fmaf(xv[i].x, xv[i].x, s2);
+                    s2 = fmaf(xv[i].y, xv[i].y, s2);
+                    s2 = fmaf(xv[i].z, xv[i].z, s2);
+                    s2 = fmaf(xv[i].w, xv[i].w, s2);
+                }
+            }
+            const float rstd = 1.0f / sqrtf(block_total(s2, red_b) / (float)p.ncols + 1.0e-5f);
+            const float4 *g4p = reinterpret_cast<const float4 *>(p.ln_g);
+            const float4 *b4p = reinterpret_cast<const float4 *>(p.ln_b);
+#pragma unroll
+            for (int i = 0; i < XP; ++i) {
+                const uint32_t g4 = tid + i * blockDim.x;
+                if (g4 < n4) {
+                    const float4 ga = g4p[g4];
+                    const float4 be = p.ln_b ? b4p[g4] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    xv[i].x = (xv[i].x * rstd) * ga.x + be.x;
+                    xv[i].y = (xv[i].y * rstd) * ga.y + be.y;
+                    xv[i].z = (xv[i].z * rstd) * ga.z + be.z;
+                    xv[i].w = (xv[i].w * rstd) * ga.w + be.w;
+                }
+            }
+        }
         auto stage_one = [&](uint32_t g4, float4 v, const float4 nw) {
             if (p.norm_w) {
                 ss = fmaf(v.x, v.x, ss);
@@ -940,6 +985,7 @@ struct FusedParams {
     uint32_t ncols;
     const float *norm_w;
     float norm_eps;
+    const float *ln_g, *ln_b;
     DynPos pos;
     uint32_t head_size;
     float rope_base;
@@ -1036,6 +1082,8 @@ __device__ __forceinline__ void fused_job_body(const FusedParams &P, const GemvJ
     xp.ncols = P.ncols;
     xp.norm_w = P.norm_w;
     xp.norm_eps = P.norm_eps;
+    xp.ln_g = P.ln_g;
+    xp.ln_b = P.ln_b;
     xp.nrows = j.nrows;
     xp.debug = P.debug;
     GemvParams pa = xp, pb = xp;
@@ -1263,6 +1311,9 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
     if (!R) R = 1;
     if (!waves) waves = (q8 && p.ncols <= 8192) ? 8 : 16;
     if (!depth) depth = (q8 && p.ncols > 8192) ? 4 : 2;
+    if (p.ln_g && (p.ncols >> 2) > 3u * (uint32_t)waves * 64u)  // XP float4 per thread
+        return set_error(WGML_E_UNSUPPORTED, "gemv_quant: %u columns are too many for the folded "
+                                             "LayerNorm", p.ncols);
     if (R == 2) {
         if (depth >= 3) return launch_rd_i8<F, 2, 3>(ctx, p, lds, waves);
         return launch_rd_i8<F, 2, 2>(ctx, p, lds, waves);
@@ -1348,6 +1399,12 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
     p.out_pos_stride = ep.out_pos_stride;
     p.norm_w = ep.norm_w;
     p.norm_eps = ep.norm_eps;
+    p.ln_g = ep.ln_gamma;
+    p.ln_b = ep.ln_beta;
+    p.act = ep.act;
+    if ((p.ln_g || p.act) && (m->type == WGML_F32 || g_f32_activations))
+        return set_error(WGML_E_UNSUPPORTED,
+                         "gemv_quant: LayerNorm / activation folding needs the integer-dot path");
     if (m->type == WGML_F32) {
         const size_t lds = (size_t)m->ncols * 4;
         if (lds > 64 * 1024)
@@ -1402,6 +1459,8 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
     P.x = f.x;
     P.norm_w = f.norm_w;
     P.norm_eps = f.norm_eps;
+    P.ln_g = f.ln_gamma;
+    P.ln_b = f.ln_beta;
     P.pos = f.pos;
     P.head_size = f.head_size ? f.head_size : 2;
     P.rope_base = f.rope_base;
@@ -1421,11 +1480,23 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
         j.out = s.out;
         j.bias = s.bias;
         j.nrows = s.a->nrows;
+        if (s.row0 || s.nrows) {  // a slice of the rows: move the plane pointers to its first row
+            const uint32_t n = s.nrows ? s.nrows : s.a->nrows - s.row0;
+            if (s.mode == JOB_SILU || (uint64_t)s.row0 + n > s.a->nrows)
+                return set_error(WGML_E_INVALID, "gemv_fused: job %d: bad row slice", i);
+            const uint64_t r = s.row0, nb = r * (ncols / 256);
+            switch (s.a->type) {
+            case WGML_Q4_K: j.a0 += nb * 144; break;
+            case WGML_Q6_K: j.a0 += nb * 128; j.a1 += nb * 64; j.a2 += nb * 16; j.a3 += nb * 2; break;
+            default: j.a0 += r * ncols; j.a1 += r * (ncols / 32) * 2; break;  // Q8_0
+            }
+            j.nrows = n;
+        }
         j.type = s.a->type;
         j.mode = s.mode;
         j.accumulate = s.accumulate;
         j.out_pos_stride = s.out_pos_stride;
-        bytes[i] = s.a->gguf_bytes;
+        bytes[i] = s.a->gguf_bytes / s.a->nrows * j.nrows;
         if (s.mode == JOB_SILU) {
             if (!s.b || s.b->type != s.a->type || s.b->nrows != s.a->nrows || s.b->ncols != ncols)
                 return set_error(WGML_E_INVALID, "gemv_fused: job %d: gate/up matrices differ", i);
@@ -1443,6 +1514,9 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
     if (lds > kMaxLds)
         return set_error(WGML_E_UNSUPPORTED, "gemv_fused: %u columns need %zu bytes of LDS", ncols,
                          lds);
+    if (P.ln_g && (ncols >> 2) > 3u * (uint32_t)MAXT)  // XP float4 per thread
+        return set_error(WGML_E_UNSUPPORTED,
+                         "gemv_fused: %u columns are too many for the folded LayerNorm", ncols);
     // one kernel per format when all matrices share it, else the mixed one
     int fmt = P.jobs[0].type, slot = 0;
     for (int i = 1; i < f.njobs; ++i)

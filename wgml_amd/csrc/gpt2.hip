@@ -12,6 +12,7 @@ namespace wgml {
 int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
                              uint32_t plan_positions, uint32_t cache_rows, const float *q,
                              const float *kc, const float *vc, float *att, float *xb);
+int reserve_attention_workspace(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions);
 }
 
 struct Gpt2Layer {
@@ -31,6 +32,14 @@ struct wgml_gpt2 {
     float *layer_input = nullptr, *curr_768 = nullptr, *curr_768_b = nullptr, *curr_2304 = nullptr,
           *curr_3072 = nullptr, *curr_vocab = nullptr;
     std::vector<void *> allocs;
+    // recorded token loop: position / token / output cursor on the device
+    DynState *dyn = nullptr;
+    uint32_t *d_prompt = nullptr, *d_tokens = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    int fusion = 1;  // 0: one launch per op group as before; 1: folded launches
+    int graph_fusion = -1;
+    uint64_t launches_last = 0;
 };
 
 namespace {
@@ -89,6 +98,15 @@ int wgml_gpt2_create(wgml_ctx *ctx, const wgml_gpt2_params *p, wgml_gpt2 **out) 
     A(&m->curr_2304, p->attn_b, true);
     A(&m->curr_3072, p->ff_len, true);
     A(&m->curr_vocab, p->n_vocab, true);
+    {
+        float *tmp = nullptr;
+        A(&tmp, 4, true);
+        m->dyn = reinterpret_cast<DynState *>(tmp);
+        A(&tmp, p->n_seq, true);
+        m->d_prompt = reinterpret_cast<uint32_t *>(tmp);
+        A(&tmp, p->n_seq, true);
+        m->d_tokens = reinterpret_cast<uint32_t *>(tmp);
+    }
     for (auto &l : m->layers) {
         A(&l.key_cache, (uint64_t)p->n_embd * p->n_seq, true);
         A(&l.value_cache, (uint64_t)p->n_embd * p->n_seq, true);
@@ -106,6 +124,8 @@ int wgml_gpt2_create(wgml_ctx *ctx, const wgml_gpt2_params *p, wgml_gpt2 **out) 
 int wgml_gpt2_destroy(wgml_gpt2 *m) {
     if (!m) return WGML_OK;
     if (m->ctx && m->ctx->stream) (void)hipStreamSynchronize(m->ctx->stream);
+    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+    if (m->graph) (void)hipGraphDestroy(m->graph);
     for (void *p : m->allocs) (void)hipFree(p);
     ctx_release(m->ctx);
     delete m;
@@ -185,56 +205,208 @@ int wgml_gpt2_set_embeddings(wgml_gpt2 *m, const float *wte, const float *wpe) {
     return WGML_OK;
 }
 
-// Gpt2::dispatch (models/gpt2/transformer.rs:265-477).  The reference's
-// mul_assign/add_assign after each layernorm and the add_assign after each
-// matmul are folded into the producing launch (affine layernorm, GEMV bias and
-// accumulate epilogues); the copies of q/k/v out of the fused qkv vector
-// (:329-353) are avoided by letting the attention read q in place and by
-// copying only k and v into their cache columns.
-int wgml_gpt2_forward(wgml_gpt2 *m, uint32_t token, uint32_t pos) {
-    WGML_REQUIRE(m != nullptr, "wgml_gpt2_forward: null model");
-    WGML_TRY(check_ready(m));
+}  // extern "C"
+
+namespace {
+
+// Gpt2::dispatch (models/gpt2/transformer.rs:265-477) for one token.  `dynamic`:
+// token and position are read from m->dyn on the device (a recorded step), else
+// they are the given values.
+// Folded launches (fusion 1): the reference's mul_assign/add_assign after each
+// layernorm and the add_assign after each matmul disappear into the GEMVs
+// (LayerNorm in the staging of x, bias / residual / GELU in the epilogue); q, k and
+// v are row slices of the one attn_w matrix, k and v written straight into their
+// cache columns (:329-353 copies them).  fusion 0 keeps layernorm, GELU and the
+// cache copies as launches of their own.
+// The folded launches exist for the quantized formats only.
+bool can_fold(const wgml_gpt2 *m) {
+    if (!gemv_fused_supported(m->lm_head)) return false;
+    for (const Gpt2Layer &w : m->layers)
+        if (!gemv_fused_supported(w.attn_w) || !gemv_fused_supported(w.proj_w) ||
+            !gemv_fused_supported(w.fc_w) || !gemv_fused_supported(w.mlp_proj_w))
+            return false;
+    return true;
+}
+
+int enqueue_step(wgml_gpt2 *m, bool dynamic, uint32_t token, uint32_t pos) {
     const wgml_gpt2_params &p = m->p;
-    WGML_REQUIRE(token < p.n_vocab, "wgml_gpt2_forward: token %u outside vocabulary %u", token,
-                 p.n_vocab);
-    WGML_REQUIRE(pos < p.n_seq, "wgml_gpt2_forward: pos %u outside n_seq %u", pos, p.n_seq);
     wgml_ctx *ctx = m->ctx;
     const uint32_t n = p.n_embd;
-    const DynPos dpos{nullptr, pos};
+    const DynPos dpos = dynamic ? DynPos{&m->dyn->pos, 0} : DynPos{nullptr, pos};
+    const DynPos dtok = dynamic ? DynPos{&m->dyn->token, 0} : DynPos{nullptr, token};
     const wgml_attn_params ap{p.n_seq, n, 1u, p.n_head, n / p.n_head, pos};
+    const uint32_t plan = dynamic ? p.n_seq : pos + 1;
+    const bool fold = m->fusion >= 1 && can_fold(m);
+    if (dynamic && !fold)
+        return set_error(WGML_E_UNSUPPORTED, "wgml_gpt2: the recorded step needs fusion 1");
 
     // layer_input = wte[:, token] + wpe[:, pos]   (:277-290)
-    WGML_CHECK_HIP(hipMemcpyAsync(m->layer_input, m->wte + (size_t)token * n, (size_t)n * 4,
-                                  hipMemcpyDeviceToDevice, ctx->stream));
-    WGML_TRY(launch_op_assign(ctx, WGML_ASSIGN_ADD, m->layer_input, m->wpe + (size_t)pos * n, n));
+    WGML_TRY(launch_embed(ctx, m->layer_input, m->wte, n, dtok, nullptr, 2, 0.f, dpos, m->wpe));
 
     for (uint32_t l = 0; l < p.n_layer; ++l) {
         const Gpt2Layer &w = m->layers[l];
-        WGML_TRY(launch_layernorm(ctx, m->curr_768, m->layer_input, w.ln_1_g, w.ln_1_b, n));
-        WGML_TRY(launch_gemv_quant(ctx, m->curr_2304, w.attn_w, m->curr_768,
-                                   GemvEpilogue{w.attn_b, 0}));
-        // k -> key_cache[:, pos], v -> value_cache[:, pos]; contiguous so one copy each
-        WGML_CHECK_HIP(hipMemcpyAsync(w.key_cache + (size_t)pos * n, m->curr_2304 + n,
-                                      (size_t)n * 4, hipMemcpyDeviceToDevice, ctx->stream));
-        WGML_CHECK_HIP(hipMemcpyAsync(w.value_cache + (size_t)pos * n, m->curr_2304 + 2 * n,
-                                      (size_t)n * 4, hipMemcpyDeviceToDevice, ctx->stream));
-        WGML_TRY(launch_attention_planned(ctx, ap, dpos, pos + 1, ap.seq_len, m->curr_2304, w.key_cache,
-                                          w.value_cache, nullptr, m->curr_768));
+        if (fold) {
+            FusedGemv f;
+            f.njobs = 3;
+            f.x = m->layer_input;
+            f.ln_gamma = w.ln_1_g;
+            f.ln_beta = w.ln_1_b;
+            f.pos = dpos;
+            float *outs[3] = {m->curr_2304, w.key_cache, w.value_cache};
+            for (int j = 0; j < 3; ++j) {
+                f.jobs[j].a = w.attn_w;
+                f.jobs[j].row0 = (uint32_t)j * n;
+                f.jobs[j].nrows = n;
+                f.jobs[j].bias = w.attn_b + (size_t)j * n;
+                f.jobs[j].out = outs[j];
+                f.jobs[j].out_pos_stride = j ? n : 0;
+            }
+            WGML_TRY(launch_gemv_fused(ctx, f));
+        } else {
+            WGML_TRY(launch_layernorm(ctx, m->curr_768, m->layer_input, w.ln_1_g, w.ln_1_b, n));
+            GemvEpilogue e;
+            e.bias = w.attn_b;
+            WGML_TRY(launch_gemv_quant(ctx, m->curr_2304, w.attn_w, m->curr_768, e));
+            // k -> key_cache[:, pos], v -> value_cache[:, pos]; contiguous so one copy each
+            WGML_CHECK_HIP(hipMemcpyAsync(w.key_cache + (size_t)pos * n, m->curr_2304 + n,
+                                          (size_t)n * 4, hipMemcpyDeviceToDevice, ctx->stream));
+            WGML_CHECK_HIP(hipMemcpyAsync(w.value_cache + (size_t)pos * n, m->curr_2304 + 2 * n,
+                                          (size_t)n * 4, hipMemcpyDeviceToDevice, ctx->stream));
+        }
+        WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, ap.seq_len, m->curr_2304,
+                                          w.key_cache, w.value_cache, nullptr, m->curr_768));
         // layer_input += proj_w * attn + proj_b   (:372-395)
-        WGML_TRY(launch_gemv_quant(ctx, m->layer_input, w.proj_w, m->curr_768,
-                                   GemvEpilogue{w.proj_b, 1}));
-        WGML_TRY(launch_layernorm(ctx, m->curr_768, m->layer_input, w.ln_2_g, w.ln_2_b, n));
-        WGML_TRY(launch_gemv_quant(ctx, m->curr_3072, w.fc_w, m->curr_768,
-                                   GemvEpilogue{w.fc_b, 0}));
-        WGML_TRY(launch_unary(ctx, WGML_UNARY_GELU, m->curr_3072, p.ff_len, nullptr));
+        {
+            GemvEpilogue e;
+            e.bias = w.proj_b;
+            e.accumulate = 1;
+            WGML_TRY(launch_gemv_quant(ctx, m->layer_input, w.proj_w, m->curr_768, e));
+        }
+        if (fold) {
+            GemvEpilogue e;  // h = gelu(fc_w * ln_2(layer_input) + fc_b)   (:397-431)
+            e.bias = w.fc_b;
+            e.ln_gamma = w.ln_2_g;
+            e.ln_beta = w.ln_2_b;
+            e.act = 1;
+            WGML_TRY(launch_gemv_quant(ctx, m->curr_3072, w.fc_w, m->layer_input, e));
+        } else {
+            WGML_TRY(launch_layernorm(ctx, m->curr_768, m->layer_input, w.ln_2_g, w.ln_2_b, n));
+            GemvEpilogue e;
+            e.bias = w.fc_b;
+            WGML_TRY(launch_gemv_quant(ctx, m->curr_3072, w.fc_w, m->curr_768, e));
+            WGML_TRY(launch_unary(ctx, WGML_UNARY_GELU, m->curr_3072, p.ff_len, nullptr));
+        }
         // layer_input += mlp_proj_w * h + mlp_proj_b   (:433-452)
-        WGML_TRY(launch_gemv_quant(ctx, m->layer_input, w.mlp_proj_w, m->curr_3072,
-                                   GemvEpilogue{w.mlp_proj_b, 1}));
+        {
+            GemvEpilogue e;
+            e.bias = w.mlp_proj_b;
+            e.accumulate = 1;
+            WGML_TRY(launch_gemv_quant(ctx, m->layer_input, w.mlp_proj_w, m->curr_3072, e));
+        }
     }
-    WGML_TRY(launch_layernorm(ctx, m->curr_768, m->layer_input, m->ln_f_g, m->ln_f_b, n));
-    WGML_TRY(launch_gemv_quant(ctx, m->curr_vocab, m->lm_head, m->curr_768, GemvEpilogue{}));
+    if (fold) {
+        GemvEpilogue e;
+        e.ln_gamma = m->ln_f_g;
+        e.ln_beta = m->ln_f_b;
+        WGML_TRY(launch_gemv_quant(ctx, m->curr_vocab, m->lm_head, m->layer_input, e));
+    } else {
+        WGML_TRY(launch_layernorm(ctx, m->curr_768, m->layer_input, m->ln_f_g, m->ln_f_b, n));
+        WGML_TRY(launch_gemv_quant(ctx, m->curr_vocab, m->lm_head, m->curr_768, GemvEpilogue{}));
+    }
     return WGML_OK;
 }
+
+void drop_graph(wgml_gpt2 *m) {
+    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+    if (m->graph) (void)hipGraphDestroy(m->graph);
+    m->graph_exec = nullptr;
+    m->graph = nullptr;
+    m->graph_fusion = -1;
+}
+
+// Records one step (+ greedy sampling and bookkeeping) into a HIP graph.
+int build_graph(wgml_gpt2 *m) {
+    if (m->graph_exec && m->graph_fusion == m->fusion) return WGML_OK;
+    drop_graph(m);
+    wgml_ctx *ctx = m->ctx;
+    const wgml_gpt2_params &p = m->p;
+    const uint32_t n = p.n_embd;
+    const wgml_attn_params ap{p.n_seq, n, 1u, p.n_head, n / p.n_head, 0};
+    WGML_TRY(reserve_attention_workspace(ctx, ap, p.n_seq));
+    // An eager step first (function attributes, lazy loading); it runs at position 0
+    // and would overwrite that column of every cache: keep a copy and put it back.
+    const size_t col = (size_t)n * 4;
+    void *saved = nullptr;
+    WGML_CHECK_HIP(hipMalloc(&saved, col * 2 * p.n_layer));
+    for (uint32_t l = 0; l < p.n_layer; ++l) {
+        (void)hipMemcpyAsync((char *)saved + col * (2 * l), m->layers[l].key_cache, col,
+                             hipMemcpyDeviceToDevice, ctx->stream);
+        (void)hipMemcpyAsync((char *)saved + col * (2 * l + 1), m->layers[l].value_cache, col,
+                             hipMemcpyDeviceToDevice, ctx->stream);
+    }
+    const DynState init{0, 0, 0, 0};
+    hipError_t ew = hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream);
+    int rcw = ew == hipSuccess ? enqueue_step(m, true, 0, 0) : WGML_E_HIP;
+    if (rcw == WGML_OK)
+        rcw = launch_argmax_next(ctx, m->curr_vocab, p.n_vocab, m->dyn, m->d_prompt, m->d_tokens);
+    for (uint32_t l = 0; l < p.n_layer; ++l) {
+        (void)hipMemcpyAsync(m->layers[l].key_cache, (char *)saved + col * (2 * l), col,
+                             hipMemcpyDeviceToDevice, ctx->stream);
+        (void)hipMemcpyAsync(m->layers[l].value_cache, (char *)saved + col * (2 * l + 1), col,
+                             hipMemcpyDeviceToDevice, ctx->stream);
+    }
+    ew = hipStreamSynchronize(ctx->stream);
+    (void)hipFree(saved);
+    if (rcw != WGML_OK) return rcw;
+    if (ew != hipSuccess)
+        return set_error(WGML_E_HIP, "wgml_gpt2: warm-up step failed: %s", hipGetErrorString(ew));
+
+    WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    const uint64_t launches0 = ctx->launches;
+    int rc = enqueue_step(m, true, 0, 0);
+    if (rc == WGML_OK)
+        rc = launch_argmax_next(ctx, m->curr_vocab, p.n_vocab, m->dyn, m->d_prompt, m->d_tokens);
+    m->launches_last = ctx->launches - launches0;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &m->graph);
+    if (rc == WGML_OK && e != hipSuccess)
+        rc = set_error(WGML_E_HIP, "wgml_gpt2: graph capture failed: %s", hipGetErrorString(e));
+    if (rc == WGML_OK) {
+        e = hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0);
+        if (e != hipSuccess)
+            rc = set_error(WGML_E_HIP, "wgml_gpt2: graph instantiate failed: %s",
+                           hipGetErrorString(e));
+    }
+    if (rc != WGML_OK) {
+        drop_graph(m);
+        return rc;
+    }
+    m->graph_fusion = m->fusion;
+    return WGML_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int wgml_gpt2_forward(wgml_gpt2 *m, uint32_t token, uint32_t pos) {
+    WGML_REQUIRE(m != nullptr, "wgml_gpt2_forward: null model");
+    WGML_TRY(check_ready(m));
+    WGML_REQUIRE(token < m->p.n_vocab, "wgml_gpt2_forward: token %u outside vocabulary %u", token,
+                 m->p.n_vocab);
+    WGML_REQUIRE(pos < m->p.n_seq, "wgml_gpt2_forward: pos %u outside n_seq %u", pos, m->p.n_seq);
+    return enqueue_step(m, false, token, pos);
+}
+
+// 0: layernorm, GELU and the cache copies are launches of their own; 1 (default):
+// folded into the GEMVs.  Same results to fp32 rounding.
+int wgml_gpt2_set_fusion(wgml_gpt2 *m, int level) {
+    WGML_REQUIRE(m != nullptr, "wgml_gpt2_set_fusion: null model");
+    WGML_REQUIRE(level == 0 || level == 1, "wgml_gpt2_set_fusion: level %d not in {0,1}", level);
+    m->fusion = level;
+    return WGML_OK;
+}
+
+int wgml_gpt2_launches_per_token(const wgml_gpt2 *m) { return m ? (int)m->launches_last : 0; }
 
 int wgml_gpt2_read_logits(wgml_gpt2 *m, float *host_out) {
     WGML_REQUIRE(m && host_out, "wgml_gpt2_read_logits: null argument");
@@ -250,18 +422,59 @@ int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_p
     WGML_REQUIRE(n_prompt >= 1, "wgml_gpt2_generate_greedy: empty prompt");
     WGML_REQUIRE(n_total <= m->p.n_seq, "wgml_gpt2_generate_greedy: %u positions exceed n_seq %u",
                  n_total, m->p.n_seq);
+    WGML_TRY(check_ready(m));
+    for (uint32_t i = 0; i < n_prompt && i < n_total; ++i)
+        WGML_REQUIRE(prompt[i] < m->p.n_vocab, "wgml_gpt2_generate_greedy: prompt token %u outside "
+                                                "the vocabulary", prompt[i]);
     wgml_ctx *ctx = m->ctx;
-    uint32_t token = prompt[0];
-    for (uint32_t pos = 0; pos < n_total; ++pos) {
-        WGML_TRY(wgml_gpt2_forward(m, token, pos));
-        WGML_TRY(launch_argmax(ctx, m->curr_vocab, m->p.n_vocab, ctx->d_scalar));
-        WGML_CHECK_HIP(hipMemcpyAsync(ctx->h_scalar, ctx->d_scalar, 4, hipMemcpyDeviceToHost,
-                                      ctx->stream));
-        WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
-        const uint32_t best = ctx->h_scalar[0];
-        out_tokens[pos] = best;
-        token = (pos + 1 < n_prompt) ? prompt[pos + 1] : best;
+    if (n_total == 0) return WGML_OK;
+    if (m->fusion < 1 || !can_fold(m)) {
+        // one launch per op group and a host round trip per token, as the reference's
+        // chat loop does (chat_gpt2.rs:61-110)
+        uint32_t token = prompt[0];
+        for (uint32_t pos = 0; pos < n_total; ++pos) {
+            const uint64_t l0 = ctx->launches;
+            WGML_TRY(enqueue_step(m, false, token, pos));
+            WGML_TRY(launch_argmax(ctx, m->curr_vocab, m->p.n_vocab, ctx->d_scalar));
+            m->launches_last = ctx->launches - l0;
+            WGML_CHECK_HIP(hipMemcpyAsync(ctx->h_scalar, ctx->d_scalar, 4, hipMemcpyDeviceToHost,
+                                          ctx->stream));
+            WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+            const uint32_t best = ctx->h_scalar[0];
+            out_tokens[pos] = best;
+            token = (pos + 1 < n_prompt) ? prompt[pos + 1] : best;
+        }
+        return WGML_OK;
     }
+    // Recorded step replayed per token: sampling and bookkeeping stay on the device,
+    // one synchronisation at the end.
+    const bool use_graph = !graphs_disabled();
+    if (use_graph) {
+        WGML_TRY(build_graph(m));
+    } else {
+        const wgml_attn_params ap{m->p.n_seq, m->p.n_embd, 1u, m->p.n_head,
+                                  m->p.n_embd / m->p.n_head, 0};
+        WGML_TRY(reserve_attention_workspace(ctx, ap, m->p.n_seq));
+    }
+    const uint32_t np = n_prompt < n_total ? n_prompt : n_total;
+    WGML_CHECK_HIP(hipMemcpyAsync(m->d_prompt, prompt, (size_t)np * 4, hipMemcpyHostToDevice,
+                                  ctx->stream));
+    const DynState init{0, prompt[0], 0, np};
+    WGML_CHECK_HIP(hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream));
+    for (uint32_t i = 0; i < n_total; ++i) {
+        if (use_graph) {
+            WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec, ctx->stream));
+        } else {
+            const uint64_t l0 = ctx->launches;
+            WGML_TRY(enqueue_step(m, true, 0, 0));
+            WGML_TRY(launch_argmax_next(ctx, m->curr_vocab, m->p.n_vocab, m->dyn, m->d_prompt,
+                                        m->d_tokens));
+            m->launches_last = ctx->launches - l0;
+        }
+    }
+    WGML_CHECK_HIP(hipMemcpyAsync(out_tokens, m->d_tokens, (size_t)n_total * 4,
+                                  hipMemcpyDeviceToHost, ctx->stream));
+    WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
     return WGML_OK;
 }
 

@@ -121,8 +121,7 @@ __device__ __forceinline__ float unary_eval(int op, float x, float4 a) {
     case WGML_UNARY_NEG: return -x;
     case WGML_UNARY_STEP: return x > 0.f ? 1.f : 0.f;
     case WGML_UNARY_ELU: return x > 0.f ? x : expf(x) - 1.f;
-    case WGML_UNARY_GELU:
-        return 0.5f * x * (1.0f + tanhf(0.79788456080286535588f * x * (1.0f + 0.044715f * x * x)));
+    case WGML_UNARY_GELU: return gelu_tanh(x);
     case WGML_UNARY_GELU_QUICK: return x * (1.0f / (1.0f + expf(-1.702f * x)));
     case WGML_UNARY_SILU: return x / (1.0f + expf(-x));
     case WGML_UNARY_TANH: return tanhf(x);
@@ -237,11 +236,17 @@ __global__ __launch_bounds__(1024) void argmax_next_kernel(const float *__restri
 // state.x.copy_from_view(token_embd.column(token)) (wgml-chat/src/chat_llama2.rs:185-187)
 // Also fills the step's RoPE table (if given): (cos, sin) of pos * theta_i for the
 // head_size/2 pairs of a head, with the angle formed exactly as ops/rope.wgsl:38-41.
+// With `pos_table` (GPT-2's learned positions) the row of the current position is added:
+// layer_input = wte[:, token] + wpe[:, pos] (models/gpt2/transformer.rs:277-290).
 __global__ void embed_kernel(float *__restrict__ x, const float *__restrict__ table, uint32_t dim,
                              DynPos token, float2 *__restrict__ rope_cs, uint32_t head_size,
-                             float rope_base, DynPos pos) {
+                             float rope_base, DynPos pos, const float *__restrict__ pos_table) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < dim) x[i] = table[(size_t)dyn_pos(token) * dim + i];
+    if (i < dim) {
+        float v = table[(size_t)dyn_pos(token) * dim + i];
+        if (pos_table) v += pos_table[(size_t)dyn_pos(pos) * dim + i];
+        x[i] = v;
+    }
     if (rope_cs && i < head_size / 2) {
         const float head_dim = (float)(2 * i);
         const float theta = powf(rope_base, -head_dim / (float)head_size);
@@ -322,9 +327,11 @@ int launch_argmax(wgml_ctx *ctx, const float *v, uint32_t n, uint32_t *d_out) {
 }
 
 int launch_embed(wgml_ctx *ctx, float *x, const float *table, uint32_t dim, DynPos token,
-                 float *rope_cs, uint32_t head_size, float rope_base, DynPos pos) {
+                 float *rope_cs, uint32_t head_size, float rope_base, DynPos pos,
+                 const float *pos_table) {
     embed_kernel<<<grid1(dim), dim3(256), 0, ctx->stream>>>(
-        x, table, dim, token, reinterpret_cast<float2 *>(rope_cs), head_size, rope_base, pos);
+        x, table, dim, token, reinterpret_cast<float2 *>(rope_cs), head_size, rope_base, pos,
+        pos_table);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;

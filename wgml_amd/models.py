@@ -271,6 +271,12 @@ class Gpt2:
         call("wgml_gpt2_set_embeddings", self._h, _ptr(wte), _ptr(wpe))
         return self
 
+    def set_fusion(self, level: int) -> None:
+        call("wgml_gpt2_set_fusion", self._h, level)
+
+    def launches_per_token(self) -> int:
+        return _lib.lib.wgml_gpt2_launches_per_token(self._h)
+
     def forward(self, token: int, pos: int) -> None:
         call("wgml_gpt2_forward", self._h, token, pos)
 
