@@ -168,9 +168,6 @@ PROTOTYPES = {
     "wgml_debug_set_gemv_rows_per_wave": (_i, [_i]),
     "wgml_debug_set_gemv_config": (_i, [_i, _i, _i, _i]),
     "wgml_debug_set_gemv_f32_activations": (_i, [_i]),
-    "wgml_debug_set_gemv_flags": (_i, [_i]),
-    "wgml_debug_set_gemv_fused_variant": (_i, [_i]),
-    "wgml_debug_set_gemv_active_waves": (_i, [_i]),
 }
 
 # calls whose return value is not a status code

@@ -38,7 +38,6 @@ struct GemvParams {
     const float *bias;
     uint32_t nrows, ncols;
     int accumulate;
-    int debug;  // experiments: bit0 skip x staging, bit1 skip the dot products
     const uint32_t *dyn_pos;  // out += *dyn_pos * out_pos_stride
     uint32_t out_pos_stride;
     const float *norm_w;  // optional fused RMSNorm of x
@@ -671,7 +670,7 @@ struct PlainPolicy {
 };
 
 // The body shared by the single-matrix and the fused multi-matrix kernels.  `p`
-// supplies x, ncols, the optional RMSNorm and the debug flags; `pol` the rows.
+// supplies x, ncols and the optional norm folding; `pol` the rows.
 // The workgroup is number `wg` of the `nwg` that share the matrix; its waves
 // w < nw take the row-groups (wg * nw + w) + i * (nwg * nw) < ngroups, so that at
 // any time the machine reads one contiguous window of the matrix.  A group is
@@ -711,14 +710,13 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
     const float4 *nw4 = reinterpret_cast<const float4 *>(p.norm_w);
     const uint32_t n4 = p.ncols >> 2;
-    const bool stage = !(p.debug & 1);
     float4 xv[XP], nv[XP];
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
         const uint32_t g4 = tid + i * blockDim.x;
         xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         nv[i] = make_float4(1.f, 1.f, 1.f, 1.f);
-        if (stage && g4 < n4) {
+        if (g4 < n4) {
             xv[i] = x4[g4];
             if (p.norm_w) nv[i] = nw4[g4];
         }
@@ -748,7 +746,7 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     // the finished dot products instead.
     __shared__ float red[16];
     float out_scale = 1.f;
-    if (stage) {
+    {
         uint32_t *xq32 = reinterpret_cast<uint32_t *>(xq);
         float ss = 0.f;
         if (p.ln_g) {
@@ -886,16 +884,7 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
             if (it < n_it) {
                 const uint32_t tile = step * 64 + lane;
                 if (tile < ntiles) {
-                    if (p.debug & 2) {
-#pragma unroll
-                        for (int r = 0; r < R; ++r) {
-                            const uint32_t *ww = reinterpret_cast<const uint32_t *>(&w[d][r]);
-                            uint32_t xx = 0;
-#pragma unroll
-                            for (int q = 0; q < (int)(sizeof(typename WF::Row) / 4); ++q) xx ^= ww[q];
-                            acc[r] += __uint_as_float(xx & 0x3fffffffu);
-                        }
-                    } else if (XREG) {
+                    if (XREG) {
                         F::template accumulate<R>(w[d], xr, tile, acc);
                     } else {
                         typename F::X xt;
@@ -990,7 +979,6 @@ struct FusedParams {
     uint32_t head_size;
     float rope_base;
     const float2 *rope_cs;  // optional: (cos, sin) of the current position per pair of a head
-    int debug;
 };
 
 // A group is a pair of rows, done as two single-row passes of one wave:
@@ -1085,7 +1073,6 @@ __device__ __forceinline__ void fused_job_body(const FusedParams &P, const GemvJ
     xp.ln_g = P.ln_g;
     xp.ln_b = P.ln_b;
     xp.nrows = j.nrows;
-    xp.debug = P.debug;
     GemvParams pa = xp, pb = xp;
     pa.p0 = j.a0; pa.p1 = j.a1; pa.p2 = j.a2; pa.p3 = j.a3;
     pb.p0 = j.b0; pb.p1 = j.b1; pb.p2 = j.b2; pb.p3 = j.b3;
@@ -1181,9 +1168,6 @@ int g_force_r = 0;      // rows per wave, 0 = heuristic
 int g_force_waves = 0;  // waves per workgroup, 0 = heuristic
 int g_force_depth = 0;  // pipeline depth, 0 = heuristic
 int g_force_wg_per_cu = 0;
-int g_debug_flags = 0;
-int g_fused_variant = 0;
-int g_force_active_waves = 0;
 int g_f32_activations = 0;  // 1: fp32-activation kernels instead of the integer-dot path
 constexpr size_t kMaxLds = 128 * 1024;
 
@@ -1249,9 +1233,7 @@ WgPlan plan_groups(uint32_t ngroups, uint32_t max_wgs, uint32_t max_waves, uint3
     const uint32_t wgs = (ngroups + c - 1) / c;
     c = (ngroups + wgs - 1) / wgs;
     const uint32_t k = (c + max_waves - 1) / max_waves;
-    uint32_t nw = (c + k - 1) / k;
-    if (g_force_active_waves > 0 && (uint32_t)g_force_active_waves <= max_waves)
-        nw = (uint32_t)g_force_active_waves;
+    const uint32_t nw = (c + k - 1) / k;
     return {c, nw, wgs};
 }
 
@@ -1394,7 +1376,6 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
     p.nrows = m->nrows;
     p.ncols = m->ncols;
     p.accumulate = ep.accumulate;
-    p.debug = g_debug_flags;
     p.dyn_pos = ep.dyn_pos;
     p.out_pos_stride = ep.out_pos_stride;
     p.norm_w = ep.norm_w;
@@ -1465,7 +1446,6 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
     P.head_size = f.head_size ? f.head_size : 2;
     P.rope_base = f.rope_base;
     P.rope_cs = reinterpret_cast<const float2 *>(f.rope_cs);
-    P.debug = g_debug_flags;
     const uint32_t ncols = f.jobs[0].a->ncols;
     P.ncols = ncols;
     size_t lds = 0;
@@ -1586,10 +1566,7 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
 }
 
 int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
-    switch (g_fused_variant) {
-    case 1: return launch_gemv_fused_variant<3, 1024, 1>(ctx, f);
-    default: return launch_gemv_fused_variant<2, 1024, 1>(ctx, f);
-    }
+    return launch_gemv_fused_variant<2, 1024, 1>(ctx, f);
 }
 
 }  // namespace wgml
@@ -1602,18 +1579,6 @@ WGML_API int wgml_debug_set_gemv_rows_per_wave(int r) {
     WGML_REQUIRE(r == 0 || r == 1 || r == 2,
                  "wgml_debug_set_gemv_rows_per_wave: %d not in {0,1,2}", r);
     g_force_r = r;
-    return WGML_OK;
-}
-WGML_API int wgml_debug_set_gemv_active_waves(int v) {
-    g_force_active_waves = v;
-    return WGML_OK;
-}
-WGML_API int wgml_debug_set_gemv_fused_variant(int v) {
-    g_fused_variant = v;
-    return WGML_OK;
-}
-WGML_API int wgml_debug_set_gemv_flags(int f) {
-    g_debug_flags = f;
     return WGML_OK;
 }
 // 1 selects the fp32-activation GEMV kernels, 0 (default) the integer-dot path.
