@@ -100,12 +100,14 @@ WGML_API int wgml_buf_zero(wgml_buf *buf);
 /* ---- quantized matrices: GpuQuantMatrix (quantized_matrix.rs:9-75) and
  *      GgufTensorData::to_gpu_matrix (gguf.rs:131-184) ---------------------- *
  * `gguf_bytes` is the tensor exactly as stored in a GGUF file: row-major,
- * nrows rows of ncols/elems_per_block blocks.  Supported tags: WGML_F32,
- * WGML_Q8_0, WGML_Q4_K, WGML_Q6_K; others give WGML_E_UNSUPPORTED.  Unlike
- * the reference there is no pairing rule (ncols % 64 / % 512) and no silent
- * fall-back to f32: any ncols that is a multiple of the block length stays
- * quantized.  The bytes are re-laid out on the device (see the layout notes
- * in csrc/common.h); the values are unchanged. */
+ * nrows rows of ncols/elems_per_block blocks.  WGML_Q8_0, WGML_Q4_K and WGML_Q6_K
+ * stay quantized (re-laid out on the device, see the layout notes in
+ * csrc/common.h; the values are unchanged).  WGML_F16, WGML_Q4_0, WGML_Q4_1,
+ * WGML_Q5_0, WGML_Q5_1, WGML_Q5_K and WGML_Q8_K are expanded to f32 on the device
+ * at creation, as to_gpu_matrix does for every format its GEMV cannot read; the
+ * matrix then reports WGML_F32.  Other tags give WGML_E_UNSUPPORTED.  Unlike the
+ * reference there is no pairing rule (ncols % 64 / % 512) for the quantized
+ * formats: any ncols that is a multiple of the block length stays quantized. */
 WGML_API int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t ncols,
                                       const void *gguf_bytes, wgml_qmat **out);
 WGML_API int wgml_quant_matrix_destroy(wgml_qmat *m);

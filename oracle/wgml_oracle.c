@@ -53,8 +53,43 @@ typedef struct { /* quantization.rs:204-209 */
     int8_t scales[QK_K / 16];
     uint16_t d;
 } block_q6_k;
+typedef struct { /* quantization.rs:47-50 */
+    uint16_t d;
+    uint8_t qs[16];
+} block_q4_0;
+typedef struct { /* quantization.rs:75-79 */
+    uint16_t d, m;
+    uint8_t qs[16];
+} block_q4_1;
+typedef struct { /* quantization.rs:105-109 */
+    uint16_t d;
+    uint8_t qh[4];
+    uint8_t qs[16];
+} block_q5_0;
+typedef struct { /* quantization.rs:138-143 */
+    uint16_t d, m;
+    uint8_t qh[4];
+    uint8_t qs[16];
+} block_q5_1;
+typedef struct { /* quantization.rs:174-178 */
+    float d;
+    int8_t qs[QK_K];
+    int16_t bsums[QK_K / 16];
+} block_q8_k;
+typedef struct { /* quantization.rs:249-255 */
+    uint16_t d, dmin;
+    uint8_t scales[K_SCALE_SIZE];
+    uint8_t qh[QK_K / 8];
+    uint8_t qs[QK_K / 2];
+} block_q5_k;
 #pragma pack(pop)
 
+_Static_assert(sizeof(block_q4_0) == 18, "q4_0 block size");
+_Static_assert(sizeof(block_q4_1) == 20, "q4_1 block size");
+_Static_assert(sizeof(block_q5_0) == 22, "q5_0 block size");
+_Static_assert(sizeof(block_q5_1) == 24, "q5_1 block size");
+_Static_assert(sizeof(block_q8_k) == 292, "q8_k block size");
+_Static_assert(sizeof(block_q5_k) == 176, "q5_k block size");
 _Static_assert(sizeof(block_q8_0) == 34, "q8_0 block size");
 _Static_assert(sizeof(block_q4_k) == 144, "q4_k block size");
 _Static_assert(sizeof(block_q6_k) == 210, "q6_k block size");
@@ -62,9 +97,16 @@ _Static_assert(sizeof(block_q6_k) == 210, "q6_k block size");
 size_t orc_block_bytes(int type) {
     switch (type) {
     case ORC_F32: return 4;
+    case ORC_F16: return 2;
+    case ORC_Q4_0: return sizeof(block_q4_0);
+    case ORC_Q4_1: return sizeof(block_q4_1);
+    case ORC_Q5_0: return sizeof(block_q5_0);
+    case ORC_Q5_1: return sizeof(block_q5_1);
     case ORC_Q8_0: return sizeof(block_q8_0);
     case ORC_Q4_K: return sizeof(block_q4_k);
+    case ORC_Q5_K: return sizeof(block_q5_k);
     case ORC_Q6_K: return sizeof(block_q6_k);
+    case ORC_Q8_K: return sizeof(block_q8_k);
     default: return 0;
     }
 }
@@ -72,9 +114,10 @@ size_t orc_block_bytes(int type) {
 size_t orc_block_elems(int type) {
     switch (type) {
     case ORC_F32: return 1;
+    case ORC_F16: return 1;
+    case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: return 32;
     case ORC_Q8_0: return QK8_0;
-    case ORC_Q4_K: return QK_K;
-    case ORC_Q6_K: return QK_K;
+    case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: case ORC_Q8_K: return QK_K;
     default: return 0;
     }
 }
@@ -152,10 +195,109 @@ void orc_dequantize_q6_k(const void *blocks, size_t nblocks, float *out) {
     }
 }
 
+/* quantization.rs:53-68 */
+void orc_dequantize_q4_0(const void *blocks, size_t nblocks, float *out) {
+    const block_q4_0 *b = (const block_q4_0 *)blocks;
+    for (size_t i = 0; i < nblocks; ++i, out += 32) {
+        const float d = orc_decode_f16(b[i].d);
+        for (int j = 0; j < 16; ++j) {
+            const int x0 = (int)(b[i].qs[j] & 0x0F) - 8, x1 = (int)(b[i].qs[j] >> 4) - 8;
+            out[j] = (float)x0 * d;
+            out[j + 16] = (float)x1 * d;
+        }
+    }
+}
+
+/* quantization.rs:82-98 */
+void orc_dequantize_q4_1(const void *blocks, size_t nblocks, float *out) {
+    const block_q4_1 *b = (const block_q4_1 *)blocks;
+    for (size_t i = 0; i < nblocks; ++i, out += 32) {
+        const float d = orc_decode_f16(b[i].d), m = orc_decode_f16(b[i].m);
+        for (int j = 0; j < 16; ++j) {
+            out[j] = (float)(b[i].qs[j] & 0x0F) * d + m;
+            out[j + 16] = (float)(b[i].qs[j] >> 4) * d + m;
+        }
+    }
+}
+
+/* quantization.rs:112-131 */
+void orc_dequantize_q5_0(const void *blocks, size_t nblocks, float *out) {
+    const block_q5_0 *b = (const block_q5_0 *)blocks;
+    for (size_t i = 0; i < nblocks; ++i, out += 32) {
+        const float d = orc_decode_f16(b[i].d);
+        uint32_t qh;
+        memcpy(&qh, b[i].qh, 4);
+        for (int j = 0; j < 16; ++j) {
+            const uint32_t xh_0 = ((qh >> j) << 4) & 0x10, xh_1 = (qh >> (j + 12)) & 0x10;
+            const int x0 = (int)((b[i].qs[j] & 0x0Fu) | xh_0) - 16;
+            const int x1 = (int)((uint32_t)(b[i].qs[j] >> 4) | xh_1) - 16;
+            out[j] = (float)x0 * d;
+            out[j + 16] = (float)x1 * d;
+        }
+    }
+}
+
+/* quantization.rs:146-167 */
+void orc_dequantize_q5_1(const void *blocks, size_t nblocks, float *out) {
+    const block_q5_1 *b = (const block_q5_1 *)blocks;
+    for (size_t i = 0; i < nblocks; ++i, out += 32) {
+        const float d = orc_decode_f16(b[i].d), m = orc_decode_f16(b[i].m);
+        uint32_t qh;
+        memcpy(&qh, b[i].qh, 4);
+        for (int j = 0; j < 16; ++j) {
+            const uint32_t xh_0 = ((qh >> j) << 4) & 0x10, xh_1 = (qh >> (j + 12)) & 0x10;
+            const uint32_t x0 = (b[i].qs[j] & 0x0Fu) | xh_0, x1 = (uint32_t)(b[i].qs[j] >> 4) | xh_1;
+            out[j] = (float)x0 * d + m;
+            out[j + 16] = (float)x1 * d + m;
+        }
+    }
+}
+
+/* quantization.rs:195-201 */
+void orc_dequantize_q8_k(const void *blocks, size_t nblocks, float *out) {
+    const block_q8_k *b = (const block_q8_k *)blocks;
+    for (size_t i = 0; i < nblocks; ++i, out += QK_K)
+        for (int j = 0; j < QK_K; ++j) out[j] = b[i].d * (float)b[i].qs[j];
+}
+
+/* quantization.rs:274-317 */
+void orc_dequantize_q5_k(const void *blocks, size_t nblocks, float *out) {
+    const block_q5_k *b = (const block_q5_k *)blocks;
+    for (size_t i = 0; i < nblocks; ++i, out += QK_K) {
+        const float d = orc_decode_f16(b[i].d), min = orc_decode_f16(b[i].dmin);
+        int iq = 0, is = 0;
+        uint8_t u1 = 1, u2 = 2, sc, m;
+        for (int j = 0; j < QK_K; j += 64) {
+            get_scale_min_k4(is, b[i].scales, &sc, &m);
+            const float d1 = d * (float)sc, m1 = min * (float)m;
+            get_scale_min_k4(is + 1, b[i].scales, &sc, &m);
+            const float d2 = d * (float)sc, m2 = min * (float)m;
+            for (int l = 0; l < 32; ++l)
+                out[j + l] = d1 * (float)((b[i].qs[iq + l] & 0xF) + ((b[i].qh[l] & u1) ? 16 : 0)) - m1;
+            for (int l = 0; l < 32; ++l)
+                out[j + l + 32] =
+                    d2 * (float)((b[i].qs[iq + l] >> 4) + ((b[i].qh[l] & u2) ? 16 : 0)) - m2;
+            iq += 32;
+            is += 2;
+            u1 = (uint8_t)(u1 << 2);
+            u2 = (uint8_t)(u2 << 2);
+        }
+    }
+}
+
 /* gguf.rs:114-129 */
 int orc_dequantize(int type, const void *blocks, size_t nelems, float *out) {
     switch (type) {
     case ORC_F32: memcpy(out, blocks, nelems * sizeof(float)); return 0;
+    case ORC_F16:
+        for (size_t i = 0; i < nelems; ++i) out[i] = orc_decode_f16(((const uint16_t *)blocks)[i]);
+        return 0;
+    case ORC_Q4_0: orc_dequantize_q4_0(blocks, nelems / 32, out); return 0;
+    case ORC_Q4_1: orc_dequantize_q4_1(blocks, nelems / 32, out); return 0;
+    case ORC_Q5_0: orc_dequantize_q5_0(blocks, nelems / 32, out); return 0;
+    case ORC_Q5_1: orc_dequantize_q5_1(blocks, nelems / 32, out); return 0;
+    case ORC_Q5_K: orc_dequantize_q5_k(blocks, nelems / QK_K, out); return 0;
+    case ORC_Q8_K: orc_dequantize_q8_k(blocks, nelems / QK_K, out); return 0;
     case ORC_Q8_0: orc_dequantize_q8_0(blocks, nelems / QK8_0, out); return 0;
     case ORC_Q4_K: orc_dequantize_q4_k(blocks, nelems / QK_K, out); return 0;
     case ORC_Q6_K: orc_dequantize_q6_k(blocks, nelems / QK_K, out); return 0;

@@ -45,9 +45,16 @@ extern "C" {
  * gguf.rs:70-103. */
 enum {
     ORC_F32 = 0,
+    ORC_F16 = 1,
+    ORC_Q4_0 = 2,
+    ORC_Q4_1 = 3,
+    ORC_Q5_0 = 6,
+    ORC_Q5_1 = 7,
     ORC_Q8_0 = 8,
     ORC_Q4_K = 12,
+    ORC_Q5_K = 13,
     ORC_Q6_K = 14,
+    ORC_Q8_K = 15,
 };
 
 /* quantization.rs:392-409 */
@@ -62,6 +69,13 @@ size_t orc_block_elems(int type);
 void orc_dequantize_q8_0(const void *blocks, size_t nblocks, float *out);
 void orc_dequantize_q4_k(const void *blocks, size_t nblocks, float *out);
 void orc_dequantize_q6_k(const void *blocks, size_t nblocks, float *out);
+/* quantization.rs:53-68, 82-98, 112-131, 146-167, 195-201, 274-317 */
+void orc_dequantize_q4_0(const void *blocks, size_t nblocks, float *out);
+void orc_dequantize_q4_1(const void *blocks, size_t nblocks, float *out);
+void orc_dequantize_q5_0(const void *blocks, size_t nblocks, float *out);
+void orc_dequantize_q5_1(const void *blocks, size_t nblocks, float *out);
+void orc_dequantize_q8_k(const void *blocks, size_t nblocks, float *out);
+void orc_dequantize_q5_k(const void *blocks, size_t nblocks, float *out);
 /* gguf.rs:114-129: dispatch on the tag; returns 0, or -1 for an unsupported tag. */
 int orc_dequantize(int type, const void *blocks, size_t nelems, float *out);
 

@@ -72,9 +72,83 @@ def dequant_q6_k(raw: np.ndarray) -> np.ndarray:
     return out.reshape(-1)
 
 
-DEQUANT = {8: dequant_q8_0, 12: dequant_q4_k, 14: dequant_q6_k}
-BLOCK_BYTES = {8: 34, 12: 144, 14: 210}
-BLOCK_ELEMS = {8: 32, 12: 256, 14: 256}
+def _nibbles_5bit(b_qs: np.ndarray, qh_bytes: np.ndarray):
+    """qs: (nb, 16) uint8, qh: (nb, 4) uint8 -> two (nb, 16) arrays of 5-bit values
+    (elements 0..15 and 16..31 of a 32-element block; ggml dequantize_row_q5_0/q5_1)."""
+    qh = qh_bytes.copy().view(np.uint32)[:, 0].astype(np.uint64)
+    j = np.arange(16, dtype=np.uint64)
+    hi0 = ((qh[:, None] >> j) & 1).astype(np.uint8)          # bit j
+    hi1 = ((qh[:, None] >> (j + 16)) & 1).astype(np.uint8)   # bit j + 16
+    return (b_qs & 0x0F) | (hi0 << 4), (b_qs >> 4) | (hi1 << 4)
+
+
+def dequant_q4_0(raw):
+    b = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1, 18)
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])[:, None]
+    q = np.concatenate([b[:, 2:] & 0x0F, b[:, 2:] >> 4], axis=1).astype(np.int16) - 8
+    return (q.astype(np.float32) * d).astype(np.float32).reshape(-1)
+
+
+def dequant_q4_1(raw):
+    b = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1, 20)
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])[:, None]
+    m = half_bits_to_f32(b[:, 2:4].copy().view(np.uint16)[:, 0])[:, None]
+    q = np.concatenate([b[:, 4:] & 0x0F, b[:, 4:] >> 4], axis=1).astype(np.float32)
+    return ((q * d).astype(np.float32) + m).astype(np.float32).reshape(-1)
+
+
+def dequant_q5_0(raw):
+    b = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1, 22)
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])[:, None]
+    lo, hi = _nibbles_5bit(b[:, 6:], b[:, 2:6])
+    q = np.concatenate([lo, hi], axis=1).astype(np.int16) - 16
+    return (q.astype(np.float32) * d).astype(np.float32).reshape(-1)
+
+
+def dequant_q5_1(raw):
+    b = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1, 24)
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])[:, None]
+    m = half_bits_to_f32(b[:, 2:4].copy().view(np.uint16)[:, 0])[:, None]
+    lo, hi = _nibbles_5bit(b[:, 8:], b[:, 4:8])
+    q = np.concatenate([lo, hi], axis=1).astype(np.float32)
+    return ((q * d).astype(np.float32) + m).astype(np.float32).reshape(-1)
+
+
+def dequant_q8_k(raw):
+    b = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1, 292)
+    d = b[:, 0:4].copy().view(np.float32)[:, 0][:, None]
+    q = b[:, 4:260].view(np.int8).astype(np.float32)
+    return (d * q).astype(np.float32).reshape(-1)
+
+
+def dequant_q5_k(raw):
+    b = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1, 176)
+    nb = b.shape[0]
+    d = half_bits_to_f32(b[:, 0:2].copy().view(np.uint16)[:, 0])
+    dmin = half_bits_to_f32(b[:, 2:4].copy().view(np.uint16)[:, 0])
+    sc, m = _scale_min_k4(b[:, 4:16])
+    qh = b[:, 16:48]                      # (nb, 32): bit s of qh[l] is the 5th bit of sub-block s
+    qs = b[:, 48:].reshape(nb, 4, 32)
+    q = np.empty((nb, 8, 32), dtype=np.float32)
+    for s_ in range(8):
+        nib = (qs[:, s_ // 2, :] & 0x0F) if s_ % 2 == 0 else (qs[:, s_ // 2, :] >> 4)
+        q[:, s_, :] = (nib + (((qh >> s_) & 1) << 4)).astype(np.float32)
+    dl = (d[:, None] * sc.astype(np.float32)).astype(np.float32)
+    ml = (dmin[:, None] * m.astype(np.float32)).astype(np.float32)
+    return ((dl[:, :, None] * q).astype(np.float32) - ml[:, :, None]).astype(np.float32).reshape(-1)
+
+
+def dequant_f16(raw):
+    return half_bits_to_f32(np.ascontiguousarray(raw, dtype=np.uint8).view(np.uint16))
+
+
+DEQUANT = {1: dequant_f16, 2: dequant_q4_0, 3: dequant_q4_1, 6: dequant_q5_0, 7: dequant_q5_1,
+           8: dequant_q8_0, 12: dequant_q4_k, 13: dequant_q5_k, 14: dequant_q6_k, 15: dequant_q8_k}
+BLOCK_BYTES = {1: 2, 2: 18, 3: 20, 6: 22, 7: 24, 8: 34, 12: 144, 13: 176, 14: 210, 15: 292}
+BLOCK_ELEMS = {1: 1, 2: 32, 3: 32, 6: 32, 7: 32, 8: 32, 12: 256, 13: 256, 14: 256, 15: 256}
+# byte offsets of the f16 scale fields of a block (forced finite in random blocks)
+_HALF_FIELDS = {1: (0,), 2: (0,), 3: (0, 2), 6: (0,), 7: (0, 2), 8: (0,), 12: (0, 2), 13: (0, 2),
+                14: (208,), 15: ()}
 
 
 def random_blocks(qtype: int, nblocks: int, seed: int) -> np.ndarray:
@@ -91,13 +165,11 @@ def random_blocks(qtype: int, nblocks: int, seed: int) -> np.ndarray:
         h = (h & 0x83FF) | (exp.astype(np.uint16) << 10)
         raw[:, col:col + 2] = h.view(np.uint8).reshape(-1, 2)
 
-    if qtype == 8:
-        fix_half(0)
-    elif qtype == 12:
-        fix_half(0)
-        fix_half(2)
-    else:
-        fix_half(208)
+    for col in _HALF_FIELDS[qtype]:
+        fix_half(col)
+    if qtype == 15:  # Q8_K: d is an f32; draw it uniformly in [-4, 4)
+        d = (rng.random(nblocks, dtype=np.float32) * 8 - 4).astype(np.float32)
+        raw[:, 0:4] = d.view(np.uint8).reshape(-1, 4)
     return raw.reshape(-1)
 
 

@@ -15,6 +15,7 @@ ORACLE_DIR = Path(__file__).resolve().parent.parent / "oracle"
 LIB = ORACLE_DIR / "libwgml_oracle.so"
 
 F32, Q8_0, Q4_K, Q6_K = 0, 8, 12, 14
+F16, Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, Q8_K = 1, 2, 3, 6, 7, 13, 15
 
 
 def build(force: bool = False) -> None:

@@ -38,7 +38,8 @@ def test_version_and_host_helpers():
     assert _lib.lib.wgml_quant_block_elems(W.Q8_0) == 32
     assert _lib.lib.wgml_quant_block_elems(W.Q4_K) == 256
     assert _lib.lib.wgml_quant_block_elems(W.Q6_K) == 256
-    assert _lib.lib.wgml_quant_block_elems(2) == 0  # Q4_0: outside this path
+    assert _lib.lib.wgml_quant_block_elems(W.Q4_0) == 32 and _lib.lib.wgml_quant_block_elems(W.Q5_K) == 256
+    assert _lib.lib.wgml_quant_block_elems(10) == 0  # Q2_K: a format the reference cannot read either
     assert W.quant_bytes(W.Q4_K, 100) == 0          # not a whole block
     assert W.quant_bytes(W.F32, 10) == 40
 

@@ -59,6 +59,41 @@ def test_dequant_random_bits_bit_exact(gpu, qtype, nrows, nblk_per_row):
     assert np.array_equal(bits(got), bits(want))
 
 
+EXPANDED = [("q4_0", W.Q4_0), ("q4_1", W.Q4_1), ("q5_0", W.Q5_0), ("q5_1", W.Q5_1),
+            ("q5_k", W.Q5_K), ("q8_k", W.Q8_K)]
+
+
+@pytest.mark.parametrize("name,qtype", EXPANDED)
+def test_formats_expanded_to_f32_at_load(gpu, name, qtype):
+    # GgufTensorData::to_gpu_matrix dequantizes these to an f32 matrix (gguf.rs:131-184); here the
+    # expansion runs on the device.  Reference fixture blocks, then random bits; bit-exact.
+    raw, want = GOLD[f"{name}_raw"], GOLD[f"{name}_expected"]
+    be = npref.BLOCK_ELEMS[qtype]
+    m = W.GpuQuantMatrix(gpu, qtype, 2, 8 * be, raw)
+    assert m.shape() == (W.F32, 2, 8 * be) and m.gguf_bytes() == 2 * 8 * be * 4
+    assert np.array_equal(bits(gpu_dequant(gpu, qtype, raw, 2, 8 * be)), bits(want))
+    nrows, nblk = 5, 7
+    rnd = npref.random_blocks(qtype, nrows * nblk, seed=500 + qtype)
+    want = orc.dequantize(qtype, rnd, nrows * nblk * be)
+    assert np.array_equal(bits(gpu_dequant(gpu, qtype, rnd, nrows, nblk * be)), bits(want))
+    # host dequantizer, same values
+    assert np.array_equal(bits(W.dequantize_host(qtype, rnd, want.size)), bits(want))
+    # and the matrix is usable by the GEMV (f32 path)
+    x = W.rng_normal(5, nblk * be)
+    out = W.GpuVector.uninit(gpu, nrows)
+    W.GemvQuant.from_device(gpu).dispatch(out, W.GpuQuantMatrix(gpu, qtype, nrows, nblk * be, rnd),
+                                          W.GpuVector.init(gpu, x))
+    ref = want.reshape(nrows, -1).astype(np.float64) @ x.astype(np.float64)
+    np.testing.assert_allclose(out.read(), ref, rtol=0, atol=1e-4 * np.abs(ref).max())
+
+
+def test_f16_matrix_expanded_at_load(gpu):
+    h = np.arange(4 * 64, dtype=np.uint16) * 97 % 31744  # finite halves
+    want = np.array([orc.decode_f16(int(b)) for b in h], dtype=np.float32)
+    assert np.array_equal(bits(gpu_dequant(gpu, W.F16, h.view(np.uint8), 4, 64)), bits(want))
+    assert np.array_equal(bits(W.dequantize_host(W.F16, h.view(np.uint8), h.size)), bits(want))
+
+
 def test_f32_matrix_round_trip(gpu):
     a = W.rng_normal(5, 12 * 64)
     got = gpu_dequant(gpu, W.F32, a.view(np.uint8), 12, 64)
@@ -76,8 +111,8 @@ def test_quantized_then_dequantized_matches_oracle(gpu):
 
 def test_matrix_create_errors(gpu):
     raw = np.zeros(144 * 4, dtype=np.uint8)
-    with pytest.raises(W.WgmlError) as ei:  # Q5_K: a tag outside this path
-        W.GpuQuantMatrix(gpu, 13, 1, 256, raw)
+    with pytest.raises(W.WgmlError) as ei:  # Q2_K: a tag the reference cannot read either
+        W.GpuQuantMatrix(gpu, 10, 1, 256, raw)
     assert ei.value.code == W._lib.E_UNSUPPORTED
     with pytest.raises(W.WgmlError) as ei:  # ncols not a whole number of blocks
         W.GpuQuantMatrix(gpu, W.Q4_K, 4, 200, raw)

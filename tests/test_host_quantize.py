@@ -78,3 +78,18 @@ def test_quantize_errors():
     assert W.quant_bytes(W.Q8_0, 4096 * 11008) == 47906816
     assert W.quant_bytes(W.Q4_K, 4096 * 11008) == 25362432
     assert W.quant_bytes(W.Q6_K, 4096 * 11008) == 36986880
+
+
+@pytest.mark.parametrize("qtype", [1, 2, 3, 6, 7, 8, 12, 13, 14, 15])
+def test_dequantize_host_matches_oracle(qtype):
+    # Block*::dequantize on the host (what the reference does for tensors it keeps in f32)
+    import npref
+    import oracle as orc
+    nb = 300
+    raw = npref.random_blocks(qtype, nb, seed=40 + qtype)
+    n = nb * npref.BLOCK_ELEMS[qtype]
+    got = W.dequantize_host(qtype, raw, n)
+    want = orc.dequantize(qtype, raw, n)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    with pytest.raises(W.WgmlError):
+        W.dequantize_host(10, raw, 256)  # Q2_K: unsupported

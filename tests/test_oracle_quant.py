@@ -30,7 +30,13 @@ def test_decode_f16_exhaustive_vs_numpy():
     assert orc.decode_f16(0x45AE) == 5.6796875
 
 
-@pytest.mark.parametrize("name,qtype", [("q8_0", orc.Q8_0), ("q4_k", orc.Q4_K), ("q6_k", orc.Q6_K)])
+ALL_FIXTURES = [("q8_0", orc.Q8_0), ("q4_k", orc.Q4_K), ("q6_k", orc.Q6_K), ("q4_0", orc.Q4_0),
+                ("q4_1", orc.Q4_1), ("q5_0", orc.Q5_0), ("q5_1", orc.Q5_1), ("q5_k", orc.Q5_K),
+                ("q8_k", orc.Q8_K)]
+ALL_TYPES = [t for _, t in ALL_FIXTURES]
+
+
+@pytest.mark.parametrize("name,qtype", ALL_FIXTURES)
 def test_dequant_reference_fixture_blocks(name, qtype):
     raw, want = GOLD[f"{name}_raw"], GOLD[f"{name}_expected"]
     got = orc.dequantize(qtype, raw, want.size)
@@ -49,9 +55,23 @@ def test_dequant_hand_computed_anchors():
     assert q4[128 + 5] == 49.375                # sub-block 4: sc 8, m 0, nibble 5
     q6 = orc.dequantize(orc.Q6_K, GOLD["q6_k_raw"], 16 * 256)
     assert q6[0] == 499872 / 2 ** 24            # (123*2^-24) * -127 * -32
+    q40 = orc.dequantize(orc.Q4_0, GOLD["q4_0_raw"], 16 * 32)
+    assert q40[0] == -8 * 1.234375 and q40[16] == -8 * 1.234375   # block 0: qs[0] = 0x00
+    assert q40[32 + 1] == (1 - 8) * 1.234375 and q40[32 + 17] == (1 - 8) * 1.234375  # 0x11
+    q41 = orc.dequantize(orc.Q4_1, GOLD["q4_1_raw"], 16 * 32)
+    assert q41[5] == np.float32(5 * 1.234375) + np.float32(3 * 2.0 ** -24)
+    q50 = orc.dequantize(orc.Q5_0, GOLD["q5_0_raw"], 16 * 32)
+    # qh = [1, 100, 200, 250] -> u32 0xFAC86401: bit 0 set (element 0 gets +16), bit 1 clear
+    assert q50[0] == (0 + 16 - 16) * 1.234375 and q50[1] == (1 - 16) * 1.234375
+    # element 16 takes bit 16 (0xC8 = 0b11001000 -> bit 0 clear), element 19 takes bit 19 (set)
+    assert q50[16] == (0 - 16) * 1.234375 and q50[19] == (0 + 16 - 16) * 1.234375
+    q8k = orc.dequantize(orc.Q8_K, GOLD["q8_k_raw"], 16 * 256)
+    assert q8k[0] == np.float32(1.234) * np.float32(-127) and q8k[255] == np.float32(1.234) * -128
+    q5k = orc.dequantize(orc.Q5_K, GOLD["q5_k_raw"], 16 * 256)
+    assert np.all(q5k[0:32:2] == -22.71875)     # block 0: sc 0 -> -(dmin * 4) whatever the quants
 
 
-@pytest.mark.parametrize("qtype", [orc.Q8_0, orc.Q4_K, orc.Q6_K])
+@pytest.mark.parametrize("qtype", ALL_TYPES + [orc.F16])
 def test_dequant_random_bits_vs_numpy(qtype):
     nb = 10000
     raw = npref.random_blocks(qtype, nb, seed=1234 + qtype)

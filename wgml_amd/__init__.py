@@ -5,7 +5,8 @@ ABI, see include/wgml_hip.h); this package is the thin host-side mirror of the
 reference's `wgml::ops` / `wgml::models` names.  Importing fails if the library
 has not been built: there is no CPU fallback.
 """
-from ._lib import (F32, Q4_K, Q6_K, Q8_0, LIB_PATH, WgmlError, lib)  # noqa: F401
+from ._lib import (F16, F32, Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0, Q8_K, LIB_PATH,  # noqa: F401
+                   WgmlError, lib)
 from .ops import *  # noqa: F401,F403
 from .models import *  # noqa: F401,F403
 from .models import prompt_tokens  # noqa: F401

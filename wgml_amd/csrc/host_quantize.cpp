@@ -373,14 +373,14 @@ extern "C" {
 
 int wgml_quantize(int type, const float *src, void *dst, uint64_t nelems, int nthreads) {
     WGML_REQUIRE(src && dst, "wgml_quantize: null argument");
-    uint32_t be = wgml_quant_block_elems(type);
-    if (!be || type == WGML_F32) {
-        if (type == WGML_F32) {
-            memcpy(dst, src, nelems * 4);
-            return WGML_OK;
-        }
-        return set_error(WGML_E_UNSUPPORTED, "wgml_quantize: unsupported type %d", type);
+    if (type == WGML_F32) {
+        memcpy(dst, src, nelems * 4);
+        return WGML_OK;
     }
+    if (type != WGML_Q8_0 && type != WGML_Q4_K && type != WGML_Q6_K)
+        return set_error(WGML_E_UNSUPPORTED,
+                         "wgml_quantize: no quantizer for type %d (Q8_0, Q4_K, Q6_K only)", type);
+    const uint32_t be = wgml_quant_block_elems(type);
     WGML_REQUIRE(nelems % be == 0, "wgml_quantize: %llu elements is not a whole number of blocks",
                  (unsigned long long)nelems);
     const uint64_t nblocks = nelems / be;
@@ -417,8 +417,72 @@ int wgml_dequantize_host(int type, const void *src, float *dst, uint64_t nelems,
         return WGML_OK;
     }
     const uint32_t be = wgml_quant_block_elems(type);
-    if (!be || (type != WGML_Q8_0 && type != WGML_Q4_K && type != WGML_Q6_K))
-        return set_error(WGML_E_UNSUPPORTED, "wgml_dequantize_host: unsupported type %d", type);
+    if (!be) return set_error(WGML_E_UNSUPPORTED, "wgml_dequantize_host: unsupported type %d", type);
+    if (type != WGML_Q8_0 && type != WGML_Q4_K && type != WGML_Q6_K) {
+        WGML_REQUIRE(nelems % be == 0,
+                     "wgml_dequantize_host: %llu elements is not a whole number of blocks",
+                     (unsigned long long)nelems);
+        const uint8_t *raw = (const uint8_t *)src;
+        auto u16 = [](const uint8_t *p) { return (uint16_t)(p[0] | ((uint16_t)p[1] << 8)); };
+        auto u32 = [](const uint8_t *p) {
+            return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+        };
+        parallel_for(nelems / be, nthreads, [=](uint64_t b0, uint64_t b1) {
+            for (uint64_t bi = b0; bi < b1; ++bi) {
+                float *y = dst + bi * be;
+                if (type == WGML_Q8_K) {  // quantization.rs:195-201
+                    const uint8_t *b = raw + bi * 292;
+                    float d;
+                    memcpy(&d, b, 4);
+                    for (int j = 0; j < QK_K; ++j) y[j] = d * (float)(int8_t)b[4 + j];
+                } else if (type == WGML_Q5_K) {  // quantization.rs:274-317
+                    const uint8_t *b = raw + bi * 176;
+                    const float d = f16_to_f32(u16(b)), dmin = f16_to_f32(u16(b + 2));
+                    const uint8_t *sc = b + 4, *qh = b + 16, *qs = b + 48;
+                    for (int sub = 0; sub < 8; ++sub) {
+                        uint8_t s8, m8;
+                        if (sub < 4) {
+                            s8 = sc[sub] & 63;
+                            m8 = sc[sub + 4] & 63;
+                        } else {
+                            s8 = (uint8_t)((sc[sub + 4] & 0xF) | ((sc[sub - 4] >> 6) << 4));
+                            m8 = (uint8_t)((sc[sub + 4] >> 4) | ((sc[sub] >> 6) << 4));
+                        }
+                        const float dl = d * (float)s8, ml = dmin * (float)m8;
+                        for (int l = 0; l < 32; ++l) {
+                            const uint8_t q = qs[(sub >> 1) * 32 + l];
+                            const int x = ((sub & 1) ? (q >> 4) : (q & 0xF)) + (((qh[l] >> sub) & 1) ? 16 : 0);
+                            y[sub * 32 + l] = dl * (float)x - ml;
+                        }
+                    }
+                } else {  // Q4_0 / Q4_1 / Q5_0 / Q5_1: quantization.rs:53-68, 82-98, 112-131, 146-167
+                    const bool has_m = type == WGML_Q4_1 || type == WGML_Q5_1;
+                    const bool has_qh = type == WGML_Q5_0 || type == WGML_Q5_1;
+                    const uint8_t *b = raw + bi * (18 + (has_m ? 2 : 0) + (has_qh ? 4 : 0));
+                    const float d = f16_to_f32(u16(b));
+                    const float m = has_m ? f16_to_f32(u16(b + 2)) : 0.f;
+                    const uint32_t qh = has_qh ? u32(b + 2 + (has_m ? 2 : 0)) : 0u;
+                    const uint8_t *qs = b + 2 + (has_m ? 2 : 0) + (has_qh ? 4 : 0);
+                    for (uint32_t j = 0; j < 16; ++j) {
+                        uint32_t x0 = qs[j] & 0x0Fu, x1 = (uint32_t)(qs[j] >> 4);
+                        if (has_qh) {
+                            x0 |= ((qh >> j) << 4) & 0x10u;
+                            x1 |= (qh >> (j + 12)) & 0x10u;
+                        }
+                        if (has_m) {
+                            y[j] = (float)x0 * d + m;
+                            y[j + 16] = (float)x1 * d + m;
+                        } else {
+                            const int off = has_qh ? 16 : 8;
+                            y[j] = (float)((int)x0 - off) * d;
+                            y[j + 16] = (float)((int)x1 - off) * d;
+                        }
+                    }
+                }
+            }
+        });
+        return WGML_OK;
+    }
     WGML_REQUIRE(nelems % be == 0,
                  "wgml_dequantize_host: %llu elements is not a whole number of blocks",
                  (unsigned long long)nelems);

@@ -114,12 +114,74 @@ __global__ void f16_to_f32_kernel(const uint16_t *__restrict__ in, float *__rest
     if (i < n) out[i] = f16_bits_to_f32(in[i]);
 }
 
+// ---- formats that the reference expands to f32 at load ----------------------
+// GgufTensorData::to_gpu_matrix (gguf.rs:131-184) keeps Q8_0 / Q4_K / Q6_K
+// quantized and dequantizes everything else; these kernels do that expansion on
+// the device from the raw GGUF bytes (one thread per element; byte loads, the
+// blocks are only 2-byte aligned).  Arithmetic as Block*::dequantize
+// (quantization.rs:16-24, 53-68, 82-98, 112-131, 146-167, 195-201, 274-317).
+__device__ __forceinline__ uint16_t ld_u16(const uint8_t *p) {
+    return (uint16_t)(p[0] | ((uint16_t)p[1] << 8));
+}
+__device__ __forceinline__ uint32_t ld_u32(const uint8_t *p) {
+    return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+
+template <int TYPE>
+__global__ void dequant_raw_kernel(const uint8_t *__restrict__ raw, float *__restrict__ out,
+                                   uint64_t n) {
+    const uint64_t e = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    if (TYPE == WGML_F16) {
+        out[e] = f16_bits_to_f32(ld_u16(raw + e * 2));
+    } else if (TYPE == WGML_Q4_0 || TYPE == WGML_Q4_1 || TYPE == WGML_Q5_0 || TYPE == WGML_Q5_1) {
+        constexpr int BYTES = TYPE == WGML_Q4_0 ? 18 : TYPE == WGML_Q4_1 ? 20 : TYPE == WGML_Q5_0 ? 22 : 24;
+        constexpr bool HAS_M = TYPE == WGML_Q4_1 || TYPE == WGML_Q5_1;
+        constexpr bool HAS_QH = TYPE == WGML_Q5_0 || TYPE == WGML_Q5_1;
+        const uint8_t *b = raw + (e / 32) * BYTES;
+        const uint32_t k = (uint32_t)(e % 32), j = k & 15;
+        const float d = f16_bits_to_f32(ld_u16(b));
+        const uint8_t *qs = b + 2 + (HAS_M ? 2 : 0) + (HAS_QH ? 4 : 0);
+        uint32_t x = k < 16 ? (qs[j] & 0x0Fu) : (uint32_t)(qs[j] >> 4);
+        if (HAS_QH) {
+            const uint32_t qh = ld_u32(b + 2 + (HAS_M ? 2 : 0));
+            x |= k < 16 ? ((qh >> j) << 4) & 0x10u : (qh >> (j + 12)) & 0x10u;
+        }
+        if (HAS_M) {
+            const float m = f16_bits_to_f32(ld_u16(b + 2));
+            out[e] = (float)x * d + m;
+        } else {
+            out[e] = (float)((int)x - (HAS_QH ? 16 : 8)) * d;
+        }
+    } else if (TYPE == WGML_Q8_K) {
+        const uint8_t *b = raw + (e / QK_K) * 292;
+        const float d = __uint_as_float(ld_u32(b));
+        out[e] = d * (float)(int8_t)b[4 + e % QK_K];
+    } else if (TYPE == WGML_Q5_K) {
+        const uint8_t *b = raw + (e / QK_K) * 176;
+        const uint32_t k = (uint32_t)(e % QK_K), sub = k >> 5, l = k & 31;  // 8 sub-blocks of 32
+        const float d = f16_bits_to_f32(ld_u16(b)), dmin = f16_bits_to_f32(ld_u16(b + 2));
+        uint8_t sc, mn;
+        get_scale_min_k4(sub, b + 4, sc, mn);
+        const uint8_t q = b[48 + (sub >> 1) * 32 + l];
+        const uint32_t nib = (sub & 1) ? (uint32_t)(q >> 4) : (q & 0x0Fu);
+        const uint32_t x = nib + ((b[16 + l] >> sub) & 1u) * 16u;
+        out[e] = (d * (float)sc) * (float)x - dmin * (float)mn;
+    }
+}
+
+// True for the formats expanded to f32 at load.
+bool expands_to_f32(int type) {
+    return type == WGML_F16 || type == WGML_Q4_0 || type == WGML_Q4_1 || type == WGML_Q5_0 ||
+           type == WGML_Q5_1 || type == WGML_Q5_K || type == WGML_Q8_K;
+}
+
 uint32_t block_elems(int type) {
     switch (type) {
-    case WGML_F32: return 1;
+    case WGML_F32: case WGML_F16: return 1;
+    case WGML_Q4_0: case WGML_Q4_1: case WGML_Q5_0: case WGML_Q5_1: return 32;
     case WGML_Q8_0: return QK8_0;
-    case WGML_Q4_K: return QK_K;
-    case WGML_Q6_K: return QK_K;
+    case WGML_Q4_K: case WGML_Q5_K: case WGML_Q6_K: case WGML_Q8_K: return QK_K;
     default: return 0;
     }
 }
@@ -127,9 +189,16 @@ uint32_t block_elems(int type) {
 uint32_t block_bytes(int type) {
     switch (type) {
     case WGML_F32: return 4;
+    case WGML_F16: return 2;
+    case WGML_Q4_0: return 18;
+    case WGML_Q4_1: return 20;
+    case WGML_Q5_0: return 22;
+    case WGML_Q5_1: return 24;
     case WGML_Q8_0: return Q8_0_BYTES;
     case WGML_Q4_K: return Q4_K_BYTES;
+    case WGML_Q5_K: return 176;
     case WGML_Q6_K: return Q6_K_BYTES;
+    case WGML_Q8_K: return 292;
     default: return 0;
     }
 }
@@ -188,7 +257,8 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
     if (!be)
         return set_error(WGML_E_UNSUPPORTED,
                          "wgml_quant_matrix_create: quantization type %d is not supported "
-                         "(supported: F32, Q8_0, Q4_K, Q6_K)",
+                         "(quantized: Q8_0, Q4_K, Q6_K; expanded to f32: F32, F16, Q4_0, Q4_1, "
+                         "Q5_0, Q5_1, Q5_K, Q8_K)",
                          type);
     WGML_REQUIRE(nrows > 0 && ncols > 0, "wgml_quant_matrix_create: empty matrix %ux%u", nrows,
                  ncols);
@@ -202,16 +272,18 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
     uint64_t nblocks = nelem / be;
     uint64_t gguf = nblocks * block_bytes(type);
 
+    const bool expand = expands_to_f32(type);
     wgml_qmat *m = new wgml_qmat();
     m->ctx = ctx;
     ctx_retain(ctx);
-    m->type = type;
+    m->type = expand ? (int)WGML_F32 : type;
     m->nrows = nrows;
     m->ncols = ncols;
-    m->gguf_bytes = gguf;
+    m->gguf_bytes = expand ? nelem * 4 : gguf;  // what a GEMV over this matrix streams
 
     uint64_t o1 = 0, o2 = 0, o3 = 0, total = 0;
-    switch (type) {
+    if (expand) total = align256(nelem * 4);
+    switch (expand ? -1 : type) {
     case WGML_F32:
     case WGML_Q4_K: total = align256(gguf); break;
     case WGML_Q8_0:
@@ -263,6 +335,18 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
             if (type == WGML_Q8_0) {
                 repack_q8_0<<<dim3((unsigned)((nblocks + T - 1) / T)), dim3(T), 0, ctx->stream>>>(
                     (const uint16_t *)raw, (uint32_t *)m->p0, (uint16_t *)m->p1, nblocks);
+            } else if (expand) {
+                const dim3 g((unsigned)((nelem + T - 1) / T)), b(T);
+                float *o = reinterpret_cast<float *>(m->p0);
+                switch (type) {
+                case WGML_F16: dequant_raw_kernel<WGML_F16><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
+                case WGML_Q4_0: dequant_raw_kernel<WGML_Q4_0><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
+                case WGML_Q4_1: dequant_raw_kernel<WGML_Q4_1><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
+                case WGML_Q5_0: dequant_raw_kernel<WGML_Q5_0><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
+                case WGML_Q5_1: dequant_raw_kernel<WGML_Q5_1><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
+                case WGML_Q5_K: dequant_raw_kernel<WGML_Q5_K><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
+                default: dequant_raw_kernel<WGML_Q8_K><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
+                }
             } else {
                 uint64_t nt = nblocks * 105;
                 repack_q6_k<<<dim3((unsigned)((nt + T - 1) / T)), dim3(T), 0, ctx->stream>>>(

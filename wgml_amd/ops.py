@@ -20,7 +20,8 @@ __all__ = [
     "GpuInstance", "GpuVector", "GpuMatrix", "GpuQuantMatrix", "GemvQuant", "Gemv", "Quantization",
     "RmsNorm", "RmsNormConfig", "LayerNorm", "RoPE", "RoPEConfig", "RoPEVariant", "SoftMax",
     "BatchedMultiqueryAttention", "BatchedMultiqueryAttentionParams", "Silu", "UnaryOp",
-    "UnaryInplace", "OpAssign", "OpAssignVariant", "Sampler", "quantize", "quant_bytes",
+    "UnaryInplace", "OpAssign", "OpAssignVariant", "Sampler", "quantize", "dequantize_host",
+    "quant_bytes",
     "rng_normal", "rng_tokens", "WgmlError",
 ]
 
