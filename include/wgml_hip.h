@@ -342,6 +342,21 @@ WGML_API int wgml_bench_gemv_fused(wgml_ctx *ctx, const wgml_qmat *const *a,
                                    uint32_t nsets, wgml_view out, uint32_t stride, wgml_view v,
                                    const wgml_view *norm_w, uint32_t iters, float *total_ms);
 
+/* ---- sampling beyond greedy: Sampler::sample (models/sampler.rs:32-130), host only ---- *
+ * temperature 0: arg-max.  Otherwise the logits are divided by the temperature,
+ * turned into probabilities (in place) and a token is drawn with `coin` in [0, 1):
+ * from the whole distribution if topp <= 0 or >= 1, else from the smallest set of
+ * most likely tokens whose probability exceeds topp. */
+WGML_API int wgml_sample(float *logits, uint32_t n, float temperature, float topp, float coin,
+                         uint32_t *out_token);
+/* The token loop of ChatLlama2::forward with that sampler (chat_llama2.rs:51-153;
+ * the reference uses temperature 0.7, top-p 0.95 there, wgml-chat/src/sampler.rs:109):
+ * logits are read back after every step and sampled on the host; the coin of position
+ * p is the p-th output of the library's counter-based generator for `seed`. */
+WGML_API int wgml_llama2_generate_sampled(wgml_llama2 *m, const uint32_t *prompt,
+                                          uint32_t n_prompt, uint32_t n_total, float temperature,
+                                          float topp, uint64_t seed, uint32_t *out_tokens);
+
 /* ---- GGUF container: Gguf::from_bytes (gguf.rs:450-607), host only -------- *
  * The file is memory-mapped (or the caller's bytes are used in place); the
  * pointers handed out below point into it and stay valid until close.
@@ -398,6 +413,8 @@ WGML_API int wgml_dequantize_host(int type, const void *src, float *dst, uint64_
  * normal: mean + std * N(0,1) by Box-Muller in f32. */
 WGML_API int wgml_rng_normal(uint64_t seed, float *out, uint64_t n, float mean, float std,
                              int nthreads);
+/* uniform floats in [0, 1) (24 random bits each). */
+WGML_API int wgml_rng_uniform_f32(uint64_t seed, float *out, uint64_t n);
 /* uniform integers in [0, bound). */
 WGML_API int wgml_rng_uniform_u32(uint64_t seed, uint32_t *out, uint64_t n, uint32_t bound);
 

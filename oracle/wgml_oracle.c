@@ -482,6 +482,71 @@ void orc_attention(const orc_attn_params *p, const float *q, const float *key_ca
     }
 }
 
+/* models/sampler.rs:58-76: `probabilities` sum to 1, coin in [0, 1). */
+uint32_t orc_sample_mult(const float *p, int n, float coin) {
+    float cdf = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        cdf += p[i];
+        if (coin < cdf) return (uint32_t)i;
+    }
+    return (uint32_t)(n - 1);
+}
+
+/* models/sampler.rs:78-130.  Candidates with p >= (1 - topp) / (n - 1), sorted by
+ * decreasing probability (stable: ties keep index order, as Rust's sort_by_key),
+ * cut where the running sum first exceeds topp, then sampled with coin * sum. */
+uint32_t orc_sample_topp(const float *p, int n, float topp, float coin) {
+    const float cutoff = (1.0f - topp) / ((float)n - 1.0f);
+    int *idx = (int *)malloc(sizeof(int) * (size_t)n);
+    int n0 = 0;
+    for (int i = 0; i < n; ++i)
+        if (p[i] >= cutoff) idx[n0++] = i;
+    if (n0 == 0) { /* the reference would index out of bounds here; it cannot happen for
+                      probabilities that sum to 1 */
+        free(idx);
+        return (uint32_t)(n - 1);
+    }
+    for (int i = 1; i < n0; ++i) { /* stable insertion sort, descending */
+        const int v = idx[i];
+        int j = i - 1;
+        while (j >= 0 && p[idx[j]] < p[v]) {
+            idx[j + 1] = idx[j];
+            --j;
+        }
+        idx[j + 1] = v;
+    }
+    float cumulative = 0.0f;
+    int last = n0 - 1;
+    for (int i = 0; i < n0; ++i) {
+        cumulative += p[idx[i]];
+        if (cumulative > topp) {
+            last = i;
+            break;
+        }
+    }
+    const float r = coin * cumulative;
+    float cdf = 0.0f;
+    uint32_t out = (uint32_t)idx[last];
+    for (int i = 0; i <= last; ++i) {
+        cdf += p[idx[i]];
+        if (r < cdf) {
+            out = (uint32_t)idx[i];
+            break;
+        }
+    }
+    free(idx);
+    return out;
+}
+
+/* models/sampler.rs:32-52: logits are modified in place (scaled, then softmax). */
+uint32_t orc_sample(float *logits, int n, float temperature, float topp, float coin) {
+    if (temperature == 0.0f) return orc_argmax(logits, n);
+    for (int i = 0; i < n; ++i) logits[i] /= temperature;
+    orc_softmax(logits, n);
+    if (topp <= 0.0f || topp >= 1.0f) return orc_sample_mult(logits, n, coin);
+    return orc_sample_topp(logits, n, topp, coin);
+}
+
 /* models/sampler.rs:54-56 */
 uint32_t orc_argmax(const float *v, int n) {
     int best = 0;

@@ -119,6 +119,10 @@ void orc_attention(const orc_attn_params *p, const float *q, const float *key_ca
 
 /* models/sampler.rs:54-56: index of the first maximum. */
 uint32_t orc_argmax(const float *v, int n);
+/* models/sampler.rs:32-130 with the random number passed in (`coin` in [0, 1)). */
+uint32_t orc_sample_mult(const float *p, int n, float coin);
+uint32_t orc_sample_topp(const float *p, int n, float topp, float coin);
+uint32_t orc_sample(float *logits, int n, float temperature, float topp, float coin);
 
 /* A matrix as the oracle sees it: a tag plus GGUF bytes (or f32 values). */
 typedef struct {

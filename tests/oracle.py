@@ -333,3 +333,27 @@ class Gpt2:
             lib.orc_gpt2_free(self._h)
         except Exception:
             pass
+
+
+lib.orc_sample.restype = C.c_uint32
+lib.orc_sample.argtypes = [_P, _i, C.c_float, C.c_float, C.c_float]
+lib.orc_sample_mult.restype = C.c_uint32
+lib.orc_sample_mult.argtypes = [_P, _i, C.c_float]
+lib.orc_sample_topp.restype = C.c_uint32
+lib.orc_sample_topp.argtypes = [_P, _i, C.c_float, C.c_float]
+
+
+def sample(logits: np.ndarray, temperature: float, topp: float, coin: float) -> int:
+    """Sampler::sample (models/sampler.rs:32-52) on a copy of `logits`."""
+    v = np.ascontiguousarray(logits, dtype=np.float32).copy()
+    return int(lib.orc_sample(_p(v), v.size, temperature, topp, coin))
+
+
+def sample_mult(p: np.ndarray, coin: float) -> int:
+    v = np.ascontiguousarray(p, dtype=np.float32)
+    return int(lib.orc_sample_mult(_p(v), v.size, coin))
+
+
+def sample_topp(p: np.ndarray, topp: float, coin: float) -> int:
+    v = np.ascontiguousarray(p, dtype=np.float32)
+    return int(lib.orc_sample_topp(_p(v), v.size, topp, coin))

@@ -134,6 +134,31 @@ def test_llama_from_gguf_file(gpu, tmp_path):
     assert np.array_equal(m.generate_greedy(prompt, 24), want)
 
 
+def test_llama_sampled_generation(gpu):
+    # temperature / top-p sampling on the host from logits read back every step, seeded coins:
+    # the same tokens as the oracle's forward + the oracle's sampler with the same coins.
+    # (Top-2 margins in probability space are wide on this model, so fp32 differences between
+    # the two forwards do not move a token across a coin.)
+    w = synth_llama(MICRO, seed=51, scheme="q8_0")
+    prompt = W.prompt_tokens(51, 3, MICRO.vocab_size)
+    n_total, temperature, topp, seed = 20, 0.7, 0.95, 1234
+    coins = W.rng_uniform(seed, n_total)
+    ref = orc.Llama2(w)
+    want, tok, gaps = [], int(prompt[0]), []
+    for pos in range(n_total):
+        logits = ref.forward(tok, pos).astype(np.float32)
+        nxt = orc.sample(logits, temperature, topp, float(coins[pos]))
+        want.append(nxt)
+        tok = int(prompt[pos + 1]) if pos + 1 < len(prompt) else nxt
+    m = Llama2(gpu, MICRO).load(w)
+    got = m.generate_sampled(prompt, n_total, temperature, topp, seed)
+    assert list(got) == want
+    assert list(m.generate_sampled(prompt, n_total, temperature, topp, seed)) == want  # seeded
+    assert len(set(want)) > 5  # it really samples
+    greedy = m.generate_sampled(prompt, n_total, 0.0, 0.9, seed)
+    assert np.array_equal(greedy, m.generate_greedy(prompt, n_total))
+
+
 def test_llama_argument_checks(gpu):
     m = Llama2(gpu, MICRO)
     with pytest.raises(W.WgmlError, match="unset weights"):

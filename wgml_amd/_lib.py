@@ -148,6 +148,8 @@ PROTOTYPES = {
     "wgml_bench_gemv_quant": (_i, [_P, _PP, _u32, View, View, _u32, _i, _fp]),
     "wgml_bench_gemv_fused": (_i, [_P, _PP, _PP, C.POINTER(C.c_int), _u32, _u32, View, _u32, View,
                                    C.POINTER(View), _u32, _fp]),
+    "wgml_sample": (_i, [_P, _u32, _f, _f, _f, _u32p]),
+    "wgml_llama2_generate_sampled": (_i, [_P, _P, _u32, _u32, _f, _f, _u64, _P]),
     "wgml_gguf_open": (_i, [C.c_char_p, _PP]),
     "wgml_gguf_open_bytes": (_i, [_P, _u64, _PP]),
     "wgml_gguf_close": (_i, [_P]),
@@ -163,6 +165,7 @@ PROTOTYPES = {
     "wgml_quantize": (_i, [_i, _P, _P, _u64, _i]),
     "wgml_dequantize_host": (_i, [_i, _P, _P, _u64, _i]),
     "wgml_rng_normal": (_i, [_u64, _P, _u64, _f, _f, _i]),
+    "wgml_rng_uniform_f32": (_i, [_u64, _P, _u64]),
     "wgml_rng_uniform_u32": (_i, [_u64, _P, _u64, _u32]),
     # debug knob, not part of the reference surface
     "wgml_debug_set_gemv_rows_per_wave": (_i, [_i]),

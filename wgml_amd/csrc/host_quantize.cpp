@@ -555,6 +555,13 @@ int wgml_rng_normal(uint64_t seed, float *out, uint64_t n, float mean, float std
     return WGML_OK;
 }
 
+int wgml_rng_uniform_f32(uint64_t seed, float *out, uint64_t n) {
+    WGML_REQUIRE(out != nullptr || n == 0, "wgml_rng_uniform_f32: null output");
+    for (uint64_t i = 0; i < n; ++i)  // top 24 bits: every value is exact in f32 and < 1
+        out[i] = (float)(counter_hash(seed ^ 0xc2b2ae35u, i) >> 40) * (1.0f / 16777216.0f);
+    return WGML_OK;
+}
+
 int wgml_rng_uniform_u32(uint64_t seed, uint32_t *out, uint64_t n, uint32_t bound) {
     WGML_REQUIRE(out != nullptr || n == 0, "wgml_rng_uniform_u32: null output");
     WGML_REQUIRE(bound > 0, "wgml_rng_uniform_u32: bound must be positive");

@@ -582,6 +582,32 @@ int wgml_llama2_decode_greedy_sync(wgml_llama2 *m, uint32_t first_token, uint32_
     return WGML_OK;
 }
 
+// ChatLlama2::forward with the CPU sampler (chat_llama2.rs:51-153): logits come
+// back to the host after every step, as in the reference.
+int wgml_llama2_generate_sampled(wgml_llama2 *m, const uint32_t *prompt, uint32_t n_prompt,
+                                 uint32_t n_total, float temperature, float topp, uint64_t seed,
+                                 uint32_t *out_tokens) {
+    WGML_REQUIRE(m && prompt && out_tokens, "wgml_llama2_generate_sampled: null argument");
+    WGML_REQUIRE(n_prompt >= 1, "wgml_llama2_generate_sampled: empty prompt");
+    WGML_REQUIRE(n_total <= m->cfg.seq_len,
+                 "wgml_llama2_generate_sampled: %u positions exceed seq_len %u", n_total,
+                 m->cfg.seq_len);
+    if (n_total == 0) return WGML_OK;
+    std::vector<float> logits(m->cfg.vocab_size), coins(n_total);
+    WGML_TRY(wgml_rng_uniform_f32(seed, coins.data(), n_total));
+    uint32_t token = prompt[0];
+    for (uint32_t pos = 0; pos < n_total; ++pos) {
+        WGML_TRY(wgml_llama2_forward(m, token, pos));
+        WGML_TRY(wgml_llama2_read_logits(m, logits.data()));
+        uint32_t next = 0;
+        WGML_TRY(wgml_sample(logits.data(), m->cfg.vocab_size, temperature, topp, coins[pos],
+                             &next));
+        out_tokens[pos] = next;
+        token = (pos + 1 < n_prompt) ? prompt[pos + 1] : next;
+    }
+    return WGML_OK;
+}
+
 static int kv_range(wgml_llama2 *m, uint32_t layer, int which, uint32_t first_pos, uint32_t n_pos,
                     float **p) {
     WGML_REQUIRE(layer < m->cfg.n_layers, "kv: layer %u of %u", layer, m->cfg.n_layers);

@@ -153,6 +153,15 @@ class Llama2:
         config = llama2_config_from_gguf(gguf, model_type)
         return cls(gpu, config, model_type).load(llama2_weights_from_gguf(gguf, config))
 
+    def generate_sampled(self, prompt, n_total: int, temperature: float, topp: float,
+                         seed: int) -> np.ndarray:
+        """Token loop with the CPU sampler (temperature / top-p), seeded."""
+        p = np.ascontiguousarray(prompt, dtype=np.uint32)
+        out = np.empty(n_total, dtype=np.uint32)
+        call("wgml_llama2_generate_sampled", self._h, _ptr(p), p.size, n_total, temperature, topp,
+             seed, _ptr(out))
+        return out
+
     def set_fusion(self, level: int) -> None:
         call("wgml_llama2_set_fusion", self._h, level)
 

@@ -22,7 +22,7 @@ __all__ = [
     "BatchedMultiqueryAttention", "BatchedMultiqueryAttentionParams", "Silu", "UnaryOp",
     "UnaryInplace", "OpAssign", "OpAssignVariant", "Sampler", "quantize", "dequantize_host",
     "quant_bytes",
-    "rng_normal", "rng_tokens", "WgmlError",
+    "rng_normal", "rng_uniform", "rng_tokens", "WgmlError",
 ]
 
 
@@ -350,10 +350,20 @@ class OpAssign:
 
 
 class Sampler:
-    """models/sampler.rs: only the greedy branch (temperature == 0)."""
+    """models/sampler.rs: `sample_argmax` on the device (the greedy branch); `sample` is the
+    CPU sampler (temperature, top-p) with the random number passed in."""
 
-    def __init__(self, gpu: GpuInstance):
-        self.gpu = gpu
+    def __init__(self, gpu: Optional[GpuInstance] = None, temperature: float = 0.0,
+                 topp: float = 0.0):
+        self.gpu, self.temperature, self.topp = gpu, temperature, topp
+
+    def sample(self, logits: np.ndarray, coin: float) -> int:
+        """Sampler::sample (models/sampler.rs:32-52); `logits` is modified in place."""
+        assert logits.dtype == np.float32 and logits.flags.c_contiguous
+        out = C.c_uint32()
+        call("wgml_sample", _ptr(logits), logits.size, self.temperature, self.topp, coin,
+             C.byref(out))
+        return out.value
 
     def sample_argmax(self, logits: GpuVector) -> int:
         out = C.c_uint32()
@@ -391,6 +401,13 @@ def rng_normal(seed: int, n: int, mean: float = 0.0, std: float = 1.0,
                nthreads: int = 0) -> np.ndarray:
     out = np.empty(n, dtype=np.float32)
     call("wgml_rng_normal", seed, _ptr(out), n, mean, std, nthreads)
+    return out
+
+
+def rng_uniform(seed: int, n: int) -> np.ndarray:
+    """Uniform f32 in [0, 1): the sampler's coins."""
+    out = np.empty(n, dtype=np.float32)
+    call("wgml_rng_uniform_f32", seed, _ptr(out), n)
     return out
 
 
