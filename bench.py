@@ -18,6 +18,12 @@ and the CPU baseline (the single-threaded C restatement of the reference's CPU
 transformer) timed on this host on a bounded sample.
 
     python bench.py [--gpus 1] [--steps 256] [--warmup 128] [--model 7b|tiny]
+
+Two further workloads print a JSON line of the same shape (no roofline / CPU
+legs): `--model gpt2` (GPT-2 124M, every matrix Q8_0: a 32-token prompt, then
+greedy tokens up to position 32 + steps) and `--model 8b-gqa` (Llama-3-8B shape
+with grouped-query attention, every matrix Q6_K, KV caches filled with N(0,1)
+up to position 8191: `--steps` decode steps from position 8192).
 """
 from __future__ import annotations
 
@@ -131,12 +137,88 @@ def cpu_baseline(weights, prompt, n_steps):
                       f"f32 weights dequantized at load, single thread"}
 
 
+def bench_gpt2(args, W, gpu):
+    """GPT-2 124M, Q8_0: tokens per second of the greedy loop (prompt positions included:
+    the decoder takes one token per step either way)."""
+    from wgml_amd.models import GPT2_124M, Gpt2, synth_gpt2
+
+    p = GPT2_124M
+    w = synth_gpt2(p, seed=3)
+    m = Gpt2(gpu, p).load(w)
+    prompt = W.prompt_tokens(3, 32, p.n_vocab)
+    n = min(32 + args.steps, p.n_seq)
+    m.generate_greedy(prompt, min(64, n))  # records the step
+    gpu.synchronize()
+    t0 = time.perf_counter()
+    toks = m.generate_greedy(prompt, n)
+    gpu.synchronize()
+    dt = time.perf_counter() - t0
+    launches = m.launches_per_token()
+    m.set_fusion(0)  # one launch per reference op, a host read-back per token
+    gpu.synchronize()
+    t0 = time.perf_counter()
+    m.generate_greedy(prompt, n)
+    gpu.synchronize()
+    dt0 = time.perf_counter() - t0
+    log(f"gpt2-124m q8_0: {n} positions in {dt * 1e3:.1f} ms -> {n / dt:.0f} tok/s, {launches} "
+        f"launches/token; launch per reference op: {n / dt0:.0f} tok/s, "
+        f"{m.launches_per_token()} launches/token")
+    return {"metric": "decode tok/s bs1 GPT-2 124M Q8_0", "value": round(n / dt, 1), "unit": "tok/s",
+            "n_gpus": 1, "steps": n, "warmup": min(64, n), "ms_per_step": round(dt * 1e3 / n, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+            "data": "synthetic",
+            "config": {"workload": f"gpt2-124m q8_0 bs1 greedy: 32-token prompt, positions 0..{n - 1}",
+                       "launches_per_token": launches,
+                       "tok_s_one_launch_per_reference_op": round(n / dt0, 1),
+                       "last_token": int(toks[-1])},
+            "roofline": None, "cpu_baseline": None}
+
+
+def bench_8b_gqa(args, W, gpu):
+    """Llama-3-8B shape (32 q heads / 8 kv heads, hidden 14336, vocab 128256), Q6_K, with the
+    KV caches pre-filled to position 8191: decode steps at a long context."""
+    from wgml_amd.models import LLAMA3_8B, Llama2, synth_llama
+
+    cfg = LLAMA3_8B
+    t0 = time.perf_counter()
+    w = synth_llama(cfg, seed=5, scheme="q6_k")
+    log(f"weights built in {time.perf_counter() - t0:.0f}s")
+    m = Llama2(gpu, cfg).load(w)
+    n_pre, n = 8192, min(args.steps, cfg.seq_len - 8192)
+    for layer in range(cfg.n_layers):
+        for which in (0, 1):
+            kv = W.rng_normal(1000 + 2 * layer + which, n_pre * cfg.kv_dim).reshape(n_pre, cfg.kv_dim)
+            m.kv_upload(layer, which, 0, kv)
+    gpu.synchronize()
+    m.decode_greedy(7, n_pre, 4)  # records the step
+    gpu.synchronize()
+    t0 = time.perf_counter()
+    toks = m.decode_greedy(7, n_pre, n)
+    gpu.synchronize()
+    dt = time.perf_counter() - t0
+    kvb = 2 * cfg.n_layers * cfg.kv_dim * 4 * (n_pre + n // 2)
+    wb = w.weight_bytes_per_token()
+    log(f"llama3-8b-shape q6_k at position {n_pre}: {n} steps in {dt * 1e3:.1f} ms -> {n / dt:.1f} "
+        f"tok/s; {(wb + kvb) / (dt / n) / 1e12:.2f} TB/s over weights + KV")
+    return {"metric": "decode tok/s bs1 Llama-3-8B-shape Q6_K at position 8192", "value": round(n / dt, 2),
+            "unit": "tok/s", "n_gpus": 1, "steps": n, "warmup": 4, "ms_per_step": round(dt * 1e3 / n, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+            "data": "synthetic",
+            "config": {"workload": f"llama3-8b-shape q6_k bs1 greedy decode, KV caches N(0,1) up to "
+                                   f"position 8191, {n} timed steps from position 8192",
+                       "weight_bytes_per_token": wb, "kv_bytes_per_token_mid_run": kvb,
+                       "roofline_tok_s_at_8TBs": round(HBM_PEAK_GBS * 1e9 / (wb + kvb), 1),
+                       "frac_of_roofline": round((n / dt) * (wb + kvb) / (HBM_PEAK_GBS * 1e9), 4),
+                       "launches_per_token": m.launches_per_token(), "last_token": int(toks[-1])},
+            "roofline": None, "cpu_baseline": None}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=128)
-    ap.add_argument("--model", default="7b", choices=["7b", "tiny"])
+    ap.add_argument("--model", default="7b", choices=["7b", "tiny", "gpt2", "8b-gqa"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--cpu-steps", type=int, default=0, help="CPU baseline steps (0 = auto)")
@@ -157,6 +239,10 @@ def main():
     gpu = W.GpuInstance(0)
     name, n_cu = gpu.info()
     log(f"device: {name}, {n_cu} CUs")
+    if args.model in ("gpt2", "8b-gqa"):
+        line = bench_gpt2(args, W, gpu) if args.model == "gpt2" else bench_8b_gqa(args, W, gpu)
+        print(json.dumps(line), flush=True)
+        return
 
     if args.model == "7b":
         cfg, scheme, label = LLAMA2_7B, "q4_k_m", "llama2-7b-shape q4_k_m"
