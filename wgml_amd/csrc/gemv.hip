@@ -1286,13 +1286,15 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
                          "gemv_quant: %u columns need %zu bytes of LDS (limit %zu)", p.ncols, lds,
                          kMaxLds);
     // Defaults from a sweep over the Llama-2-7B shapes on MI355X: one row per
-    // wave and 16-wave workgroups (x is staged once per 16 rows in flight);
-    // Q8_0 rows span more steps, so long rows get a deeper pipeline.
+    // wave and 16-wave workgroups (x is staged once per 16 rows in flight), and
+    // no register ring: with 16 waves per CU one tile in flight per wave already
+    // exceeds what HBM needs to stay busy, and every deeper pipeline measured
+    // slower (4096x11008 Q4_K: 8.4 us at depth 1, 9.2 at 2, 9.6 at 4).
     int R = g_force_r, waves = g_force_waves, depth = g_force_depth;
     const bool q8 = F::TILE == 32;
     if (!R) R = 1;
-    if (!waves) waves = (q8 && p.ncols <= 8192) ? 8 : 16;
-    if (!depth) depth = (q8 && p.ncols > 8192) ? 4 : 2;
+    if (!waves) waves = (q8 && p.ncols <= 1024) ? 8 : 16;  // short rows: less staging per row
+    if (!depth) depth = 1;
     if (p.ln_g && (p.ncols >> 2) > 3u * (uint32_t)waves * 64u)  // XP float4 per thread
         return set_error(WGML_E_UNSUPPORTED, "gemv_quant: %u columns are too many for the folded "
                                              "LayerNorm", p.ncols);
@@ -1302,7 +1304,8 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
     }
     if (depth >= 4) return launch_rd_i8<F, 1, 4>(ctx, p, lds, waves);
     if (depth == 3) return launch_rd_i8<F, 1, 3>(ctx, p, lds, waves);
-    return launch_rd_i8<F, 1, 2>(ctx, p, lds, waves);
+    if (depth == 2) return launch_rd_i8<F, 1, 2>(ctx, p, lds, waves);
+    return launch_rd_i8<F, 1, 1>(ctx, p, lds, waves);
 }
 
 // fp32-activation path: one configuration per format
@@ -1566,7 +1569,8 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
 }
 
 int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
-    return launch_gemv_fused_variant<2, 1024, 1>(ctx, f);
+    if (g_force_depth == 2) return launch_gemv_fused_variant<2, 1024, 1>(ctx, f);
+    return launch_gemv_fused_variant<1, 1024, 1>(ctx, f);
 }
 
 }  // namespace wgml
@@ -1590,8 +1594,8 @@ WGML_API int wgml_debug_set_gemv_config(int rows_per_wave, int waves_per_wg, int
                                         int depth) {
     WGML_REQUIRE(rows_per_wave == 0 || rows_per_wave == 1 || rows_per_wave == 2,
                  "wgml_debug_set_gemv_config: rows_per_wave %d not in {0,1,2}", rows_per_wave);
-    WGML_REQUIRE(depth == 0 || (depth >= 2 && depth <= 4),
-                 "wgml_debug_set_gemv_config: depth %d not in {0,2,3,4}", depth);
+    WGML_REQUIRE(depth >= 0 && depth <= 4,
+                 "wgml_debug_set_gemv_config: depth %d not in 0..4", depth);
     g_force_depth = depth;
     WGML_REQUIRE(waves_per_wg == 0 || waves_per_wg == 4 || waves_per_wg == 8 || waves_per_wg == 16,
                  "wgml_debug_set_gemv_config: waves_per_wg %d not in {0,4,8,16}", waves_per_wg);
