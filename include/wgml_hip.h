@@ -342,6 +342,55 @@ WGML_API int wgml_bench_gemv_fused(wgml_ctx *ctx, const wgml_qmat *const *a,
                                    uint32_t nsets, wgml_view out, uint32_t stride, wgml_view v,
                                    const wgml_view *norm_w, uint32_t iters, float *total_ms);
 
+/* ---- tokenizers (host only) ------------------------------------------------ *
+ * The vocabulary is handed over as one block of UTF-8 bytes plus n + 1 offsets
+ * (token i is bytes offsets[i] .. offsets[i+1]), the way the string arrays
+ * `tokenizer.ggml.tokens` / `tokenizer.ggml.merges` lie in a GGUF file.
+ * encode/decode follow the two-call pattern: *n_out is the full length, at most
+ * `cap` elements are written (out / buf may be NULL with cap 0). */
+typedef struct wgml_tokenizer wgml_tokenizer;
+/* LlamaTokenizer::from_gguf (models/llama2/tokenizer.rs:23-51): tokens, scores
+ * (`tokenizer.ggml.scores`) and the bos / eos / unknown ids. */
+WGML_API int wgml_llama_tokenizer_create(const char *tokens, const uint64_t *offsets,
+                                         uint32_t n_tokens, const float *scores, uint32_t bos,
+                                         uint32_t eos, uint32_t unk, wgml_tokenizer **out);
+/* Gpt2Tokenizer::from_gguf (models/gpt2/tokenizer.rs:54-95): tokens and the ranked
+ * merges ("first second" per entry). */
+WGML_API int wgml_gpt2_tokenizer_create(const char *tokens, const uint64_t *token_offsets,
+                                        uint32_t n_tokens, const char *merges,
+                                        const uint64_t *merge_offsets, uint32_t n_merges,
+                                        uint32_t bos, uint32_t eos, wgml_tokenizer **out);
+WGML_API int wgml_tokenizer_destroy(wgml_tokenizer *t);
+/* eos() / bos() / unk() and bos_str() / eos_str() (llama2/tokenizer.rs:53-71,
+ * gpt2/tokenizer.rs:97-152): the ids, and the string of any id. */
+WGML_API uint32_t wgml_tokenizer_vocab_size(const wgml_tokenizer *t);
+WGML_API uint32_t wgml_tokenizer_bos(const wgml_tokenizer *t);
+WGML_API uint32_t wgml_tokenizer_eos(const wgml_tokenizer *t);
+WGML_API uint32_t wgml_tokenizer_unk(const wgml_tokenizer *t);
+WGML_API int wgml_tokenizer_token(const wgml_tokenizer *t, uint32_t id, const char **str,
+                                  uint64_t *len);
+/* LlamaTokenizer::encode(text, bos, eos) (llama2/tokenizer.rs:73-166).  Where the
+ * reference panics (nothing to merge: empty text without bos; a fallback byte id
+ * beyond the vocabulary) this returns WGML_E_INVALID. */
+WGML_API int wgml_llama_tokenizer_encode(const wgml_tokenizer *t, const char *text,
+                                         uint64_t text_len, int bos, int eos, uint32_t *out,
+                                         uint64_t cap, uint64_t *n_out);
+/* LlamaTokenizer::decode(prev_token, token) (llama2/tokenizer.rs:168-180): the text
+ * of one token given the one before it. */
+WGML_API int wgml_llama_tokenizer_decode(const wgml_tokenizer *t, uint32_t prev_token,
+                                         uint32_t token, char *buf, uint64_t cap, uint64_t *n_out);
+/* Gpt2Tokenizer::encode(text) (gpt2/tokenizer.rs:105-144).  A "<...>" string that is
+ * not in the vocabulary is WGML_E_INVALID (the reference panics). */
+WGML_API int wgml_gpt2_tokenizer_encode(const wgml_tokenizer *t, const char *text,
+                                        uint64_t text_len, uint32_t *out, uint64_t cap,
+                                        uint64_t *n_out);
+/* Gpt2Tokenizer::decode(tokens) (gpt2/tokenizer.rs:154-166).  raw_bytes 0: every
+ * decoded byte becomes the character of that value, as the reference does (text
+ * beyond ASCII comes out as Latin-1); 1: the bytes themselves (UTF-8 stays UTF-8). */
+WGML_API int wgml_gpt2_tokenizer_decode(const wgml_tokenizer *t, const uint32_t *tokens,
+                                        uint64_t n_tokens, int raw_bytes, char *buf, uint64_t cap,
+                                        uint64_t *n_out);
+
 /* ---- sampling beyond greedy: Sampler::sample (models/sampler.rs:32-130), host only ---- *
  * temperature 0: arg-max.  Otherwise the logits are divided by the temperature,
  * turned into probabilities (in place) and a token is drawn with `coin` in [0, 1):

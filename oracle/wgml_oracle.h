@@ -27,6 +27,10 @@
  *                         float64 forward agrees to 1e-4.  The reference
  *                         holds no end-to-end logits, so the greedy ids are
  *                         pinned by construction only.
+ *   tokenizers            restated in oracle/tokenizers.py (Python); pinned by merge
+ *                         sequences traced by hand on small vocabularies and by the
+ *                         library's independent scanner; ids on a real vocabulary are
+ *                         parity unpinned (no vocabulary or golden ids exist offline)
  *   parity unpinned:      the exact f32 summation order of nalgebra's gemv
  *                         (source not in the reference tree; restated from
  *                         its documented column-sweep axpy form).

@@ -11,3 +11,4 @@ from .ops import *  # noqa: F401,F403
 from .models import *  # noqa: F401,F403
 from .models import prompt_tokens  # noqa: F401
 from .gguf import Gguf, GgufTensor, llama2_config_from_gguf, llama2_weights_from_gguf  # noqa: F401
+from .tokenizer import Gpt2Tokenizer, LlamaTokenizer  # noqa: F401

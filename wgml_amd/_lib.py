@@ -162,6 +162,18 @@ PROTOTYPES = {
     "wgml_gguf_metadata": (_i, [_P, _u64, C.POINTER(GgufKv)]),
     "wgml_gguf_metadata_string": (_i, [_P, _u64, _u64, C.POINTER(C.c_char_p), C.POINTER(_u64)]),
     "wgml_gguf_tensor": (_i, [_P, _u64, C.POINTER(GgufTensorInfo)]),
+    "wgml_llama_tokenizer_create": (_i, [_P, _P, _u32, _P, _u32, _u32, _u32, _PP]),
+    "wgml_gpt2_tokenizer_create": (_i, [_P, _P, _u32, _P, _P, _u32, _u32, _u32, _PP]),
+    "wgml_tokenizer_destroy": (_i, [_P]),
+    "wgml_tokenizer_vocab_size": (_u32, [_P]),
+    "wgml_tokenizer_bos": (_u32, [_P]),
+    "wgml_tokenizer_eos": (_u32, [_P]),
+    "wgml_tokenizer_unk": (_u32, [_P]),
+    "wgml_tokenizer_token": (_i, [_P, _u32, C.POINTER(C.c_char_p), C.POINTER(_u64)]),
+    "wgml_llama_tokenizer_encode": (_i, [_P, _P, _u64, _i, _i, _P, _u64, C.POINTER(_u64)]),
+    "wgml_llama_tokenizer_decode": (_i, [_P, _u32, _u32, _P, _u64, C.POINTER(_u64)]),
+    "wgml_gpt2_tokenizer_encode": (_i, [_P, _P, _u64, _P, _u64, C.POINTER(_u64)]),
+    "wgml_gpt2_tokenizer_decode": (_i, [_P, _P, _u64, _i, _P, _u64, C.POINTER(_u64)]),
     "wgml_quantize": (_i, [_i, _P, _P, _u64, _i]),
     "wgml_dequantize_host": (_i, [_i, _P, _P, _u64, _i]),
     "wgml_rng_normal": (_i, [_u64, _P, _u64, _f, _f, _i]),
@@ -177,6 +189,8 @@ PROTOTYPES = {
 _NON_STATUS = {"wgml_last_error", "wgml_version", "wgml_buf_size", "wgml_quant_matrix_gguf_bytes",
                "wgml_quant_bytes", "wgml_quant_block_elems", "wgml_llama2_launches_per_token",
                "wgml_gpt2_launches_per_token",
+               "wgml_tokenizer_vocab_size", "wgml_tokenizer_bos", "wgml_tokenizer_eos",
+               "wgml_tokenizer_unk",
                "wgml_gguf_version", "wgml_gguf_alignment", "wgml_gguf_n_metadata",
                "wgml_gguf_n_tensors", "wgml_gguf_find_metadata", "wgml_gguf_find_tensor"}
 

@@ -893,6 +893,20 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
                         F::template accumulate<R>(w[d], xt, tile, acc);
                     }
                 }
+                // refill this register set with the triple D positions ahead; the
+                // request goes out before the reduction below, which then runs while
+                // it is in flight
+                if (it + D < n_it) {
+                    const uint32_t tile_n = ls * 64 + lane;
+                    if (tile_n < ntiles) pol.template load<WF, R>(w[d], lg, lsub, tile_n);
+                    if (++ls == nsteps) {
+                        ls = 0;
+                        if (++lsub == S) {
+                            lsub = 0;
+                            lg += GW;
+                        }
+                    }
+                }
                 if (++step == nsteps) {
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
@@ -909,18 +923,6 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
                             pol.template finish<R>(mine, nres, gseg, GW, lane, gseg == first);
                             nres = 0;
                             gseg = g;
-                        }
-                    }
-                }
-                // refill this register set with the triple D positions ahead
-                if (it + D < n_it) {
-                    const uint32_t tile_n = ls * 64 + lane;
-                    if (tile_n < ntiles) pol.template load<WF, R>(w[d], lg, lsub, tile_n);
-                    if (++ls == nsteps) {
-                        ls = 0;
-                        if (++lsub == S) {
-                            lsub = 0;
-                            lg += GW;
                         }
                     }
                 }
