@@ -132,3 +132,42 @@ def llama_to_gguf(path, weights, model_name="llama", token_embd_type=0):
     tensors.append(("output_norm.weight", 0, [weights.output_norm.size],
                     weights.output_norm.astype("<f4").tobytes()))
     return write_gguf(path, md, tensors)
+
+
+def gpt2_to_gguf(path, weights, embd_type=0):
+    """Writes Gpt2HostWeights under the tensor and key names Gpt2Weights::from_gguf and
+    Gpt2Params::from_gguf read (models/gpt2/transformer.rs:115-127,179-188;
+    models/gpt2/cpu.rs:34-47).  `embd_type`: GGUF type of token_embd / position_embd."""
+    import wgml_amd as W
+
+    p = weights.params
+    md = [("general.architecture", STRING, "gpt2"), ("general.file_type", U32, 1),
+          ("gpt2.context_length", U32, p.n_seq), ("gpt2.embedding_length", U32, p.n_embd),
+          ("gpt2.attention.head_count", U32, p.n_head), ("gpt2.block_count", U32, p.n_layer),
+          ("gpt2.feed_forward_length", U32, p.ff_len),
+          ("tokenizer.ggml.tokens", ARRAY, (STRING, [f"t{i}" for i in range(p.n_vocab)]))]
+    names = {"attn_w": "attn_qkv.weight", "attn_b": "attn_qkv.bias",
+             "attn_proj_w": "attn_output.weight", "attn_proj_b": "attn_output.bias",
+             "mlp_fc_w": "ffn_up.weight", "mlp_fc_b": "ffn_up.bias",
+             "mlp_proj_w": "ffn_down.weight", "mlp_proj_b": "ffn_down.bias",
+             "ln_1_g": "attn_norm.weight", "ln_1_b": "attn_norm.bias",
+             "ln_2_g": "ffn_norm.weight", "ln_2_b": "ffn_norm.bias"}
+    tensors = []
+    for l, layer in enumerate(weights.layers):
+        for name, v in layer.items():
+            if hasattr(v, "qtype"):
+                tensors.append((f"blk.{l}.{names[name]}", v.qtype, [v.ncols, v.nrows],
+                                np.ascontiguousarray(v.data).tobytes()))
+            else:
+                tensors.append((f"blk.{l}.{names[name]}", 0, [v.size], v.astype("<f4").tobytes()))
+
+    def embd(name, a):
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        raw = a.tobytes() if embd_type == 0 else W.quantize(embd_type, a.reshape(-1)).tobytes()
+        tensors.append((name, embd_type, [a.shape[1], a.shape[0]], raw))
+
+    embd("token_embd.weight", weights.wte)
+    embd("position_embd.weight", weights.wpe)
+    tensors.append(("output_norm.weight", 0, [p.n_embd], weights.ln_f_g.astype("<f4").tobytes()))
+    tensors.append(("output_norm.bias", 0, [p.n_embd], weights.ln_f_b.astype("<f4").tobytes()))
+    return write_gguf(path, md, tensors)

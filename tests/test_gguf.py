@@ -154,3 +154,51 @@ def test_defaults_and_tied_output(tmp_path):
     np.testing.assert_array_equal(np.asarray(w2.output.data).reshape(-1), q)
     import oracle as orc
     np.testing.assert_array_equal(w2.token_embd.reshape(-1), orc.dequantize(W.Q8_0, q, q.size // 34 * 32))
+
+
+def test_gpt2_round_trip_through_a_file(tmp_path):
+    # Gpt2Params::from_gguf / Gpt2Weights::from_gguf key and tensor names
+    from wgml_amd.models import Gpt2Params, synth_gpt2
+
+    p = Gpt2Params(n_vocab=320, n_seq=32, n_embd=64, n_head=4, n_layer=2, ff_len=256, attn_b=192)
+    w = synth_gpt2(p, seed=21)
+    rng = np.random.default_rng(1)
+    for l in w.layers:
+        l["ln_1_b"] = rng.standard_normal(p.n_embd).astype(np.float32)
+        l["ln_2_g"] = rng.standard_normal(p.n_embd).astype(np.float32)
+    w.ln_f_b = rng.standard_normal(p.n_embd).astype(np.float32)
+    path = tmp_path / "gpt2.gguf"
+    gw.gpt2_to_gguf(path, w)
+    g = W.Gguf(path)
+    p2 = W.gpt2_params_from_gguf(g)
+    assert p2 == p
+    w2 = W.gpt2_weights_from_gguf(g, p2)
+    assert len(w2.layers) == p.n_layer
+    for a, b in zip(w.layers, w2.layers):
+        assert set(a) == set(b)
+        for k in a:
+            if isinstance(a[k], HostMatrix):
+                assert (a[k].qtype, a[k].nrows, a[k].ncols) == (b[k].qtype, b[k].nrows, b[k].ncols)
+                np.testing.assert_array_equal(np.asarray(a[k].data).view(np.uint8).reshape(-1),
+                                              np.asarray(b[k].data).view(np.uint8).reshape(-1))
+            else:
+                np.testing.assert_array_equal(a[k], b[k])
+    np.testing.assert_array_equal(w.wte, w2.wte)
+    np.testing.assert_array_equal(w.wpe, w2.wpe)
+    np.testing.assert_array_equal(w.ln_f_g, w2.ln_f_g)
+    np.testing.assert_array_equal(w.ln_f_b, w2.ln_f_b)
+    # lm_head is the token_embd tensor (tied): f32 here, one row per token
+    assert (w2.lm_head.qtype, w2.lm_head.nrows, w2.lm_head.ncols) == (W.F32, p.n_vocab, p.n_embd)
+    np.testing.assert_array_equal(np.asarray(w2.lm_head.data).view(np.float32).reshape(p.n_vocab, -1),
+                                  w.wte)
+
+    # quantized embeddings are expanded for the look-ups and kept quantized for lm_head
+    path = tmp_path / "gpt2_q8.gguf"
+    gw.gpt2_to_gguf(path, w, embd_type=W.Q8_0)
+    g = W.Gguf(path)
+    w3 = W.gpt2_weights_from_gguf(g, W.gpt2_params_from_gguf(g))
+    q = W.quantize(W.Q8_0, np.ascontiguousarray(w.wte, np.float32).reshape(-1))
+    np.testing.assert_array_equal(np.asarray(w3.lm_head.data).reshape(-1), q)
+    np.testing.assert_array_equal(w3.wte.reshape(-1), W.dequantize_host(W.Q8_0, q, w.wte.size))
+    with pytest.raises(KeyError):
+        W.gpt2_params_from_gguf(W.Gguf(DUMMY))

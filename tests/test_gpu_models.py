@@ -7,7 +7,7 @@ import pytest
 
 import oracle as orc
 import wgml_amd as W
-from wgml_amd.models import (GPT2_124M, TINY_LLAMA, Gpt2, Gpt2Params, Llama2, Llama2Config,
+from wgml_amd.models import (GPT2_124M, TINY_LLAMA, Gpt2, Gpt2Params, HostMatrix, Llama2, Llama2Config,
                              LlamaModelType, synth_gpt2, synth_llama)
 
 pytestmark = pytest.mark.gpu
@@ -192,6 +192,25 @@ def test_gpt2_micro_logits(gpu, fusion):
         m.forward(t, pos)
         ok, e = logits_close(m.logits(), want)
         assert ok, (pos, e)
+
+
+def test_gpt2_from_gguf_file(gpu, tmp_path):
+    # weights written under the reference's GPT-2 tensor / key names and loaded back through
+    # the GGUF reader: same greedy tokens as the oracle on the original weights (lm_head is the
+    # f32 token_embd tensor here, as in the reference)
+    import gguf_writer as gw
+
+    p = Gpt2Params(n_vocab=320, n_seq=32, n_embd=64, n_head=4, n_layer=2, ff_len=256, attn_b=192)
+    w = synth_gpt2(p, seed=9)
+    w.lm_head = HostMatrix(W.F32, p.n_vocab, p.n_embd,
+                           np.ascontiguousarray(w.wte, np.float32).view(np.uint8).reshape(-1))
+    path = tmp_path / "gpt2.gguf"
+    gw.gpt2_to_gguf(path, w)
+    prompt = W.prompt_tokens(9, 4, p.n_vocab)
+    want, _ = orc.Gpt2(w).generate_greedy(prompt, 20)
+    m = Gpt2.from_gguf(gpu, W.Gguf(path))
+    assert m.params == p
+    assert np.array_equal(m.generate_greedy(prompt, 20), want)
 
 
 def test_gpt2_124m_greedy_prefix(gpu):

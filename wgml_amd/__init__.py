@@ -10,5 +10,6 @@ from ._lib import (F16, F32, Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0, Q8_
 from .ops import *  # noqa: F401,F403
 from .models import *  # noqa: F401,F403
 from .models import prompt_tokens  # noqa: F401
-from .gguf import Gguf, GgufTensor, llama2_config_from_gguf, llama2_weights_from_gguf  # noqa: F401
+from .gguf import (Gguf, GgufTensor, gpt2_params_from_gguf, gpt2_weights_from_gguf,  # noqa: F401
+                   llama2_config_from_gguf, llama2_weights_from_gguf)
 from .tokenizer import Gpt2Tokenizer, LlamaTokenizer  # noqa: F401

@@ -151,3 +151,74 @@ def llama2_weights_from_gguf(gguf: Gguf, config):
     w.output = HostMatrix(out.qtype, c.vocab_size, c.dim, out.data)
     w.output_norm = gguf.tensors["output_norm.weight"].as_f32().copy()
     return w
+
+
+# reference tensor name -> host weight name (models/gpt2/transformer.rs:115-127)
+_GPT2_MATS = {"attn_qkv": "attn_w", "attn_output": "attn_proj_w", "ffn_up": "mlp_fc_w",
+              "ffn_down": "mlp_proj_w"}
+_GPT2_BIAS = {"attn_qkv": "attn_b", "attn_output": "attn_proj_b", "ffn_up": "mlp_fc_b",
+              "ffn_down": "mlp_proj_b"}
+_GPT2_NORMS = {"attn_norm": "ln_1", "ffn_norm": "ln_2"}
+
+
+def gpt2_params_from_gguf(gguf: Gguf):
+    """Gpt2Params::from_gguf (models/gpt2/cpu.rs:34-47)."""
+    from .models import Gpt2Params
+
+    md = gguf.metadata
+    return Gpt2Params(n_vocab=len(md["tokenizer.ggml.tokens"]),
+                      n_seq=int(md["gpt2.context_length"]),
+                      n_embd=int(md["gpt2.embedding_length"]),
+                      n_head=int(md["gpt2.attention.head_count"]),
+                      n_layer=int(md["gpt2.block_count"]),
+                      ff_len=int(md["gpt2.feed_forward_length"]),
+                      attn_b=int(gguf.tensors["blk.0.attn_qkv.bias"].dimensions[0]))
+
+
+def gpt2_weights_from_gguf(gguf: Gguf, params):
+    """Gpt2Weights::from_gguf (models/gpt2/transformer.rs:108-205) as host weights.  The
+    reference expands every matrix to f32; here a matrix keeps its GGUF quantization where the
+    GEMV reads it directly, the values are the same.  wte and wpe are expanded to f32 (they
+    are looked up, not multiplied); lm_head is the token_embd tensor itself (GPT-2 ties them)."""
+    from . import ops
+    from .models import Gpt2HostWeights, HostMatrix
+
+    p = params
+
+    def matrix(tname: str, nrows: int, ncols: int) -> HostMatrix:
+        t = gguf.tensors[tname]
+        if t.dimensions[0] != ncols or t.dimensions[1] != nrows:
+            raise ValueError(f"tensor '{tname}' is {t.dimensions[1]}x{t.dimensions[0]}, "
+                             f"expected {nrows}x{ncols}")
+        return HostMatrix(t.qtype, nrows, ncols, t.data)
+
+    def f32(tname: str, n: int) -> np.ndarray:
+        a = gguf.tensors[tname].as_f32()
+        if a.size != n:
+            raise ValueError(f"tensor '{tname}' has {a.size} elements, expected {n}")
+        return a.copy()
+
+    def expanded(tname: str, nrows: int, ncols: int) -> np.ndarray:
+        m = matrix(tname, nrows, ncols)
+        if m.qtype == _lib.F32:
+            return np.asarray(m.data).view(np.float32).reshape(nrows, ncols).copy()
+        return ops.dequantize_host(m.qtype, m.data, nrows * ncols).reshape(nrows, ncols)
+
+    shapes = {"attn_qkv": (p.attn_b, p.n_embd), "attn_output": (p.n_embd, p.n_embd),
+              "ffn_up": (p.ff_len, p.n_embd), "ffn_down": (p.n_embd, p.ff_len)}
+    w = Gpt2HostWeights(params=p)
+    for l in range(p.n_layer):
+        layer: Dict[str, object] = {}
+        for tname, (nr, nc) in shapes.items():
+            layer[_GPT2_MATS[tname]] = matrix(f"blk.{l}.{tname}.weight", nr, nc)
+            layer[_GPT2_BIAS[tname]] = f32(f"blk.{l}.{tname}.bias", nr)
+        for tname, name in _GPT2_NORMS.items():
+            layer[name + "_g"] = f32(f"blk.{l}.{tname}.weight", p.n_embd)
+            layer[name + "_b"] = f32(f"blk.{l}.{tname}.bias", p.n_embd)
+        w.layers.append(layer)
+    w.ln_f_g = f32("output_norm.weight", p.n_embd)
+    w.ln_f_b = f32("output_norm.bias", p.n_embd)
+    w.wte = expanded("token_embd.weight", p.n_vocab, p.n_embd)
+    w.wpe = expanded("position_embd.weight", p.n_seq, p.n_embd)
+    w.lm_head = matrix("token_embd.weight", p.n_vocab, p.n_embd)
+    return w

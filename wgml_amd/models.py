@@ -280,6 +280,15 @@ class Gpt2:
         call("wgml_gpt2_set_embeddings", self._h, _ptr(wte), _ptr(wpe))
         return self
 
+    @classmethod
+    def from_gguf(cls, gpu: GpuInstance, gguf) -> "Gpt2":
+        """Gpt2Params::from_gguf + Gpt2Weights::from_gguf (models/gpt2/cpu.rs:34-47,
+        models/gpt2/transformer.rs:108-205) from a `wgml_amd.Gguf`."""
+        from .gguf import gpt2_params_from_gguf, gpt2_weights_from_gguf
+
+        params = gpt2_params_from_gguf(gguf)
+        return cls(gpu, params).load(gpt2_weights_from_gguf(gguf, params))
+
     def set_fusion(self, level: int) -> None:
         call("wgml_gpt2_set_fusion", self._h, level)
 
