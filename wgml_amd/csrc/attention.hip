@@ -237,6 +237,44 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnArgs a, uint3
     }
 }
 
+// Merge of the fast kernel's partials: every workgroup of the grid has written one
+// (a neutral one if it had no position), so nothing depends on the current position
+// and all loads go out at once: lane y of every wave fetches (max, sum) of partial y,
+// thread d the d-th value of every partial; the weights are formed in registers.
+__global__ __launch_bounds__(256) void attn_merge_fast_kernel(const AttnArgs a, uint32_t hsp) {
+    const uint32_t h = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const uint32_t stride = 2 + hsp, ny = a.n_wg_y;  // ny <= MERGE_MAX_Y = 64
+    const float *base = a.ws + (size_t)h * ny * stride;
+    const float my = lane < ny ? base[(size_t)lane * stride] : -INFINITY;
+    const float ly = lane < ny ? base[(size_t)lane * stride + 1] : 0.f;
+    constexpr int B = 16;
+    float v[B];
+    const bool has_d = tid < a.head_size;  // head sizes up to 256: one dimension per thread
+#pragma unroll
+    for (int k = 0; k < B; ++k)
+        v[k] = (has_d && (uint32_t)k < ny) ? base[(size_t)k * stride + 2 + tid] : 0.f;
+    const float M = wave_max(my);
+    const float wgt = my == -INFINITY ? 0.f : __expf(my - M);
+    const float L = wave_sum(ly * wgt);
+    float o = 0.f;
+#pragma unroll
+    for (int k = 0; k < B; ++k) {
+        const float wk = readlane_f32(wgt, k);
+        o = fmaf(wk > 0.f ? v[k] : 0.f, wk, o);  // values of neutral partials were never written
+    }
+    for (uint32_t y0 = B; y0 < ny; y0 += B) {
+#pragma unroll
+        for (int k = 0; k < B; ++k)
+            v[k] = (has_d && y0 + k < ny) ? base[(size_t)(y0 + k) * stride + 2 + tid] : 0.f;
+#pragma unroll
+        for (int k = 0; k < B; ++k) {
+            const float wk = __shfl(wgt, (int)(y0 + k), 64);
+            o = fmaf(wk > 0.f ? v[k] : 0.f, wk, o);
+        }
+    }
+    if (has_d) a.xb[(size_t)h * a.head_size + tid] = o / L;
+}
+
 // ---------------------------------------------------------------- fast kernel
 __device__ __forceinline__ float dot4(const float4 a, const float4 b, float acc) {
     acc = fmaf(a.x, b.x, acc);
@@ -317,7 +355,16 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
 
     const uint32_t pos = dyn_pos(a.pos);
     const uint32_t n_used = fast_n_used(pos, a.n_wg_y, NW);  // workgroups with work
-    if (blockIdx.y >= n_used) return;
+    if (blockIdx.y >= n_used) {
+        // no position for this workgroup: a neutral partial (max -inf, sum 0), so that the
+        // merge need not know the position to tell which partials count
+        if (threadIdx.x < KM) {
+            float *p = a.ws + ((size_t)(h0 + threadIdx.x) * a.n_wg_y + blockIdx.y) * (2 + HSP);
+            p[0] = -INFINITY;
+            p[1] = 0.f;
+        }
+        return;
+    }
     const uint32_t nq = pos / 4 + 1;
     // online-softmax update with the two quads of a set
     auto consume = [&](const float4(&kk)[2][NV4], const float4(&vv)[2][NV4], uint32_t i0) {
@@ -589,7 +636,7 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
         WGML_TRY(ensure_ws(ctx, (size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4));
         a.ws = ctx->attn_ws;
         WGML_TRY(launch_fast<WAVES>(ctx, a, pl.nv, pl.km, grid));
-        attn_merge_kernel<<<dim3(p.n_heads), dim3(256), 0, ctx->stream>>>(a, pl.hsp);
+        attn_merge_fast_kernel<<<dim3(p.n_heads), dim3(256), 0, ctx->stream>>>(a, pl.hsp);
         WGML_CHECK_LAUNCH();
         ctx->launches++;
         return WGML_OK;
