@@ -634,9 +634,12 @@ struct IFmtQ8_0 {
 struct PlainPolicy {
     static constexpr int S = 1;  // passes per group
     const GemvParams &p;
+    // `ok` false: the load still happens, from row-group 0 (a wave's loads are never
+    // skipped, see gemv_i8_body)
     template <class WF, int R>
-    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t, uint32_t tile) const {
-        load_group<WF, R>(w, p, g, tile);
+    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t, uint32_t tile,
+                         bool ok) const {
+        load_group<WF, R>(w, p, ok ? g : 0u, tile);
     }
     // Lane n holds finished result n of the segment that starts at group g0:
     // result n belongs to row (g0 + (n / R) * GW) * R + n % R.  The operands the
@@ -710,6 +713,9 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
     const float4 *nw4 = reinterpret_cast<const float4 *>(p.norm_w);
     const uint32_t n4 = p.ncols >> 2;
+    // (The x loads stay under their conditions: clamping the out-of-range ones to a
+    // valid address instead makes every idle thread of the machine hit the same
+    // cache line, which cost 1 us on a 4096x4096 launch.)
     float4 xv[XP], nv[XP];
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
@@ -722,19 +728,24 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
         }
     }
 
+    // The weight loads below and in the main loop are issued unconditionally (a lane
+    // without a tile re-reads tile 0, a wave without work row-group 0).  Only then
+    // can the compiler count the loads in flight and wait for exactly the one it
+    // needs: with a load under a condition it falls back to waiting for all of
+    // them, and the staging of x, a cache hit, would wait for the first weight
+    // tile to arrive from HBM.
     typename WF::Row w[D][R];
     uint32_t lg = first, lsub = 0, ls = 0;  // (group, pass, step) of the next load
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-        if ((uint32_t)d < n_it) {
-            const uint32_t tile = ls * 64 + lane;
-            if (tile < ntiles) pol.template load<WF, R>(w[d], lg, lsub, tile);
-            if (++ls == nsteps) {
-                ls = 0;
-                if (++lsub == S) {
-                    lsub = 0;
-                    lg += GW;
-                }
+        const uint32_t tile = ls * 64 + lane;
+        const bool ok = (uint32_t)d < n_it;
+        pol.template load<WF, R>(w[d], lg, lsub, ok && tile < ntiles ? tile : 0u, ok);
+        if (++ls == nsteps) {
+            ls = 0;
+            if (++lsub == S) {
+                lsub = 0;
+                lg += GW;
             }
         }
     }
@@ -865,71 +876,90 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     }
     if (n_it == 0) return;
 
-    // Finished row sums are parked one per lane (result n in lane n) and handed
-    // to the policy 64 at a time: the epilogue's loads and stores (bias, RoPE table,
-    // accumulate) would otherwise sit between the weight loads in flight, and a
-    // wave waits for its memory operations in order.
     typename F::X xr;
     if (XREG && lane < ntiles) F::load_x(xr, xq + lane, meta + (size_t)lane * MF);
     uint32_t g = first, sub = 0, step = 0;  // (group, pass, step) being computed
-    uint32_t nres = 0, gseg = first;
-    float mine = 0.f;
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
-    for (uint32_t base = 0; base < n_it; base += D) {
-#pragma unroll
-        for (int d = 0; d < D; ++d) {
-            const uint32_t it = base + d;
-            if (it < n_it) {
-                const uint32_t tile = step * 64 + lane;
-                if (tile < ntiles) {
-                    if (XREG) {
-                        F::template accumulate<R>(w[d], xr, tile, acc);
-                    } else {
-                        typename F::X xt;
-                        F::load_x(xt, xq + (size_t)step * 2 * PCH * 64 + lane,
-                                  meta + (size_t)tile * MF);
-                        F::template accumulate<R>(w[d], xt, tile, acc);
-                    }
-                }
-                // refill this register set with the triple D positions ahead; the
-                // request goes out before the reduction below, which then runs while
-                // it is in flight
-                if (it + D < n_it) {
-                    const uint32_t tile_n = ls * 64 + lane;
-                    if (tile_n < ntiles) pol.template load<WF, R>(w[d], lg, lsub, tile_n);
-                    if (++ls == nsteps) {
-                        ls = 0;
-                        if (++lsub == S) {
-                            lsub = 0;
-                            lg += GW;
-                        }
-                    }
-                }
-                if (++step == nsteps) {
-#pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        const float t = wave_sum(acc[r]) * out_scale;
-                        mine = lane == nres ? t : mine;
-                        ++nres;
-                        acc[r] = 0.f;
-                    }
-                    step = 0;
-                    if (++sub == S) {
-                        sub = 0;
-                        g += GW;
-                        if (nres + S * R > 64) {
-                            pol.template finish<R>(mine, nres, gseg, GW, lane, gseg == first);
-                            nres = 0;
-                            gseg = g;
-                        }
-                    }
-                }
+    // The iterations are cut into segments of whole groups, a multiple of D long (so
+    // that register set d always holds iteration d mod D) and with at most 64
+    // results; the policy's epilogue runs between segments, never inside the loop.
+    const uint32_t per_group = S * nsteps;
+    uint32_t unit = per_group;
+    while (unit % D) unit += per_group;
+    const uint32_t unit_groups = unit / per_group;
+    const uint32_t seg_len = ((64u / (S * R)) / unit_groups) * unit;
+    uint32_t nres = 0;
+    float mine = 0.f;
+    // one iteration on a register set: the dot products of a tile, and the row
+    // reduction when the row is complete (no memory operation, LDS aside)
+    auto compute = [&](typename WF::Row(&wd)[R]) {
+        const uint32_t tile = step * 64 + lane;
+        if (tile < ntiles) {
+            if (XREG) {
+                F::template accumulate<R>(wd, xr, tile, acc);
+            } else {
+                typename F::X xt;
+                F::load_x(xt, xq + (size_t)step * 2 * PCH * 64 + lane, meta + (size_t)tile * MF);
+                F::template accumulate<R>(wd, xt, tile, acc);
             }
         }
+        if (++step == nsteps) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float t = wave_sum(acc[r]) * out_scale;
+                mine = lane == nres ? t : mine;
+                ++nres;
+                acc[r] = 0.f;
+            }
+            step = 0;
+            if (++sub == S) {
+                sub = 0;
+                g += GW;
+            }
+        }
+    };
+    // refills a register set with the next triple of the load cursor
+    auto refill = [&](typename WF::Row(&wd)[R]) {
+        const uint32_t tile_n = ls * 64 + lane;
+        pol.template load<WF, R>(wd, lg, lsub, tile_n < ntiles ? tile_n : 0u, true);
+        if (++ls == nsteps) {
+            ls = 0;
+            if (++lsub == S) {
+                lsub = 0;
+                lg += GW;
+            }
+        }
+    };
+    for (uint32_t it0 = 0; it0 < n_it; it0 += seg_len) {
+        const uint32_t seg_end = min(n_it, it0 + seg_len);
+        const uint32_t gseg = g;
+        nres = 0;
+        uint32_t base = it0;
+        // rounds of D iterations whose refills all exist: straight-line loads
+        for (; base < seg_end && base + 2 * D <= n_it; base += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                compute(w[d]);
+                refill(w[d]);
+            }
+        }
+        // the last rounds of the launch: refills only while iterations remain (a
+        // wave cannot end before a load it issued has returned)
+        for (; base < seg_end; base += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                const uint32_t it = base + d;
+                if (it < seg_end) compute(w[d]);
+                if (it + D < n_it) refill(w[d]);
+            }
+        }
+        // Finished row sums are parked one per lane (result n in lane n) and handed
+        // to the policy here: its loads and stores (bias, RoPE table, accumulate)
+        // stay out of the weight stream.
+        pol.template finish<R>(mine, nres, gseg, GW, lane, it0 == 0);
     }
-    if (nres) pol.template finish<R>(mine, nres, gseg, GW, lane, gseg == first);
 }
 
 template <class F, int R, int D, int MAXT>
@@ -994,8 +1024,10 @@ struct JobPolicy {
     float rope_base;
     const float2 *rope_cs;
     template <class WF, int R>
-    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t sub, uint32_t tile) const {
+    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t sub, uint32_t tile,
+                         bool ok) const {
         static_assert(R == 1, "fused launches make single-row passes");
+        if (!ok) g = 0;
         // plane pointers are picked one by one (wave-uniform selects): choosing between
         // the two parameter blocks by reference would force them into memory
         const bool second = j.mode == JOB_SILU && sub;
@@ -1291,7 +1323,7 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
     // wave and 16-wave workgroups (x is staged once per 16 rows in flight), and
     // no register ring: with 16 waves per CU one tile in flight per wave already
     // exceeds what HBM needs to stay busy, and every deeper pipeline measured
-    // slower (4096x11008 Q4_K: 8.4 us at depth 1, 9.2 at 2, 9.6 at 4).
+    // slower, also with exact waits (11008x4096 Q4_K: 8.4 us at depth 1, 9.4 at 2).
     int R = g_force_r, waves = g_force_waves, depth = g_force_depth;
     const bool q8 = F::TILE == 32;
     if (!R) R = 1;
