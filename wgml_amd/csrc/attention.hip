@@ -304,9 +304,16 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
     const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
     const float *kb = a.kc + (size_t)kvh * hs;
     const float *vb = a.vc + (size_t)kvh * hs;
-    bool dv[NV4];  // this lane's float4 number v lies inside the head
+    // this lane's float4 number v lies inside the head; if not, it re-reads the head's
+    // last float4 (loads stay unconditional 16-byte loads) and q is zero there, so
+    // that it adds nothing to a score; its slots of the output are never stored
+    bool dv[NV4];
+    uint32_t cv[NV4];
 #pragma unroll
-    for (int v = 0; v < NV4; ++v) dv[v] = (sub + 16 * v) * 4 < hs;
+    for (int v = 0; v < NV4; ++v) {
+        dv[v] = (sub + 16 * v) * 4 < hs;
+        cv[v] = min(sub + 16 * v, hs / 4 - 1);
+    }
 
     // This wave's quads are gid, gid + total, ...  Two register sets of two quads
     // each take turns: while one is consumed the other's loads are in flight.  The
@@ -330,9 +337,9 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
                 const float4 *kp = reinterpret_cast<const float4 *>(kb + (size_t)tt * a.kv_dim);
                 const float4 *vp = reinterpret_cast<const float4 *>(vb + (size_t)tt * a.kv_dim);
 #pragma unroll
-                for (int v = 0; v < NV4; ++v) kk[u][v] = dv[v] ? kp[sub + 16 * v] : zero4;
+                for (int v = 0; v < NV4; ++v) kk[u][v] = kp[cv[v]];
 #pragma unroll
-                for (int v = 0; v < NV4; ++v) vv[u][v] = dv[v] ? vp[sub + 16 * v] : zero4;
+                for (int v = 0; v < NV4; ++v) vv[u][v] = vp[cv[v]];
             }
         }
     };
@@ -347,8 +354,9 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
         l[m] = 0.f;
 #pragma unroll
         for (int v = 0; v < NV4; ++v) {
-            q[m][v] = dv[v] ? reinterpret_cast<const float4 *>(a.q + (size_t)(h0 + m) * hs)[sub + 16 * v]
-                            : zero4;
+            const float4 qv = reinterpret_cast<const float4 *>(a.q + (size_t)(h0 + m) * hs)[cv[v]];
+            q[m][v] = make_float4(dv[v] ? qv.x : 0.f, dv[v] ? qv.y : 0.f, dv[v] ? qv.z : 0.f,
+                                  dv[v] ? qv.w : 0.f);
             acc[m][v] = zero4;
         }
     }
