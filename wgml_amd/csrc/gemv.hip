@@ -716,15 +716,22 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     // (The x loads stay under their conditions: clamping the out-of-range ones to a
     // valid address instead makes every idle thread of the machine hit the same
     // cache line, which cost 1 us on a 4096x4096 launch.)
-    float4 xv[XP], nv[XP];
+    // nv: the RMSNorm weights, or gamma of a folded LayerNorm; bv: its beta.  They are
+    // requested here, ahead of the weights, so that waiting for them later does not
+    // mean waiting for a weight tile.
+    float4 xv[XP], nv[XP], bv[XP];
+    const float4 *gsrc = p.ln_g ? reinterpret_cast<const float4 *>(p.ln_g) : nw4;
+    const float4 *bsrc = reinterpret_cast<const float4 *>(p.ln_b);
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
         const uint32_t g4 = tid + i * blockDim.x;
         xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         nv[i] = make_float4(1.f, 1.f, 1.f, 1.f);
+        bv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (g4 < n4) {
             xv[i] = x4[g4];
-            if (p.norm_w) nv[i] = nw4[g4];
+            if (gsrc) nv[i] = gsrc[g4];
+            if (p.ln_g && bsrc) bv[i] = bsrc[g4];
         }
     }
 
@@ -792,14 +799,11 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
                 }
             }
             const float rstd = 1.0f / sqrtf(block_total(s2, red_b) / (float)p.ncols + 1.0e-5f);
-            const float4 *g4p = reinterpret_cast<const float4 *>(p.ln_g);
-            const float4 *b4p = reinterpret_cast<const float4 *>(p.ln_b);
 #pragma unroll
             for (int i = 0; i < XP; ++i) {
                 const uint32_t g4 = tid + i * blockDim.x;
                 if (g4 < n4) {
-                    const float4 ga = g4p[g4];
-                    const float4 be = p.ln_b ? b4p[g4] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    const float4 ga = nv[i], be = bv[i];
                     xv[i].x = (xv[i].x * rstd) * ga.x + be.x;
                     xv[i].y = (xv[i].y * rstd) * ga.y + be.y;
                     xv[i].z = (xv[i].z * rstd) * ga.z + be.z;
