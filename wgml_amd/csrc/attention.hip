@@ -294,7 +294,9 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
     __shared__ float sm_m[NW][KM], sm_l[NW][KM];
     __shared__ float sm_acc[NW][KM][HSP];
 
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63;
+    // readfirstlane: tells the compiler that the wave index is uniform (scalar loop control)
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint32_t sub = lane & 15, quarter = lane >> 4;
     const uint32_t hs = a.head_size;
     const uint32_t h0 = blockIdx.x * KM;

@@ -693,7 +693,11 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     constexpr int LPB = F::XB / 4;            // lanes (float4) per activation block
     extern __shared__ float4 smem4[];
     uint4 *xq = reinterpret_cast<uint4 *>(smem4);
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // the wave index is read through readfirstlane: the compiler then knows that it,
+    // and the loop control derived from it, are the same in every lane (scalar registers
+    // and branches instead of vector compares and masks)
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t nwaves = blockDim.x >> 6;
     const uint32_t ntiles = p.ncols / F::TILE;
     const uint32_t nsteps = (ntiles + 63) >> 6;
