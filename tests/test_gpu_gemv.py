@@ -183,3 +183,43 @@ def test_gemv_dimension_mismatch(gpu):
         op.dispatch(W.GpuVector.uninit(gpu, 8), m, W.GpuVector.uninit(gpu, 32))
     with pytest.raises(W.WgmlError, match="dimension mismatch"):
         op.dispatch(W.GpuVector.uninit(gpu, 4), m, W.GpuVector.uninit(gpu, 64))
+
+
+@pytest.mark.parametrize("qtype,nrows,ncols", [(W.Q8_0, 300000, 64), (W.Q4_K, 270000, 256),
+                                               (W.Q6_K, 135001, 256)])
+def test_gemv_more_than_64_rows_per_wave(gpu, qtype, nrows, ncols):
+    # tall matrices: a wave owns more rows than it has lanes to park results in, so its rows
+    # are handled in several segments with the epilogue in between
+    raw = weights(qtype, nrows, ncols, 77)
+    x = W.rng_normal(78, ncols)
+    _, ref = orc.gemv_quant(qtype, raw, nrows, ncols, x)
+    ok, e = close(gemv(gpu, qtype, raw, nrows, ncols, x), ref)
+    assert ok, e
+
+
+@pytest.mark.parametrize("nrows,ncols", [(140000, 256), (1001, 512), (11008, 4096)])
+def test_fused_gate_up_silu_launch(gpu, nrows, ncols):
+    # the decoder's fused gate/up launch on its own (through the benchmark entry point, one
+    # launch): out = up * silu(gate) with the RMSNorm of x folded in.  140000 rows make a wave
+    # own more than 32 (gate, up) pairs, i.e. several segments.
+    import ctypes as C
+
+    from wgml_amd._lib import call
+
+    gate_raw, up_raw = weights(W.Q4_K, nrows, ncols, 5), weights(W.Q4_K, nrows, ncols, 6)
+    x = W.rng_normal(7, ncols)
+    nw = (1.0 + 0.1 * W.rng_normal(8, ncols)).astype(np.float32)
+    gate = W.GpuQuantMatrix(gpu, W.Q4_K, nrows, ncols, gate_raw)
+    up = W.GpuQuantMatrix(gpu, W.Q4_K, nrows, ncols, up_raw)
+    out = W.GpuVector.init(gpu, np.full(nrows, np.nan, dtype=np.float32))
+    xv, nwv = W.GpuVector.init(gpu, x), W.GpuVector.init(gpu, nw)
+    a, b = (C.c_void_p * 1)(gate.handle), (C.c_void_p * 1)(up.handle)
+    modes, ms, nview = (C.c_int * 1)(2), C.c_float(), nwv.view()
+    call("wgml_bench_gemv_fused", gpu.handle, a, b, modes, 1, 1, out.view(), nrows, xv.view(),
+         C.byref(nview), 1, C.byref(ms))
+    xn = orc.rms_norm(x, nw, 1e-5)
+    _, g = orc.gemv_quant(W.Q4_K, gate_raw, nrows, ncols, xn)
+    _, u = orc.gemv_quant(W.Q4_K, up_raw, nrows, ncols, xn)
+    ref = u * (g / (1.0 + np.exp(-g)))
+    ok, e = close(out.read(), ref)
+    assert ok, e
