@@ -202,3 +202,37 @@ def test_gpt2_round_trip_through_a_file(tmp_path):
     np.testing.assert_array_equal(w3.wte.reshape(-1), W.dequantize_host(W.Q8_0, q, w.wte.size))
     with pytest.raises(KeyError):
         W.gpt2_params_from_gguf(W.Gguf(DUMMY))
+
+
+def test_mutated_files_never_crash_the_reader():
+    # seeded byte flips, length-field overwrites and truncations of the fixture: the reader
+    # either parses the result or reports an error (the reference panics on several of these,
+    # gguf.rs:248-294); it must not read outside the buffer
+    raw = open(DUMMY, "rb").read()
+    rng = np.random.default_rng(1234)
+    header_len = 1216  # metadata + tensor infos of the fixture end here
+    parsed = refused = 0
+    for case in range(600):
+        b = bytearray(raw)
+        kind = case % 3
+        if kind == 0:  # flip a few bytes in the header region
+            for _ in range(int(rng.integers(1, 4))):
+                b[int(rng.integers(0, header_len))] = int(rng.integers(0, 256))
+        elif kind == 1:  # overwrite an aligned 8-byte field with a huge or odd value
+            off = int(rng.integers(1, header_len // 8)) * 8
+            vals = [0, 1, 7, 1 << 31, (1 << 63) - 1, (1 << 64) - 1]
+            struct.pack_into("<Q", b, off, vals[int(rng.integers(0, len(vals)))])
+        else:  # truncate
+            b = b[:int(rng.integers(0, len(raw)))]
+        try:
+            g = W.Gguf(bytes(b))
+            for t in g.tensors.values():  # every view must be readable
+                if t.data.size:
+                    int(t.data[0]) + int(t.data[-1])
+            for v in g.metadata.values():
+                repr(v)[:10]
+            g.close()
+            parsed += 1
+        except W.WgmlError:
+            refused += 1
+    assert parsed + refused == 600 and refused > 100

@@ -226,3 +226,23 @@ def test_tokenizers_from_gguf(tmp_path, llama, gpt2):
     tok2 = W.Gpt2Tokenizer.from_gguf(g2)
     assert tok2.encode("hello world") == gpt2[0].encode("hello world")
     assert np.array_equal(tok2.encode("I'm 12"), gpt2[0].encode("I'm 12"))
+
+
+def test_invalid_utf8_does_not_crash(llama, gpt2):
+    # raw bytes through the C entry points (the Python classes only ever pass valid UTF-8):
+    # malformed sequences are taken byte by byte as U+FFFD, nothing is read past the end
+    rng = random.Random(3)
+    ltok, gtok = llama[0], gpt2[0]
+    for case in range(300):
+        raw = bytes(rng.randrange(256) for _ in range(rng.randint(1, 24)))
+        ids = ltok._ids("wgml_llama_tokenizer_encode", ltok._h, raw, len(raw), 1, 0)
+        assert ids[0] == 1 and all(0 <= t < len(ltok) for t in ids)
+        try:
+            ids = gtok._ids("wgml_gpt2_tokenizer_encode", gtok._h, raw, len(raw))
+            assert all(0 <= t < len(gtok) for t in ids)
+        except WgmlError:
+            pass  # a "<...>" run that is no token
+    for bad in (b"\xe2\x96", b"\xf0\x9f\x98", b"\xc3", b"\xed\xa0\x80", b"\xf4\x90\x80\x80"):
+        ids = ltok._ids("wgml_llama_tokenizer_encode", ltok._h, bad, len(bad), 0, 0)
+        assert ids  # U+FFFD is no token of the vocabulary: its bytes EF BF BD + 3, per malformed byte
+        assert all(t in (0xEF + 3, 0xBF + 3, 0xBD + 3) for t in ids)
