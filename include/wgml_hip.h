@@ -127,6 +127,17 @@ WGML_API uint32_t wgml_quant_block_elems(int type); /* QuantizedValue::DEQUANTIZ
  * out.len == nrows, v.len == ncols. */
 WGML_API int wgml_gemv_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, wgml_view v);
 
+/* The same product for n_tokens <= 128 vectors at once, on the matrix cores:
+ * out[t] = m * x[t], with x n_tokens x ncols and out n_tokens x nrows, both row-major.
+ * No counterpart in the reference, which multiplies one vector at a time
+ * (GemvQuant::dispatch above); it is the building block of wgml_llama2_prefill.
+ * The weights are expanded with the reference's dequantization arithmetic and
+ * rounded to f16, the vectors are rounded to f16, sums are fp32: results agree
+ * with n_tokens calls of wgml_gemv_quant to about 1e-3 of a row's magnitude, not
+ * to the last bits.  m must be WGML_Q8_0, WGML_Q4_K or WGML_Q6_K. */
+WGML_API int wgml_gemm_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, wgml_view x,
+                             uint32_t n_tokens);
+
 /* Quantization shader `dequantize_*` (ops/quantization.wgsl, exercised by
  * ops/quantization.rs:37-408) == Block*::dequantize (quantization.rs): writes
  * the nrows*ncols f32 values, row-major, bit-exact with the CPU twin. */

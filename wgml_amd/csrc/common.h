@@ -55,6 +55,11 @@ struct wgml_ctx {
     float *attn_ws = nullptr;
     size_t attn_ws_bytes = 0;
     std::vector<void *> retired;  // outgrown workspaces, freed with the context
+    // f16 copy of the activations of a batched matrix product (+ one scale per token),
+    // grown on demand
+    void *prefill_xh = nullptr;
+    size_t prefill_xh_bytes = 0;
+    float *prefill_xscale = nullptr;
     uint64_t launches = 0;  // kernels enqueued so far (diagnostics)
     // Buffers, matrices and models keep their context alive: the device objects
     // are torn down when the last reference goes, whatever order handles are
@@ -191,5 +196,25 @@ int launch_embed(wgml_ctx *ctx, float *x, const float *table, uint32_t dim, DynP
 int launch_argmax_next(wgml_ctx *ctx, const float *v, uint32_t n, DynState *dyn,
                        const uint32_t *prompt, uint32_t *tokens_out);
 int launch_dequantize(wgml_ctx *ctx, float *out, const wgml_qmat *m);
+
+// ---- batched products for prompt processing (prefill.hip) ---------------------
+constexpr uint32_t kPrefillMaxTokens = 128;
+uint32_t prefill_tpad(uint32_t T);  // tokens rounded up to 16, 32, 64 or 128
+uint32_t prefill_kpad(uint32_t K);  // columns rounded up to a multiple of 64
+int ensure_prefill_scratch(wgml_ctx *ctx, size_t xh_bytes);
+// xh[tpad][kpad] (f16) <- x[T][K] (f32, rows x_stride apart), RMS-normalised with
+// norm_w first when that is non-null; xscale[tpad] receives what a token's
+// products must be multiplied with.
+int launch_prefill_prep(wgml_ctx *ctx, const float *x, uint32_t x_stride, const float *norm_w,
+                        float eps, void *xh, float *xscale, uint32_t K, uint32_t T);
+// out[t][r] (rows out_stride apart) = (or +=) sum_k M[r][k] x[t][k] + bias[r]
+int launch_gemm_quant(wgml_ctx *ctx, float *out, uint32_t out_stride, const wgml_qmat *m,
+                      const void *xh, const float *xscale, uint32_t T, const float *bias,
+                      int accumulate);
+int launch_embed_rows(wgml_ctx *ctx, float *x, const float *table, const uint32_t *d_tokens,
+                      uint32_t dim, uint32_t T);
+int launch_rope_rows(wgml_ctx *ctx, int variant, uint32_t head_size, uint32_t kv_dim, uint32_t pos0,
+                     float base_freq, float *q, uint32_t q_len, uint32_t q_stride, float *k,
+                     uint32_t k_stride, uint32_t T);
 
 }  // namespace wgml

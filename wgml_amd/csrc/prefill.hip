@@ -1,0 +1,439 @@
+// Batched prompt processing ("prefill"): the decoder's matrix products for up to 128
+// tokens at once, as a GEMM on the matrix cores.  The reference has no such path -- it
+// pushes the prompt through its batch-1 step one token at a time
+// (wgml-chat/src/chat_llama2.rs:155-228 with the forced-token rule of
+// wgml-chat/src/sampler.rs:102-107) -- so this is new functionality whose results are
+// held against exactly that: N sequential decode steps.
+//
+//   out[t][r] = sum_k W[r][k] * X[t][k]      W: Q4_K / Q6_K / Q8_0 as stored for the GEMV
+//
+// Weights are expanded to f16 in registers with the reference's dequantization
+// arithmetic (fp32, then rounded to f16), activations are f16 (scaled per token by a
+// power of two so that they stay in range), products accumulate in fp32 on
+// v_mfma_f32_16x16x16_f16.  With f16 inputs the results differ from the fp32 path
+// by about 3e-4 of a row's RMS (the tests bound it at 1e-3).
+//
+// Tiling: a workgroup is 4 waves; a wave owns 16 matrix rows and NT blocks of 16
+// tokens (NT accumulators of 16x16).  The K dimension is walked in chunks of 64: the
+// chunk of X (all tokens) is staged once per workgroup in LDS, every wave expands its
+// 16 x 64 weight elements once and uses them for all its token blocks.
+#include <hip/hip_fp16.h>
+
+#include "common.h"
+#include "device_utils.h"
+
+using namespace wgml;
+
+namespace {
+
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t KC = 64;  // elements of K per chunk
+
+struct GemmArgs {
+    const uint8_t *p0, *p1, *p2, *p3;  // matrix planes (as wgml_qmat)
+    const _Float16 *xh;                // [tpad][kpad] activations
+    const float *xscale;               // [tpad] factor to multiply a token's results with
+    float *out;                        // [T][out_stride]
+    const float *bias;                 // optional, per row
+    uint32_t nrows, ncols, kpad, T, tpad, out_stride;
+    int accumulate;                    // out += result
+    uint32_t tg;                       // token groups per workgroup (tpad / 16 / NT)
+};
+
+__device__ __forceinline__ half4 to_half4(float a, float b, float c, float d) {
+    half4 h;
+    h[0] = (_Float16)a;
+    h[1] = (_Float16)b;
+    h[2] = (_Float16)c;
+    h[3] = (_Float16)d;
+    return h;
+}
+
+// ---- weight fragments -----------------------------------------------------------
+// frag(a, row, chunk, g, a4): the 16 elements  k = 64*chunk + 16*s + 4*g + i  (s, i in
+// 0..3) of matrix row `row`, expanded as the reference's dequantize does
+// (quantization.rs:29-42, 204-244, 322-389) and rounded to f16; a4[s] is the A operand
+// of step s.  `valid`: elements of the chunk that exist (ncols - 64*chunk, capped at 64).
+struct GemmQ4K {
+    __device__ static void frag(const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g,
+                                uint32_t, half4 (&a4)[4]) {
+        const uint8_t *blk = a.p0 + ((size_t)row * (a.ncols / 256) + (chunk >> 2)) * 144;
+        const uint32_t j = chunk & 3;
+        const uint4 hdr = *reinterpret_cast<const uint4 *>(blk);
+        const uint32_t q0 = *reinterpret_cast<const uint32_t *>(blk + 16 + j * 32 + 4 * g);
+        const uint32_t q1 = *reinterpret_cast<const uint32_t *>(blk + 16 + j * 32 + 16 + 4 * g);
+        const float d = f16_bits_to_f32((uint16_t)(hdr.x & 0xffffu));
+        const float dmin = f16_bits_to_f32((uint16_t)(hdr.x >> 16));
+        // get_scale_min_k4 for sub-blocks 2j and 2j + 1, on the three words of packed scales
+        // (no byte array: the index is not a compile-time constant)
+        uint32_t s1, m1, s2, m2;
+        if (j < 2) {
+            const uint32_t sh = 16 * j;
+            s1 = (hdr.y >> sh) & 63u;
+            m1 = (hdr.z >> sh) & 63u;
+            s2 = (hdr.y >> (sh + 8)) & 63u;
+            m2 = (hdr.z >> (sh + 8)) & 63u;
+        } else {
+            const uint32_t sh = 16 * (j - 2);
+            s1 = ((hdr.w >> sh) & 15u) | (((hdr.y >> (sh + 6)) & 3u) << 4);
+            m1 = ((hdr.w >> (sh + 4)) & 15u) | (((hdr.z >> (sh + 6)) & 3u) << 4);
+            s2 = ((hdr.w >> (sh + 8)) & 15u) | (((hdr.y >> (sh + 14)) & 3u) << 4);
+            m2 = ((hdr.w >> (sh + 12)) & 15u) | (((hdr.z >> (sh + 14)) & 3u) << 4);
+        }
+        const float d1 = d * (float)s1, mm1 = dmin * (float)m1;
+        const float d2 = d * (float)s2, mm2 = dmin * (float)m2;
+        auto lo = [&](uint32_t q, float dd, float mm) {
+            return to_half4(dd * (float)(q & 15u) - mm, dd * (float)((q >> 8) & 15u) - mm,
+                            dd * (float)((q >> 16) & 15u) - mm, dd * (float)((q >> 24) & 15u) - mm);
+        };
+        a4[0] = lo(q0, d1, mm1);
+        a4[1] = lo(q1, d1, mm1);
+        a4[2] = lo(q0 >> 4, d2, mm2);
+        a4[3] = lo(q1 >> 4, d2, mm2);
+    }
+};
+
+struct GemmQ6K {
+    __device__ static void frag(const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g,
+                                uint32_t, half4 (&a4)[4]) {
+        const size_t blk = (size_t)row * (a.ncols / 256) + (chunk >> 2);
+        const uint32_t c = chunk & 3, i = c >> 1, hi_nib = c & 1;
+        const uint8_t *ql = a.p0 + blk * 128 + 64 * i + 4 * g;
+        const uint8_t *qh = a.p1 + blk * 64 + 32 * i + 4 * g;
+        const uint32_t scw = *reinterpret_cast<const uint32_t *>(a.p2 + blk * 16 + 8 * i + 4 * hi_nib);
+        const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(a.p3 + blk * 2));
+        const uint32_t h0 = *reinterpret_cast<const uint32_t *>(qh);
+        const uint32_t h1 = *reinterpret_cast<const uint32_t *>(qh + 16);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            uint32_t l = *reinterpret_cast<const uint32_t *>(ql + 16 * s);
+            if (hi_nib) l >>= 4;
+            const uint32_t h = ((s & 1) ? h1 : h0) >> (2 * (2 * hi_nib + (s >> 1)));
+            const float ds = d * (float)(int8_t)((scw >> (8 * s)) & 0xffu);
+            float v[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int q = (int)(((l >> (8 * b)) & 15u) | (((h >> (8 * b)) & 3u) << 4)) - 32;
+                v[b] = ds * (float)q;
+            }
+            a4[s] = to_half4(v[0], v[1], v[2], v[3]);
+        }
+    }
+};
+
+struct GemmQ8_0 {
+    __device__ static void frag(const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g,
+                                uint32_t valid, half4 (&a4)[4]) {
+        const uint8_t *qs = a.p0 + (size_t)row * a.ncols + chunk * 64 + 4 * g;
+        const uint8_t *dp = a.p1 + ((size_t)row * (a.ncols / 32) + chunk * 2) * 2;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            a4[s] = to_half4(0.f, 0.f, 0.f, 0.f);
+            if ((uint32_t)(16 * s) < valid) {  // rows are a multiple of 32 elements long
+                const uint32_t q = *reinterpret_cast<const uint32_t *>(qs + 16 * s);
+                const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(dp + 2 * (s >> 1)));
+                a4[s] = to_half4((float)(int8_t)(q & 0xffu) * d, (float)(int8_t)((q >> 8) & 0xffu) * d,
+                                 (float)(int8_t)((q >> 16) & 0xffu) * d, (float)((int32_t)q >> 24) * d);
+            }
+        }
+    }
+};
+
+template <class F, int NT>
+__global__ __launch_bounds__(256) void gemm_quant_f16_kernel(const GemmArgs a) {
+    // X chunk in LDS: entry (k4, tok) = the four halves X[tok][64*chunk + 4*k4 .. +3]
+    extern __shared__ uint2 xs[];  // [16][tp]
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t j = lane & 15, g = lane >> 4;
+    const uint32_t tp = a.tpad + 1;  // padded row of the LDS table
+    const uint32_t tgi = wave % a.tg, rb = wave / a.tg;  // token group, row block of this wave
+    const uint32_t rbw = 4 / a.tg;                        // row blocks per workgroup
+    const uint32_t row0 = (blockIdx.x * rbw + rb) * 16;
+    const uint32_t row = min(row0 + j, a.nrows - 1);  // this lane's row of the A operand
+    const uint32_t nchunks = a.kpad / KC;
+
+    floatx4 acc[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) acc[n] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    for (uint32_t c = 0; c < nchunks; ++c) {
+        // stage X[:, chunk] (8 threads per token: 16 bytes each)
+        __syncthreads();
+        for (uint32_t e = tid; e < a.tpad * 8; e += 256) {
+            const uint32_t tok = e >> 3, part = e & 7;
+            const uint4 v = *reinterpret_cast<const uint4 *>(a.xh + (size_t)tok * a.kpad + c * KC + part * 8);
+            xs[(2 * part) * tp + tok] = make_uint2(v.x, v.y);
+            xs[(2 * part + 1) * tp + tok] = make_uint2(v.z, v.w);
+        }
+        half4 a4[4];
+        const uint32_t valid = min(KC, a.ncols - min(a.ncols, c * KC));
+        F::frag(a, row, c, g, valid, a4);
+        __syncthreads();
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+#pragma unroll
+            for (int n = 0; n < NT; ++n) {
+                const uint32_t tok = (tgi * NT + n) * 16 + j;
+                const uint2 bw = xs[(4 * s + g) * tp + tok];
+                half4 b;
+                __builtin_memcpy(&b, &bw, 8);
+                acc[n] = __builtin_amdgcn_mfma_f32_16x16x16f16(a4[s], b, acc[n], 0, 0, 0);
+            }
+        }
+    }
+    // acc[n][i] = out[token (tgi*NT + n)*16 + j][row0 + 4g + i]
+    const uint32_t r4 = row0 + 4 * g;
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+        const uint32_t tok = (tgi * NT + n) * 16 + j;
+        if (tok >= a.T || r4 >= a.nrows) continue;
+        const float xs_t = a.xscale ? a.xscale[tok] : 1.f;
+        float *o = a.out + (size_t)tok * a.out_stride + r4;
+        if (r4 + 3 < a.nrows && (reinterpret_cast<uintptr_t>(o) & 15u) == 0) {
+            float4 v = make_float4(acc[n][0] * xs_t, acc[n][1] * xs_t, acc[n][2] * xs_t, acc[n][3] * xs_t);
+            if (a.bias) {
+                v.x += a.bias[r4];
+                v.y += a.bias[r4 + 1];
+                v.z += a.bias[r4 + 2];
+                v.w += a.bias[r4 + 3];
+            }
+            if (a.accumulate) {
+                const float4 p = *reinterpret_cast<const float4 *>(o);
+                v = make_float4(p.x + v.x, p.y + v.y, p.z + v.z, p.w + v.w);
+            }
+            *reinterpret_cast<float4 *>(o) = v;
+            continue;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (r4 + i < a.nrows) {
+                float v = acc[n][i] * xs_t;
+                if (a.bias) v += a.bias[r4 + i];
+                o[i] = a.accumulate ? o[i] + v : v;
+            }
+        }
+    }
+}
+
+// One workgroup per token: X[t] (fp32, optionally RMS-normalised with weights w as
+// the reference does: (x * rsqrt(mean(x^2) + eps)) * w, ops/rms_norm.rs:55-63) -> f16,
+// divided by a power of two if needed so that |x| <= 1024; the factor to undo it goes
+// to xscale[t].  Tokens from T on and columns from K on are zero.
+__global__ __launch_bounds__(256) void prep_x_kernel(const float *__restrict__ x, uint32_t x_stride,
+                                                     const float *__restrict__ norm_w, float eps,
+                                                     _Float16 *__restrict__ xh,
+                                                     float *__restrict__ xscale, uint32_t K,
+                                                     uint32_t kpad, uint32_t T) {
+    __shared__ float red[16];
+    const uint32_t t = blockIdx.x, tid = threadIdx.x;
+    _Float16 *o = xh + (size_t)t * kpad;
+    if (t >= T) {
+        for (uint32_t k = tid; k < kpad; k += 256) o[k] = (_Float16)0.f;
+        if (tid == 0) xscale[t] = 0.f;
+        return;
+    }
+    const float *xr = x + (size_t)t * x_stride;
+    float rs = 1.f;
+    if (norm_w) {
+        float ss = 0.f;
+        for (uint32_t k = tid; k < K; k += 256) ss = fmaf(xr[k], xr[k], ss);
+        rs = 1.0f / sqrtf(block_sum(ss, red) / (float)K + eps);
+    }
+    float amax = 0.f;
+    for (uint32_t k = tid; k < K; k += 256) {
+        const float v = norm_w ? (xr[k] * rs) * norm_w[k] : xr[k];
+        amax = fmaxf(amax, fabsf(v));
+    }
+    amax = block_max(amax, red);
+    float down = 1.f, up = 1.f;
+    for (int it = 0; it < 120 && amax * down > 1024.f; ++it) {  // uniform over the workgroup
+        down *= 0.5f;
+        up *= 2.f;
+    }
+    for (uint32_t k = tid; k < kpad; k += 256) {
+        float v = 0.f;
+        if (k < K) v = (norm_w ? (xr[k] * rs) * norm_w[k] : xr[k]) * down;
+        o[k] = (_Float16)v;
+    }
+    if (tid == 0) xscale[t] = up;
+}
+
+// X[t] = table[tokens[t]]  (embedding rows of the prompt tokens)
+__global__ void embed_rows_kernel(float *__restrict__ x, const float *__restrict__ table,
+                                  const uint32_t *__restrict__ tokens, uint32_t dim) {
+    const uint32_t t = blockIdx.y, i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < dim) x[(size_t)t * dim + i] = table[(size_t)tokens[t] * dim + i];
+}
+
+// RoPE of q[t] and of the K-cache row of position pos0 + t, for every token t
+// (the arithmetic of rope_kernel in ops.hip; ops/rope.wgsl:35-78 of the reference).
+__global__ void rope_rows_kernel(float *__restrict__ q, uint32_t q_stride, float *__restrict__ k,
+                                 uint32_t k_stride, uint32_t n_pairs, uint32_t head_size,
+                                 uint32_t kv_dim, uint32_t pos0, float base_freq, int neox) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
+    if (i >= n_pairs) return;
+    const uint32_t p = pos0 + t;
+    float *qt = q + (size_t)t * q_stride, *kt = k + (size_t)t * k_stride;
+    const float head_dim = (float)((i * 2) % head_size);
+    const float theta = powf(base_freq, -head_dim / (float)head_size);
+    float sn, cs;
+    sincosf((float)p * theta, &sn, &cs);
+    uint32_t a, b;
+    if (!neox) {
+        a = i * 2;
+        b = a + 1;
+    } else {
+        const uint32_t head_id = (i * 2) / head_size;
+        a = i + head_id * head_size / 2;
+        b = a + head_size / 2;
+    }
+    {
+        const float x = qt[a], y = qt[b];
+        qt[a] = cs * x - sn * y;
+        qt[b] = sn * x + cs * y;
+    }
+    if (i * 2 < kv_dim) {
+        const float x = kt[a], y = kt[b];
+        kt[a] = cs * x - sn * y;
+        kt[b] = sn * x + cs * y;
+    }
+}
+
+template <class F>
+int launch_gemm_fmt(wgml_ctx *ctx, GemmArgs &a) {
+    const uint32_t tb = a.tpad / 16;  // token blocks: 1, 2, 4 or 8
+    // token blocks per wave: as many as keep about one workgroup per CU busy
+    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
+    uint32_t nt = tb;
+    while (nt > 1 && tb / nt < 4 && (a.nrows + 16 * (4 / (tb / nt)) - 1) / (16 * (4 / (tb / nt))) < cu)
+        nt >>= 1;
+    a.tg = tb / nt;
+    if (a.tg > 4) {  // at most four token groups fit a workgroup: more blocks per wave
+        a.tg = 4;
+        nt = tb / 4;
+    }
+    const uint32_t rows_per_wg = 16 * (4 / a.tg);
+    const dim3 grid((a.nrows + rows_per_wg - 1) / rows_per_wg), block(256);
+    const size_t lds = (size_t)16 * (a.tpad + 1) * 8;
+    switch (nt) {
+    case 8: gemm_quant_f16_kernel<F, 8><<<grid, block, lds, ctx->stream>>>(a); break;
+    case 4: gemm_quant_f16_kernel<F, 4><<<grid, block, lds, ctx->stream>>>(a); break;
+    case 2: gemm_quant_f16_kernel<F, 2><<<grid, block, lds, ctx->stream>>>(a); break;
+    default: gemm_quant_f16_kernel<F, 1><<<grid, block, lds, ctx->stream>>>(a); break;
+    }
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
+}  // namespace
+
+namespace wgml {
+
+uint32_t prefill_tpad(uint32_t T) { return T <= 16 ? 16 : T <= 32 ? 32 : T <= 64 ? 64 : 128; }
+uint32_t prefill_kpad(uint32_t K) { return (K + KC - 1) / KC * KC; }
+
+int ensure_prefill_scratch(wgml_ctx *ctx, size_t xh_bytes) {
+    if (!ctx->prefill_xscale)
+        WGML_CHECK_HIP(hipMalloc((void **)&ctx->prefill_xscale, kPrefillMaxTokens * sizeof(float)));
+    if (xh_bytes <= ctx->prefill_xh_bytes) return WGML_OK;
+    // work already enqueued may still read the old buffer: retire it, free with the context
+    if (ctx->prefill_xh) ctx->retired.push_back(ctx->prefill_xh);
+    ctx->prefill_xh = nullptr;
+    ctx->prefill_xh_bytes = 0;
+    WGML_CHECK_HIP(hipMalloc(&ctx->prefill_xh, xh_bytes));
+    ctx->prefill_xh_bytes = xh_bytes;
+    return WGML_OK;
+}
+
+int launch_prefill_prep(wgml_ctx *ctx, const float *x, uint32_t x_stride, const float *norm_w,
+                        float eps, void *xh, float *xscale, uint32_t K, uint32_t T) {
+    prep_x_kernel<<<dim3(prefill_tpad(T)), dim3(256), 0, ctx->stream>>>(
+        x, x_stride, norm_w, eps, reinterpret_cast<_Float16 *>(xh), xscale, K, prefill_kpad(K), T);
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
+int launch_gemm_quant(wgml_ctx *ctx, float *out, uint32_t out_stride, const wgml_qmat *m,
+                      const void *xh, const float *xscale, uint32_t T, const float *bias,
+                      int accumulate) {
+    if (T == 0 || T > kPrefillMaxTokens)
+        return set_error(WGML_E_INVALID, "gemm_quant: %u tokens (1..%u)", T, kPrefillMaxTokens);
+    GemmArgs a{};
+    a.p0 = m->p0;
+    a.p1 = m->p1;
+    a.p2 = m->p2;
+    a.p3 = m->p3;
+    a.xh = reinterpret_cast<const _Float16 *>(xh);
+    a.xscale = xscale;
+    a.out = out;
+    a.bias = bias;
+    a.nrows = m->nrows;
+    a.ncols = m->ncols;
+    a.kpad = prefill_kpad(m->ncols);
+    a.T = T;
+    a.tpad = prefill_tpad(T);
+    a.out_stride = out_stride;
+    a.accumulate = accumulate;
+    switch (m->type) {
+    case WGML_Q4_K: return launch_gemm_fmt<GemmQ4K>(ctx, a);
+    case WGML_Q6_K: return launch_gemm_fmt<GemmQ6K>(ctx, a);
+    case WGML_Q8_0: return launch_gemm_fmt<GemmQ8_0>(ctx, a);
+    default:
+        return set_error(WGML_E_UNSUPPORTED, "gemm_quant: matrix type %d (Q8_0, Q4_K, Q6_K only)",
+                         m->type);
+    }
+}
+
+int launch_embed_rows(wgml_ctx *ctx, float *x, const float *table, const uint32_t *d_tokens,
+                      uint32_t dim, uint32_t T) {
+    embed_rows_kernel<<<dim3((dim + 255) / 256, T), dim3(256), 0, ctx->stream>>>(x, table, d_tokens,
+                                                                                 dim);
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
+int launch_rope_rows(wgml_ctx *ctx, int variant, uint32_t head_size, uint32_t kv_dim, uint32_t pos0,
+                     float base_freq, float *q, uint32_t q_len, uint32_t q_stride, float *k,
+                     uint32_t k_stride, uint32_t T) {
+    const uint32_t n_pairs = q_len / 2;
+    rope_rows_kernel<<<dim3((n_pairs + 63) / 64, T), dim3(64), 0, ctx->stream>>>(
+        q, q_stride, k, k_stride, n_pairs, head_size, kv_dim, pos0, base_freq,
+        variant == WGML_ROPE_NEOX);
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
+}  // namespace wgml
+
+extern "C" {
+
+// out[t] = M x[t] for T <= 128 vectors at once (x: T x ncols, out: T x nrows, both
+// row-major f32) on the matrix cores; the batched counterpart of wgml_gemv_quant.
+int wgml_gemm_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, wgml_view x, uint32_t n_tokens) {
+    WGML_REQUIRE(ctx && m, "wgml_gemm_quant: null argument");
+    WGML_TRY(check_view(out, "wgml_gemm_quant: out"));
+    WGML_TRY(check_view(x, "wgml_gemm_quant: x"));
+    WGML_REQUIRE(n_tokens >= 1 && n_tokens <= kPrefillMaxTokens,
+                 "wgml_gemm_quant: %u tokens (1..%u)", n_tokens, kPrefillMaxTokens);
+    WGML_REQUIRE((uint64_t)x.len == (uint64_t)n_tokens * m->ncols,
+                 "Gemm: dimension mismatch (x has %u elements, expected %u x %u)", x.len, n_tokens,
+                 m->ncols);
+    WGML_REQUIRE((uint64_t)out.len == (uint64_t)n_tokens * m->nrows,
+                 "Gemm: dimension mismatch (out has %u elements, expected %u x %u)", out.len,
+                 n_tokens, m->nrows);
+    const size_t xh_bytes = (size_t)kPrefillMaxTokens * prefill_kpad(m->ncols) * 2;
+    WGML_TRY(ensure_prefill_scratch(ctx, xh_bytes));
+    WGML_TRY(launch_prefill_prep(ctx, view_ptr(x), m->ncols, nullptr, 0.f, ctx->prefill_xh,
+                                 ctx->prefill_xscale, m->ncols, n_tokens));
+    return launch_gemm_quant(ctx, view_ptr(out), m->nrows, m, ctx->prefill_xh, ctx->prefill_xscale,
+                             n_tokens, nullptr, 0);
+}
+
+}  // extern "C"

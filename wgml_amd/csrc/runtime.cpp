@@ -37,6 +37,8 @@ void ctx_release(wgml_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->attn_ws) (void)hipFree(ctx->attn_ws);
+    if (ctx->prefill_xh) (void)hipFree(ctx->prefill_xh);
+    if (ctx->prefill_xscale) (void)hipFree(ctx->prefill_xscale);
     for (void *p : ctx->retired) (void)hipFree(p);
     if (ctx->d_scalar) (void)hipFree(ctx->d_scalar);
     if (ctx->h_scalar) (void)hipHostFree(ctx->h_scalar);

@@ -17,7 +17,7 @@ from . import _lib
 from ._lib import AttnParams, RopeConfig, View, WgmlError, call
 
 __all__ = [
-    "GpuInstance", "GpuVector", "GpuMatrix", "GpuQuantMatrix", "GemvQuant", "Gemv", "Quantization",
+    "GpuInstance", "GpuVector", "GpuMatrix", "GpuQuantMatrix", "GemvQuant", "GemmQuant", "Gemv", "Quantization",
     "RmsNorm", "RmsNormConfig", "LayerNorm", "RoPE", "RoPEConfig", "RoPEVariant", "SoftMax",
     "BatchedMultiqueryAttention", "BatchedMultiqueryAttentionParams", "Silu", "UnaryOp",
     "UnaryInplace", "OpAssign", "OpAssignVariant", "Sampler", "quantize", "dequantize_host",
@@ -210,6 +210,17 @@ class GemvQuant(_Op):
 
     def dispatch(self, out: GpuVector, m: GpuQuantMatrix, v: GpuVector) -> None:
         call("wgml_gemv_quant", self.gpu.handle, out.view(), m.handle, v.view())
+
+
+class GemmQuant(_Op):
+    """The product of a quantized matrix with up to 128 vectors at once, on the matrix cores
+    (f16 operands, fp32 sums).  The reference multiplies one vector at a time
+    (ops/gemv_quant.rs:243-348); this is that product for the tokens of a prompt."""
+
+    MAX_TOKENS = 128
+
+    def dispatch(self, out: GpuVector, m: GpuQuantMatrix, x: GpuVector, n_tokens: int) -> None:
+        call("wgml_gemm_quant", self.gpu.handle, out.view(), m.handle, x.view(), n_tokens)
 
 
 class Gemv(_Op):
