@@ -272,6 +272,28 @@ WGML_API int wgml_llama2_decode_greedy(wgml_llama2 *m, uint32_t first_token, uin
 WGML_API int wgml_llama2_decode_greedy_sync(wgml_llama2 *m, uint32_t first_token,
                                             uint32_t start_pos, uint32_t n_steps,
                                             uint32_t *out_tokens);
+/* Batched prompt pass ("prefill").  No counterpart in the reference, which feeds the
+ * prompt through the single-token step one position at a time with the sampled
+ * token overridden (chat_llama2.rs:155-228, sampler.rs:102-107); this produces the
+ * state those n_tokens steps leave behind -- KV-cache rows start_pos ..
+ * start_pos + n_tokens - 1 of every layer and the logits of the last token (read
+ * them with wgml_llama2_read_logits) -- with every matrix-vector product of the
+ * step replaced by one product with up to 128 token vectors on the matrix cores
+ * (wgml_gemm_quant; longer prompts go through in runs of 128).  Arithmetic: f16
+ * operands, fp32 sums for the layer matrices; norms, RoPE, attention and the
+ * output matrix in fp32 as in the step, so logits agree with the step-by-step
+ * pass to about 1e-3 of their range rather than to fp32 rounding.  The layer matrices
+ * must be WGML_Q8_0, WGML_Q4_K or WGML_Q6_K (WGML_E_UNSUPPORTED otherwise).
+ * Enqueues and returns. */
+WGML_API int wgml_llama2_prefill(wgml_llama2 *m, const uint32_t *tokens, uint32_t n_tokens,
+                                 uint32_t start_pos);
+/* wgml_llama2_prefill of the prompt at position 0 followed by greedy decoding:
+ * out_tokens[0] is the arg-max after the last prompt token, out_tokens[i] the
+ * arg-max after out_tokens[i-1] was consumed (n_new entries): the tokens
+ * wgml_llama2_generate_greedy returns from index n_prompt - 1 on. */
+WGML_API int wgml_llama2_prefill_decode_greedy(wgml_llama2 *m, const uint32_t *prompt,
+                                               uint32_t n_prompt, uint32_t n_new,
+                                               uint32_t *out_tokens);
 /* Direct KV-cache access (tests; pre-filled long-context runs). which: 0 = key,
  * 1 = value; `n_pos` positions starting at `first_pos`, kv_dim floats each. */
 WGML_API int wgml_llama2_kv_upload(wgml_llama2 *m, uint32_t layer, int which, uint32_t first_pos,

@@ -123,3 +123,128 @@ def test_gemm_rejects_bad_arguments(gpu):
     f = W.GpuQuantMatrix(gpu, W.F16, 8, 64, np.zeros(8 * 64 * 2, dtype=np.uint8))
     with pytest.raises(W.WgmlError):
         op.dispatch(out, f, x, 3)
+
+
+# ---- the whole prompt pass against the oracle's token-by-token steps -----------------
+from wgml_amd.models import TINY_LLAMA, Llama2, Llama2Config, LlamaModelType, synth_llama  # noqa: E402
+
+MICRO = Llama2Config(dim=256, hidden_dim=512, n_layers=2, n_q_heads=4, n_kv_heads=2,
+                     vocab_size=320, seq_len=40, rope_base_freq=10000.0, rms_norm_eps=1e-5)
+
+
+def spice(w, cfg, seed, biases):
+    rng = np.random.default_rng(seed)
+    for l in w.layers:
+        l["attn_norm"] = (1 + 0.1 * rng.standard_normal(cfg.dim)).astype(np.float32)
+        l["ffn_norm"] = (1 + 0.1 * rng.standard_normal(cfg.dim)).astype(np.float32)
+        if biases:
+            l["attn_q_bias"] = (0.1 * rng.standard_normal(cfg.dim)).astype(np.float32)
+            l["attn_k_bias"] = (0.1 * rng.standard_normal(cfg.kv_dim)).astype(np.float32)
+            l["attn_v_bias"] = (0.1 * rng.standard_normal(cfg.kv_dim)).astype(np.float32)
+    w.output_norm = (1 + 0.1 * rng.standard_normal(cfg.dim)).astype(np.float32)
+
+
+def assert_state_matches(m, ref, cfg, n_pos, want_logits, tol=3e-3):
+    got = m.logits()
+    scale = float(np.abs(want_logits).max())
+    err = float(np.abs(got.astype(np.float64) - want_logits).max()) / scale
+    assert err <= tol, err
+    for layer in range(cfg.n_layers):
+        for which, ref_c in ((0, ref.key_cache(layer)), (1, ref.value_cache(layer))):
+            want_c = ref_c[:n_pos]
+            np.testing.assert_allclose(m.kv_download(layer, which, 0, n_pos), want_c, rtol=0,
+                                       atol=tol * np.abs(want_c).max())
+    return err
+
+
+@pytest.mark.parametrize("scheme", ["q8_0", "q4_k", "q6_k", "q4_k_m"])
+@pytest.mark.parametrize("model_type", [LlamaModelType.Llama, LlamaModelType.Qwen2])
+@pytest.mark.parametrize("n_prompt", [1, 9, 33])
+def test_prefill_matches_stepwise_oracle(gpu, scheme, model_type, n_prompt):
+    w = synth_llama(MICRO, seed=21, scheme=scheme)
+    spice(w, MICRO, 5, biases=model_type == LlamaModelType.Qwen2)
+    ref = orc.Llama2(w, rope_variant=model_type)
+    toks = W.prompt_tokens(3, n_prompt, MICRO.vocab_size)
+    for pos, t in enumerate(toks):
+        want = ref.forward(int(t), pos)
+    m = Llama2(gpu, MICRO, model_type).load(w)
+    m.prefill(toks)
+    assert_state_matches(m, ref, MICRO, n_prompt, want)
+    # decoding continues from the state the prompt pass left
+    nxt = int(np.argmax(want))
+    want2 = ref.forward(nxt, n_prompt)
+    got2 = m.forward_logits(n_prompt, nxt)
+    assert np.abs(got2 - want2).max() <= 3e-3 * np.abs(want2).max()
+
+
+def test_prefill_in_two_calls_and_in_runs_of_128(gpu):
+    cfg = Llama2Config(dim=256, hidden_dim=512, n_layers=2, n_q_heads=4, n_kv_heads=4,
+                       vocab_size=320, seq_len=300, rope_base_freq=10000.0, rms_norm_eps=1e-5)
+    w = synth_llama(cfg, seed=4, scheme="q4_k_m")
+    spice(w, cfg, 6, biases=False)
+    ref = orc.Llama2(w)
+    toks = W.prompt_tokens(9, 290, cfg.vocab_size)
+    for pos, t in enumerate(toks):
+        want = ref.forward(int(t), pos)
+    m = Llama2(gpu, cfg).load(w)
+    m.prefill(toks[:37])  # one call
+    m.prefill(toks[37:], start_pos=37)  # 253 tokens: runs of 128 + 125
+    assert_state_matches(m, ref, cfg, 290, want)
+
+
+@pytest.mark.parametrize("dim,heads,kv_heads,hidden", [(320, 4, 2, 448), (96, 2, 1, 160), (512, 4, 4, 1024),
+                                                       (512, 2, 1, 768)])
+def test_prefill_head_sizes_and_partial_chunks(gpu, dim, heads, kv_heads, hidden):
+    # head sizes 80, 48, 128 and 256; row lengths that are not multiples of 64 (Q8_0 only)
+    cfg = Llama2Config(dim=dim, hidden_dim=hidden, n_layers=2, n_q_heads=heads, n_kv_heads=kv_heads,
+                       vocab_size=300, seq_len=24, rope_base_freq=10000.0, rms_norm_eps=1e-5)
+    w = synth_llama(cfg, seed=2, scheme="q8_0")
+    spice(w, cfg, 3, biases=True)
+    ref = orc.Llama2(w, rope_variant=LlamaModelType.Qwen2)
+    toks = W.prompt_tokens(5, 19, cfg.vocab_size)
+    for pos, t in enumerate(toks):
+        want = ref.forward(int(t), pos)
+    m = Llama2(gpu, cfg, LlamaModelType.Qwen2).load(w)
+    m.prefill(toks)
+    assert_state_matches(m, ref, cfg, 19, want)
+
+
+def test_prefill_then_greedy_tokens_on_tiny_llama(gpu):
+    # the tiny configuration: Q8_0, 16-token seeded prompt, greedy continuation.  The prompt
+    # pass rounds operands to f16, so a near-tie between the two best logits may resolve
+    # differently: tokens must be identical up to the first step whose top-2 margin in the
+    # oracle is below the error bound of the logits (3e-3 of their range)
+    cfg = TINY_LLAMA
+    w = synth_llama(cfg, seed=1, scheme="q8_0")
+    prompt = W.prompt_tokens(1, 16, cfg.vocab_size)
+    n_new = 64
+    oracle_model = orc.Llama2(w, predequantize=True)
+    want, margins = oracle_model.generate_greedy(prompt, 16 + n_new - 1)
+    m = Llama2(gpu, cfg).load(w)
+    got = m.prefill_decode_greedy(prompt, n_new)
+    want_new, margins_new = want[15:], np.asarray(margins)[15:]
+    m.prefill(prompt)
+    logit_range = float(np.abs(m.logits()).max())
+    risky = np.nonzero(margins_new < 3e-3 * logit_range)[0]
+    upto = int(risky[0]) if risky.size else n_new
+    print(f"identical tokens required for the first {upto} of {n_new}; min margin "
+          f"{margins_new.min():.3e}, logit range {logit_range:.3e}")
+    assert upto >= 8
+    assert np.array_equal(got[:upto], want_new[:upto])
+    # and the token-by-token device loop gives the same continuation from the same state
+    stepwise = m.generate_greedy(prompt, 16 + n_new - 1)[15:]
+    assert np.array_equal(got[:upto], stepwise[:upto])
+
+
+def test_prefill_rejects_bad_arguments(gpu):
+    w = synth_llama(MICRO, seed=21, scheme="q8_0")
+    m = Llama2(gpu, MICRO).load(w)
+    with pytest.raises(W.WgmlError):
+        m.prefill([])
+    with pytest.raises(W.WgmlError):
+        m.prefill([1, 2, MICRO.vocab_size])
+    with pytest.raises(W.WgmlError):
+        m.prefill([1] * 10, start_pos=MICRO.seq_len - 9)
+    f = Llama2(gpu, MICRO).load(synth_llama(MICRO, seed=21, scheme="f32"))
+    with pytest.raises(W.WgmlError):
+        f.prefill([1, 2, 3])

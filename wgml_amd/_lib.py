@@ -130,6 +130,8 @@ PROTOTYPES = {
     "wgml_llama2_forward": (_i, [_P, _u32, _u32]),
     "wgml_llama2_read_logits": (_i, [_P, _P]),
     "wgml_llama2_generate_greedy": (_i, [_P, _P, _u32, _u32, _P]),
+    "wgml_llama2_prefill": (_i, [_P, _P, _u32, _u32]),
+    "wgml_llama2_prefill_decode_greedy": (_i, [_P, _P, _u32, _u32, _P]),
     "wgml_llama2_decode_greedy": (_i, [_P, _u32, _u32, _u32, _P]),
     "wgml_llama2_decode_greedy_sync": (_i, [_P, _u32, _u32, _u32, _P]),
     "wgml_llama2_kv_upload": (_i, [_P, _u32, _i, _u32, _u32, _P]),

@@ -202,11 +202,16 @@ constexpr uint32_t kPrefillMaxTokens = 128;
 uint32_t prefill_tpad(uint32_t T);  // tokens rounded up to 16, 32, 64 or 128
 uint32_t prefill_kpad(uint32_t K);  // columns rounded up to a multiple of 64
 int ensure_prefill_scratch(wgml_ctx *ctx, size_t xh_bytes);
-// xh[tpad][kpad] (f16) <- x[T][K] (f32, rows x_stride apart), RMS-normalised with
-// norm_w first when that is non-null; xscale[tpad] receives what a token's
-// products must be multiplied with.
-int launch_prefill_prep(wgml_ctx *ctx, const float *x, uint32_t x_stride, const float *norm_w,
-                        float eps, void *xh, float *xscale, uint32_t K, uint32_t T);
+// xh[tpad][kpad] (f16) <- x[T][K] (f32, rows x_stride apart): RMS-normalised with
+// norm_w first when that is non-null; replaced by up[t][k] * silu(x[t][k]) when `up`
+// is non-null.  xscale[tpad] receives what a token's products must be multiplied with.
+int launch_prefill_prep(wgml_ctx *ctx, const float *x, uint32_t x_stride, const float *up,
+                        const float *norm_w, float eps, void *xh, float *xscale, uint32_t K,
+                        uint32_t T);
+// xb[t] = attention of q[t] (position pos0 + t) over cache rows 0 .. pos0 + t
+int launch_attention_rows(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pos0, uint32_t T,
+                          const float *q, uint32_t q_stride, const float *kc, const float *vc,
+                          float *xb, uint32_t xb_stride);
 // out[t][r] (rows out_stride apart) = (or +=) sum_k M[r][k] x[t][k] + bias[r]
 int launch_gemm_quant(wgml_ctx *ctx, float *out, uint32_t out_stride, const wgml_qmat *m,
                       const void *xh, const float *xscale, uint32_t T, const float *bias,

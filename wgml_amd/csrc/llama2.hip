@@ -48,6 +48,10 @@ struct wgml_llama2 {
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     int graph_fusion = -1;
+    // state of the batched prompt pass, allocated at its first use: one row per token
+    // of a run (up to kPrefillMaxTokens)
+    float *pf_x = nullptr, *pf_xb = nullptr, *pf_q = nullptr, *pf_hb = nullptr, *pf_hb2 = nullptr;
+    uint32_t *pf_tokens = nullptr;
     std::vector<void *> allocs;
     uint64_t launches_last = 0;
 };
@@ -347,6 +351,54 @@ int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint3
     return WGML_OK;
 }
 
+bool gemm_supported(const wgml_qmat *q) {
+    return q->type == WGML_Q8_0 || q->type == WGML_Q4_K || q->type == WGML_Q6_K;
+}
+
+// One run of T <= kPrefillMaxTokens prompt tokens at positions pos0 .. pos0 + T - 1: the
+// launches of enqueue_step with every matrix-vector product replaced by a product
+// with the T vectors at once.  Leaves the last token's residual stream in m->x.
+int enqueue_prefill_run(wgml_llama2 *m, const uint32_t *tokens, uint32_t T, uint32_t pos0) {
+    const wgml_llama2_config &c = m->cfg;
+    wgml_ctx *ctx = m->ctx;
+    const uint32_t dim = c.dim, kv_dim = m->kv_dim, hidden = c.hidden_dim;
+    const int variant = m->model_type == WGML_MODEL_QWEN2 ? WGML_ROPE_NEOX : WGML_ROPE_ORIGINAL;
+    const wgml_attn_params ap{c.seq_len, kv_dim, m->kv_mul, c.n_q_heads, m->head_size, pos0};
+    void *xh = ctx->prefill_xh;
+    float *xs = ctx->prefill_xscale;
+
+    // the caller's token array may be reused as soon as this returns
+    WGML_CHECK_HIP(hipMemcpyAsync(m->pf_tokens, tokens, (size_t)T * 4, hipMemcpyHostToDevice,
+                                  ctx->stream));
+    WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    WGML_TRY(launch_embed_rows(ctx, m->pf_x, m->token_embd, m->pf_tokens, dim, T));
+    for (uint32_t l = 0; l < c.n_layers; ++l) {
+        const LlamaLayer &w = m->layers[l];
+        float *kc = w.key_cache + (size_t)pos0 * kv_dim, *vc = w.value_cache + (size_t)pos0 * kv_dim;
+        WGML_TRY(launch_prefill_prep(ctx, m->pf_x, dim, nullptr, w.attn_norm, c.rms_norm_eps, xh, xs,
+                                     dim, T));
+        WGML_TRY(launch_gemm_quant(ctx, m->pf_q, dim, w.attn_q, xh, xs, T, w.bq, 0));
+        WGML_TRY(launch_gemm_quant(ctx, kc, kv_dim, w.attn_k, xh, xs, T, w.bk, 0));
+        WGML_TRY(launch_gemm_quant(ctx, vc, kv_dim, w.attn_v, xh, xs, T, w.bv, 0));
+        WGML_TRY(launch_rope_rows(ctx, variant, m->head_size, kv_dim, pos0, c.rope_base_freq,
+                                  m->pf_q, dim, dim, kc, kv_dim, T));
+        WGML_TRY(launch_attention_rows(ctx, ap, pos0, T, m->pf_q, dim, w.key_cache, w.value_cache,
+                                       m->pf_xb, dim));
+        WGML_TRY(launch_prefill_prep(ctx, m->pf_xb, dim, nullptr, nullptr, 0.f, xh, xs, dim, T));
+        WGML_TRY(launch_gemm_quant(ctx, m->pf_x, dim, w.attn_output, xh, xs, T, nullptr, 1));
+        WGML_TRY(launch_prefill_prep(ctx, m->pf_x, dim, nullptr, w.ffn_norm, c.rms_norm_eps, xh, xs,
+                                     dim, T));
+        WGML_TRY(launch_gemm_quant(ctx, m->pf_hb, hidden, w.ffn_gate, xh, xs, T, nullptr, 0));
+        WGML_TRY(launch_gemm_quant(ctx, m->pf_hb2, hidden, w.ffn_up, xh, xs, T, nullptr, 0));
+        WGML_TRY(launch_prefill_prep(ctx, m->pf_hb, hidden, m->pf_hb2, nullptr, 0.f, xh, xs, hidden,
+                                     T));
+        WGML_TRY(launch_gemm_quant(ctx, m->pf_x, dim, w.ffn_down, xh, xs, T, nullptr, 1));
+    }
+    WGML_CHECK_HIP(hipMemcpyAsync(m->x, m->pf_x + (size_t)(T - 1) * dim, (size_t)dim * 4,
+                                  hipMemcpyDeviceToDevice, ctx->stream));
+    return WGML_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -525,6 +577,72 @@ int wgml_llama2_forward(wgml_llama2 *m, uint32_t token, uint32_t pos) {
     WGML_TRY(enqueue_step(m, false, token, pos));
     m->launches_last = m->ctx->launches - launches0;
     return WGML_OK;
+}
+
+int wgml_llama2_prefill(wgml_llama2 *m, const uint32_t *tokens, uint32_t n_tokens,
+                        uint32_t start_pos) {
+    WGML_REQUIRE(m && tokens, "wgml_llama2_prefill: null argument");
+    WGML_TRY(check_ready(m));
+    const wgml_llama2_config &c = m->cfg;
+    WGML_REQUIRE(n_tokens >= 1, "wgml_llama2_prefill: empty prompt");
+    WGML_REQUIRE((uint64_t)start_pos + n_tokens <= c.seq_len,
+                 "wgml_llama2_prefill: %u tokens from position %u exceed seq_len %u", n_tokens,
+                 start_pos, c.seq_len);
+    for (uint32_t i = 0; i < n_tokens; ++i)
+        WGML_REQUIRE(tokens[i] < c.vocab_size,
+                     "wgml_llama2_prefill: token %u outside vocabulary %u", tokens[i], c.vocab_size);
+    for (const LlamaLayer &w : m->layers)
+        for (const wgml_qmat *q : {w.attn_q, w.attn_k, w.attn_v, w.attn_output, w.ffn_gate, w.ffn_up,
+                                   w.ffn_down})
+            if (!gemm_supported(q))
+                return set_error(WGML_E_UNSUPPORTED,
+                                 "wgml_llama2_prefill: layer matrices must be Q8_0, Q4_K or Q6_K "
+                                 "(found type %d)", q->type);
+    wgml_ctx *ctx = m->ctx;
+    if (!m->pf_x) {
+        int rc = WGML_OK;
+        auto A = [&](float **p, uint64_t n) {
+            if (rc == WGML_OK) rc = dev_alloc(m, p, n, false);
+        };
+        A(&m->pf_xb, (uint64_t)kPrefillMaxTokens * c.dim);
+        A(&m->pf_q, (uint64_t)kPrefillMaxTokens * c.dim);
+        A(&m->pf_hb, (uint64_t)kPrefillMaxTokens * c.hidden_dim);
+        A(&m->pf_hb2, (uint64_t)kPrefillMaxTokens * c.hidden_dim);
+        if (rc == WGML_OK) rc = dev_alloc_bytes(m, (void **)&m->pf_tokens, kPrefillMaxTokens * 4, false);
+        A(&m->pf_x, (uint64_t)kPrefillMaxTokens * c.dim);  // last: marks the set as complete
+        WGML_TRY(rc);
+    }
+    const uint32_t kmax = c.dim > c.hidden_dim ? c.dim : c.hidden_dim;
+    WGML_TRY(ensure_prefill_scratch(ctx, (size_t)kPrefillMaxTokens * prefill_kpad(kmax) * 2));
+    const uint64_t launches0 = ctx->launches;
+    for (uint32_t done = 0; done < n_tokens; done += kPrefillMaxTokens) {
+        const uint32_t T = n_tokens - done < kPrefillMaxTokens ? n_tokens - done : kPrefillMaxTokens;
+        WGML_TRY(enqueue_prefill_run(m, tokens + done, T, start_pos + done));
+    }
+    // logits of the last token, as a decode step ends (final norm folded into the product)
+    GemvEpilogue eo;
+    eo.norm_w = m->output_norm;
+    eo.norm_eps = c.rms_norm_eps;
+    WGML_TRY(launch_gemv_quant(ctx, m->logits, m->output, m->x, eo));
+    m->launches_last = ctx->launches - launches0;
+    return WGML_OK;
+}
+
+int wgml_llama2_prefill_decode_greedy(wgml_llama2 *m, const uint32_t *prompt, uint32_t n_prompt,
+                                      uint32_t n_new, uint32_t *out_tokens) {
+    WGML_REQUIRE(m && prompt && out_tokens, "wgml_llama2_prefill_decode_greedy: null argument");
+    WGML_REQUIRE((uint64_t)n_prompt + n_new <= (uint64_t)m->cfg.seq_len + 1,
+                 "wgml_llama2_prefill_decode_greedy: %u + %u positions exceed seq_len %u", n_prompt,
+                 n_new, m->cfg.seq_len);
+    WGML_TRY(wgml_llama2_prefill(m, prompt, n_prompt, 0));
+    if (n_new == 0) return WGML_OK;
+    wgml_ctx *ctx = m->ctx;
+    WGML_TRY(launch_argmax(ctx, m->logits, m->cfg.vocab_size, ctx->d_scalar));
+    WGML_CHECK_HIP(hipMemcpyAsync(ctx->h_scalar, ctx->d_scalar, 4, hipMemcpyDeviceToHost, ctx->stream));
+    WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    out_tokens[0] = ctx->h_scalar[0];
+    if (n_new == 1) return WGML_OK;
+    return run_recorded(m, out_tokens[0], n_prompt, n_new - 1, nullptr, 0, out_tokens + 1);
 }
 
 int wgml_llama2_read_logits(wgml_llama2 *m, float *host_out) {

@@ -222,7 +222,10 @@ __global__ __launch_bounds__(256) void gemm_quant_f16_kernel(const GemmArgs a) {
 // the reference does: (x * rsqrt(mean(x^2) + eps)) * w, ops/rms_norm.rs:55-63) -> f16,
 // divided by a power of two if needed so that |x| <= 1024; the factor to undo it goes
 // to xscale[t].  Tokens from T on and columns from K on are zero.
+// With `up` non-null the input is the gated activation up[k] * silu(x[k])
+// (ops/silu.wgsl:13-27) instead of x itself (no normalisation then).
 __global__ __launch_bounds__(256) void prep_x_kernel(const float *__restrict__ x, uint32_t x_stride,
+                                                     const float *__restrict__ up,
                                                      const float *__restrict__ norm_w, float eps,
                                                      _Float16 *__restrict__ xh,
                                                      float *__restrict__ xscale, uint32_t K,
@@ -236,29 +239,32 @@ __global__ __launch_bounds__(256) void prep_x_kernel(const float *__restrict__ x
         return;
     }
     const float *xr = x + (size_t)t * x_stride;
+    const float *ur = up ? up + (size_t)t * x_stride : nullptr;
     float rs = 1.f;
     if (norm_w) {
         float ss = 0.f;
         for (uint32_t k = tid; k < K; k += 256) ss = fmaf(xr[k], xr[k], ss);
         rs = 1.0f / sqrtf(block_sum(ss, red) / (float)K + eps);
     }
+    auto value = [&](uint32_t k) {
+        const float xv = xr[k];
+        if (ur) return ur[k] * (xv / (1.0f + expf(-xv)));
+        return norm_w ? (xv * rs) * norm_w[k] : xv;
+    };
     float amax = 0.f;
-    for (uint32_t k = tid; k < K; k += 256) {
-        const float v = norm_w ? (xr[k] * rs) * norm_w[k] : xr[k];
-        amax = fmaxf(amax, fabsf(v));
-    }
+    for (uint32_t k = tid; k < K; k += 256) amax = fmaxf(amax, fabsf(value(k)));
     amax = block_max(amax, red);
-    float down = 1.f, up = 1.f;
+    float down = 1.f, undo = 1.f;
     for (int it = 0; it < 120 && amax * down > 1024.f; ++it) {  // uniform over the workgroup
         down *= 0.5f;
-        up *= 2.f;
+        undo *= 2.f;
     }
     for (uint32_t k = tid; k < kpad; k += 256) {
         float v = 0.f;
-        if (k < K) v = (norm_w ? (xr[k] * rs) * norm_w[k] : xr[k]) * down;
+        if (k < K) v = value(k) * down;
         o[k] = (_Float16)v;
     }
-    if (tid == 0) xscale[t] = up;
+    if (tid == 0) xscale[t] = undo;
 }
 
 // X[t] = table[tokens[t]]  (embedding rows of the prompt tokens)
@@ -299,6 +305,122 @@ __global__ void rope_rows_kernel(float *__restrict__ q, uint32_t q_stride, float
         const float x = kt[a], y = kt[b];
         kt[a] = cs * x - sn * y;
         kt[b] = sn * x + cs * y;
+    }
+}
+
+
+// Causal attention for a run of tokens: workgroup (h, t) computes head h of token t,
+// which sits at position pos0 + t and attends to cache rows 0 .. pos0 + t (the rows of
+// this run were written by the K and V products before).  Same arithmetic as the decode
+// kernels (ops/batched_multiquery_attention.wgsl:24-97: scores q.k / sqrt(head_size),
+// softmax, weighted sum of values), as an online softmax: 16 lanes share a position,
+// a wave covers four positions at a time, the four waves stride over the positions.
+struct AttnRowsArgs {
+    const float *q;  // [T][q_stride]
+    const float *kc, *vc;  // caches: rows kv_dim apart
+    float *xb;  // [T][xb_stride]
+    uint32_t q_stride, xb_stride, kv_dim, kv_mul, head_size, pos0;
+};
+
+__device__ __forceinline__ float dot4f(const float4 a, const float4 b, float acc) {
+    acc = fmaf(a.x, b.x, acc);
+    acc = fmaf(a.y, b.y, acc);
+    acc = fmaf(a.z, b.z, acc);
+    return fmaf(a.w, b.w, acc);
+}
+__device__ __forceinline__ float4 axpby4f(const float4 a, float sa, const float4 b, float sb) {
+    return make_float4(fmaf(a.x, sa, b.x * sb), fmaf(a.y, sa, b.y * sb), fmaf(a.z, sa, b.z * sb),
+                       fmaf(a.w, sa, b.w * sb));
+}
+
+template <int NV4>
+__global__ __launch_bounds__(256) void attn_rows_kernel(const AttnRowsArgs a) {
+    constexpr int HSP = NV4 * 64;
+    __shared__ float sm_m[4], sm_l[4];
+    __shared__ float sm_acc[4][HSP];
+    const uint32_t h = blockIdx.x, t = blockIdx.y, pos = a.pos0 + t;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t sub = lane & 15, quarter = lane >> 4, hs = a.head_size;
+    const float *kb = a.kc + (size_t)(h / a.kv_mul) * hs;
+    const float *vb = a.vc + (size_t)(h / a.kv_mul) * hs;
+    const float inv_sqrt_hs = 1.0f / sqrtf((float)hs);
+    // float4 number sub + 16 v of the head; lanes beyond the head re-read its last one
+    // with a zero q and never store
+    uint32_t cv[NV4];
+    float4 q[NV4], acc[NV4];
+#pragma unroll
+    for (int v = 0; v < NV4; ++v) {
+        const bool inside = (sub + 16 * v) * 4 < hs;
+        cv[v] = min(sub + 16 * v, hs / 4 - 1);
+        const float4 qv =
+            reinterpret_cast<const float4 *>(a.q + (size_t)t * a.q_stride + (size_t)h * hs)[cv[v]];
+        q[v] = inside ? qv : make_float4(0.f, 0.f, 0.f, 0.f);
+        acc[v] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float mx = -INFINITY, l = 0.f;
+    for (uint32_t p0 = wave * 4; p0 <= pos; p0 += 16) {  // uniform over the wave
+        const uint32_t tt = p0 + quarter;
+        const uint32_t tc = min(tt, pos);
+        const float4 *kp = reinterpret_cast<const float4 *>(kb + (size_t)tc * a.kv_dim);
+        const float4 *vp = reinterpret_cast<const float4 *>(vb + (size_t)tc * a.kv_dim);
+        float4 kk[NV4], vv[NV4];
+#pragma unroll
+        for (int v = 0; v < NV4; ++v) kk[v] = kp[cv[v]];
+#pragma unroll
+        for (int v = 0; v < NV4; ++v) vv[v] = vp[cv[v]];
+        float part = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV4; ++v) part = dot4f(q[v], kk[v], part);
+        const float s = row16_sum(part) * inv_sqrt_hs;
+        if (tt <= pos) {  // uniform within a 16-lane row
+            const float mn = fmaxf(mx, s);
+            const float sc = __expf(mx - mn), p = __expf(s - mn);
+            l = fmaf(l, sc, p);
+#pragma unroll
+            for (int v = 0; v < NV4; ++v) acc[v] = axpby4f(acc[v], sc, vv[v], p);
+            mx = mn;
+        }
+    }
+    // the four quarters of the wave
+#pragma unroll
+    for (int step = 16; step <= 32; step <<= 1) {
+        const float om = __shfl_xor(mx, step, 64), ol = __shfl_xor(l, step, 64);
+        const float M = fmaxf(mx, om);
+        const float sa = mx == -INFINITY ? 0.f : __expf(mx - M);
+        const float sb = om == -INFINITY ? 0.f : __expf(om - M);
+        l = fmaf(l, sa, ol * sb);
+#pragma unroll
+        for (int v = 0; v < NV4; ++v) {
+            float4 o;
+            o.x = __shfl_xor(acc[v].x, step, 64);
+            o.y = __shfl_xor(acc[v].y, step, 64);
+            o.z = __shfl_xor(acc[v].z, step, 64);
+            o.w = __shfl_xor(acc[v].w, step, 64);
+            acc[v] = axpby4f(acc[v], sa, o, sb);
+        }
+        mx = M;
+    }
+    // the four waves
+    if (lane == 0) {
+        sm_m[wave] = mx;
+        sm_l[wave] = l;
+    }
+    if (quarter == 0) {
+#pragma unroll
+        for (int v = 0; v < NV4; ++v) reinterpret_cast<float4 *>(&sm_acc[wave][0])[sub + 16 * v] = acc[v];
+    }
+    __syncthreads();
+    for (uint32_t d = threadIdx.x; d < hs; d += 256) {
+        const float M = fmaxf(fmaxf(sm_m[0], sm_m[1]), fmaxf(sm_m[2], sm_m[3]));
+        float L = 0.f, o = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float wgt = sm_m[w] == -INFINITY ? 0.f : __expf(sm_m[w] - M);
+            L = fmaf(sm_l[w], wgt, L);
+            o = fmaf(wgt > 0.f ? sm_acc[w][d] : 0.f, wgt, o);
+        }
+        a.xb[(size_t)t * a.xb_stride + (size_t)h * hs + d] = o / L;
     }
 }
 
@@ -349,10 +471,11 @@ int ensure_prefill_scratch(wgml_ctx *ctx, size_t xh_bytes) {
     return WGML_OK;
 }
 
-int launch_prefill_prep(wgml_ctx *ctx, const float *x, uint32_t x_stride, const float *norm_w,
-                        float eps, void *xh, float *xscale, uint32_t K, uint32_t T) {
+int launch_prefill_prep(wgml_ctx *ctx, const float *x, uint32_t x_stride, const float *up,
+                        const float *norm_w, float eps, void *xh, float *xscale, uint32_t K,
+                        uint32_t T) {
     prep_x_kernel<<<dim3(prefill_tpad(T)), dim3(256), 0, ctx->stream>>>(
-        x, x_stride, norm_w, eps, reinterpret_cast<_Float16 *>(xh), xscale, K, prefill_kpad(K), T);
+        x, x_stride, up, norm_w, eps, reinterpret_cast<_Float16 *>(xh), xscale, K, prefill_kpad(K), T);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
@@ -410,6 +533,26 @@ int launch_rope_rows(wgml_ctx *ctx, int variant, uint32_t head_size, uint32_t kv
     return WGML_OK;
 }
 
+int launch_attention_rows(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pos0, uint32_t T,
+                          const float *q, uint32_t q_stride, const float *kc, const float *vc,
+                          float *xb, uint32_t xb_stride) {
+    if (p.head_size % 4 != 0 || p.head_size > 256 || p.kv_dim % 4 != 0 || q_stride % 4 != 0)
+        return set_error(WGML_E_UNSUPPORTED,
+                         "attention over a run of tokens: head_size %u (multiple of 4, <= 256)",
+                         p.head_size);
+    AttnRowsArgs a{q, kc, vc, xb, q_stride, xb_stride, p.kv_dim, p.kv_mul, p.head_size, pos0};
+    const dim3 grid(p.n_heads, T), block(256);
+    switch ((p.head_size + 63) / 64) {
+    case 1: attn_rows_kernel<1><<<grid, block, 0, ctx->stream>>>(a); break;
+    case 2: attn_rows_kernel<2><<<grid, block, 0, ctx->stream>>>(a); break;
+    case 3: attn_rows_kernel<3><<<grid, block, 0, ctx->stream>>>(a); break;
+    default: attn_rows_kernel<4><<<grid, block, 0, ctx->stream>>>(a); break;
+    }
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
 }  // namespace wgml
 
 extern "C" {
@@ -430,7 +573,7 @@ int wgml_gemm_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, wgml_view 
                  n_tokens, m->nrows);
     const size_t xh_bytes = (size_t)kPrefillMaxTokens * prefill_kpad(m->ncols) * 2;
     WGML_TRY(ensure_prefill_scratch(ctx, xh_bytes));
-    WGML_TRY(launch_prefill_prep(ctx, view_ptr(x), m->ncols, nullptr, 0.f, ctx->prefill_xh,
+    WGML_TRY(launch_prefill_prep(ctx, view_ptr(x), m->ncols, nullptr, nullptr, 0.f, ctx->prefill_xh,
                                  ctx->prefill_xscale, m->ncols, n_tokens));
     return launch_gemm_quant(ctx, view_ptr(out), m->nrows, m, ctx->prefill_xh, ctx->prefill_xscale,
                              n_tokens, nullptr, 0);

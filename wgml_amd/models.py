@@ -184,6 +184,20 @@ class Llama2:
         call("wgml_llama2_generate_greedy", self._h, _ptr(p), p.size, n_total, _ptr(out))
         return out
 
+    def prefill(self, tokens, start_pos: int = 0) -> None:
+        """Batched prompt pass on the matrix cores: fills the KV cache for the tokens'
+        positions and leaves the last token's logits (`logits()`).  The reference has no
+        batched pass (it steps through the prompt, chat_llama2.rs:155-228)."""
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        call("wgml_llama2_prefill", self._h, _ptr(t), t.size, start_pos)
+
+    def prefill_decode_greedy(self, prompt, n_new: int) -> np.ndarray:
+        """`prefill(prompt)` then greedy decoding; returns the n_new generated tokens."""
+        p = np.ascontiguousarray(prompt, dtype=np.uint32)
+        out = np.empty(n_new, dtype=np.uint32)
+        call("wgml_llama2_prefill_decode_greedy", self._h, _ptr(p), p.size, n_new, _ptr(out))
+        return out
+
     def decode_greedy(self, first_token: int, start_pos: int, n_steps: int) -> np.ndarray:
         out = np.empty(n_steps, dtype=np.uint32)
         call("wgml_llama2_decode_greedy", self._h, first_token, start_pos, n_steps, _ptr(out))
