@@ -306,6 +306,32 @@ def main():
         f"{model.launches_per_token()} launches/token; with a host read-back per token: "
         f"{tok_s_sync:.1f} tok/s")
 
+    # the batched prompt pass over the same prompt (f16 MFMA products, 128 tokens per run);
+    # untimed first call allocates its buffers.  It rewrites KV rows 0..warmup-1 with values
+    # that agree with the step-by-step ones to ~1e-3, which nothing after this point reads.
+    prefill = None
+    if args.warmup >= 2:
+        model.prefill(prompt)
+        gpu.synchronize()
+        reps = 3
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            model.prefill(prompt)
+        gpu.synchronize()
+        pdt = (time.perf_counter() - t0) / reps
+        layer_elems = cfg.n_layers * (2 * cfg.dim * cfg.dim + 2 * cfg.kv_dim * cfg.dim +
+                                      3 * cfg.dim * cfg.hidden_dim)
+        flops = 2.0 * layer_elems * args.warmup
+        prefill = {"tokens": args.warmup, "ms": round(pdt * 1e3, 3),
+                   "tok_s": round(args.warmup / pdt, 1),
+                   "TFLOP/s": round(flops / pdt * 1e-12, 1),
+                   "ms_step_by_step_at_decode_rate": round(args.warmup / tok_s * 1e3, 1),
+                   "first_token_matches_step_by_step": int(np.argmax(model.logits())) == first,
+                   "launches": model.launches_per_token()}
+        log(f"prefill: {args.warmup} tokens in {pdt * 1e3:.2f} ms -> {args.warmup / pdt:.0f} tok/s, "
+            f"{flops / pdt * 1e-12:.1f} TFLOP/s (step by step: {args.warmup / tok_s * 1e3:.0f} ms); "
+            f"first token matches: {prefill['first_token_matches_step_by_step']}")
+
     # dominant kernel: the fused gate/up launch (27% of a step), timed live over the model's
     # own per-layer matrices; the plain single-matrix Q4_K GEMV of the same shape beside it
     roofline = None
@@ -361,7 +387,7 @@ def main():
                    "launches_per_token": model.launches_per_token(),
                    "tok_s_with_per_token_host_sync": round(tok_s_sync, 2),
                    "last_token": int(toks[-1])},
-        "roofline": roofline, "cpu_baseline": cpu, "gemv_sweep": sweep,
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "gemv_sweep": sweep,
     }
     print(json.dumps(line), flush=True)
 

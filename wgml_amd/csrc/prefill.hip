@@ -13,10 +13,20 @@
 // v_mfma_f32_16x16x16_f16.  With f16 inputs the results differ from the fp32 path
 // by about 3e-4 of a row's RMS (the tests bound it at 1e-3).
 //
-// Tiling: a workgroup is 4 waves; a wave owns 16 matrix rows and NT blocks of 16
-// tokens (NT accumulators of 16x16).  The K dimension is walked in chunks of 64: the
-// chunk of X (all tokens) is staged once per workgroup in LDS, every wave expands its
-// 16 x 64 weight elements once and uses them for all its token blocks.
+// Tiling.  A workgroup owns 16 matrix rows and all tokens; its 8 waves split K: wave w
+// takes the 64-element chunks w, w + 8, ...  so that every weight element is expanded
+// exactly once, by one wave, and used for all NT blocks of 16 tokens (NT accumulators
+// of 16x16 per wave).  The 8 partial sums meet in LDS at the end, added in a fixed order.
+// Nothing is shared between the waves before that, so the loop has no barrier: each wave
+// keeps the loads of its next chunk (weights and activations) in flight while it
+// multiplies the current one.
+//
+// Activations are stored in the order the B operand wants them (written by
+// prep_x_kernel): for chunk c, token block n, half s2 of the chunk, lane (g, j) finds
+// the 8 halves  X[16 n + j][64 c + 32 s2 + 8 g .. + 7]  as one 16-byte word at
+// word index ((c * NT + n) * 2 + s2) * 64 + 16 g + j: a wave's load is 1 KiB contiguous.
+// The first four halves are the B operand of MFMA step 2 s2, the last four of step
+// 2 s2 + 1; the A operand follows the same assignment of k to (step, lane, slot).
 #include <hip/hip_fp16.h>
 
 #include "common.h"
@@ -29,17 +39,17 @@ namespace {
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr uint32_t KC = 64;  // elements of K per chunk
+constexpr uint32_t KC = 64;    // elements of K per chunk
+constexpr uint32_t KWAVES = 8;  // waves of a workgroup = ways K is split
 
 struct GemmArgs {
     const uint8_t *p0, *p1, *p2, *p3;  // matrix planes (as wgml_qmat)
-    const _Float16 *xh;                // [tpad][kpad] activations
+    const uint4 *xh;                   // packed f16 activations (see above)
     const float *xscale;               // [tpad] factor to multiply a token's results with
     float *out;                        // [T][out_stride]
     const float *bias;                 // optional, per row
     uint32_t nrows, ncols, kpad, T, tpad, out_stride;
     int accumulate;                    // out += result
-    uint32_t tg;                       // token groups per workgroup (tpad / 16 / NT)
 };
 
 __device__ __forceinline__ half4 to_half4(float a, float b, float c, float d) {
@@ -52,18 +62,24 @@ __device__ __forceinline__ half4 to_half4(float a, float b, float c, float d) {
 }
 
 // ---- weight fragments -----------------------------------------------------------
-// frag(a, row, chunk, g, a4): the 16 elements  k = 64*chunk + 16*s + 4*g + i  (s, i in
-// 0..3) of matrix row `row`, expanded as the reference's dequantize does
-// (quantization.rs:29-42, 204-244, 322-389) and rounded to f16; a4[s] is the A operand
-// of step s.  `valid`: elements of the chunk that exist (ncols - 64*chunk, capped at 64).
+// Lane (g, j) of a wave holds, for chunk c of row j of the tile, the 16 elements
+//     k = 64 c + 32 s2 + 8 g + 4 e + i        (s2, e in 0..1, i in 0..3)
+// load() fetches their bytes, frag() expands them as the reference's dequantize does
+// (quantization.rs:29-42, 204-244, 322-389) and rounds to f16: a4[2 s2 + e][i].
 struct GemmQ4K {
-    __device__ static void frag(const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g,
-                                uint32_t, half4 (&a4)[4]) {
+    struct Raw {
+        uint4 hdr;  // d, dmin, 12 bytes of packed scales
+        uint2 qs;   // bytes 8 g .. 8 g + 7 of the chunk's 32: low nibbles s2 = 0, high s2 = 1
+    };
+    __device__ static void load(Raw &r, const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g) {
         const uint8_t *blk = a.p0 + ((size_t)row * (a.ncols / 256) + (chunk >> 2)) * 144;
+        r.hdr = *reinterpret_cast<const uint4 *>(blk);
+        r.qs = *reinterpret_cast<const uint2 *>(blk + 16 + (chunk & 3) * 32 + 8 * g);
+    }
+    __device__ static void frag(const Raw &r, const GemmArgs &, uint32_t chunk, uint32_t,
+                                half4 (&a4)[4]) {
+        const uint4 hdr = r.hdr;
         const uint32_t j = chunk & 3;
-        const uint4 hdr = *reinterpret_cast<const uint4 *>(blk);
-        const uint32_t q0 = *reinterpret_cast<const uint32_t *>(blk + 16 + j * 32 + 4 * g);
-        const uint32_t q1 = *reinterpret_cast<const uint32_t *>(blk + 16 + j * 32 + 16 + 4 * g);
         const float d = f16_bits_to_f32((uint16_t)(hdr.x & 0xffffu));
         const float dmin = f16_bits_to_f32((uint16_t)(hdr.x >> 16));
         // get_scale_min_k4 for sub-blocks 2j and 2j + 1, on the three words of packed scales
@@ -84,116 +100,167 @@ struct GemmQ4K {
         }
         const float d1 = d * (float)s1, mm1 = dmin * (float)m1;
         const float d2 = d * (float)s2, mm2 = dmin * (float)m2;
-        auto lo = [&](uint32_t q, float dd, float mm) {
+        auto four = [&](uint32_t q, float dd, float mm) {
             return to_half4(dd * (float)(q & 15u) - mm, dd * (float)((q >> 8) & 15u) - mm,
                             dd * (float)((q >> 16) & 15u) - mm, dd * (float)((q >> 24) & 15u) - mm);
         };
-        a4[0] = lo(q0, d1, mm1);
-        a4[1] = lo(q1, d1, mm1);
-        a4[2] = lo(q0 >> 4, d2, mm2);
-        a4[3] = lo(q1 >> 4, d2, mm2);
+        a4[0] = four(r.qs.x, d1, mm1);
+        a4[1] = four(r.qs.y, d1, mm1);
+        a4[2] = four(r.qs.x >> 4, d2, mm2);
+        a4[3] = four(r.qs.y >> 4, d2, mm2);
     }
 };
 
 struct GemmQ6K {
-    __device__ static void frag(const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g,
-                                uint32_t, half4 (&a4)[4]) {
+    struct Raw {
+        uint2 ql[2];  // per s2: 8 bytes of low nibbles
+        uint2 qh;     // 8 bytes of high bit pairs
+        uint32_t scw;  // the four scales of this 64-element chunk
+        uint32_t d;
+    };
+    __device__ static void load(Raw &r, const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g) {
         const size_t blk = (size_t)row * (a.ncols / 256) + (chunk >> 2);
-        const uint32_t c = chunk & 3, i = c >> 1, hi_nib = c & 1;
-        const uint8_t *ql = a.p0 + blk * 128 + 64 * i + 4 * g;
-        const uint8_t *qh = a.p1 + blk * 64 + 32 * i + 4 * g;
-        const uint32_t scw = *reinterpret_cast<const uint32_t *>(a.p2 + blk * 16 + 8 * i + 4 * hi_nib);
-        const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(a.p3 + blk * 2));
-        const uint32_t h0 = *reinterpret_cast<const uint32_t *>(qh);
-        const uint32_t h1 = *reinterpret_cast<const uint32_t *>(qh + 16);
+        const uint32_t c = chunk & 3, i = c >> 1;
+        const uint8_t *ql = a.p0 + blk * 128 + 64 * i + 8 * g;
+        r.ql[0] = *reinterpret_cast<const uint2 *>(ql);
+        r.ql[1] = *reinterpret_cast<const uint2 *>(ql + 32);
+        r.qh = *reinterpret_cast<const uint2 *>(a.p1 + blk * 64 + 32 * i + 8 * g);
+        r.scw = *reinterpret_cast<const uint32_t *>(a.p2 + blk * 16 + 8 * i + 4 * (c & 1));
+        r.d = *reinterpret_cast<const uint16_t *>(a.p3 + blk * 2);
+    }
+    __device__ static void frag(const Raw &r, const GemmArgs &, uint32_t chunk, uint32_t g,
+                                half4 (&a4)[4]) {
+        // element e = 64 (c & 1) + 32 s2 + 8 g + b of the 128-element half: quarter
+        // e / 32 = 2 (c & 1) + s2 picks the nibble (high for quarters 2, 3), the bit pair of
+        // qh[8 g + b] (shift 2 * quarter) and the scale (8 g + b) / 16 + 2 * quarter
+        const uint32_t hi_nib = chunk & 1;
+        const float d = f16_bits_to_f32((uint16_t)r.d);
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            uint32_t l = *reinterpret_cast<const uint32_t *>(ql + 16 * s);
-            if (hi_nib) l >>= 4;
-            const uint32_t h = ((s & 1) ? h1 : h0) >> (2 * (2 * hi_nib + (s >> 1)));
-            const float ds = d * (float)(int8_t)((scw >> (8 * s)) & 0xffu);
-            float v[4];
+        for (int s2 = 0; s2 < 2; ++s2) {
+            const float ds = d * (float)(int8_t)((r.scw >> (8 * ((g >> 1) + 2 * s2))) & 0xffu);
+            const uint32_t hsh = 2 * (2 * hi_nib + s2);
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                const int q = (int)(((l >> (8 * b)) & 15u) | (((h >> (8 * b)) & 3u) << 4)) - 32;
-                v[b] = ds * (float)q;
+            for (int e = 0; e < 2; ++e) {
+                uint32_t l = e ? r.ql[s2].y : r.ql[s2].x;
+                if (hi_nib) l >>= 4;
+                const uint32_t h = (e ? r.qh.y : r.qh.x) >> hsh;
+                float v[4];
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const int q = (int)(((l >> (8 * b)) & 15u) | (((h >> (8 * b)) & 3u) << 4)) - 32;
+                    v[b] = ds * (float)q;
+                }
+                a4[2 * s2 + e] = to_half4(v[0], v[1], v[2], v[3]);
             }
-            a4[s] = to_half4(v[0], v[1], v[2], v[3]);
         }
     }
 };
 
 struct GemmQ8_0 {
-    __device__ static void frag(const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g,
-                                uint32_t valid, half4 (&a4)[4]) {
-        const uint8_t *qs = a.p0 + (size_t)row * a.ncols + chunk * 64 + 4 * g;
-        const uint8_t *dp = a.p1 + ((size_t)row * (a.ncols / 32) + chunk * 2) * 2;
+    struct Raw {
+        uint2 q[2];  // per s2 (= 32-element block of the chunk): 8 quants
+        uint32_t d[2];
+    };
+    // rows are a multiple of 32 elements long: the second half of the last chunk may not
+    // exist; it is then read from the first half and expanded to zeros
+    __device__ static void load(Raw &r, const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g) {
+        const uint32_t b0 = chunk * 2, nb = a.ncols / 32;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            a4[s] = to_half4(0.f, 0.f, 0.f, 0.f);
-            if ((uint32_t)(16 * s) < valid) {  // rows are a multiple of 32 elements long
-                const uint32_t q = *reinterpret_cast<const uint32_t *>(qs + 16 * s);
-                const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(dp + 2 * (s >> 1)));
-                a4[s] = to_half4((float)(int8_t)(q & 0xffu) * d, (float)(int8_t)((q >> 8) & 0xffu) * d,
-                                 (float)(int8_t)((q >> 16) & 0xffu) * d, (float)((int32_t)q >> 24) * d);
-            }
+        for (int s2 = 0; s2 < 2; ++s2) {
+            const uint32_t b = min(b0 + s2, nb - 1);
+            r.q[s2] = *reinterpret_cast<const uint2 *>(a.p0 + (size_t)row * a.ncols + b * 32 + 8 * g);
+            r.d[s2] = *reinterpret_cast<const uint16_t *>(a.p1 + ((size_t)row * nb + b) * 2);
+        }
+    }
+    __device__ static void frag(const Raw &r, const GemmArgs &a, uint32_t chunk, uint32_t,
+                                half4 (&a4)[4]) {
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            const bool exists = chunk * 2 + s2 < a.ncols / 32;
+            const float d = exists ? f16_bits_to_f32((uint16_t)r.d[s2]) : 0.f;
+            const uint32_t x = exists ? r.q[s2].x : 0u, y = exists ? r.q[s2].y : 0u;
+            a4[2 * s2] = to_half4(sb0(x) * d, sb1(x) * d, sb2(x) * d, sb3(x) * d);
+            a4[2 * s2 + 1] = to_half4(sb0(y) * d, sb1(y) * d, sb2(y) * d, sb3(y) * d);
         }
     }
 };
 
 template <class F, int NT>
-__global__ __launch_bounds__(256) void gemm_quant_f16_kernel(const GemmArgs a) {
-    // X chunk in LDS: entry (k4, tok) = the four halves X[tok][64*chunk + 4*k4 .. +3]
-    extern __shared__ uint2 xs[];  // [16][tp]
+__global__ __launch_bounds__(KWAVES * 64) void gemm_quant_f16_kernel(const GemmArgs a) {
+    extern __shared__ float4 red[];  // [KWAVES][NT][64]
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t j = lane & 15, g = lane >> 4;
-    const uint32_t tp = a.tpad + 1;  // padded row of the LDS table
-    const uint32_t tgi = wave % a.tg, rb = wave / a.tg;  // token group, row block of this wave
-    const uint32_t rbw = 4 / a.tg;                        // row blocks per workgroup
-    const uint32_t row0 = (blockIdx.x * rbw + rb) * 16;
+    const uint32_t row0 = blockIdx.x * 16;
     const uint32_t row = min(row0 + j, a.nrows - 1);  // this lane's row of the A operand
     const uint32_t nchunks = a.kpad / KC;
+    // chunks of this wave: wave, wave + 8, ...
+    const uint32_t n_my = nchunks > wave ? (nchunks - wave + KWAVES - 1) / KWAVES : 0;
 
     floatx4 acc[NT];
 #pragma unroll
     for (int n = 0; n < NT; ++n) acc[n] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    for (uint32_t c = 0; c < nchunks; ++c) {
-        // stage X[:, chunk] (8 threads per token: 16 bytes each)
-        __syncthreads();
-        for (uint32_t e = tid; e < a.tpad * 8; e += 256) {
-            const uint32_t tok = e >> 3, part = e & 7;
-            const uint4 v = *reinterpret_cast<const uint4 *>(a.xh + (size_t)tok * a.kpad + c * KC + part * 8);
-            xs[(2 * part) * tp + tok] = make_uint2(v.x, v.y);
-            xs[(2 * part + 1) * tp + tok] = make_uint2(v.z, v.w);
-        }
-        half4 a4[4];
-        const uint32_t valid = min(KC, a.ncols - min(a.ncols, c * KC));
-        F::frag(a, row, c, g, valid, a4);
-        __syncthreads();
+    typename F::Raw ra, rb;
+    uint4 ba[NT][2], bb[NT][2];
+    // every load is unconditional (a chunk number past the end re-reads the last chunk and
+    // is never multiplied): the compiler can then count outstanding loads exactly instead
+    // of draining them all before each use
+    auto load = [&](typename F::Raw &r, uint4(&b)[NT][2], uint32_t i) {
+        const uint32_t c = min(wave + KWAVES * i, nchunks - 1);
+        F::load(r, a, row, c, g);
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
+        for (int n = 0; n < NT; ++n) {
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) b[n][s2] = a.xh[(((size_t)c * NT + n) * 2 + s2) * 64 + lane];
+        }
+    };
+    auto compute = [&](const typename F::Raw &r, const uint4(&b)[NT][2], uint32_t i) {
+        const uint32_t c = wave + KWAVES * i;
+        half4 a4[4];
+        F::frag(r, a, c, g, a4);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
 #pragma unroll
             for (int n = 0; n < NT; ++n) {
-                const uint32_t tok = (tgi * NT + n) * 16 + j;
-                const uint2 bw = xs[(4 * s + g) * tp + tok];
-                half4 b;
-                __builtin_memcpy(&b, &bw, 8);
-                acc[n] = __builtin_amdgcn_mfma_f32_16x16x16f16(a4[s], b, acc[n], 0, 0, 0);
+                const uint2 lo = make_uint2(b[n][s2].x, b[n][s2].y), hi = make_uint2(b[n][s2].z, b[n][s2].w);
+                half4 b0, b1;
+                __builtin_memcpy(&b0, &lo, 8);
+                __builtin_memcpy(&b1, &hi, 8);
+                acc[n] = __builtin_amdgcn_mfma_f32_16x16x16f16(a4[2 * s2], b0, acc[n], 0, 0, 0);
+                acc[n] = __builtin_amdgcn_mfma_f32_16x16x16f16(a4[2 * s2 + 1], b1, acc[n], 0, 0, 0);
             }
         }
+    };
+    if (n_my > 0) {
+        load(ra, ba, 0);
+        for (uint32_t i = 0; i < n_my; i += 2) {
+            load(rb, bb, i + 1);
+            compute(ra, ba, i);
+            load(ra, ba, i + 2);
+            if (i + 1 < n_my) compute(rb, bb, i + 1);
+        }
     }
-    // acc[n][i] = out[token (tgi*NT + n)*16 + j][row0 + 4g + i]
-    const uint32_t r4 = row0 + 4 * g;
+    // the partial sums of the 8 waves, added in wave order
 #pragma unroll
-    for (int n = 0; n < NT; ++n) {
-        const uint32_t tok = (tgi * NT + n) * 16 + j;
+    for (int n = 0; n < NT; ++n)
+        red[(wave * NT + n) * 64 + lane] = make_float4(acc[n][0], acc[n][1], acc[n][2], acc[n][3]);
+    __syncthreads();
+    for (uint32_t idx = tid; idx < NT * 64; idx += KWAVES * 64) {
+        const uint32_t n = idx >> 6, l = idx & 63;
+        float4 v = red[n * 64 + l];
+#pragma unroll
+        for (uint32_t w = 1; w < KWAVES; ++w) {
+            const float4 p = red[(w * NT + n) * 64 + l];
+            v = make_float4(v.x + p.x, v.y + p.y, v.z + p.z, v.w + p.w);
+        }
+        // v = out[token 16 n + (l & 15)][row0 + 4 (l >> 4) .. + 3]
+        const uint32_t tok = n * 16 + (l & 15), r4 = row0 + 4 * (l >> 4);
         if (tok >= a.T || r4 >= a.nrows) continue;
         const float xs_t = a.xscale ? a.xscale[tok] : 1.f;
+        v = make_float4(v.x * xs_t, v.y * xs_t, v.z * xs_t, v.w * xs_t);
         float *o = a.out + (size_t)tok * a.out_stride + r4;
         if (r4 + 3 < a.nrows && (reinterpret_cast<uintptr_t>(o) & 15u) == 0) {
-            float4 v = make_float4(acc[n][0] * xs_t, acc[n][1] * xs_t, acc[n][2] * xs_t, acc[n][3] * xs_t);
             if (a.bias) {
                 v.x += a.bias[r4];
                 v.y += a.bias[r4 + 1];
@@ -207,34 +274,39 @@ __global__ __launch_bounds__(256) void gemm_quant_f16_kernel(const GemmArgs a) {
             *reinterpret_cast<float4 *>(o) = v;
             continue;
         }
+        const float vv[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             if (r4 + i < a.nrows) {
-                float v = acc[n][i] * xs_t;
-                if (a.bias) v += a.bias[r4 + i];
-                o[i] = a.accumulate ? o[i] + v : v;
+                float e = vv[i];
+                if (a.bias) e += a.bias[r4 + i];
+                o[i] = a.accumulate ? o[i] + e : e;
             }
         }
     }
 }
 
 // One workgroup per token: X[t] (fp32, optionally RMS-normalised with weights w as
-// the reference does: (x * rsqrt(mean(x^2) + eps)) * w, ops/rms_norm.rs:55-63) -> f16,
-// divided by a power of two if needed so that |x| <= 1024; the factor to undo it goes
-// to xscale[t].  Tokens from T on and columns from K on are zero.
-// With `up` non-null the input is the gated activation up[k] * silu(x[k])
-// (ops/silu.wgsl:13-27) instead of x itself (no normalisation then).
+// the reference does: (x * rsqrt(mean(x^2) + eps)) * w, ops/rms_norm.rs:55-63) -> f16
+// in the packed order described at the top, divided by a power of two if needed so that
+// |x| <= 1024; the factor to undo it goes to xscale[t].  Tokens from T on and columns
+// from K on are zero.  With `up` non-null the input is the gated activation
+// up[k] * silu(x[k]) (ops/silu.wgsl:13-27) instead of x itself (no normalisation then).
 __global__ __launch_bounds__(256) void prep_x_kernel(const float *__restrict__ x, uint32_t x_stride,
                                                      const float *__restrict__ up,
                                                      const float *__restrict__ norm_w, float eps,
-                                                     _Float16 *__restrict__ xh,
+                                                     uint4 *__restrict__ xh,
                                                      float *__restrict__ xscale, uint32_t K,
                                                      uint32_t kpad, uint32_t T) {
     __shared__ float red[16];
-    const uint32_t t = blockIdx.x, tid = threadIdx.x;
-    _Float16 *o = xh + (size_t)t * kpad;
+    const uint32_t t = blockIdx.x, tid = threadIdx.x, nt = gridDim.x / 16;
+    // 16-byte word of (token t, columns 8 k8 .. 8 k8 + 7)
+    auto word = [&](uint32_t k8) -> uint4 & {
+        const uint32_t c = k8 >> 3, s2 = (k8 >> 2) & 1, g = k8 & 3;
+        return xh[(((size_t)c * nt + (t >> 4)) * 2 + s2) * 64 + 16 * g + (t & 15)];
+    };
     if (t >= T) {
-        for (uint32_t k = tid; k < kpad; k += 256) o[k] = (_Float16)0.f;
+        for (uint32_t k8 = tid; k8 < kpad / 8; k8 += 256) word(k8) = make_uint4(0, 0, 0, 0);
         if (tid == 0) xscale[t] = 0.f;
         return;
     }
@@ -259,10 +331,16 @@ __global__ __launch_bounds__(256) void prep_x_kernel(const float *__restrict__ x
         down *= 0.5f;
         undo *= 2.f;
     }
-    for (uint32_t k = tid; k < kpad; k += 256) {
-        float v = 0.f;
-        if (k < K) v = value(k) * down;
-        o[k] = (_Float16)v;
+    for (uint32_t k8 = tid; k8 < kpad / 8; k8 += 256) {
+        _Float16 h[8];
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const uint32_t k = 8 * k8 + b;
+            h[b] = (_Float16)(k < K ? value(k) * down : 0.f);
+        }
+        uint4 w;
+        __builtin_memcpy(&w, h, 16);
+        word(k8) = w;
     }
     if (tid == 0) xscale[t] = undo;
 }
@@ -425,21 +503,10 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const AttnRowsArgs a) {
 }
 
 template <class F>
-int launch_gemm_fmt(wgml_ctx *ctx, GemmArgs &a) {
-    const uint32_t tb = a.tpad / 16;  // token blocks: 1, 2, 4 or 8
-    // token blocks per wave: as many as keep about one workgroup per CU busy
-    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
-    uint32_t nt = tb;
-    while (nt > 1 && tb / nt < 4 && (a.nrows + 16 * (4 / (tb / nt)) - 1) / (16 * (4 / (tb / nt))) < cu)
-        nt >>= 1;
-    a.tg = tb / nt;
-    if (a.tg > 4) {  // at most four token groups fit a workgroup: more blocks per wave
-        a.tg = 4;
-        nt = tb / 4;
-    }
-    const uint32_t rows_per_wg = 16 * (4 / a.tg);
-    const dim3 grid((a.nrows + rows_per_wg - 1) / rows_per_wg), block(256);
-    const size_t lds = (size_t)16 * (a.tpad + 1) * 8;
+int launch_gemm_fmt(wgml_ctx *ctx, const GemmArgs &a) {
+    const uint32_t nt = a.tpad / 16;  // token blocks: 1, 2, 4 or 8
+    const dim3 grid((a.nrows + 15) / 16), block(KWAVES * 64);
+    const size_t lds = (size_t)KWAVES * nt * 64 * sizeof(float4);
     switch (nt) {
     case 8: gemm_quant_f16_kernel<F, 8><<<grid, block, lds, ctx->stream>>>(a); break;
     case 4: gemm_quant_f16_kernel<F, 4><<<grid, block, lds, ctx->stream>>>(a); break;
@@ -475,7 +542,7 @@ int launch_prefill_prep(wgml_ctx *ctx, const float *x, uint32_t x_stride, const 
                         const float *norm_w, float eps, void *xh, float *xscale, uint32_t K,
                         uint32_t T) {
     prep_x_kernel<<<dim3(prefill_tpad(T)), dim3(256), 0, ctx->stream>>>(
-        x, x_stride, up, norm_w, eps, reinterpret_cast<_Float16 *>(xh), xscale, K, prefill_kpad(K), T);
+        x, x_stride, up, norm_w, eps, reinterpret_cast<uint4 *>(xh), xscale, K, prefill_kpad(K), T);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
@@ -491,7 +558,7 @@ int launch_gemm_quant(wgml_ctx *ctx, float *out, uint32_t out_stride, const wgml
     a.p1 = m->p1;
     a.p2 = m->p2;
     a.p3 = m->p3;
-    a.xh = reinterpret_cast<const _Float16 *>(xh);
+    a.xh = reinterpret_cast<const uint4 *>(xh);
     a.xscale = xscale;
     a.out = out;
     a.bias = bias;
