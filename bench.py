@@ -226,6 +226,9 @@ def main():
                     help="only the dominant-kernel measurement (for profiler runs): the fused "
                          "gate/up launches, then three plain copies of 256 MiB (op_assign Copy) "
                          "as the known-size kernel that calibrates the HBM byte counters")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="only the batched prompt pass over a --warmup-token prompt, 1 untimed + "
+                         "3 timed calls (for profiler runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every kernel uses a single device; "
@@ -272,6 +275,18 @@ def main():
         return
     model = Llama2(gpu, cfg).load(weights)
     prompt = W.prompt_tokens(4, args.warmup, cfg.vocab_size)
+    if args.prefill_only:
+        model.prefill(prompt)
+        gpu.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(3):
+            model.prefill(prompt)
+        gpu.synchronize()
+        pdt = (time.perf_counter() - t0) / 3
+        print(json.dumps({"prefill_tokens": args.warmup, "ms": round(pdt * 1e3, 3),
+                          "tok_s": round(args.warmup / pdt, 1),
+                          "launches": model.launches_per_token()}), flush=True)
+        return
 
     # warm-up: the prompt, one token at a time (the reference has no batched prefill)
     out = model.generate_greedy(prompt, args.warmup)
@@ -298,12 +313,13 @@ def main():
     dt = time.perf_counter() - t0
     tok_s = args.steps / dt
     assert np.array_equal(toks[:n_sync], toks_sync), "recorded and synchronous loops disagree"
+    launches_per_token = model.launches_per_token()
     wbytes = weights.weight_bytes_per_token()
     kv_bytes_mid = 2 * cfg.n_layers * cfg.kv_dim * 4 * (args.warmup + args.steps // 2)
     roof_tok_s = HBM_PEAK_GBS * 1e9 / wbytes
     log(f"decode: {args.steps} steps in {dt * 1e3:.1f} ms -> {tok_s:.1f} tok/s "
         f"({100 * tok_s / roof_tok_s:.1f}% of the weight-bytes roofline {roof_tok_s:.0f} tok/s); "
-        f"{model.launches_per_token()} launches/token; with a host read-back per token: "
+        f"{launches_per_token} launches/token; with a host read-back per token: "
         f"{tok_s_sync:.1f} tok/s")
 
     # the batched prompt pass over the same prompt (f16 MFMA products, 128 tokens per run);
@@ -384,7 +400,7 @@ def main():
                    "weight_bytes_per_token": wbytes, "kv_bytes_per_token_mid_run": kv_bytes_mid,
                    "roofline_tok_s_at_8TBs": round(roof_tok_s, 1),
                    "frac_of_weight_roofline": round(tok_s / roof_tok_s, 4),
-                   "launches_per_token": model.launches_per_token(),
+                   "launches_per_token": launches_per_token,
                    "tok_s_with_per_token_host_sync": round(tok_s_sync, 2),
                    "last_token": int(toks[-1])},
         "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "gemv_sweep": sweep,

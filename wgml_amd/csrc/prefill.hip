@@ -10,7 +10,7 @@
 // Weights are expanded to f16 in registers with the reference's dequantization
 // arithmetic (fp32, then rounded to f16), activations are f16 (scaled per token by a
 // power of two so that they stay in range), products accumulate in fp32 on
-// v_mfma_f32_16x16x16_f16.  With f16 inputs the results differ from the fp32 path
+// v_mfma_f32_16x16x32_f16.  With f16 inputs the results differ from the fp32 path
 // by about 3e-4 of a row's RMS (the tests bound it at 1e-3).
 //
 // Tiling.  A workgroup owns 16 matrix rows and all tokens; its 8 waves split K: wave w
@@ -25,8 +25,8 @@
 // prep_x_kernel): for chunk c, token block n, half s2 of the chunk, lane (g, j) finds
 // the 8 halves  X[16 n + j][64 c + 32 s2 + 8 g .. + 7]  as one 16-byte word at
 // word index ((c * NT + n) * 2 + s2) * 64 + 16 g + j: a wave's load is 1 KiB contiguous.
-// The first four halves are the B operand of MFMA step 2 s2, the last four of step
-// 2 s2 + 1; the A operand follows the same assignment of k to (step, lane, slot).
+// That word is the B operand of one 16x16x32 MFMA (lane (g, j) supplies k = 8 g .. 8 g + 7
+// of the 32 for token j); the A operand follows the same assignment of k to lanes.
 #include <hip/hip_fp16.h>
 
 #include "common.h"
@@ -37,6 +37,7 @@ using namespace wgml;
 namespace {
 
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t KC = 64;    // elements of K per chunk
@@ -185,102 +186,126 @@ struct GemmQ8_0 {
     }
 };
 
-template <class F, int NT>
+template <class F, int NT, int RB>
 __global__ __launch_bounds__(KWAVES * 64) void gemm_quant_f16_kernel(const GemmArgs a) {
     extern __shared__ float4 red[];  // [KWAVES][NT][64]
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t j = lane & 15, g = lane >> 4;
-    const uint32_t row0 = blockIdx.x * 16;
-    const uint32_t row = min(row0 + j, a.nrows - 1);  // this lane's row of the A operand
+    const uint32_t row0 = blockIdx.x * (16 * RB);
+    uint32_t row[RB];  // this lane's rows of the A operands
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) row[rb] = min(row0 + 16 * rb + j, a.nrows - 1);
     const uint32_t nchunks = a.kpad / KC;
     // chunks of this wave: wave, wave + 8, ...
     const uint32_t n_my = nchunks > wave ? (nchunks - wave + KWAVES - 1) / KWAVES : 0;
 
-    floatx4 acc[NT];
+    floatx4 acc[RB][NT];
 #pragma unroll
-    for (int n = 0; n < NT; ++n) acc[n] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+        for (int n = 0; n < NT; ++n) acc[rb][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
 
-    typename F::Raw ra, rb;
-    uint4 ba[NT][2], bb[NT][2];
-    // every load is unconditional (a chunk number past the end re-reads the last chunk and
+    // Every load is unconditional (a chunk number past the end re-reads the last chunk and
     // is never multiplied): the compiler can then count outstanding loads exactly instead
-    // of draining them all before each use
-    auto load = [&](typename F::Raw &r, uint4(&b)[NT][2], uint32_t i) {
-        const uint32_t c = min(wave + KWAVES * i, nchunks - 1);
-        F::load(r, a, row, c, g);
+    // of draining them all before each use.  The weight bytes of the next chunk are
+    // requested when a chunk's arithmetic starts; each activation word of the next chunk
+    // is requested into the register of the one it replaces right after that one's last use.
+    typename F::Raw ra[RB], rb_[RB];
+    uint4 b[NT][2];
+    auto chunk_of = [&](uint32_t i) { return min(wave + KWAVES * i, nchunks - 1); };
+    auto load_a = [&](typename F::Raw(&r)[RB], uint32_t i) {
+        const uint32_t c = chunk_of(i);
 #pragma unroll
-        for (int n = 0; n < NT; ++n) {
-#pragma unroll
-            for (int s2 = 0; s2 < 2; ++s2) b[n][s2] = a.xh[(((size_t)c * NT + n) * 2 + s2) * 64 + lane];
-        }
+        for (int rb = 0; rb < RB; ++rb) F::load(r[rb], a, row[rb], c, g);
     };
-    auto compute = [&](const typename F::Raw &r, const uint4(&b)[NT][2], uint32_t i) {
+    auto compute = [&](const typename F::Raw(&r)[RB], uint32_t i) {
         const uint32_t c = wave + KWAVES * i;
-        half4 a4[4];
-        F::frag(r, a, c, g, a4);
+        const uint4 *next = a.xh + (size_t)chunk_of(i + 1) * NT * 128 + lane;
+        half4 a4[RB][4];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) F::frag(r[rb], a, c, g, a4[rb]);
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
 #pragma unroll
             for (int n = 0; n < NT; ++n) {
-                const uint2 lo = make_uint2(b[n][s2].x, b[n][s2].y), hi = make_uint2(b[n][s2].z, b[n][s2].w);
-                half4 b0, b1;
-                __builtin_memcpy(&b0, &lo, 8);
-                __builtin_memcpy(&b1, &hi, 8);
-                acc[n] = __builtin_amdgcn_mfma_f32_16x16x16f16(a4[2 * s2], b0, acc[n], 0, 0, 0);
-                acc[n] = __builtin_amdgcn_mfma_f32_16x16x16f16(a4[2 * s2 + 1], b1, acc[n], 0, 0, 0);
+                half8 bw;
+                __builtin_memcpy(&bw, &b[n][s2], 16);
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) {
+                    half8 aw;
+                    __builtin_memcpy(&aw, &a4[rb][2 * s2], 16);  // a4[2 s2], a4[2 s2 + 1]: 8 consecutive k
+                    acc[rb][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw, bw, acc[rb][n], 0, 0, 0);
+                }
+                b[n][s2] = next[(n * 2 + s2) * 64];
             }
         }
     };
     if (n_my > 0) {
-        load(ra, ba, 0);
+        load_a(ra, 0);
+        {
+            const uint4 *first = a.xh + (size_t)chunk_of(0) * NT * 128 + lane;
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+#pragma unroll
+                for (int n = 0; n < NT; ++n) b[n][s2] = first[(n * 2 + s2) * 64];
+            }
+        }
         for (uint32_t i = 0; i < n_my; i += 2) {
-            load(rb, bb, i + 1);
-            compute(ra, ba, i);
-            load(ra, ba, i + 2);
-            if (i + 1 < n_my) compute(rb, bb, i + 1);
+            load_a(rb_, i + 1);
+            compute(ra, i);
+            if (i + 1 < n_my) {
+                load_a(ra, i + 2);
+                compute(rb_, i + 1);
+            }
         }
     }
-    // the partial sums of the 8 waves, added in wave order
+    // the partial sums of the 8 waves, added in wave order, one row block at a time
 #pragma unroll
-    for (int n = 0; n < NT; ++n)
-        red[(wave * NT + n) * 64 + lane] = make_float4(acc[n][0], acc[n][1], acc[n][2], acc[n][3]);
-    __syncthreads();
-    for (uint32_t idx = tid; idx < NT * 64; idx += KWAVES * 64) {
-        const uint32_t n = idx >> 6, l = idx & 63;
-        float4 v = red[n * 64 + l];
+    for (int rb = 0; rb < RB; ++rb) {
+        if (rb > 0) __syncthreads();
 #pragma unroll
-        for (uint32_t w = 1; w < KWAVES; ++w) {
-            const float4 p = red[(w * NT + n) * 64 + l];
-            v = make_float4(v.x + p.x, v.y + p.y, v.z + p.z, v.w + p.w);
-        }
-        // v = out[token 16 n + (l & 15)][row0 + 4 (l >> 4) .. + 3]
-        const uint32_t tok = n * 16 + (l & 15), r4 = row0 + 4 * (l >> 4);
-        if (tok >= a.T || r4 >= a.nrows) continue;
-        const float xs_t = a.xscale ? a.xscale[tok] : 1.f;
-        v = make_float4(v.x * xs_t, v.y * xs_t, v.z * xs_t, v.w * xs_t);
-        float *o = a.out + (size_t)tok * a.out_stride + r4;
-        if (r4 + 3 < a.nrows && (reinterpret_cast<uintptr_t>(o) & 15u) == 0) {
-            if (a.bias) {
-                v.x += a.bias[r4];
-                v.y += a.bias[r4 + 1];
-                v.z += a.bias[r4 + 2];
-                v.w += a.bias[r4 + 3];
+        for (int n = 0; n < NT; ++n)
+            red[(wave * NT + n) * 64 + lane] =
+                make_float4(acc[rb][n][0], acc[rb][n][1], acc[rb][n][2], acc[rb][n][3]);
+        __syncthreads();
+        for (uint32_t idx = tid; idx < NT * 64; idx += KWAVES * 64) {
+            const uint32_t n = idx >> 6, l = idx & 63;
+            float4 v = red[n * 64 + l];
+#pragma unroll
+            for (uint32_t w = 1; w < KWAVES; ++w) {
+                const float4 p = red[(w * NT + n) * 64 + l];
+                v = make_float4(v.x + p.x, v.y + p.y, v.z + p.z, v.w + p.w);
             }
-            if (a.accumulate) {
-                const float4 p = *reinterpret_cast<const float4 *>(o);
-                v = make_float4(p.x + v.x, p.y + v.y, p.z + v.z, p.w + v.w);
+            // v = out[token 16 n + (l & 15)][first row of the block + 4 (l >> 4) .. + 3]
+            const uint32_t tok = n * 16 + (l & 15), r4 = row0 + 16 * rb + 4 * (l >> 4);
+            if (tok >= a.T || r4 >= a.nrows) continue;
+            const float xs_t = a.xscale ? a.xscale[tok] : 1.f;
+            v = make_float4(v.x * xs_t, v.y * xs_t, v.z * xs_t, v.w * xs_t);
+            float *o = a.out + (size_t)tok * a.out_stride + r4;
+            if (r4 + 3 < a.nrows && (reinterpret_cast<uintptr_t>(o) & 15u) == 0) {
+                if (a.bias) {
+                    v.x += a.bias[r4];
+                    v.y += a.bias[r4 + 1];
+                    v.z += a.bias[r4 + 2];
+                    v.w += a.bias[r4 + 3];
+                }
+                if (a.accumulate) {
+                    const float4 p = *reinterpret_cast<const float4 *>(o);
+                    v = make_float4(p.x + v.x, p.y + v.y, p.z + v.z, p.w + v.w);
+                }
+                *reinterpret_cast<float4 *>(o) = v;
+                continue;
             }
-            *reinterpret_cast<float4 *>(o) = v;
-            continue;
-        }
-        const float vv[4] = {v.x, v.y, v.z, v.w};
+            const float vv[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if (r4 + i < a.nrows) {
-                float e = vv[i];
-                if (a.bias) e += a.bias[r4 + i];
-                o[i] = a.accumulate ? o[i] + e : e;
+            for (int i = 0; i < 4; ++i) {
+                if (r4 + i < a.nrows) {
+                    float e = vv[i];
+                    if (a.bias) e += a.bias[r4 + i];
+                    o[i] = a.accumulate ? o[i] + e : e;
+                }
             }
         }
     }
@@ -292,7 +317,9 @@ __global__ __launch_bounds__(KWAVES * 64) void gemm_quant_f16_kernel(const GemmA
 // |x| <= 1024; the factor to undo it goes to xscale[t].  Tokens from T on and columns
 // from K on are zero.  With `up` non-null the input is the gated activation
 // up[k] * silu(x[k]) (ops/silu.wgsl:13-27) instead of x itself (no normalisation then).
-__global__ __launch_bounds__(256) void prep_x_kernel(const float *__restrict__ x, uint32_t x_stride,
+constexpr int PREP_THREADS = 1024;
+constexpr int PREP_GROUPS = 2;  // groups of 8 columns a thread keeps in registers
+__global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(const float *__restrict__ x, uint32_t x_stride,
                                                      const float *__restrict__ up,
                                                      const float *__restrict__ norm_w, float eps,
                                                      uint4 *__restrict__ xh,
@@ -305,42 +332,87 @@ __global__ __launch_bounds__(256) void prep_x_kernel(const float *__restrict__ x
         const uint32_t c = k8 >> 3, s2 = (k8 >> 2) & 1, g = k8 & 3;
         return xh[(((size_t)c * nt + (t >> 4)) * 2 + s2) * 64 + 16 * g + (t & 15)];
     };
+    const uint32_t ngroups = kpad / 8;
     if (t >= T) {
-        for (uint32_t k8 = tid; k8 < kpad / 8; k8 += 256) word(k8) = make_uint4(0, 0, 0, 0);
+        for (uint32_t k8 = tid; k8 < ngroups; k8 += PREP_THREADS) word(k8) = make_uint4(0, 0, 0, 0);
         if (tid == 0) xscale[t] = 0.f;
         return;
     }
     const float *xr = x + (size_t)t * x_stride;
     const float *ur = up ? up + (size_t)t * x_stride : nullptr;
+    // Rows of up to 8 * PREP_GROUPS * PREP_THREADS columns are read once and kept in
+    // registers (v); longer rows are re-read from memory by the later passes.
+    const bool cached = ngroups <= PREP_GROUPS * PREP_THREADS;
+    float v[PREP_GROUPS][8];
+    auto raw = [&](uint32_t k) -> float {  // the value before normalisation
+        if (k >= K) return 0.f;
+        const float xv = xr[k];
+        return ur ? ur[k] * (xv / (1.0f + expf(-xv))) : xv;
+    };
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < PREP_GROUPS; ++i) {
+            const uint32_t k0 = 8 * (tid + i * PREP_THREADS);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[i][e] = k0 + e < kpad ? raw(k0 + e) : 0.f;
+        }
+    }
     float rs = 1.f;
     if (norm_w) {
         float ss = 0.f;
-        for (uint32_t k = tid; k < K; k += 256) ss = fmaf(xr[k], xr[k], ss);
+        if (cached) {
+#pragma unroll
+            for (int i = 0; i < PREP_GROUPS; ++i) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss = fmaf(v[i][e], v[i][e], ss);
+            }
+        } else {
+            for (uint32_t k = tid; k < K; k += PREP_THREADS) ss = fmaf(xr[k], xr[k], ss);
+        }
         rs = 1.0f / sqrtf(block_sum(ss, red) / (float)K + eps);
     }
-    auto value = [&](uint32_t k) {
-        const float xv = xr[k];
-        if (ur) return ur[k] * (xv / (1.0f + expf(-xv)));
-        return norm_w ? (xv * rs) * norm_w[k] : xv;
-    };
+    auto value = [&](uint32_t k, float r) { return norm_w && k < K ? (r * rs) * norm_w[k] : r; };
     float amax = 0.f;
-    for (uint32_t k = tid; k < K; k += 256) amax = fmaxf(amax, fabsf(value(k)));
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < PREP_GROUPS; ++i) {
+            const uint32_t k0 = 8 * (tid + i * PREP_THREADS);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                v[i][e] = value(k0 + e, v[i][e]);
+                amax = fmaxf(amax, fabsf(v[i][e]));
+            }
+        }
+    } else {
+        for (uint32_t k = tid; k < K; k += PREP_THREADS) amax = fmaxf(amax, fabsf(value(k, raw(k))));
+    }
     amax = block_max(amax, red);
     float down = 1.f, undo = 1.f;
     for (int it = 0; it < 120 && amax * down > 1024.f; ++it) {  // uniform over the workgroup
         down *= 0.5f;
         undo *= 2.f;
     }
-    for (uint32_t k8 = tid; k8 < kpad / 8; k8 += 256) {
+    auto store = [&](uint32_t k8, const float(&f)[8]) {
         _Float16 h[8];
 #pragma unroll
-        for (int b = 0; b < 8; ++b) {
-            const uint32_t k = 8 * k8 + b;
-            h[b] = (_Float16)(k < K ? value(k) * down : 0.f);
-        }
+        for (int e = 0; e < 8; ++e) h[e] = (_Float16)(f[e] * down);
         uint4 w;
         __builtin_memcpy(&w, h, 16);
         word(k8) = w;
+    };
+    if (cached) {
+#pragma unroll
+        for (int i = 0; i < PREP_GROUPS; ++i) {
+            const uint32_t k8 = tid + i * PREP_THREADS;
+            if (k8 < ngroups) store(k8, v[i]);
+        }
+    } else {
+        for (uint32_t k8 = tid; k8 < ngroups; k8 += PREP_THREADS) {
+            float f[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] = value(8 * k8 + e, raw(8 * k8 + e));
+            store(k8, f);
+        }
     }
     if (tid == 0) xscale[t] = undo;
 }
@@ -502,20 +574,32 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const AttnRowsArgs a) {
     }
 }
 
-template <class F>
-int launch_gemm_fmt(wgml_ctx *ctx, const GemmArgs &a) {
+int g_force_row_blocks = 0;  // 0: by matrix height; 1 or 2: forced (tests)
+
+template <class F, int RB>
+int launch_gemm_rb(wgml_ctx *ctx, const GemmArgs &a) {
     const uint32_t nt = a.tpad / 16;  // token blocks: 1, 2, 4 or 8
-    const dim3 grid((a.nrows + 15) / 16), block(KWAVES * 64);
+    const dim3 grid((a.nrows + 16 * RB - 1) / (16 * RB)), block(KWAVES * 64);
     const size_t lds = (size_t)KWAVES * nt * 64 * sizeof(float4);
     switch (nt) {
-    case 8: gemm_quant_f16_kernel<F, 8><<<grid, block, lds, ctx->stream>>>(a); break;
-    case 4: gemm_quant_f16_kernel<F, 4><<<grid, block, lds, ctx->stream>>>(a); break;
-    case 2: gemm_quant_f16_kernel<F, 2><<<grid, block, lds, ctx->stream>>>(a); break;
-    default: gemm_quant_f16_kernel<F, 1><<<grid, block, lds, ctx->stream>>>(a); break;
+    case 8: gemm_quant_f16_kernel<F, 8, RB><<<grid, block, lds, ctx->stream>>>(a); break;
+    case 4: gemm_quant_f16_kernel<F, 4, RB><<<grid, block, lds, ctx->stream>>>(a); break;
+    case 2: gemm_quant_f16_kernel<F, 2, RB><<<grid, block, lds, ctx->stream>>>(a); break;
+    default: gemm_quant_f16_kernel<F, 1, RB><<<grid, block, lds, ctx->stream>>>(a); break;
     }
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
+}
+
+// Two row blocks per wave halve the activation traffic per product (each activation word
+// serves 32 rows) at the price of half as many workgroups: worth it once those still
+// cover half of the compute units.
+template <class F>
+int launch_gemm_fmt(wgml_ctx *ctx, const GemmArgs &a) {
+    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
+    const bool two = g_force_row_blocks ? g_force_row_blocks == 2 : a.nrows / 32 >= cu / 2;
+    return two ? launch_gemm_rb<F, 2>(ctx, a) : launch_gemm_rb<F, 1>(ctx, a);
 }
 
 }  // namespace
@@ -541,7 +625,7 @@ int ensure_prefill_scratch(wgml_ctx *ctx, size_t xh_bytes) {
 int launch_prefill_prep(wgml_ctx *ctx, const float *x, uint32_t x_stride, const float *up,
                         const float *norm_w, float eps, void *xh, float *xscale, uint32_t K,
                         uint32_t T) {
-    prep_x_kernel<<<dim3(prefill_tpad(T)), dim3(256), 0, ctx->stream>>>(
+    prep_x_kernel<<<dim3(prefill_tpad(T)), dim3(PREP_THREADS), 0, ctx->stream>>>(
         x, x_stride, up, norm_w, eps, reinterpret_cast<uint4 *>(xh), xscale, K, prefill_kpad(K), T);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
@@ -623,6 +707,12 @@ int launch_attention_rows(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pos
 }  // namespace wgml
 
 extern "C" {
+
+// Test hook: 0 = choose rows per workgroup by matrix height, 1 = 16 rows, 2 = 32 rows.
+WGML_API int wgml_debug_set_gemm_row_blocks(int n) {
+    g_force_row_blocks = n == 1 || n == 2 ? n : 0;
+    return WGML_OK;
+}
 
 // out[t] = M x[t] for T <= 128 vectors at once (x: T x ncols, out: T x nrows, both
 // row-major f32) on the matrix cores; the batched counterpart of wgml_gemv_quant.
