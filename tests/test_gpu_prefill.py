@@ -20,12 +20,13 @@ pytestmark = pytest.mark.gpu
 QT = [W.Q8_0, W.Q4_K, W.Q6_K]
 
 
-@pytest.fixture(params=[0, 1, 2], ids=["rows_auto", "rows16", "rows32"])
+@pytest.fixture(params=[0, 1, 2, 3, 8], ids=["ksplit_auto", "ksplit1", "ksplit2", "ksplit3", "ksplit8"])
 def row_blocks(request):
-    # rows of the matrix per workgroup of the product kernel: chosen by matrix height, or forced
-    W._lib.lib.wgml_debug_set_gemm_row_blocks(request.param)
+    # workgroups that share the K range of a product (their partial sums are added by a
+    # second kernel): chosen by matrix shape, or forced
+    W._lib.lib.wgml_debug_set_gemm_k_split(request.param)
     yield request.param
-    W._lib.lib.wgml_debug_set_gemm_row_blocks(0)
+    W._lib.lib.wgml_debug_set_gemm_k_split(0)
 
 
 def gemm(gpu, qtype, raw, nrows, ncols, x):

@@ -186,7 +186,7 @@ PROTOTYPES = {
     "wgml_debug_set_gemv_rows_per_wave": (_i, [_i]),
     "wgml_debug_set_gemv_config": (_i, [_i, _i, _i, _i]),
     "wgml_debug_set_gemv_f32_activations": (_i, [_i]),
-    "wgml_debug_set_gemm_row_blocks": (_i, [_i]),
+    "wgml_debug_set_gemm_k_split": (_i, [_i]),
 }
 
 # calls whose return value is not a status code

@@ -60,6 +60,9 @@ struct wgml_ctx {
     void *prefill_xh = nullptr;
     size_t prefill_xh_bytes = 0;
     float *prefill_xscale = nullptr;
+    // partial sums of batched products whose K range is split between workgroups
+    float *gemm_part = nullptr;
+    size_t gemm_part_bytes = 0;
     uint64_t launches = 0;  // kernels enqueued so far (diagnostics)
     // Buffers, matrices and models keep their context alive: the device objects
     // are torn down when the last reference goes, whatever order handles are
@@ -216,6 +219,16 @@ int launch_attention_rows(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pos
 int launch_gemm_quant(wgml_ctx *ctx, float *out, uint32_t out_stride, const wgml_qmat *m,
                       const void *xh, const float *xscale, uint32_t T, const float *bias,
                       int accumulate);
+// The same for up to three matrices of one format and width that multiply the same
+// activations, in one launch.
+struct GemmTarget {
+    const wgml_qmat *m;
+    float *out;
+    uint32_t out_stride;
+    const float *bias;
+};
+int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, const void *xh,
+                            const float *xscale, uint32_t T, int accumulate);
 int launch_embed_rows(wgml_ctx *ctx, float *x, const float *table, const uint32_t *d_tokens,
                       uint32_t dim, uint32_t T);
 int launch_rope_rows(wgml_ctx *ctx, int variant, uint32_t head_size, uint32_t kv_dim, uint32_t pos0,

@@ -377,9 +377,26 @@ int enqueue_prefill_run(wgml_llama2 *m, const uint32_t *tokens, uint32_t T, uint
         float *kc = w.key_cache + (size_t)pos0 * kv_dim, *vc = w.value_cache + (size_t)pos0 * kv_dim;
         WGML_TRY(launch_prefill_prep(ctx, m->pf_x, dim, nullptr, w.attn_norm, c.rms_norm_eps, xh, xs,
                                      dim, T));
-        WGML_TRY(launch_gemm_quant(ctx, m->pf_q, dim, w.attn_q, xh, xs, T, w.bq, 0));
-        WGML_TRY(launch_gemm_quant(ctx, kc, kv_dim, w.attn_k, xh, xs, T, w.bk, 0));
-        WGML_TRY(launch_gemm_quant(ctx, vc, kv_dim, w.attn_v, xh, xs, T, w.bv, 0));
+        // Q, K and V in as few launches as their formats allow (one launch takes matrices
+        // of one format); K and V go straight to their cache rows
+        {
+            const GemmTarget tq{w.attn_q, m->pf_q, dim, w.bq}, tk{w.attn_k, kc, kv_dim, w.bk},
+                tv{w.attn_v, vc, kv_dim, w.bv};
+            GemmTarget group[3] = {tq, tk, tv};
+            bool done[3] = {false, false, false};
+            for (int i = 0; i < 3; ++i) {
+                if (done[i]) continue;
+                GemmTarget launch[3];
+                int n = 0;
+                for (int k = i; k < 3; ++k) {
+                    if (!done[k] && group[k].m->type == group[i].m->type) {
+                        launch[n++] = group[k];
+                        done[k] = true;
+                    }
+                }
+                WGML_TRY(launch_gemm_quant_multi(ctx, launch, n, xh, xs, T, 0));
+            }
+        }
         WGML_TRY(launch_rope_rows(ctx, variant, m->head_size, kv_dim, pos0, c.rope_base_freq,
                                   m->pf_q, dim, dim, kc, kv_dim, T));
         WGML_TRY(launch_attention_rows(ctx, ap, pos0, T, m->pf_q, dim, w.key_cache, w.value_cache,
@@ -388,8 +405,14 @@ int enqueue_prefill_run(wgml_llama2 *m, const uint32_t *tokens, uint32_t T, uint
         WGML_TRY(launch_gemm_quant(ctx, m->pf_x, dim, w.attn_output, xh, xs, T, nullptr, 1));
         WGML_TRY(launch_prefill_prep(ctx, m->pf_x, dim, nullptr, w.ffn_norm, c.rms_norm_eps, xh, xs,
                                      dim, T));
-        WGML_TRY(launch_gemm_quant(ctx, m->pf_hb, hidden, w.ffn_gate, xh, xs, T, nullptr, 0));
-        WGML_TRY(launch_gemm_quant(ctx, m->pf_hb2, hidden, w.ffn_up, xh, xs, T, nullptr, 0));
+        if (w.ffn_gate->type == w.ffn_up->type) {
+            const GemmTarget gu[2] = {{w.ffn_gate, m->pf_hb, hidden, nullptr},
+                                      {w.ffn_up, m->pf_hb2, hidden, nullptr}};
+            WGML_TRY(launch_gemm_quant_multi(ctx, gu, 2, xh, xs, T, 0));
+        } else {
+            WGML_TRY(launch_gemm_quant(ctx, m->pf_hb, hidden, w.ffn_gate, xh, xs, T, nullptr, 0));
+            WGML_TRY(launch_gemm_quant(ctx, m->pf_hb2, hidden, w.ffn_up, xh, xs, T, nullptr, 0));
+        }
         WGML_TRY(launch_prefill_prep(ctx, m->pf_hb, hidden, m->pf_hb2, nullptr, 0.f, xh, xs, hidden,
                                      T));
         WGML_TRY(launch_gemm_quant(ctx, m->pf_x, dim, w.ffn_down, xh, xs, T, nullptr, 1));

@@ -13,18 +13,25 @@
 // v_mfma_f32_16x16x32_f16.  With f16 inputs the results differ from the fp32 path
 // by about 3e-4 of a row's RMS (the tests bound it at 1e-3).
 //
-// Tiling.  A workgroup owns 16 matrix rows and all tokens; its 8 waves split K: wave w
-// takes the 64-element chunks w, w + 8, ...  so that every weight element is expanded
-// exactly once, by one wave, and used for all NT blocks of 16 tokens (NT accumulators
-// of 16x16 per wave).  The 8 partial sums meet in LDS at the end, added in a fixed order.
-// Nothing is shared between the waves before that, so the loop has no barrier: each wave
-// keeps the loads of its next chunk (weights and activations) in flight while it
-// multiplies the current one.
+// Tiling.  A workgroup (8 waves) owns 64 rows of one matrix -- four blocks of 16 -- and
+// a contiguous range of K, walked in iterations of two 64-element chunks.  Per iteration
+// the workgroup stages both chunks of the activations (all tokens) in LDS; waves 0-3
+// multiply the first chunk with their row block's weights, waves 4-7 the second, so an
+// activation word fetched from L2 serves 64 rows and every weight element is expanded
+// exactly once, by one wave, for all NT blocks of 16 tokens (NT accumulators of 16x16 per
+// wave).  Two LDS buffers: the next pair of chunks is on its way from memory while the
+// current one is multiplied, one barrier per iteration.  At the end waves 4-7 hand
+// their sums to waves 0-3 through LDS.
+//
+// One launch can cover up to three matrices that multiply the same activations (Q, K
+// and V; gate and up): their row tiles are laid side by side in grid.x.  A matrix too
+// short to give every compute unit a tile has its K range split between grid.y
+// workgroups; they leave partial sums that gemm_reduce_kernel adds in a fixed order.
 //
 // Activations are stored in the order the B operand wants them (written by
 // prep_x_kernel): for chunk c, token block n, half s2 of the chunk, lane (g, j) finds
 // the 8 halves  X[16 n + j][64 c + 32 s2 + 8 g .. + 7]  as one 16-byte word at
-// word index ((c * NT + n) * 2 + s2) * 64 + 16 g + j: a wave's load is 1 KiB contiguous.
+// word index ((c * NT + n) * 2 + s2) * 64 + 16 g + j: a chunk is NT KiB contiguous.
 // That word is the B operand of one 16x16x32 MFMA (lane (g, j) supplies k = 8 g .. 8 g + 7
 // of the 32 for token j); the A operand follows the same assignment of k to lanes.
 #include <hip/hip_fp16.h>
@@ -39,18 +46,28 @@ namespace {
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // plain vector: arrays of it stay in registers
 
 constexpr uint32_t KC = 64;    // elements of K per chunk
 constexpr uint32_t KWAVES = 8;  // waves of a workgroup = ways K is split
 
-struct GemmArgs {
+struct GemmMat {
     const uint8_t *p0, *p1, *p2, *p3;  // matrix planes (as wgml_qmat)
-    const uint4 *xh;                   // packed f16 activations (see above)
-    const float *xscale;               // [tpad] factor to multiply a token's results with
     float *out;                        // [T][out_stride]
     const float *bias;                 // optional, per row
-    uint32_t nrows, ncols, kpad, T, tpad, out_stride;
+    uint32_t nrows, out_stride;
+    uint32_t tile0;                    // first 64-row tile of this matrix in grid.x
+};
+
+struct GemmArgs {
+    GemmMat m[3];
+    uint32_t nmat;
+    const u32x4 *xh;                   // packed f16 activations (see above)
+    const float *xscale;               // [tpad] factor to multiply a token's results with
+    uint32_t ncols, kpad, T, tpad;
     int accumulate;                    // out += result
+    float *part;                       // [ks][T][nrows] partial sums (ks > 1, one matrix)
+    uint32_t ks;                       // ways K is split between workgroups (grid.y)
 };
 
 __device__ __forceinline__ half4 to_half4(float a, float b, float c, float d) {
@@ -72,13 +89,13 @@ struct GemmQ4K {
         uint4 hdr;  // d, dmin, 12 bytes of packed scales
         uint2 qs;   // bytes 8 g .. 8 g + 7 of the chunk's 32: low nibbles s2 = 0, high s2 = 1
     };
-    __device__ static void load(Raw &r, const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g) {
-        const uint8_t *blk = a.p0 + ((size_t)row * (a.ncols / 256) + (chunk >> 2)) * 144;
+    __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, uint32_t row, uint32_t chunk,
+                                uint32_t g) {
+        const uint8_t *blk = m.p0 + ((size_t)row * (ncols / 256) + (chunk >> 2)) * 144;
         r.hdr = *reinterpret_cast<const uint4 *>(blk);
         r.qs = *reinterpret_cast<const uint2 *>(blk + 16 + (chunk & 3) * 32 + 8 * g);
     }
-    __device__ static void frag(const Raw &r, const GemmArgs &, uint32_t chunk, uint32_t,
-                                half4 (&a4)[4]) {
+    __device__ static void frag(const Raw &r, uint32_t, uint32_t chunk, uint32_t, half4 (&a4)[4]) {
         const uint4 hdr = r.hdr;
         const uint32_t j = chunk & 3;
         const float d = f16_bits_to_f32((uint16_t)(hdr.x & 0xffffu));
@@ -119,18 +136,18 @@ struct GemmQ6K {
         uint32_t scw;  // the four scales of this 64-element chunk
         uint32_t d;
     };
-    __device__ static void load(Raw &r, const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g) {
-        const size_t blk = (size_t)row * (a.ncols / 256) + (chunk >> 2);
+    __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, uint32_t row, uint32_t chunk,
+                                uint32_t g) {
+        const size_t blk = (size_t)row * (ncols / 256) + (chunk >> 2);
         const uint32_t c = chunk & 3, i = c >> 1;
-        const uint8_t *ql = a.p0 + blk * 128 + 64 * i + 8 * g;
+        const uint8_t *ql = m.p0 + blk * 128 + 64 * i + 8 * g;
         r.ql[0] = *reinterpret_cast<const uint2 *>(ql);
         r.ql[1] = *reinterpret_cast<const uint2 *>(ql + 32);
-        r.qh = *reinterpret_cast<const uint2 *>(a.p1 + blk * 64 + 32 * i + 8 * g);
-        r.scw = *reinterpret_cast<const uint32_t *>(a.p2 + blk * 16 + 8 * i + 4 * (c & 1));
-        r.d = *reinterpret_cast<const uint16_t *>(a.p3 + blk * 2);
+        r.qh = *reinterpret_cast<const uint2 *>(m.p1 + blk * 64 + 32 * i + 8 * g);
+        r.scw = *reinterpret_cast<const uint32_t *>(m.p2 + blk * 16 + 8 * i + 4 * (c & 1));
+        r.d = *reinterpret_cast<const uint16_t *>(m.p3 + blk * 2);
     }
-    __device__ static void frag(const Raw &r, const GemmArgs &, uint32_t chunk, uint32_t g,
-                                half4 (&a4)[4]) {
+    __device__ static void frag(const Raw &r, uint32_t, uint32_t chunk, uint32_t g, half4 (&a4)[4]) {
         // element e = 64 (c & 1) + 32 s2 + 8 g + b of the 128-element half: quarter
         // e / 32 = 2 (c & 1) + s2 picks the nibble (high for quarters 2, 3), the bit pair of
         // qh[8 g + b] (shift 2 * quarter) and the scale (8 g + b) / 16 + 2 * quarter
@@ -164,20 +181,20 @@ struct GemmQ8_0 {
     };
     // rows are a multiple of 32 elements long: the second half of the last chunk may not
     // exist; it is then read from the first half and expanded to zeros
-    __device__ static void load(Raw &r, const GemmArgs &a, uint32_t row, uint32_t chunk, uint32_t g) {
-        const uint32_t b0 = chunk * 2, nb = a.ncols / 32;
+    __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, uint32_t row, uint32_t chunk,
+                                uint32_t g) {
+        const uint32_t b0 = chunk * 2, nb = ncols / 32;
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
             const uint32_t b = min(b0 + s2, nb - 1);
-            r.q[s2] = *reinterpret_cast<const uint2 *>(a.p0 + (size_t)row * a.ncols + b * 32 + 8 * g);
-            r.d[s2] = *reinterpret_cast<const uint16_t *>(a.p1 + ((size_t)row * nb + b) * 2);
+            r.q[s2] = *reinterpret_cast<const uint2 *>(m.p0 + (size_t)row * ncols + b * 32 + 8 * g);
+            r.d[s2] = *reinterpret_cast<const uint16_t *>(m.p1 + ((size_t)row * nb + b) * 2);
         }
     }
-    __device__ static void frag(const Raw &r, const GemmArgs &a, uint32_t chunk, uint32_t,
-                                half4 (&a4)[4]) {
+    __device__ static void frag(const Raw &r, uint32_t ncols, uint32_t chunk, uint32_t, half4 (&a4)[4]) {
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
-            const bool exists = chunk * 2 + s2 < a.ncols / 32;
+            const bool exists = chunk * 2 + s2 < ncols / 32;
             const float d = exists ? f16_bits_to_f32((uint16_t)r.d[s2]) : 0.f;
             const uint32_t x = exists ? r.q[s2].x : 0u, y = exists ? r.q[s2].y : 0u;
             a4[2 * s2] = to_half4(sb0(x) * d, sb1(x) * d, sb2(x) * d, sb3(x) * d);
@@ -186,129 +203,148 @@ struct GemmQ8_0 {
     }
 };
 
-template <class F, int NT, int RB>
-__global__ __launch_bounds__(KWAVES * 64) void gemm_quant_f16_kernel(const GemmArgs a) {
-    extern __shared__ float4 red[];  // [KWAVES][NT][64]
+template <class F, int NT>
+__global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a) {
+    extern __shared__ u32x4 xs[];  // [2 buffers][2 chunks][NT * 128 words]
+    constexpr uint32_t CW = NT * 128;  // words of one chunk
+    constexpr uint32_t NTHREADS = KWAVES * 64;
+    constexpr int SW = (2 * CW + NTHREADS - 1) / NTHREADS;  // staged words per thread
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t j = lane & 15, g = lane >> 4;
-    const uint32_t row0 = blockIdx.x * (16 * RB);
-    uint32_t row[RB];  // this lane's rows of the A operands
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) row[rb] = min(row0 + 16 * rb + j, a.nrows - 1);
+    const uint32_t rb = wave & 3, kh = wave >> 2;
+    // which matrix this tile belongs to (uniform over the workgroup)
+    uint32_t mi = 0;
+    if (a.nmat > 1 && blockIdx.x >= a.m[1].tile0) mi = 1;
+    if (a.nmat > 2 && blockIdx.x >= a.m[2].tile0) mi = 2;
+    const GemmMat &m = a.m[mi];
+    const uint32_t row0 = (blockIdx.x - m.tile0) * 64 + 16 * rb;
+    const uint32_t row = min(row0 + j, m.nrows - 1);  // this lane's row of the A operand
     const uint32_t nchunks = a.kpad / KC;
-    // chunks of this wave: wave, wave + 8, ...
-    const uint32_t n_my = nchunks > wave ? (nchunks - wave + KWAVES - 1) / KWAVES : 0;
+    const uint32_t per = (nchunks + a.ks - 1) / a.ks;
+    const uint32_t c0 = min(blockIdx.y * per, nchunks), c1 = min(nchunks, c0 + per);
+    const uint32_t n_it = (c1 - c0 + 1) / 2;
 
-    floatx4 acc[RB][NT];
+    floatx4 acc[NT];
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-#pragma unroll
-        for (int n = 0; n < NT; ++n) acc[rb][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-    }
+    for (int n = 0; n < NT; ++n) acc[n] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // Every load is unconditional (a chunk number past the end re-reads the last chunk and
-    // is never multiplied): the compiler can then count outstanding loads exactly instead
-    // of draining them all before each use.  The weight bytes of the next chunk are
-    // requested when a chunk's arithmetic starts; each activation word of the next chunk
-    // is requested into the register of the one it replaces right after that one's last use.
-    typename F::Raw ra[RB], rb_[RB];
-    uint4 b[NT][2];
-    auto chunk_of = [&](uint32_t i) { return min(wave + KWAVES * i, nchunks - 1); };
-    auto load_a = [&](typename F::Raw(&r)[RB], uint32_t i) {
-        const uint32_t c = chunk_of(i);
+    // Staged words of this thread: word tid + 512 q of the pair of chunks, q < SW.  All
+    // loads are unconditional (chunks past the end re-read the last one and are not used).
+    u32x4 st[SW];
+    typename F::Raw cur, nxt;
+    if (n_it > 0) {
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) F::load(r[rb], a, row[rb], c, g);
-    };
-    auto compute = [&](const typename F::Raw(&r)[RB], uint32_t i) {
-        const uint32_t c = wave + KWAVES * i;
-        const uint4 *next = a.xh + (size_t)chunk_of(i + 1) * NT * 128 + lane;
-        half4 a4[RB][4];
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) F::frag(r[rb], a, c, g, a4[rb]);
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-#pragma unroll
-            for (int n = 0; n < NT; ++n) {
-                half8 bw;
-                __builtin_memcpy(&bw, &b[n][s2], 16);
-#pragma unroll
-                for (int rb = 0; rb < RB; ++rb) {
-                    half8 aw;
-                    __builtin_memcpy(&aw, &a4[rb][2 * s2], 16);  // a4[2 s2], a4[2 s2 + 1]: 8 consecutive k
-                    acc[rb][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw, bw, acc[rb][n], 0, 0, 0);
-                }
-                b[n][s2] = next[(n * 2 + s2) * 64];
-            }
+        for (int q = 0; q < SW; ++q) {
+            const uint32_t w = min(tid + NTHREADS * q, 2 * CW - 1);
+            st[q] = a.xh[(size_t)min(c0 + w / CW, nchunks - 1) * CW + w % CW];
         }
-    };
-    if (n_my > 0) {
-        load_a(ra, 0);
-        {
-            const uint4 *first = a.xh + (size_t)chunk_of(0) * NT * 128 + lane;
+        F::load(cur, m, a.ncols, row, min(c0 + kh, nchunks - 1), g);
+    }
+    for (uint32_t it = 0; it < n_it; ++it) {
+        u32x4 *buf = xs + (it & 1) * 2 * CW;
+#pragma unroll
+        for (int q = 0; q < SW; ++q) {
+            if (2 * CW % NTHREADS == 0 || tid + NTHREADS * q < 2 * CW) buf[tid + NTHREADS * q] = st[q];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < SW; ++q) {
+            const uint32_t w = min(tid + NTHREADS * q, 2 * CW - 1);
+            st[q] = a.xh[(size_t)min(c0 + 2 * (it + 1) + w / CW, nchunks - 1) * CW + w % CW];
+        }
+        F::load(nxt, m, a.ncols, row, min(c0 + 2 * (it + 1) + kh, nchunks - 1), g);
+        const uint32_t c = c0 + 2 * it + kh;
+        if (c < c1) {  // uniform over the wave
+            const u32x4 *bsrc = buf + kh * CW + lane;
+            // the LDS words of the first half are requested before the weights are expanded,
+            // those of the second half while the first half is multiplied
+            u32x4 bw[NT];
+#pragma unroll
+            for (int n = 0; n < NT; ++n) bw[n] = bsrc[(n * 2) * 64];
+            half4 a4[4];
+            F::frag(cur, a.ncols, c, g, a4);
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2) {
+                half8 aw;
+                __builtin_memcpy(&aw, &a4[2 * s2], 16);
 #pragma unroll
-                for (int n = 0; n < NT; ++n) b[n][s2] = first[(n * 2 + s2) * 64];
+                for (int n = 0; n < NT; ++n) {
+                    half8 b8;
+                    __builtin_memcpy(&b8, &bw[n], 16);
+                    acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw, b8, acc[n], 0, 0, 0);
+                    if (s2 == 0) bw[n] = bsrc[(n * 2 + 1) * 64];
+                }
             }
         }
-        for (uint32_t i = 0; i < n_my; i += 2) {
-            load_a(rb_, i + 1);
-            compute(ra, i);
-            if (i + 1 < n_my) {
-                load_a(ra, i + 2);
-                compute(rb_, i + 1);
-            }
-        }
+        cur = nxt;
     }
-    // the partial sums of the 8 waves, added in wave order, one row block at a time
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-        if (rb > 0) __syncthreads();
+    // waves 4-7 hand their sums to waves 0-3 through LDS
+    __syncthreads();
+    float4 *red = reinterpret_cast<float4 *>(xs);  // [4 row blocks][NT][64]
+    if (kh == 1) {
 #pragma unroll
         for (int n = 0; n < NT; ++n)
-            red[(wave * NT + n) * 64 + lane] =
-                make_float4(acc[rb][n][0], acc[rb][n][1], acc[rb][n][2], acc[rb][n][3]);
-        __syncthreads();
-        for (uint32_t idx = tid; idx < NT * 64; idx += KWAVES * 64) {
-            const uint32_t n = idx >> 6, l = idx & 63;
-            float4 v = red[n * 64 + l];
+            red[(rb * NT + n) * 64 + lane] = make_float4(acc[n][0], acc[n][1], acc[n][2], acc[n][3]);
+    }
+    __syncthreads();
+    if (kh == 1) return;
+    const uint32_t r4 = row0 + 4 * g;  // acc[n] = rows r4 .. r4 + 3 of token 16 n + j
 #pragma unroll
-            for (uint32_t w = 1; w < KWAVES; ++w) {
-                const float4 p = red[(w * NT + n) * 64 + l];
-                v = make_float4(v.x + p.x, v.y + p.y, v.z + p.z, v.w + p.w);
-            }
-            // v = out[token 16 n + (l & 15)][first row of the block + 4 (l >> 4) .. + 3]
-            const uint32_t tok = n * 16 + (l & 15), r4 = row0 + 16 * rb + 4 * (l >> 4);
-            if (tok >= a.T || r4 >= a.nrows) continue;
+    for (int n = 0; n < NT; ++n) {
+        const float4 p = red[(rb * NT + n) * 64 + lane];
+        float4 v = make_float4(acc[n][0] + p.x, acc[n][1] + p.y, acc[n][2] + p.z, acc[n][3] + p.w);
+        const uint32_t tok = n * 16 + j;
+        if (tok >= a.T || r4 >= m.nrows) continue;
+        float *o;
+        bool add = false;
+        if (a.ks > 1) {
+            o = a.part + ((size_t)blockIdx.y * a.T + tok) * m.nrows + r4;  // plain partial sum
+        } else {
             const float xs_t = a.xscale ? a.xscale[tok] : 1.f;
             v = make_float4(v.x * xs_t, v.y * xs_t, v.z * xs_t, v.w * xs_t);
-            float *o = a.out + (size_t)tok * a.out_stride + r4;
-            if (r4 + 3 < a.nrows && (reinterpret_cast<uintptr_t>(o) & 15u) == 0) {
-                if (a.bias) {
-                    v.x += a.bias[r4];
-                    v.y += a.bias[r4 + 1];
-                    v.z += a.bias[r4 + 2];
-                    v.w += a.bias[r4 + 3];
-                }
-                if (a.accumulate) {
-                    const float4 p = *reinterpret_cast<const float4 *>(o);
-                    v = make_float4(p.x + v.x, p.y + v.y, p.z + v.z, p.w + v.w);
-                }
-                *reinterpret_cast<float4 *>(o) = v;
-                continue;
-            }
-            const float vv[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if (r4 + i < a.nrows) {
-                    float e = vv[i];
-                    if (a.bias) e += a.bias[r4 + i];
-                    o[i] = a.accumulate ? o[i] + e : e;
+            if (m.bias) {
+                if (r4 + 3 < m.nrows) {
+                    v.x += m.bias[r4];
+                    v.y += m.bias[r4 + 1];
+                    v.z += m.bias[r4 + 2];
+                    v.w += m.bias[r4 + 3];
+                } else {
+                    v.x += m.bias[r4];
+                    if (r4 + 1 < m.nrows) v.y += m.bias[r4 + 1];
+                    if (r4 + 2 < m.nrows) v.z += m.bias[r4 + 2];
                 }
             }
+            o = m.out + (size_t)tok * m.out_stride + r4;
+            add = a.accumulate != 0;
+        }
+        if (r4 + 3 < m.nrows && (reinterpret_cast<uintptr_t>(o) & 15u) == 0) {
+            if (add) {
+                const float4 q = *reinterpret_cast<const float4 *>(o);
+                v = make_float4(q.x + v.x, q.y + v.y, q.z + v.z, q.w + v.w);
+            }
+            *reinterpret_cast<float4 *>(o) = v;
+        } else {
+            o[0] = add ? o[0] + v.x : v.x;
+            if (r4 + 1 < m.nrows) o[1] = add ? o[1] + v.y : v.y;
+            if (r4 + 2 < m.nrows) o[2] = add ? o[2] + v.z : v.z;
+            if (r4 + 3 < m.nrows) o[3] = add ? o[3] + v.w : v.w;
         }
     }
+}
+
+// out[t][r] (= or +=) xscale[t] * (part[0][t][r] + part[1][t][r] + ...) + bias[r]
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmArgs a) {
+    const GemmMat &m = a.m[0];
+    const uint32_t r = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
+    if (r >= m.nrows) return;
+    const float *p = a.part + (size_t)t * m.nrows + r;
+    float v = p[0];
+    for (uint32_t y = 1; y < a.ks; ++y) v += p[(size_t)y * a.T * m.nrows];
+    v *= a.xscale ? a.xscale[t] : 1.f;
+    if (m.bias) v += m.bias[r];
+    float *o = m.out + (size_t)t * m.out_stride + r;
+    *o = a.accumulate ? *o + v : v;
 }
 
 // One workgroup per token: X[t] (fp32, optionally RMS-normalised with weights w as
@@ -574,32 +610,38 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const AttnRowsArgs a) {
     }
 }
 
-int g_force_row_blocks = 0;  // 0: by matrix height; 1 or 2: forced (tests)
+int g_force_k_split = 0;  // 0: by matrix shape; 1..8: forced (tests)
 
-template <class F, int RB>
-int launch_gemm_rb(wgml_ctx *ctx, const GemmArgs &a) {
+// How many workgroups split K: enough that tiles x ks covers the compute units about
+// 1.5 times (two workgroups fit a unit), a power of two, and at least 4 iterations each.
+uint32_t gemm_k_split(const wgml_ctx *ctx, uint32_t tiles, uint32_t kpad) {
+    const uint32_t nchunks = kpad / KC;
+    if (g_force_k_split) return min((uint32_t)g_force_k_split, max(nchunks, 1u));
+    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
+    uint32_t ks = 1;
+    while (ks < 8 && tiles * ks * 2 <= cu + cu / 2 && nchunks / (ks * 2) >= 8) ks *= 2;
+    return ks;
+}
+
+template <class F>
+int launch_gemm_fmt(wgml_ctx *ctx, GemmArgs &a, uint32_t tiles) {
     const uint32_t nt = a.tpad / 16;  // token blocks: 1, 2, 4 or 8
-    const dim3 grid((a.nrows + 16 * RB - 1) / (16 * RB)), block(KWAVES * 64);
-    const size_t lds = (size_t)KWAVES * nt * 64 * sizeof(float4);
+    const dim3 grid(tiles, a.ks), block(KWAVES * 64);
+    const size_t lds = (size_t)nt * 8192;  // 2 buffers x 2 chunks x nt x 2 KiB
     switch (nt) {
-    case 8: gemm_quant_f16_kernel<F, 8, RB><<<grid, block, lds, ctx->stream>>>(a); break;
-    case 4: gemm_quant_f16_kernel<F, 4, RB><<<grid, block, lds, ctx->stream>>>(a); break;
-    case 2: gemm_quant_f16_kernel<F, 2, RB><<<grid, block, lds, ctx->stream>>>(a); break;
-    default: gemm_quant_f16_kernel<F, 1, RB><<<grid, block, lds, ctx->stream>>>(a); break;
+    case 8: gemm_lds_kernel<F, 8><<<grid, block, lds, ctx->stream>>>(a); break;
+    case 4: gemm_lds_kernel<F, 4><<<grid, block, lds, ctx->stream>>>(a); break;
+    case 2: gemm_lds_kernel<F, 2><<<grid, block, lds, ctx->stream>>>(a); break;
+    default: gemm_lds_kernel<F, 1><<<grid, block, lds, ctx->stream>>>(a); break;
     }
     WGML_CHECK_LAUNCH();
     ctx->launches++;
+    if (a.ks > 1) {
+        gemm_reduce_kernel<<<dim3((a.m[0].nrows + 255) / 256, a.T), dim3(256), 0, ctx->stream>>>(a);
+        WGML_CHECK_LAUNCH();
+        ctx->launches++;
+    }
     return WGML_OK;
-}
-
-// Two row blocks per wave halve the activation traffic per product (each activation word
-// serves 32 rows) at the price of half as many workgroups: worth it once those still
-// cover half of the compute units.
-template <class F>
-int launch_gemm_fmt(wgml_ctx *ctx, const GemmArgs &a) {
-    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
-    const bool two = g_force_row_blocks ? g_force_row_blocks == 2 : a.nrows / 32 >= cu / 2;
-    return two ? launch_gemm_rb<F, 2>(ctx, a) : launch_gemm_rb<F, 1>(ctx, a);
 }
 
 }  // namespace
@@ -632,35 +674,69 @@ int launch_prefill_prep(wgml_ctx *ctx, const float *x, uint32_t x_stride, const 
     return WGML_OK;
 }
 
+int ensure_gemm_partials(wgml_ctx *ctx, size_t bytes) {
+    if (bytes <= ctx->gemm_part_bytes) return WGML_OK;
+    if (ctx->gemm_part) ctx->retired.push_back(ctx->gemm_part);  // may still be read by queued work
+    ctx->gemm_part = nullptr;
+    ctx->gemm_part_bytes = 0;
+    bytes = (bytes + (size_t(8) << 20)) & ~((size_t(1) << 20) - 1);  // grow in steps
+    WGML_CHECK_HIP(hipMalloc((void **)&ctx->gemm_part, bytes));
+    ctx->gemm_part_bytes = bytes;
+    return WGML_OK;
+}
+
+int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, const void *xh,
+                            const float *xscale, uint32_t T, int accumulate) {
+    if (T == 0 || T > kPrefillMaxTokens)
+        return set_error(WGML_E_INVALID, "gemm_quant: %u tokens (1..%u)", T, kPrefillMaxTokens);
+    if (n < 1 || n > 3) return set_error(WGML_E_INVALID, "gemm_quant: %d matrices (1..3)", n);
+    const wgml_qmat *first = targets[0].m;
+    GemmArgs a{};
+    uint32_t tiles = 0;
+    for (int i = 0; i < n; ++i) {
+        const wgml_qmat *q = targets[i].m;
+        if (q->type != first->type || q->ncols != first->ncols)
+            return set_error(WGML_E_INVALID, "gemm_quant: matrices of one launch differ in format or width");
+        GemmMat &g = a.m[i];
+        g.p0 = q->p0;
+        g.p1 = q->p1;
+        g.p2 = q->p2;
+        g.p3 = q->p3;
+        g.out = targets[i].out;
+        g.bias = targets[i].bias;
+        g.nrows = q->nrows;
+        g.out_stride = targets[i].out_stride;
+        g.tile0 = tiles;
+        tiles += (q->nrows + 63) / 64;
+    }
+    a.nmat = (uint32_t)n;
+    a.xh = reinterpret_cast<const u32x4 *>(xh);
+    a.xscale = xscale;
+    a.ncols = first->ncols;
+    a.kpad = prefill_kpad(first->ncols);
+    a.T = T;
+    a.tpad = prefill_tpad(T);
+    a.accumulate = accumulate;
+    a.ks = n == 1 ? gemm_k_split(ctx, tiles, a.kpad) : 1;
+    if (a.ks > 1) {
+        WGML_TRY(ensure_gemm_partials(ctx, (size_t)a.ks * T * first->nrows * sizeof(float)));
+        a.part = ctx->gemm_part;
+    }
+    switch (first->type) {
+    case WGML_Q4_K: return launch_gemm_fmt<GemmQ4K>(ctx, a, tiles);
+    case WGML_Q6_K: return launch_gemm_fmt<GemmQ6K>(ctx, a, tiles);
+    case WGML_Q8_0: return launch_gemm_fmt<GemmQ8_0>(ctx, a, tiles);
+    default:
+        return set_error(WGML_E_UNSUPPORTED, "gemm_quant: matrix type %d (Q8_0, Q4_K, Q6_K only)",
+                         first->type);
+    }
+}
+
 int launch_gemm_quant(wgml_ctx *ctx, float *out, uint32_t out_stride, const wgml_qmat *m,
                       const void *xh, const float *xscale, uint32_t T, const float *bias,
                       int accumulate) {
-    if (T == 0 || T > kPrefillMaxTokens)
-        return set_error(WGML_E_INVALID, "gemm_quant: %u tokens (1..%u)", T, kPrefillMaxTokens);
-    GemmArgs a{};
-    a.p0 = m->p0;
-    a.p1 = m->p1;
-    a.p2 = m->p2;
-    a.p3 = m->p3;
-    a.xh = reinterpret_cast<const uint4 *>(xh);
-    a.xscale = xscale;
-    a.out = out;
-    a.bias = bias;
-    a.nrows = m->nrows;
-    a.ncols = m->ncols;
-    a.kpad = prefill_kpad(m->ncols);
-    a.T = T;
-    a.tpad = prefill_tpad(T);
-    a.out_stride = out_stride;
-    a.accumulate = accumulate;
-    switch (m->type) {
-    case WGML_Q4_K: return launch_gemm_fmt<GemmQ4K>(ctx, a);
-    case WGML_Q6_K: return launch_gemm_fmt<GemmQ6K>(ctx, a);
-    case WGML_Q8_0: return launch_gemm_fmt<GemmQ8_0>(ctx, a);
-    default:
-        return set_error(WGML_E_UNSUPPORTED, "gemm_quant: matrix type %d (Q8_0, Q4_K, Q6_K only)",
-                         m->type);
-    }
+    const GemmTarget t{m, out, out_stride, bias};
+    return launch_gemm_quant_multi(ctx, &t, 1, xh, xscale, T, accumulate);
 }
 
 int launch_embed_rows(wgml_ctx *ctx, float *x, const float *table, const uint32_t *d_tokens,
@@ -708,9 +784,9 @@ int launch_attention_rows(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pos
 
 extern "C" {
 
-// Test hook: 0 = choose rows per workgroup by matrix height, 1 = 16 rows, 2 = 32 rows.
-WGML_API int wgml_debug_set_gemm_row_blocks(int n) {
-    g_force_row_blocks = n == 1 || n == 2 ? n : 0;
+// Test hook: 0 = choose by matrix shape how many workgroups split K, 1..8 = that many.
+WGML_API int wgml_debug_set_gemm_k_split(int n) {
+    g_force_k_split = n >= 1 && n <= 8 ? n : 0;
     return WGML_OK;
 }
 

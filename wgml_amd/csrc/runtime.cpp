@@ -39,6 +39,7 @@ void ctx_release(wgml_ctx *ctx) {
     if (ctx->attn_ws) (void)hipFree(ctx->attn_ws);
     if (ctx->prefill_xh) (void)hipFree(ctx->prefill_xh);
     if (ctx->prefill_xscale) (void)hipFree(ctx->prefill_xscale);
+    if (ctx->gemm_part) (void)hipFree(ctx->gemm_part);
     for (void *p : ctx->retired) (void)hipFree(p);
     if (ctx->d_scalar) (void)hipFree(ctx->d_scalar);
     if (ctx->h_scalar) (void)hipHostFree(ctx->h_scalar);
