@@ -63,6 +63,9 @@ struct wgml_ctx {
     // partial sums of batched products whose K range is split between workgroups
     float *gemm_part = nullptr;
     size_t gemm_part_bytes = 0;
+    // > 0: the last batched product left this many partial sums per element in gemm_part
+    // for the next kernel to add to its output (launch_prefill_prep or launch_gemm_flush)
+    uint32_t gemm_pending_ks = 0;
     uint64_t launches = 0;  // kernels enqueued so far (diagnostics)
     // Buffers, matrices and models keep their context alive: the device objects
     // are torn down when the last reference goes, whatever order handles are
@@ -208,17 +211,25 @@ int ensure_prefill_scratch(wgml_ctx *ctx, size_t xh_bytes);
 // xh[tpad][kpad] (f16) <- x[T][K] (f32, rows x_stride apart): RMS-normalised with
 // norm_w first when that is non-null; replaced by up[t][k] * silu(x[t][k]) when `up`
 // is non-null.  xscale[tpad] receives what a token's products must be multiplied with.
-int launch_prefill_prep(wgml_ctx *ctx, const float *x, uint32_t x_stride, const float *up,
+// If the product before left partial sums for x (defer_reduce), they are added to x first.
+int launch_prefill_prep(wgml_ctx *ctx, float *x, uint32_t x_stride, const float *up,
                         const float *norm_w, float eps, void *xh, float *xscale, uint32_t K,
                         uint32_t T);
+// Adds partial sums left for x by a product with defer_reduce (no-op if there are none).
+int launch_gemm_flush(wgml_ctx *ctx, float *x, uint32_t x_stride, const float *xscale, uint32_t K,
+                      uint32_t T);
 // xb[t] = attention of q[t] (position pos0 + t) over cache rows 0 .. pos0 + t
 int launch_attention_rows(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pos0, uint32_t T,
                           const float *q, uint32_t q_stride, const float *kc, const float *vc,
                           float *xb, uint32_t xb_stride);
 // out[t][r] (rows out_stride apart) = (or +=) sum_k M[r][k] x[t][k] + bias[r]
+// defer_reduce: when the product's K range is split between workgroups and it is a plain
+// `out += ` of one matrix, the partial sums are left for the caller's next kernel on out
+// (launch_prefill_prep or launch_gemm_flush), which must come before anything else reads out
+// or writes xscale.
 int launch_gemm_quant(wgml_ctx *ctx, float *out, uint32_t out_stride, const wgml_qmat *m,
                       const void *xh, const float *xscale, uint32_t T, const float *bias,
-                      int accumulate);
+                      int accumulate, bool defer_reduce = false);
 // The same for up to three matrices of one format and width that multiply the same
 // activations, in one launch.
 struct GemmTarget {
@@ -228,7 +239,8 @@ struct GemmTarget {
     const float *bias;
 };
 int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, const void *xh,
-                            const float *xscale, uint32_t T, int accumulate);
+                            const float *xscale, uint32_t T, int accumulate,
+                            bool defer_reduce = false);
 int launch_embed_rows(wgml_ctx *ctx, float *x, const float *table, const uint32_t *d_tokens,
                       uint32_t dim, uint32_t T);
 int launch_rope_rows(wgml_ctx *ctx, int variant, uint32_t head_size, uint32_t kv_dim, uint32_t pos0,

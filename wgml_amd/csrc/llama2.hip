@@ -402,7 +402,7 @@ int enqueue_prefill_run(wgml_llama2 *m, const uint32_t *tokens, uint32_t T, uint
         WGML_TRY(launch_attention_rows(ctx, ap, pos0, T, m->pf_q, dim, w.key_cache, w.value_cache,
                                        m->pf_xb, dim));
         WGML_TRY(launch_prefill_prep(ctx, m->pf_xb, dim, nullptr, nullptr, 0.f, xh, xs, dim, T));
-        WGML_TRY(launch_gemm_quant(ctx, m->pf_x, dim, w.attn_output, xh, xs, T, nullptr, 1));
+        WGML_TRY(launch_gemm_quant(ctx, m->pf_x, dim, w.attn_output, xh, xs, T, nullptr, 1, true));
         WGML_TRY(launch_prefill_prep(ctx, m->pf_x, dim, nullptr, w.ffn_norm, c.rms_norm_eps, xh, xs,
                                      dim, T));
         if (w.ffn_gate->type == w.ffn_up->type) {
@@ -415,8 +415,9 @@ int enqueue_prefill_run(wgml_llama2 *m, const uint32_t *tokens, uint32_t T, uint
         }
         WGML_TRY(launch_prefill_prep(ctx, m->pf_hb, hidden, m->pf_hb2, nullptr, 0.f, xh, xs, hidden,
                                      T));
-        WGML_TRY(launch_gemm_quant(ctx, m->pf_x, dim, w.ffn_down, xh, xs, T, nullptr, 1));
+        WGML_TRY(launch_gemm_quant(ctx, m->pf_x, dim, w.ffn_down, xh, xs, T, nullptr, 1, true));
     }
+    WGML_TRY(launch_gemm_flush(ctx, m->pf_x, dim, xs, dim, T));  // the last layer's down projection
     WGML_CHECK_HIP(hipMemcpyAsync(m->x, m->pf_x + (size_t)(T - 1) * dim, (size_t)dim * 4,
                                   hipMemcpyDeviceToDevice, ctx->stream));
     return WGML_OK;

@@ -57,6 +57,7 @@ struct GemmMat {
     const float *bias;                 // optional, per row
     uint32_t nrows, out_stride;
     uint32_t tile0;                    // first 64-row tile of this matrix in grid.x
+    uint32_t roff;                     // rows of the matrices before this one in the launch
 };
 
 struct GemmArgs {
@@ -66,8 +67,10 @@ struct GemmArgs {
     const float *xscale;               // [tpad] factor to multiply a token's results with
     uint32_t ncols, kpad, T, tpad;
     int accumulate;                    // out += result
-    float *part;                       // [ks][T][nrows] partial sums (ks > 1, one matrix)
+    float *part;                       // [ks][T][total_rows] partial sums (ks > 1)
     uint32_t ks;                       // ways K is split between workgroups (grid.y)
+    uint32_t total_rows;               // rows of all matrices of the launch
+    int defer;                         // ks > 1: leave the partial sums to the next kernel
 };
 
 __device__ __forceinline__ half4 to_half4(float a, float b, float c, float d) {
@@ -299,7 +302,8 @@ __global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a)
         float *o;
         bool add = false;
         if (a.ks > 1) {
-            o = a.part + ((size_t)blockIdx.y * a.T + tok) * m.nrows + r4;  // plain partial sum
+            // plain partial sum
+            o = a.part + ((size_t)blockIdx.y * a.T + tok) * a.total_rows + m.roff + r4;
         } else {
             const float xs_t = a.xscale ? a.xscale[tok] : 1.f;
             v = make_float4(v.x * xs_t, v.y * xs_t, v.z * xs_t, v.w * xs_t);
@@ -335,12 +339,16 @@ __global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a)
 
 // out[t][r] (= or +=) xscale[t] * (part[0][t][r] + part[1][t][r] + ...) + bias[r]
 __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmArgs a) {
-    const GemmMat &m = a.m[0];
-    const uint32_t r = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
-    if (r >= m.nrows) return;
-    const float *p = a.part + (size_t)t * m.nrows + r;
+    const uint32_t rg = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;  // row among all matrices
+    if (rg >= a.total_rows) return;
+    uint32_t mi = 0;
+    if (a.nmat > 1 && rg >= a.m[1].roff) mi = 1;
+    if (a.nmat > 2 && rg >= a.m[2].roff) mi = 2;
+    const GemmMat &m = a.m[mi];
+    const uint32_t r = rg - m.roff;
+    const float *p = a.part + (size_t)t * a.total_rows + rg;
     float v = p[0];
-    for (uint32_t y = 1; y < a.ks; ++y) v += p[(size_t)y * a.T * m.nrows];
+    for (uint32_t y = 1; y < a.ks; ++y) v += p[(size_t)y * a.T * a.total_rows];
     v *= a.xscale ? a.xscale[t] : 1.f;
     if (m.bias) v += m.bias[r];
     float *o = m.out + (size_t)t * m.out_stride + r;
@@ -355,7 +363,8 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmArgs a) {
 // up[k] * silu(x[k]) (ops/silu.wgsl:13-27) instead of x itself (no normalisation then).
 constexpr int PREP_THREADS = 1024;
 constexpr int PREP_GROUPS = 2;  // groups of 8 columns a thread keeps in registers
-__global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(const float *__restrict__ x, uint32_t x_stride,
+__global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict__ x, uint32_t x_stride,
+                                                     const float *__restrict__ part, uint32_t part_ks,
                                                      const float *__restrict__ up,
                                                      const float *__restrict__ norm_w, float eps,
                                                      uint4 *__restrict__ xh,
@@ -374,8 +383,20 @@ __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(const float *__res
         if (tid == 0) xscale[t] = 0.f;
         return;
     }
-    const float *xr = x + (size_t)t * x_stride;
+    float *xr = x + (size_t)t * x_stride;
     const float *ur = up ? up + (size_t)t * x_stride : nullptr;
+    if (part_ks) {
+        // the product before this kernel left x[t] += xscale[t] * (part[0][t] + part[1][t] + ...)
+        // to be done here (part: [part_ks][T][K], xscale[t] still that product's factor)
+        const float old_scale = xscale[t];
+        for (uint32_t k = tid; k < K; k += PREP_THREADS) {
+            const float *p = part + (size_t)t * K + k;
+            float sum = p[0];
+            for (uint32_t y = 1; y < part_ks; ++y) sum += p[(size_t)y * T * K];
+            xr[k] += sum * old_scale;
+        }
+        __syncthreads();  // every thread reads what others wrote (same workgroup only)
+    }
     // Rows of up to 8 * PREP_GROUPS * PREP_THREADS columns are read once and kept in
     // registers (v); longer rows are re-read from memory by the later passes.
     const bool cached = ngroups <= PREP_GROUPS * PREP_THREADS;
@@ -636,8 +657,8 @@ int launch_gemm_fmt(wgml_ctx *ctx, GemmArgs &a, uint32_t tiles) {
     }
     WGML_CHECK_LAUNCH();
     ctx->launches++;
-    if (a.ks > 1) {
-        gemm_reduce_kernel<<<dim3((a.m[0].nrows + 255) / 256, a.T), dim3(256), 0, ctx->stream>>>(a);
+    if (a.ks > 1 && !a.defer) {
+        gemm_reduce_kernel<<<dim3((a.total_rows + 255) / 256, a.T), dim3(256), 0, ctx->stream>>>(a);
         WGML_CHECK_LAUNCH();
         ctx->launches++;
     }
@@ -664,11 +685,39 @@ int ensure_prefill_scratch(wgml_ctx *ctx, size_t xh_bytes) {
     return WGML_OK;
 }
 
-int launch_prefill_prep(wgml_ctx *ctx, const float *x, uint32_t x_stride, const float *up,
+int launch_prefill_prep(wgml_ctx *ctx, float *x, uint32_t x_stride, const float *up,
                         const float *norm_w, float eps, void *xh, float *xscale, uint32_t K,
                         uint32_t T) {
+    // partial sums a product with defer_reduce left for x (they are K wide: x is its output)
+    const uint32_t pending = ctx->gemm_pending_ks;
+    ctx->gemm_pending_ks = 0;
     prep_x_kernel<<<dim3(prefill_tpad(T)), dim3(PREP_THREADS), 0, ctx->stream>>>(
-        x, x_stride, up, norm_w, eps, reinterpret_cast<uint4 *>(xh), xscale, K, prefill_kpad(K), T);
+        x, x_stride, pending ? ctx->gemm_part : nullptr, pending, up, norm_w, eps,
+        reinterpret_cast<uint4 *>(xh), xscale, K, prefill_kpad(K), T);
+    WGML_CHECK_LAUNCH();
+    ctx->launches++;
+    return WGML_OK;
+}
+
+// x[t] += the partial sums a product with defer_reduce left, for callers whose next
+// kernel is not launch_prefill_prep.
+__global__ void gemm_flush_kernel(float *x, uint32_t x_stride, const float *part, uint32_t ks,
+                                  const float *xscale, uint32_t K, uint32_t T) {
+    const uint32_t k = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
+    if (k >= K) return;
+    const float *p = part + (size_t)t * K + k;
+    float sum = p[0];
+    for (uint32_t y = 1; y < ks; ++y) sum += p[(size_t)y * T * K];
+    x[(size_t)t * x_stride + k] += sum * xscale[t];
+}
+
+int launch_gemm_flush(wgml_ctx *ctx, float *x, uint32_t x_stride, const float *xscale, uint32_t K,
+                      uint32_t T) {
+    const uint32_t pending = ctx->gemm_pending_ks;
+    ctx->gemm_pending_ks = 0;
+    if (!pending) return WGML_OK;
+    gemm_flush_kernel<<<dim3((K + 255) / 256, T), dim3(256), 0, ctx->stream>>>(x, x_stride, ctx->gemm_part,
+                                                                          pending, xscale, K, T);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
@@ -686,7 +735,7 @@ int ensure_gemm_partials(wgml_ctx *ctx, size_t bytes) {
 }
 
 int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, const void *xh,
-                            const float *xscale, uint32_t T, int accumulate) {
+                            const float *xscale, uint32_t T, int accumulate, bool defer_reduce) {
     if (T == 0 || T > kPrefillMaxTokens)
         return set_error(WGML_E_INVALID, "gemm_quant: %u tokens (1..%u)", T, kPrefillMaxTokens);
     if (n < 1 || n > 3) return set_error(WGML_E_INVALID, "gemm_quant: %d matrices (1..3)", n);
@@ -707,7 +756,9 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
         g.nrows = q->nrows;
         g.out_stride = targets[i].out_stride;
         g.tile0 = tiles;
+        g.roff = a.total_rows;
         tiles += (q->nrows + 63) / 64;
+        a.total_rows += q->nrows;
     }
     a.nmat = (uint32_t)n;
     a.xh = reinterpret_cast<const u32x4 *>(xh);
@@ -717,10 +768,14 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
     a.T = T;
     a.tpad = prefill_tpad(T);
     a.accumulate = accumulate;
-    a.ks = n == 1 ? gemm_k_split(ctx, tiles, a.kpad) : 1;
+    a.ks = gemm_k_split(ctx, tiles, a.kpad);
+    ctx->gemm_pending_ks = 0;
     if (a.ks > 1) {
-        WGML_TRY(ensure_gemm_partials(ctx, (size_t)a.ks * T * first->nrows * sizeof(float)));
+        WGML_TRY(ensure_gemm_partials(ctx, (size_t)a.ks * T * a.total_rows * sizeof(float)));
         a.part = ctx->gemm_part;
+        // the caller's next kernel adds the partial sums up itself (one matrix, plain += only)
+        a.defer = defer_reduce && n == 1 && accumulate && !targets[0].bias;
+        if (a.defer) ctx->gemm_pending_ks = a.ks;
     }
     switch (first->type) {
     case WGML_Q4_K: return launch_gemm_fmt<GemmQ4K>(ctx, a, tiles);
@@ -734,9 +789,9 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
 
 int launch_gemm_quant(wgml_ctx *ctx, float *out, uint32_t out_stride, const wgml_qmat *m,
                       const void *xh, const float *xscale, uint32_t T, const float *bias,
-                      int accumulate) {
+                      int accumulate, bool defer_reduce) {
     const GemmTarget t{m, out, out_stride, bias};
-    return launch_gemm_quant_multi(ctx, &t, 1, xh, xscale, T, accumulate);
+    return launch_gemm_quant_multi(ctx, &t, 1, xh, xscale, T, accumulate, defer_reduce);
 }
 
 int launch_embed_rows(wgml_ctx *ctx, float *x, const float *table, const uint32_t *d_tokens,
@@ -809,7 +864,7 @@ int wgml_gemm_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, wgml_view 
     WGML_TRY(launch_prefill_prep(ctx, view_ptr(x), m->ncols, nullptr, nullptr, 0.f, ctx->prefill_xh,
                                  ctx->prefill_xscale, m->ncols, n_tokens));
     return launch_gemm_quant(ctx, view_ptr(out), m->nrows, m, ctx->prefill_xh, ctx->prefill_xscale,
-                             n_tokens, nullptr, 0);
+                             n_tokens, nullptr, 0, false);
 }
 
 }  // extern "C"
