@@ -385,10 +385,14 @@ __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict_
     }
     float *xr = x + (size_t)t * x_stride;
     const float *ur = up ? up + (size_t)t * x_stride : nullptr;
-    if (part_ks) {
-        // the product before this kernel left x[t] += xscale[t] * (part[0][t] + part[1][t] + ...)
-        // to be done here (part: [part_ks][T][K], xscale[t] still that product's factor)
-        const float old_scale = xscale[t];
+    // Rows of up to 8 * PREP_GROUPS * PREP_THREADS columns are read once, 8 consecutive
+    // columns per thread and group, and kept in registers (v); longer rows are re-read from
+    // memory by the later passes.  (K is a multiple of 32 for every quantized format.)
+    const bool cached = ngroups <= PREP_GROUPS * PREP_THREADS && K % 8 == 0 && x_stride % 4 == 0;
+    // the product before this kernel may have left  x[t] += xscale[t] * (part[0][t] + part[1][t]
+    // + ...)  to be done here (part: [part_ks][T][K], xscale[t] still that product's factor)
+    const float old_scale = part_ks ? xscale[t] : 0.f;
+    if (part_ks && !cached) {
         for (uint32_t k = tid; k < K; k += PREP_THREADS) {
             const float *p = part + (size_t)t * K + k;
             float sum = p[0];
@@ -397,9 +401,6 @@ __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict_
         }
         __syncthreads();  // every thread reads what others wrote (same workgroup only)
     }
-    // Rows of up to 8 * PREP_GROUPS * PREP_THREADS columns are read once and kept in
-    // registers (v); longer rows are re-read from memory by the later passes.
-    const bool cached = ngroups <= PREP_GROUPS * PREP_THREADS;
     float v[PREP_GROUPS][8];
     auto raw = [&](uint32_t k) -> float {  // the value before normalisation
         if (k >= K) return 0.f;
@@ -411,7 +412,38 @@ __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict_
         for (int i = 0; i < PREP_GROUPS; ++i) {
             const uint32_t k0 = 8 * (tid + i * PREP_THREADS);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[i][e] = k0 + e < kpad ? raw(k0 + e) : 0.f;
+            for (int e = 0; e < 8; ++e) v[i][e] = 0.f;
+            if (k0 < K) {
+                float4 *xp = reinterpret_cast<float4 *>(xr + k0);
+                float4 a0 = xp[0], a1 = xp[1];
+                if (part_ks) {
+                    const float4 *pp = reinterpret_cast<const float4 *>(part + (size_t)t * K + k0);
+                    float4 s0 = pp[0], s1 = pp[1];
+                    for (uint32_t y = 1; y < part_ks; ++y) {
+                        const float4 *py = reinterpret_cast<const float4 *>(part + ((size_t)y * T + t) * K + k0);
+                        const float4 q0 = py[0], q1 = py[1];
+                        s0 = make_float4(s0.x + q0.x, s0.y + q0.y, s0.z + q0.z, s0.w + q0.w);
+                        s1 = make_float4(s1.x + q1.x, s1.y + q1.y, s1.z + q1.z, s1.w + q1.w);
+                    }
+                    a0 = make_float4(a0.x + s0.x * old_scale, a0.y + s0.y * old_scale,
+                                     a0.z + s0.z * old_scale, a0.w + s0.w * old_scale);
+                    a1 = make_float4(a1.x + s1.x * old_scale, a1.y + s1.y * old_scale,
+                                     a1.z + s1.z * old_scale, a1.w + s1.w * old_scale);
+                    xp[0] = a0;
+                    xp[1] = a1;
+                }
+                const float xv[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+                if (ur) {
+                    const float4 *up4 = reinterpret_cast<const float4 *>(ur + k0);
+                    const float4 u0 = up4[0], u1 = up4[1];
+                    const float uv[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[i][e] = uv[e] * (xv[e] / (1.0f + expf(-xv[e])));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[i][e] = xv[e];
+                }
+            }
         }
     }
     float rs = 1.f;
