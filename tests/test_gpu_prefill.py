@@ -21,7 +21,7 @@ QT = [W.Q8_0, W.Q4_K, W.Q6_K]
 
 
 @pytest.fixture(params=[0, 1, 2, 3, 8], ids=["ksplit_auto", "ksplit1", "ksplit2", "ksplit3", "ksplit8"])
-def row_blocks(request):
+def k_split(request):
     # workgroups that share the K range of a product (their partial sums are added by a
     # second kernel): chosen by matrix shape, or forced
     W._lib.lib.wgml_debug_set_gemm_k_split(request.param)
@@ -54,7 +54,7 @@ def check(got, ref):
 @pytest.mark.parametrize("qtype", QT)
 @pytest.mark.parametrize("T", [1, 5, 16, 17, 37, 64, 100, 128])
 @pytest.mark.parametrize("nrows,ncols", [(16, 256), (5, 512), (100, 768), (333, 2048)])
-def test_gemm_matches_dequantized_product(gpu, row_blocks, qtype, T, nrows, ncols):
+def test_gemm_matches_dequantized_product(gpu, k_split, qtype, T, nrows, ncols):
     raw = W.quantize(qtype, W.rng_normal(10 + nrows, nrows * ncols, 0, 0.02))
     x = W.rng_normal(20 + T, T * ncols).reshape(T, ncols)
     check(gemm(gpu, qtype, raw, nrows, ncols, x), reference(qtype, raw, nrows, ncols, x))
@@ -62,7 +62,7 @@ def test_gemm_matches_dequantized_product(gpu, row_blocks, qtype, T, nrows, ncol
 
 @pytest.mark.parametrize("ncols", [32, 96, 160, 2080])
 @pytest.mark.parametrize("T", [3, 40])
-def test_gemm_q8_0_rows_not_a_multiple_of_64(gpu, row_blocks, ncols, T):
+def test_gemm_q8_0_rows_not_a_multiple_of_64(gpu, k_split, ncols, T):
     nrows = 21
     raw = W.quantize(W.Q8_0, W.rng_normal(3, nrows * ncols, 0, 0.02))
     x = W.rng_normal(4, T * ncols).reshape(T, ncols)
@@ -84,7 +84,7 @@ def test_gemm_agrees_with_gemv_per_token(gpu, qtype):
 
 
 @pytest.mark.parametrize("qtype", QT)
-def test_gemm_large_activations_stay_finite(gpu, row_blocks, qtype):
+def test_gemm_large_activations_stay_finite(gpu, k_split, qtype):
     # values far beyond the f16 range (65504): the per-token power-of-two scale absorbs them
     nrows, ncols, T = 48, 1024, 9
     raw = W.quantize(qtype, W.rng_normal(1, nrows * ncols, 0, 0.02))
@@ -203,7 +203,7 @@ def test_prefill_in_two_calls_and_in_runs_of_128(gpu):
 
 @pytest.mark.parametrize("dim,heads,kv_heads,hidden", [(320, 4, 2, 448), (96, 2, 1, 160), (512, 4, 4, 1024),
                                                        (512, 2, 1, 768)])
-def test_prefill_head_sizes_and_partial_chunks(gpu, row_blocks, dim, heads, kv_heads, hidden):
+def test_prefill_head_sizes_and_partial_chunks(gpu, k_split, dim, heads, kv_heads, hidden):
     # head sizes 80, 48, 128 and 256; row lengths that are not multiples of 64 (Q8_0 only)
     cfg = Llama2Config(dim=dim, hidden_dim=hidden, n_layers=2, n_q_heads=heads, n_kv_heads=kv_heads,
                        vocab_size=300, seq_len=24, rope_base_freq=10000.0, rms_norm_eps=1e-5)

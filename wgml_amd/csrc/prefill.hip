@@ -26,7 +26,8 @@
 // One launch can cover up to three matrices that multiply the same activations (Q, K
 // and V; gate and up): their row tiles are laid side by side in grid.x.  A matrix too
 // short to give every compute unit a tile has its K range split between grid.y
-// workgroups; they leave partial sums that gemm_reduce_kernel adds in a fixed order.
+// workgroups; they leave partial sums that gemm_reduce_kernel adds in a fixed order (or,
+// for a plain `x += W h`, the prep_x_kernel that reads x next).
 //
 // Activations are stored in the order the B operand wants them (written by
 // prep_x_kernel): for chunk c, token block n, half s2 of the chunk, lane (g, j) finds
@@ -49,7 +50,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // plain vector: arrays of it stay in registers
 
 constexpr uint32_t KC = 64;    // elements of K per chunk
-constexpr uint32_t KWAVES = 8;  // waves of a workgroup = ways K is split
+constexpr uint32_t KWAVES = 8;  // waves of a workgroup: 4 row blocks x 2 chunks per iteration
 
 struct GemmMat {
     const uint8_t *p0, *p1, *p2, *p3;  // matrix planes (as wgml_qmat)
