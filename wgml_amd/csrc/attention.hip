@@ -241,13 +241,15 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnArgs a, uint3
 // (a neutral one if it had no position), so nothing depends on the current position
 // and all loads go out at once: lane y of every wave fetches (max, sum) of partial y,
 // thread d the d-th value of every partial; the weights are formed in registers.
+// B: partials fetched per round of loads (16 for short grids; 64 = all in one round for the
+// long-context grids, where every extra round is another trip to memory).
+template <int B>
 __global__ __launch_bounds__(256) void attn_merge_fast_kernel(const AttnArgs a, uint32_t hsp) {
     const uint32_t h = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
     const uint32_t stride = 2 + hsp, ny = a.n_wg_y;  // ny <= MERGE_MAX_Y = 64
     const float *base = a.ws + (size_t)h * ny * stride;
     const float my = lane < ny ? base[(size_t)lane * stride] : -INFINITY;
     const float ly = lane < ny ? base[(size_t)lane * stride + 1] : 0.f;
-    constexpr int B = 16;
     float v[B];
     const bool has_d = tid < a.head_size;  // head sizes up to 256: one dimension per thread
 #pragma unroll
@@ -646,7 +648,10 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
         WGML_TRY(ensure_ws(ctx, (size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4));
         a.ws = ctx->attn_ws;
         WGML_TRY(launch_fast<WAVES>(ctx, a, pl.nv, pl.km, grid));
-        attn_merge_fast_kernel<<<dim3(p.n_heads), dim3(256), 0, ctx->stream>>>(a, pl.hsp);
+        if (pl.n_wg_y > 16)
+            attn_merge_fast_kernel<64><<<dim3(p.n_heads), dim3(256), 0, ctx->stream>>>(a, pl.hsp);
+        else
+            attn_merge_fast_kernel<16><<<dim3(p.n_heads), dim3(256), 0, ctx->stream>>>(a, pl.hsp);
         WGML_CHECK_LAUNCH();
         ctx->launches++;
         return WGML_OK;
