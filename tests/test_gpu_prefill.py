@@ -197,7 +197,9 @@ def test_prefill_in_two_calls_and_in_runs_of_128(gpu):
         want = ref.forward(int(t), pos)
     m = Llama2(gpu, cfg).load(w)
     m.prefill(toks[:37])  # one call
-    m.prefill(toks[37:], start_pos=37)  # 253 tokens: runs of 128 + 125
+    m.prefill(toks[37:287], start_pos=37)  # 250 tokens: runs of 128 + 122
+    for pos in (287, 288, 289):  # and runs of a single token
+        m.prefill(toks[pos:pos + 1], start_pos=pos)
     assert_state_matches(m, ref, cfg, 290, want)
 
 
