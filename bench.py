@@ -216,8 +216,10 @@ def bench_8b_gqa(args, W, gpu):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=256)
-    ap.add_argument("--warmup", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed decode steps (default 256; 128 for --model tiny)")
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="prompt tokens before the timed steps (default 128; 16 for --model tiny)")
     ap.add_argument("--model", default="7b", choices=["7b", "tiny", "gpt2", "8b-gqa"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
@@ -230,6 +232,10 @@ def main():
                     help="only the batched prompt pass over a --warmup-token prompt, 1 untimed + "
                          "3 timed calls (for profiler runs)")
     args = ap.parse_args()
+    if args.steps is None:
+        args.steps = 128 if args.model == "tiny" else 256
+    if args.warmup is None:
+        args.warmup = 16 if args.model == "tiny" else 128
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every kernel uses a single device; "
                  "no collectives are built). Use --gpus 1.")
