@@ -801,8 +801,10 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
     a.T = T;
     a.tpad = prefill_tpad(T);
     a.accumulate = accumulate;
+    if (ctx->gemm_pending_ks)
+        return set_error(WGML_E_INVALID, "gemm_quant: the partial sums a previous product left for its "
+                                         "output were not added yet (launch_prefill_prep / launch_gemm_flush)");
     a.ks = gemm_k_split(ctx, tiles, a.kpad);
-    ctx->gemm_pending_ks = 0;
     if (a.ks > 1) {
         WGML_TRY(ensure_gemm_partials(ctx, (size_t)a.ks * T * a.total_rows * sizeof(float)));
         a.part = ctx->gemm_part;
