@@ -639,6 +639,7 @@ int wgml_llama2_prefill(wgml_llama2 *m, const uint32_t *tokens, uint32_t n_token
     const uint32_t kmax = c.dim > c.hidden_dim ? c.dim : c.hidden_dim;
     WGML_TRY(ensure_prefill_scratch(ctx, (size_t)kPrefillMaxTokens * prefill_kpad(kmax) * 2));
     const uint64_t launches0 = ctx->launches;
+    ctx->gemm_pending_ks = 0;  // nothing is owed from an earlier call that failed half way
     for (uint32_t done = 0; done < n_tokens; done += kPrefillMaxTokens) {
         const uint32_t T = n_tokens - done < kPrefillMaxTokens ? n_tokens - done : kPrefillMaxTokens;
         WGML_TRY(enqueue_prefill_run(m, tokens + done, T, start_pos + done));
