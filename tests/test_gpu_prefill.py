@@ -153,6 +153,15 @@ def spice(w, cfg, seed, biases):
     w.output_norm = (1 + 0.1 * rng.standard_normal(cfg.dim)).astype(np.float32)
 
 
+@pytest.fixture(params=[0, 1], ids=["attn16tok", "attn1tok"])
+def attn_mode(request):
+    # attention over a run: 16 tokens per workgroup on the fp32 matrix cores (head sizes that are
+    # multiples of 16 up to 128), or one workgroup per (head, token) for every head size
+    W._lib.lib.wgml_debug_set_prefill_attention(request.param)
+    yield request.param
+    W._lib.lib.wgml_debug_set_prefill_attention(0)
+
+
 def assert_state_matches(m, ref, cfg, n_pos, want_logits, tol=3e-3):
     got = m.logits()
     scale = float(np.abs(want_logits).max())
@@ -169,7 +178,7 @@ def assert_state_matches(m, ref, cfg, n_pos, want_logits, tol=3e-3):
 @pytest.mark.parametrize("scheme", ["q8_0", "q4_k", "q6_k", "q4_k_m"])
 @pytest.mark.parametrize("model_type", [LlamaModelType.Llama, LlamaModelType.Qwen2])
 @pytest.mark.parametrize("n_prompt", [1, 9, 33])
-def test_prefill_matches_stepwise_oracle(gpu, scheme, model_type, n_prompt):
+def test_prefill_matches_stepwise_oracle(gpu, attn_mode, scheme, model_type, n_prompt):
     w = synth_llama(MICRO, seed=21, scheme=scheme)
     spice(w, MICRO, 5, biases=model_type == LlamaModelType.Qwen2)
     ref = orc.Llama2(w, rope_variant=model_type)
@@ -186,7 +195,7 @@ def test_prefill_matches_stepwise_oracle(gpu, scheme, model_type, n_prompt):
     assert np.abs(got2 - want2).max() <= 3e-3 * np.abs(want2).max()
 
 
-def test_prefill_in_two_calls_and_in_runs_of_128(gpu):
+def test_prefill_in_two_calls_and_in_runs_of_128(gpu, attn_mode):
     cfg = Llama2Config(dim=256, hidden_dim=512, n_layers=2, n_q_heads=4, n_kv_heads=4,
                        vocab_size=320, seq_len=300, rope_base_freq=10000.0, rms_norm_eps=1e-5)
     w = synth_llama(cfg, seed=4, scheme="q4_k_m")
@@ -205,7 +214,7 @@ def test_prefill_in_two_calls_and_in_runs_of_128(gpu):
 
 @pytest.mark.parametrize("dim,heads,kv_heads,hidden", [(320, 4, 2, 448), (96, 2, 1, 160), (512, 4, 4, 1024),
                                                        (512, 2, 1, 768)])
-def test_prefill_head_sizes_and_partial_chunks(gpu, k_split, dim, heads, kv_heads, hidden):
+def test_prefill_head_sizes_and_partial_chunks(gpu, attn_mode, k_split, dim, heads, kv_heads, hidden):
     # head sizes 80, 48, 128 and 256; row lengths that are not multiples of 64 (Q8_0 only)
     cfg = Llama2Config(dim=dim, hidden_dim=hidden, n_layers=2, n_q_heads=heads, n_kv_heads=kv_heads,
                        vocab_size=300, seq_len=24, rope_base_freq=10000.0, rms_norm_eps=1e-5)

@@ -187,6 +187,7 @@ PROTOTYPES = {
     "wgml_debug_set_gemv_config": (_i, [_i, _i, _i, _i]),
     "wgml_debug_set_gemv_f32_activations": (_i, [_i]),
     "wgml_debug_set_gemm_k_split": (_i, [_i]),
+    "wgml_debug_set_prefill_attention": (_i, [_i]),
 }
 
 # calls whose return value is not a status code

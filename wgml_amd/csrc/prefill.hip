@@ -664,6 +664,116 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const AttnRowsArgs a) {
     }
 }
 
+// The same attention for 16 tokens of a run at once, on the fp32 matrix cores
+// (v_mfma_f32_16x16x4_f32: operands and sums are fp32, so the arithmetic stays that of the
+// step).  Workgroup (h, tb) computes head h of tokens 16 tb .. 16 tb + 15; its four waves
+// share out the blocks of 16 cache rows and merge at the end, so a K or V row is read once
+// per 16 tokens instead of once per token.  Per block of rows, with lane = (g, n):
+//   S^T[row][token] = K · Q^T : A = K rows (lane n = row, k-slot g = dimension 16 c + 4 g + e in
+//                     step (c, e)), B = Q^T (lane n = token), 4 HS16 steps -> each lane holds
+//                     the scores of rows 4 g + i (i < 4) for token n;
+//   online softmax per token: maximum and sum over the lane's 4 rows and the 4 lane groups;
+//   O^T[dim][token] += V^T · P^T : A = V^T (lane n = dimension 16 b + n, k-slot g = row 4 g + i
+//                     in step i), B = the lane's own P values -- no transposition anywhere.
+template <int HS16>
+__global__ __launch_bounds__(256) void attn_block_kernel(const AttnRowsArgs a, uint32_t T) {
+    constexpr int HS = HS16 * 16;
+    __shared__ float sm_m[4][16], sm_l[4][16];
+    __shared__ float sm_o[4][HS][17];
+    const uint32_t h = blockIdx.x, t0 = blockIdx.y * 16;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t n = lane & 15, g = lane >> 4;
+    const size_t head_off = (size_t)(h / a.kv_mul) * HS;
+    const float inv_sqrt_hs = 1.0f / sqrtf((float)HS);
+    // this lane's token (the B operand of the score product); tokens past the run repeat the last
+    const uint32_t tq = min(t0 + n, T - 1), pos_q = a.pos0 + tq;
+    const uint32_t last_pos = a.pos0 + min(t0 + 15, T - 1);  // rows 0 .. last_pos exist
+    const uint32_t nblk = last_pos / 16 + 1;
+    float4 q[HS16];
+#pragma unroll
+    for (int c = 0; c < HS16; ++c)
+        q[c] = *reinterpret_cast<const float4 *>(a.q + (size_t)tq * a.q_stride + (size_t)h * HS + 16 * c + 4 * g);
+    floatx4 acc[HS16];
+#pragma unroll
+    for (int b = 0; b < HS16; ++b) acc[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    for (uint32_t blk = wave; blk < nblk; blk += 4) {  // uniform over the wave
+        const uint32_t pbase = blk * 16;
+        const float *krow = a.kc + (size_t)min(pbase + n, last_pos) * a.kv_dim + head_off + 4 * g;
+        float4 k[HS16];
+#pragma unroll
+        for (int c = 0; c < HS16; ++c) k[c] = *reinterpret_cast<const float4 *>(krow + 16 * c);
+        float v[HS16][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float *vrow = a.vc + (size_t)min(pbase + 4 * g + i, last_pos) * a.kv_dim + head_off + n;
+#pragma unroll
+            for (int b = 0; b < HS16; ++b) v[b][i] = vrow[16 * b];
+        }
+        floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < HS16; ++c) {
+            s = __builtin_amdgcn_mfma_f32_16x16x4f32(k[c].x, q[c].x, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_16x16x4f32(k[c].y, q[c].y, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_16x16x4f32(k[c].z, q[c].z, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_16x16x4f32(k[c].w, q[c].w, s, 0, 0, 0);
+        }
+        // s[i] = score of row pbase + 4 g + i for token n; rows after the token's position do not count
+        float sc[4], mloc = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            sc[i] = pbase + 4 * g + i <= pos_q ? s[i] * inv_sqrt_hs : -INFINITY;
+            mloc = fmaxf(mloc, sc[i]);
+        }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+        const float mn = fmaxf(m, mloc);
+        const float scale = mn == -INFINITY ? 1.f : __expf(m - mn);
+        float p[4], lsum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            p[i] = sc[i] == -INFINITY ? 0.f : __expf(sc[i] - mn);
+            lsum += p[i];
+        }
+        lsum += __shfl_xor(lsum, 16, 64);
+        lsum += __shfl_xor(lsum, 32, 64);
+        l = fmaf(l, scale, lsum);
+        m = mn;
+#pragma unroll
+        for (int b = 0; b < HS16; ++b) {
+            acc[b] = floatx4{acc[b][0] * scale, acc[b][1] * scale, acc[b][2] * scale, acc[b][3] * scale};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(v[b][i], p[i], acc[b], 0, 0, 0);
+        }
+    }
+    // acc[b][i] = O^T[dimension 16 b + 4 g + i][token n] of this wave's rows; merge the four waves
+    if (g == 0) {
+        sm_m[wave][n] = m;
+        sm_l[wave][n] = l;
+    }
+#pragma unroll
+    for (int b = 0; b < HS16; ++b) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sm_o[wave][16 * b + 4 * g + i][n] = acc[b][i];
+    }
+    __syncthreads();
+    for (uint32_t idx = threadIdx.x; idx < 16 * HS; idx += 256) {
+        const uint32_t tok = idx / HS, d = idx % HS;
+        if (t0 + tok >= T) continue;
+        const float M = fmaxf(fmaxf(sm_m[0][tok], sm_m[1][tok]), fmaxf(sm_m[2][tok], sm_m[3][tok]));
+        float L = 0.f, o = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float wgt = sm_m[w][tok] == -INFINITY ? 0.f : __expf(sm_m[w][tok] - M);
+            L = fmaf(sm_l[w][tok], wgt, L);
+            o = fmaf(sm_o[w][d][tok], wgt, o);
+        }
+        a.xb[(size_t)(t0 + tok) * a.xb_stride + (size_t)h * HS + d] = o / L;
+    }
+}
+
+int g_attn_rows_per_token = 0;  // 1: one workgroup per (head, token) for every head size (tests)
 int g_force_k_split = 0;  // 0: by matrix shape; 1..8: forced (tests)
 
 // How many workgroups split K: enough that tiles x ks covers the compute units about
@@ -858,6 +968,23 @@ int launch_attention_rows(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pos
                          "attention over a run of tokens: head_size %u (multiple of 4, <= 256)",
                          p.head_size);
     AttnRowsArgs a{q, kc, vc, xb, q_stride, xb_stride, p.kv_dim, p.kv_mul, p.head_size, pos0};
+    if (p.head_size % 16 == 0 && p.head_size <= 128 && !g_attn_rows_per_token) {
+        // 16 tokens per workgroup on the fp32 matrix cores
+        const dim3 bgrid(p.n_heads, (T + 15) / 16), bblock(256);
+        switch (p.head_size / 16) {
+        case 1: attn_block_kernel<1><<<bgrid, bblock, 0, ctx->stream>>>(a, T); break;
+        case 2: attn_block_kernel<2><<<bgrid, bblock, 0, ctx->stream>>>(a, T); break;
+        case 3: attn_block_kernel<3><<<bgrid, bblock, 0, ctx->stream>>>(a, T); break;
+        case 4: attn_block_kernel<4><<<bgrid, bblock, 0, ctx->stream>>>(a, T); break;
+        case 5: attn_block_kernel<5><<<bgrid, bblock, 0, ctx->stream>>>(a, T); break;
+        case 6: attn_block_kernel<6><<<bgrid, bblock, 0, ctx->stream>>>(a, T); break;
+        case 7: attn_block_kernel<7><<<bgrid, bblock, 0, ctx->stream>>>(a, T); break;
+        default: attn_block_kernel<8><<<bgrid, bblock, 0, ctx->stream>>>(a, T); break;
+        }
+        WGML_CHECK_LAUNCH();
+        ctx->launches++;
+        return WGML_OK;
+    }
     const dim3 grid(p.n_heads, T), block(256);
     switch ((p.head_size + 63) / 64) {
     case 1: attn_rows_kernel<1><<<grid, block, 0, ctx->stream>>>(a); break;
@@ -874,6 +1001,12 @@ int launch_attention_rows(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pos
 
 extern "C" {
 
+// Test hook: 1 = the attention of a run uses one workgroup per (head, token) for every head
+// size, 0 = 16 tokens per workgroup where the head size allows it.
+WGML_API int wgml_debug_set_prefill_attention(int per_token) {
+    g_attn_rows_per_token = per_token ? 1 : 0;
+    return WGML_OK;
+}
 // Test hook: 0 = choose by matrix shape how many workgroups split K, 1..8 = that many.
 WGML_API int wgml_debug_set_gemm_k_split(int n) {
     g_force_k_split = n >= 1 && n <= 8 ? n : 0;
