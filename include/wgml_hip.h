@@ -281,8 +281,9 @@ WGML_API int wgml_llama2_decode_greedy_sync(wgml_llama2 *m, uint32_t first_token
  * step replaced by one product with up to 128 token vectors on the matrix cores
  * (wgml_gemm_quant; longer prompts go through in runs of 128).  Arithmetic: f16
  * operands, fp32 sums for the layer matrices; norms, RoPE, attention and the
- * output matrix in fp32 as in the step, so logits agree with the step-by-step
- * pass to about 1e-3 of their range rather than to fp32 rounding.  The layer matrices
+ * output matrix in fp32 as in the step.  A product is within about 3e-4 of its
+ * fp32 value; over a whole model that adds up (3e-3 of the logits' range on 2-layer
+ * models, 6e-3 on the 32-layer 7B shape) rather than staying at fp32 rounding.  The layer matrices
  * must be WGML_Q8_0, WGML_Q4_K or WGML_Q6_K (WGML_E_UNSUPPORTED otherwise).
  * Enqueues and returns. */
 WGML_API int wgml_llama2_prefill(wgml_llama2 *m, const uint32_t *tokens, uint32_t n_tokens,
