@@ -117,6 +117,20 @@ def test_gemm_7b_shapes(gpu, qtype):
     check(got2[64:], 2.0 * got[:64].astype(np.float64))
 
 
+def test_gemm_with_views_that_are_not_16_byte_aligned(gpu):
+    # x and out are views at odd offsets into larger buffers (the reference's ops take views)
+    nrows, ncols, T = 40, 512, 7
+    raw = W.quantize(W.Q4_K, W.rng_normal(1, nrows * ncols, 0, 0.02))
+    m = W.GpuQuantMatrix(gpu, W.Q4_K, nrows, ncols, raw)
+    x = W.rng_normal(2, T * ncols).reshape(T, ncols)
+    xbuf = W.GpuVector.init(gpu, np.concatenate([np.zeros(3, np.float32), x.reshape(-1)]))
+    obuf = W.GpuVector.init(gpu, np.full(5 + T * nrows, np.nan, dtype=np.float32))
+    W.GemmQuant.from_device(gpu).dispatch(obuf.rows(5, T * nrows), m, xbuf.rows(3, T * ncols), T)
+    got = obuf.read()
+    assert np.isnan(got[:5]).all()
+    check(got[5:].reshape(T, nrows), reference(W.Q4_K, raw, nrows, ncols, x))
+
+
 def test_gemm_rejects_bad_arguments(gpu):
     raw = W.quantize(W.Q8_0, W.rng_normal(1, 8 * 64, 0, 0.02))
     m = W.GpuQuantMatrix(gpu, W.Q8_0, 8, 64, raw)

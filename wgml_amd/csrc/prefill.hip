@@ -389,7 +389,9 @@ __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict_
     // Rows of up to 8 * PREP_GROUPS * PREP_THREADS columns are read once, 8 consecutive
     // columns per thread and group, and kept in registers (v); longer rows are re-read from
     // memory by the later passes.  (K is a multiple of 32 for every quantized format.)
-    const bool cached = ngroups <= PREP_GROUPS * PREP_THREADS && K % 8 == 0 && x_stride % 4 == 0;
+    const bool cached = ngroups <= PREP_GROUPS * PREP_THREADS && K % 8 == 0 && x_stride % 4 == 0 &&
+                        ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(up) |
+                          reinterpret_cast<uintptr_t>(part)) & 15u) == 0;  // 16-byte loads below
     // the product before this kernel may have left  x[t] += xscale[t] * (part[0][t] + part[1][t]
     // + ...)  to be done here (part: [part_ks][T][K], xscale[t] still that product's factor)
     const float old_scale = part_ks ? xscale[t] : 0.f;
