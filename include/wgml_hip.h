@@ -131,10 +131,14 @@ WGML_API int wgml_gemv_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, w
  * out[t] = m * x[t], with x n_tokens x ncols and out n_tokens x nrows, both row-major.
  * No counterpart in the reference, which multiplies one vector at a time
  * (GemvQuant::dispatch above); it is the building block of wgml_llama2_prefill.
- * The weights are expanded with the reference's dequantization arithmetic and
- * rounded to f16, the vectors are rounded to f16, sums are fp32: results agree
- * with n_tokens calls of wgml_gemv_quant to about 1e-3 of a row's magnitude, not
- * to the last bits.  m must be WGML_Q8_0, WGML_Q4_K or WGML_Q6_K. */
+ * The weights are expanded with the reference's dequantization arithmetic (fp32).
+ * Precision (wgml_ctx_set_gemm_precision): level 1, the default, feeds the matrix
+ * cores pairs of f16 numbers per operand (high part + low part), three MFMAs per
+ * product term group, fp32 sums: results agree with n_tokens calls of
+ * wgml_gemv_quant to fp32 rounding (about 1e-6 of a row's magnitude).  Level 0 rounds
+ * weights and vectors to f16 once: 1.6x faster, about 3e-4 of a row's magnitude
+ * (up to 1.4e-3 for single elements).  m must be WGML_Q8_0, WGML_Q4_K or WGML_Q6_K. */
+WGML_API int wgml_ctx_set_gemm_precision(wgml_ctx *ctx, int level);
 WGML_API int wgml_gemm_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, wgml_view x,
                              uint32_t n_tokens);
 

@@ -110,6 +110,7 @@ PROTOTYPES = {
     "wgml_quant_block_elems": (_u32, [_i]),
     "wgml_gemv_quant": (_i, [_P, View, _P, View]),
     "wgml_gemm_quant": (_i, [_P, View, _P, View, _u32]),
+    "wgml_ctx_set_gemm_precision": (_i, [_P, _i]),
     "wgml_dequantize": (_i, [_P, View, _P]),
     "wgml_f16_to_f32": (_i, [_P, View, _P, _u64]),
     "wgml_gemv_f32": (_i, [_P, View, View, _u32, _u32, _i, View]),

@@ -58,7 +58,9 @@ struct wgml_ctx {
     // f16 copy of the activations of a batched matrix product (+ one scale per token),
     // grown on demand
     void *prefill_xh = nullptr;
+    void *prefill_xl = nullptr;  // low parts of the same activations (inside the same allocation)
     size_t prefill_xh_bytes = 0;
+    int gemm_precise = 1;  // batched products: 1 = split-f16 operands (fp32-grade), 0 = f16
     float *prefill_xscale = nullptr;
     // partial sums of batched products whose K range is split between workgroups
     float *gemm_part = nullptr;

@@ -65,6 +65,7 @@ struct GemmArgs {
     GemmMat m[3];
     uint32_t nmat;
     const u32x4 *xh;                   // packed f16 activations (see above)
+    const u32x4 *xl;                   // their low parts in the same order (split precision only)
     const float *xscale;               // [tpad] factor to multiply a token's results with
     uint32_t ncols, kpad, T, tpad;
     int accumulate;                    // out += result
@@ -83,11 +84,34 @@ __device__ __forceinline__ half4 to_half4(float a, float b, float c, float d) {
     return h;
 }
 
+constexpr float kSplitScale = 2048.f;  // the low parts are stored times 2^11 (f16 range)
+
+__device__ __forceinline__ void pack_f16(const float (&w)[16], half8 (&a)[2]) {
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[s2][i] = (_Float16)w[8 * s2 + i];
+    }
+}
+__device__ __forceinline__ void pack_split(const float (&w)[16], half8 (&hi)[2], half8 (&lo)[2]) {
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const _Float16 h = (_Float16)w[8 * s2 + i];
+            hi[s2][i] = h;
+            lo[s2][i] = (_Float16)((w[8 * s2 + i] - (float)h) * kSplitScale);
+        }
+    }
+}
+
 // ---- weight fragments -----------------------------------------------------------
 // Lane (g, j) of a wave holds, for chunk c of row j of the tile, the 16 elements
 //     k = 64 c + 32 s2 + 8 g + 4 e + i        (s2, e in 0..1, i in 0..3)
-// load() fetches their bytes, frag() expands them as the reference's dequantize does
-// (quantization.rs:29-42, 204-244, 322-389) and rounds to f16: a4[2 s2 + e][i].
+// load() fetches their bytes, expand() computes them as the reference's dequantize does
+// (quantization.rs:29-42, 204-244, 322-389), in fp32: w[4 (2 s2 + e) + i].  They reach the
+// matrix cores either rounded to f16 (pack_f16) or as a pair of f16 numbers whose sum is the
+// fp32 value to about 2^-22 (pack_split: hi = f16(w), lo = f16((w - hi) * 2048)).
 struct GemmQ4K {
     struct Raw {
         uint4 hdr;  // d, dmin, 12 bytes of packed scales
@@ -99,7 +123,7 @@ struct GemmQ4K {
         r.hdr = *reinterpret_cast<const uint4 *>(blk);
         r.qs = *reinterpret_cast<const uint2 *>(blk + 16 + (chunk & 3) * 32 + 8 * g);
     }
-    __device__ static void frag(const Raw &r, uint32_t, uint32_t chunk, uint32_t, half4 (&a4)[4]) {
+    __device__ static void expand(const Raw &r, uint32_t, uint32_t chunk, uint32_t, float (&w)[16]) {
         const uint4 hdr = r.hdr;
         const uint32_t j = chunk & 3;
         const float d = f16_bits_to_f32((uint16_t)(hdr.x & 0xffffu));
@@ -122,14 +146,16 @@ struct GemmQ4K {
         }
         const float d1 = d * (float)s1, mm1 = dmin * (float)m1;
         const float d2 = d * (float)s2, mm2 = dmin * (float)m2;
-        auto four = [&](uint32_t q, float dd, float mm) {
-            return to_half4(dd * (float)(q & 15u) - mm, dd * (float)((q >> 8) & 15u) - mm,
-                            dd * (float)((q >> 16) & 15u) - mm, dd * (float)((q >> 24) & 15u) - mm);
+        auto four = [&](float *o, uint32_t q, float dd, float mm) {
+            o[0] = dd * (float)(q & 15u) - mm;
+            o[1] = dd * (float)((q >> 8) & 15u) - mm;
+            o[2] = dd * (float)((q >> 16) & 15u) - mm;
+            o[3] = dd * (float)((q >> 24) & 15u) - mm;
         };
-        a4[0] = four(r.qs.x, d1, mm1);
-        a4[1] = four(r.qs.y, d1, mm1);
-        a4[2] = four(r.qs.x >> 4, d2, mm2);
-        a4[3] = four(r.qs.y >> 4, d2, mm2);
+        four(w, r.qs.x, d1, mm1);
+        four(w + 4, r.qs.y, d1, mm1);
+        four(w + 8, r.qs.x >> 4, d2, mm2);
+        four(w + 12, r.qs.y >> 4, d2, mm2);
     }
 };
 
@@ -151,7 +177,7 @@ struct GemmQ6K {
         r.scw = *reinterpret_cast<const uint32_t *>(m.p2 + blk * 16 + 8 * i + 4 * (c & 1));
         r.d = *reinterpret_cast<const uint16_t *>(m.p3 + blk * 2);
     }
-    __device__ static void frag(const Raw &r, uint32_t, uint32_t chunk, uint32_t g, half4 (&a4)[4]) {
+    __device__ static void expand(const Raw &r, uint32_t, uint32_t chunk, uint32_t g, float (&w)[16]) {
         // element e = 64 (c & 1) + 32 s2 + 8 g + b of the 128-element half: quarter
         // e / 32 = 2 (c & 1) + s2 picks the nibble (high for quarters 2, 3), the bit pair of
         // qh[8 g + b] (shift 2 * quarter) and the scale (8 g + b) / 16 + 2 * quarter
@@ -166,13 +192,11 @@ struct GemmQ6K {
                 uint32_t l = e ? r.ql[s2].y : r.ql[s2].x;
                 if (hi_nib) l >>= 4;
                 const uint32_t h = (e ? r.qh.y : r.qh.x) >> hsh;
-                float v[4];
 #pragma unroll
                 for (int b = 0; b < 4; ++b) {
                     const int q = (int)(((l >> (8 * b)) & 15u) | (((h >> (8 * b)) & 3u) << 4)) - 32;
-                    v[b] = ds * (float)q;
+                    w[4 * (2 * s2 + e) + b] = ds * (float)q;
                 }
-                a4[2 * s2 + e] = to_half4(v[0], v[1], v[2], v[3]);
             }
         }
     }
@@ -195,24 +219,35 @@ struct GemmQ8_0 {
             r.d[s2] = *reinterpret_cast<const uint16_t *>(m.p1 + ((size_t)row * nb + b) * 2);
         }
     }
-    __device__ static void frag(const Raw &r, uint32_t ncols, uint32_t chunk, uint32_t, half4 (&a4)[4]) {
+    __device__ static void expand(const Raw &r, uint32_t ncols, uint32_t chunk, uint32_t, float (&w)[16]) {
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
             const bool exists = chunk * 2 + s2 < ncols / 32;
             const float d = exists ? f16_bits_to_f32((uint16_t)r.d[s2]) : 0.f;
             const uint32_t x = exists ? r.q[s2].x : 0u, y = exists ? r.q[s2].y : 0u;
-            a4[2 * s2] = to_half4(sb0(x) * d, sb1(x) * d, sb2(x) * d, sb3(x) * d);
-            a4[2 * s2 + 1] = to_half4(sb0(y) * d, sb1(y) * d, sb2(y) * d, sb3(y) * d);
+            float *o = w + 8 * s2;
+            o[0] = sb0(x) * d;
+            o[1] = sb1(x) * d;
+            o[2] = sb2(x) * d;
+            o[3] = sb3(x) * d;
+            o[4] = sb0(y) * d;
+            o[5] = sb1(y) * d;
+            o[6] = sb2(y) * d;
+            o[7] = sb3(y) * d;
         }
     }
 };
 
-template <class F, int NT>
+// SPLIT: both operands are pairs of f16 numbers (high part, low part times 2^11); the product is
+// W_hi X_hi + 2^-11 (W_hi X_lo + W_lo X_hi), three MFMAs per sub-block instead of one, which
+// leaves an error of about 2^-22 per term instead of 2^-11.
+template <class F, int NT, bool SPLIT>
 __global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a) {
-    extern __shared__ u32x4 xs[];  // [2 buffers][2 chunks][NT * 128 words]
-    constexpr uint32_t CW = NT * 128;  // words of one chunk
+    extern __shared__ u32x4 xs[];  // [2 buffers][2 chunks][high: NT * 128 words (, low: the same)]
+    constexpr uint32_t CW = NT * 128;               // words of one chunk of one part
+    constexpr uint32_t CWX = SPLIT ? 2 * CW : CW;   // words of one chunk in LDS
     constexpr uint32_t NTHREADS = KWAVES * 64;
-    constexpr int SW = (2 * CW + NTHREADS - 1) / NTHREADS;  // staged words per thread
+    constexpr int SW = (2 * CWX + NTHREADS - 1) / NTHREADS;  // staged words per thread
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t j = lane & 15, g = lane >> 4;
@@ -229,59 +264,80 @@ __global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a)
     const uint32_t c0 = min(blockIdx.y * per, nchunks), c1 = min(nchunks, c0 + per);
     const uint32_t n_it = (c1 - c0 + 1) / 2;
 
-    floatx4 acc[NT];
+    floatx4 acc[NT], accl[SPLIT ? NT : 1];
 #pragma unroll
     for (int n = 0; n < NT; ++n) acc[n] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int n = 0; n < (SPLIT ? NT : 1); ++n) accl[n] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     // Staged words of this thread: word tid + 512 q of the pair of chunks, q < SW.  All
     // loads are unconditional (chunks past the end re-read the last one and are not used).
+    // In memory the low parts form a second array behind the high parts (a.xl).
+    auto gword = [&](uint32_t first_chunk, uint32_t q) {
+        const uint32_t w = min(tid + NTHREADS * q, 2 * CWX - 1);
+        const uint32_t c = min(first_chunk + w / CWX, nchunks - 1), ww = w % CWX;
+        if (SPLIT && ww >= CW) return a.xl[(size_t)c * CW + ww - CW];
+        return a.xh[(size_t)c * CW + ww];
+    };
     u32x4 st[SW];
     typename F::Raw cur, nxt;
     if (n_it > 0) {
 #pragma unroll
-        for (int q = 0; q < SW; ++q) {
-            const uint32_t w = min(tid + NTHREADS * q, 2 * CW - 1);
-            st[q] = a.xh[(size_t)min(c0 + w / CW, nchunks - 1) * CW + w % CW];
-        }
+        for (int q = 0; q < SW; ++q) st[q] = gword(c0, q);
         F::load(cur, m, a.ncols, row, min(c0 + kh, nchunks - 1), g);
     }
     for (uint32_t it = 0; it < n_it; ++it) {
-        u32x4 *buf = xs + (it & 1) * 2 * CW;
+        u32x4 *buf = xs + (it & 1) * 2 * CWX;
 #pragma unroll
         for (int q = 0; q < SW; ++q) {
-            if (2 * CW % NTHREADS == 0 || tid + NTHREADS * q < 2 * CW) buf[tid + NTHREADS * q] = st[q];
+            if (2 * CWX % NTHREADS == 0 || tid + NTHREADS * q < 2 * CWX) buf[tid + NTHREADS * q] = st[q];
         }
         __syncthreads();
 #pragma unroll
-        for (int q = 0; q < SW; ++q) {
-            const uint32_t w = min(tid + NTHREADS * q, 2 * CW - 1);
-            st[q] = a.xh[(size_t)min(c0 + 2 * (it + 1) + w / CW, nchunks - 1) * CW + w % CW];
-        }
+        for (int q = 0; q < SW; ++q) st[q] = gword(c0 + 2 * (it + 1), q);
         F::load(nxt, m, a.ncols, row, min(c0 + 2 * (it + 1) + kh, nchunks - 1), g);
         const uint32_t c = c0 + 2 * it + kh;
         if (c < c1) {  // uniform over the wave
-            const u32x4 *bsrc = buf + kh * CW + lane;
+            const u32x4 *bsrc = buf + kh * CWX + lane;
             // the LDS words of the first half are requested before the weights are expanded,
             // those of the second half while the first half is multiplied
             u32x4 bw[NT];
 #pragma unroll
             for (int n = 0; n < NT; ++n) bw[n] = bsrc[(n * 2) * 64];
-            half4 a4[4];
-            F::frag(cur, a.ncols, c, g, a4);
+            float w[16];
+            F::expand(cur, a.ncols, c, g, w);
+            half8 ah[2], al[2];
+            if (SPLIT) {
+                pack_split(w, ah, al);
+            } else {
+                pack_f16(w, ah);
+            }
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2) {
-                half8 aw;
-                __builtin_memcpy(&aw, &a4[2 * s2], 16);
 #pragma unroll
                 for (int n = 0; n < NT; ++n) {
                     half8 b8;
                     __builtin_memcpy(&b8, &bw[n], 16);
-                    acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw, b8, acc[n], 0, 0, 0);
+                    acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah[s2], b8, acc[n], 0, 0, 0);
+                    if (SPLIT) {
+                        accl[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al[s2], b8, accl[n], 0, 0, 0);
+                        const u32x4 lw = bsrc[CW + (n * 2 + s2) * 64];
+                        half8 l8;
+                        __builtin_memcpy(&l8, &lw, 16);
+                        accl[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah[s2], l8, accl[n], 0, 0, 0);
+                    }
                     if (s2 == 0) bw[n] = bsrc[(n * 2 + 1) * 64];
                 }
             }
         }
         cur = nxt;
+    }
+    if (SPLIT) {
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[n][i] = fmaf(accl[n][i], 1.0f / kSplitScale, acc[n][i]);
+        }
     }
     // waves 4-7 hand their sums to waves 0-3 through LDS
     __syncthreads();
@@ -368,19 +424,22 @@ __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict_
                                                      const float *__restrict__ part, uint32_t part_ks,
                                                      const float *__restrict__ up,
                                                      const float *__restrict__ norm_w, float eps,
-                                                     uint4 *__restrict__ xh,
+                                                     uint4 *__restrict__ xh, uint4 *__restrict__ xl,
                                                      float *__restrict__ xscale, uint32_t K,
                                                      uint32_t kpad, uint32_t T) {
     __shared__ float red[16];
     const uint32_t t = blockIdx.x, tid = threadIdx.x, nt = gridDim.x / 16;
     // 16-byte word of (token t, columns 8 k8 .. 8 k8 + 7)
-    auto word = [&](uint32_t k8) -> uint4 & {
+    auto word_index = [&](uint32_t k8) {
         const uint32_t c = k8 >> 3, s2 = (k8 >> 2) & 1, g = k8 & 3;
-        return xh[(((size_t)c * nt + (t >> 4)) * 2 + s2) * 64 + 16 * g + (t & 15)];
+        return (((size_t)c * nt + (t >> 4)) * 2 + s2) * 64 + 16 * g + (t & 15);
     };
     const uint32_t ngroups = kpad / 8;
     if (t >= T) {
-        for (uint32_t k8 = tid; k8 < ngroups; k8 += PREP_THREADS) word(k8) = make_uint4(0, 0, 0, 0);
+        for (uint32_t k8 = tid; k8 < ngroups; k8 += PREP_THREADS) {
+            xh[word_index(k8)] = make_uint4(0, 0, 0, 0);
+            if (xl) xl[word_index(k8)] = make_uint4(0, 0, 0, 0);
+        }
         if (tid == 0) xscale[t] = 0.f;
         return;
     }
@@ -484,13 +543,22 @@ __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict_
         down *= 0.5f;
         undo *= 2.f;
     }
+    // high parts f16(v); low parts f16((v - high) * 2^11) when the split-precision product is on
     auto store = [&](uint32_t k8, const float(&f)[8]) {
-        _Float16 h[8];
+        _Float16 h[8], lo[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) h[e] = (_Float16)(f[e] * down);
+        for (int e = 0; e < 8; ++e) {
+            const float v = f[e] * down;
+            h[e] = (_Float16)v;
+            lo[e] = (_Float16)((v - (float)h[e]) * kSplitScale);
+        }
         uint4 w;
         __builtin_memcpy(&w, h, 16);
-        word(k8) = w;
+        xh[word_index(k8)] = w;
+        if (xl) {
+            __builtin_memcpy(&w, lo, 16);
+            xl[word_index(k8)] = w;
+        }
     };
     if (cached) {
 #pragma unroll
@@ -789,25 +857,42 @@ uint32_t gemm_k_split(const wgml_ctx *ctx, uint32_t tiles, uint32_t kpad) {
     return ks;
 }
 
-template <class F>
-int launch_gemm_fmt(wgml_ctx *ctx, GemmArgs &a, uint32_t tiles) {
-    const uint32_t nt = a.tpad / 16;  // token blocks: 1, 2, 4 or 8
-    const dim3 grid(tiles, a.ks), block(KWAVES * 64);
-    const size_t lds = (size_t)nt * 8192;  // 2 buffers x 2 chunks x nt x 2 KiB
-    switch (nt) {
-    case 8: gemm_lds_kernel<F, 8><<<grid, block, lds, ctx->stream>>>(a); break;
-    case 4: gemm_lds_kernel<F, 4><<<grid, block, lds, ctx->stream>>>(a); break;
-    case 2: gemm_lds_kernel<F, 2><<<grid, block, lds, ctx->stream>>>(a); break;
-    default: gemm_lds_kernel<F, 1><<<grid, block, lds, ctx->stream>>>(a); break;
+template <class F, int NT, bool SPLIT>
+int launch_gemm_kernel(wgml_ctx *ctx, const GemmArgs &a, dim3 grid) {
+    const size_t lds = (size_t)NT * 8192 * (SPLIT ? 2 : 1);  // 2 buffers x 2 chunks x NT x 2 KiB (x 2 parts)
+    static bool opted_in = false;
+    if (lds > 64 * 1024 && !opted_in) {
+        // gfx950 has 160 KB of LDS per CU; above 64 KB a kernel must opt in once
+        WGML_CHECK_HIP(hipFuncSetAttribute((const void *)gemm_lds_kernel<F, NT, SPLIT>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        opted_in = true;
     }
+    gemm_lds_kernel<F, NT, SPLIT><<<grid, dim3(KWAVES * 64), lds, ctx->stream>>>(a);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
+    return WGML_OK;
+}
+
+template <class F, bool SPLIT>
+int launch_gemm_prec(wgml_ctx *ctx, GemmArgs &a, uint32_t tiles) {
+    const dim3 grid(tiles, a.ks);
+    switch (a.tpad / 16) {  // token blocks: 1, 2, 4 or 8
+    case 8: WGML_TRY((launch_gemm_kernel<F, 8, SPLIT>(ctx, a, grid))); break;
+    case 4: WGML_TRY((launch_gemm_kernel<F, 4, SPLIT>(ctx, a, grid))); break;
+    case 2: WGML_TRY((launch_gemm_kernel<F, 2, SPLIT>(ctx, a, grid))); break;
+    default: WGML_TRY((launch_gemm_kernel<F, 1, SPLIT>(ctx, a, grid))); break;
+    }
     if (a.ks > 1 && !a.defer) {
         gemm_reduce_kernel<<<dim3((a.total_rows + 255) / 256, a.T), dim3(256), 0, ctx->stream>>>(a);
         WGML_CHECK_LAUNCH();
         ctx->launches++;
     }
     return WGML_OK;
+}
+
+template <class F>
+int launch_gemm_fmt(wgml_ctx *ctx, GemmArgs &a, uint32_t tiles) {
+    return a.xl ? launch_gemm_prec<F, true>(ctx, a, tiles) : launch_gemm_prec<F, false>(ctx, a, tiles);
 }
 
 }  // namespace
@@ -825,7 +910,10 @@ int ensure_prefill_scratch(wgml_ctx *ctx, size_t xh_bytes) {
     if (ctx->prefill_xh) ctx->retired.push_back(ctx->prefill_xh);
     ctx->prefill_xh = nullptr;
     ctx->prefill_xh_bytes = 0;
-    WGML_CHECK_HIP(hipMalloc(&ctx->prefill_xh, xh_bytes));
+    xh_bytes = (xh_bytes + 255) & ~(size_t)255;
+    // two arrays: the f16 activations and, behind them, their low parts (split precision)
+    WGML_CHECK_HIP(hipMalloc(&ctx->prefill_xh, 2 * xh_bytes));
+    ctx->prefill_xl = (char *)ctx->prefill_xh + xh_bytes;
     ctx->prefill_xh_bytes = xh_bytes;
     return WGML_OK;
 }
@@ -838,7 +926,8 @@ int launch_prefill_prep(wgml_ctx *ctx, float *x, uint32_t x_stride, const float 
     ctx->gemm_pending_ks = 0;
     prep_x_kernel<<<dim3(prefill_tpad(T)), dim3(PREP_THREADS), 0, ctx->stream>>>(
         x, x_stride, pending ? ctx->gemm_part : nullptr, pending, up, norm_w, eps,
-        reinterpret_cast<uint4 *>(xh), xscale, K, prefill_kpad(K), T);
+        reinterpret_cast<uint4 *>(xh), ctx->gemm_precise ? reinterpret_cast<uint4 *>(ctx->prefill_xl) : nullptr,
+        xscale, K, prefill_kpad(K), T);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
@@ -907,6 +996,7 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
     }
     a.nmat = (uint32_t)n;
     a.xh = reinterpret_cast<const u32x4 *>(xh);
+    a.xl = ctx->gemm_precise ? reinterpret_cast<const u32x4 *>(ctx->prefill_xl) : nullptr;
     a.xscale = xscale;
     a.ncols = first->ncols;
     a.kpad = prefill_kpad(first->ncols);
@@ -1012,6 +1102,15 @@ WGML_API int wgml_debug_set_prefill_attention(int per_token) {
 // Test hook: 0 = choose by matrix shape how many workgroups split K, 1..8 = that many.
 WGML_API int wgml_debug_set_gemm_k_split(int n) {
     g_force_k_split = n >= 1 && n <= 8 ? n : 0;
+    return WGML_OK;
+}
+
+// 1 (default): products of the batched path take both operands as pairs of f16 numbers (error
+// about 2^-22 per term, three MFMAs per sub-block); 0: plain f16 operands (2^-11, one MFMA).
+int wgml_ctx_set_gemm_precision(wgml_ctx *ctx, int level) {
+    WGML_REQUIRE(ctx != nullptr, "wgml_ctx_set_gemm_precision: null context");
+    WGML_REQUIRE(level == 0 || level == 1, "wgml_ctx_set_gemm_precision: level %d not in {0, 1}", level);
+    ctx->gemm_precise = level;
     return WGML_OK;
 }
 

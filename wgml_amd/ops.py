@@ -45,6 +45,11 @@ class GpuInstance:
     def synchronize(self) -> None:
         call("wgml_ctx_synchronize", self._h)
 
+    def set_gemm_precision(self, level: int) -> None:
+        """Batched products (GemmQuant, Llama2.prefill): 1 = split-f16 operands, results to fp32
+        rounding (default); 0 = plain f16 operands, faster, about 3e-4 of a row's magnitude."""
+        call("wgml_ctx_set_gemm_precision", self._h, level)
+
     def info(self):
         name = C.create_string_buffer(128)
         n_cu = C.c_int()
