@@ -231,6 +231,8 @@ def main():
     ap.add_argument("--prefill-only", action="store_true",
                     help="only the batched prompt pass over a --warmup-token prompt, 1 untimed + "
                          "3 timed calls (for profiler runs)")
+    ap.add_argument("--gemm-precision", type=int, default=1, choices=[0, 1],
+                    help="with --prefill-only: 1 = split-f16 operands (default), 0 = plain f16")
     args = ap.parse_args()
     if args.steps is None:
         args.steps = 128 if args.model == "tiny" else 256
@@ -282,6 +284,7 @@ def main():
     model = Llama2(gpu, cfg).load(weights)
     prompt = W.prompt_tokens(4, args.warmup, cfg.vocab_size)
     if args.prefill_only:
+        gpu.set_gemm_precision(args.gemm_precision)
         model.prefill(prompt)
         gpu.synchronize()
         t0 = time.perf_counter()
@@ -289,7 +292,8 @@ def main():
             model.prefill(prompt)
         gpu.synchronize()
         pdt = (time.perf_counter() - t0) / 3
-        print(json.dumps({"prefill_tokens": args.warmup, "ms": round(pdt * 1e3, 3),
+        print(json.dumps({"prefill_tokens": args.warmup, "gemm_precision": args.gemm_precision,
+                          "ms": round(pdt * 1e3, 3),
                           "tok_s": round(args.warmup / pdt, 1),
                           "launches": model.launches_per_token()}), flush=True)
         return
@@ -333,26 +337,32 @@ def main():
     # that agree with the step-by-step ones to ~1e-3, which nothing after this point reads.
     prefill = None
     if args.warmup >= 2:
-        model.prefill(prompt)
-        gpu.synchronize()
-        reps = 3
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            model.prefill(prompt)
-        gpu.synchronize()
-        pdt = (time.perf_counter() - t0) / reps
         layer_elems = cfg.n_layers * (2 * cfg.dim * cfg.dim + 2 * cfg.kv_dim * cfg.dim +
                                       3 * cfg.dim * cfg.hidden_dim)
         flops = 2.0 * layer_elems * args.warmup
-        prefill = {"tokens": args.warmup, "ms": round(pdt * 1e3, 3),
-                   "tok_s": round(args.warmup / pdt, 1),
-                   "TFLOP/s": round(flops / pdt * 1e-12, 1),
-                   "ms_step_by_step_at_decode_rate": round(args.warmup / tok_s * 1e3, 1),
-                   "first_token_matches_step_by_step": int(np.argmax(model.logits())) == first,
-                   "launches": model.launches_per_token()}
-        log(f"prefill: {args.warmup} tokens in {pdt * 1e3:.2f} ms -> {args.warmup / pdt:.0f} tok/s, "
-            f"{flops / pdt * 1e-12:.1f} TFLOP/s (step by step: {args.warmup / tok_s * 1e3:.0f} ms); "
-            f"first token matches: {prefill['first_token_matches_step_by_step']}")
+        stepwise_logits = None
+        prefill = {"tokens": args.warmup,
+                   "ms_step_by_step_at_decode_rate": round(args.warmup / tok_s * 1e3, 1)}
+        # level 1 (default): split-f16 operands, results to fp32 rounding; level 0: plain f16
+        for level, key in ((1, "split_f16"), (0, "plain_f16")):
+            gpu.set_gemm_precision(level)
+            model.prefill(prompt)
+            gpu.synchronize()
+            reps = 3
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                model.prefill(prompt)
+            gpu.synchronize()
+            pdt = (time.perf_counter() - t0) / reps
+            prefill[key] = {"ms": round(pdt * 1e3, 3), "tok_s": round(args.warmup / pdt, 1),
+                            "model_TFLOP/s": round(flops / pdt * 1e-12, 1),
+                            "first_token_matches_step_by_step": int(np.argmax(model.logits())) == first,
+                            "launches": model.launches_per_token()}
+            log(f"prefill ({key}): {args.warmup} tokens in {pdt * 1e3:.2f} ms -> {args.warmup / pdt:.0f} "
+                f"tok/s, {flops / pdt * 1e-12:.1f} model TFLOP/s (step by step: "
+                f"{args.warmup / tok_s * 1e3:.0f} ms); first token matches: "
+                f"{prefill[key]['first_token_matches_step_by_step']}")
+        gpu.set_gemm_precision(1)
 
     # dominant kernel: the fused gate/up launch (27% of a step), timed live over the model's
     # own per-layer matrices; the plain single-matrix Q4_K GEMV of the same shape beside it

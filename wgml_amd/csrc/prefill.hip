@@ -846,15 +846,30 @@ __global__ __launch_bounds__(256) void attn_block_kernel(const AttnRowsArgs a, u
 int g_attn_rows_per_token = 0;  // 1: one workgroup per (head, token) for every head size (tests)
 int g_force_k_split = 0;  // 0: by matrix shape; 1..8: forced (tests)
 
-// How many workgroups split K: enough that tiles x ks covers the compute units about
-// 1.5 times (two workgroups fit a unit), a power of two, and at least 4 iterations each.
-uint32_t gemm_k_split(const wgml_ctx *ctx, uint32_t tiles, uint32_t kpad) {
+// How many workgroups split K (a power of two, at least 8 iterations each).
+//   plain f16: two workgroups fit a compute unit; split while tiles x ks stays within 1.5 per unit.
+//   split f16: one workgroup per unit (128 KB of LDS); pick the ks that minimises the number
+//   of rounds the grid needs, counted in whole-K units (rounds / ks), with a charge per
+//   doubling for the partial sums it adds.
+uint32_t gemm_k_split(const wgml_ctx *ctx, uint32_t tiles, uint32_t kpad, bool split) {
     const uint32_t nchunks = kpad / KC;
     if (g_force_k_split) return min((uint32_t)g_force_k_split, max(nchunks, 1u));
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
-    uint32_t ks = 1;
-    while (ks < 8 && tiles * ks * 2 <= cu + cu / 2 && nchunks / (ks * 2) >= 8) ks *= 2;
-    return ks;
+    if (!split) {
+        uint32_t ks = 1;
+        while (ks < 8 && tiles * ks * 2 <= cu + cu / 2 && nchunks / (ks * 2) >= 8) ks *= 2;
+        return ks;
+    }
+    uint32_t best = 1;
+    float best_cost = 1e30f, charge = 0.f;
+    for (uint32_t ks = 1; ks <= 8 && (ks == 1 || nchunks / ks >= 8); ks *= 2, charge += 0.08f) {
+        const float cost = (float)((tiles * ks + cu - 1) / cu) / (float)ks + charge;
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = ks;
+        }
+    }
+    return best;
 }
 
 template <class F, int NT, bool SPLIT>
@@ -1006,7 +1021,7 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
     if (ctx->gemm_pending_ks)
         return set_error(WGML_E_INVALID, "gemm_quant: the partial sums a previous product left for its "
                                          "output were not added yet (launch_prefill_prep / launch_gemm_flush)");
-    a.ks = gemm_k_split(ctx, tiles, a.kpad);
+    a.ks = gemm_k_split(ctx, tiles, a.kpad, a.xl != nullptr);
     if (a.ks > 1) {
         WGML_TRY(ensure_gemm_partials(ctx, (size_t)a.ks * T * a.total_rows * sizeof(float)));
         a.part = ctx->gemm_part;
