@@ -68,6 +68,7 @@ struct wgml_ctx {
     // > 0: the last batched product left this many partial sums per element in gemm_part
     // for the next kernel to add to its output (launch_prefill_prep or launch_gemm_flush)
     uint32_t gemm_pending_ks = 0;
+    uint32_t gemm_pending_pair = 0;  // those sums are a gate / up pair for a gated launch_prefill_prep
     uint64_t launches = 0;  // kernels enqueued so far (diagnostics)
     // Buffers, matrices and models keep their context alive: the device objects
     // are torn down when the last reference goes, whatever order handles are
@@ -228,7 +229,9 @@ int launch_attention_rows(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pos
 // defer_reduce: when the product's K range is split between workgroups and it is a plain
 // `out += ` of one matrix, the partial sums are left for the caller's next kernel on out
 // (launch_prefill_prep or launch_gemm_flush), which must come before anything else reads out
-// or writes xscale.
+// or writes xscale.  The same for a gate / up pair (two matrices of equal height, `out =`)
+// whose next kernel is the gated launch_prefill_prep(gate out, up out): the outputs are then
+// never written.
 int launch_gemm_quant(wgml_ctx *ctx, float *out, uint32_t out_stride, const wgml_qmat *m,
                       const void *xh, const float *xscale, uint32_t T, const float *bias,
                       int accumulate, bool defer_reduce = false);

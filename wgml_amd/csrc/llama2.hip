@@ -408,7 +408,7 @@ int enqueue_prefill_run(wgml_llama2 *m, const uint32_t *tokens, uint32_t T, uint
         if (w.ffn_gate->type == w.ffn_up->type) {
             const GemmTarget gu[2] = {{w.ffn_gate, m->pf_hb, hidden, nullptr},
                                       {w.ffn_up, m->pf_hb2, hidden, nullptr}};
-            WGML_TRY(launch_gemm_quant_multi(ctx, gu, 2, xh, xs, T, 0));
+            WGML_TRY(launch_gemm_quant_multi(ctx, gu, 2, xh, xs, T, 0, true));
         } else {
             WGML_TRY(launch_gemm_quant(ctx, m->pf_hb, hidden, w.ffn_gate, xh, xs, T, nullptr, 0));
             WGML_TRY(launch_gemm_quant(ctx, m->pf_hb2, hidden, w.ffn_up, xh, xs, T, nullptr, 0));
@@ -640,6 +640,7 @@ int wgml_llama2_prefill(wgml_llama2 *m, const uint32_t *tokens, uint32_t n_token
     WGML_TRY(ensure_prefill_scratch(ctx, (size_t)kPrefillMaxTokens * prefill_kpad(kmax) * 2));
     const uint64_t launches0 = ctx->launches;
     ctx->gemm_pending_ks = 0;  // nothing is owed from an earlier call that failed half way
+    ctx->gemm_pending_pair = 0;
     for (uint32_t done = 0; done < n_tokens; done += kPrefillMaxTokens) {
         const uint32_t T = n_tokens - done < kPrefillMaxTokens ? n_tokens - done : kPrefillMaxTokens;
         WGML_TRY(enqueue_prefill_run(m, tokens + done, T, start_pos + done));

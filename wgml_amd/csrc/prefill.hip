@@ -422,6 +422,7 @@ constexpr int PREP_THREADS = 1024;
 constexpr int PREP_GROUPS = 2;  // groups of 8 columns a thread keeps in registers
 __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict__ x, uint32_t x_stride,
                                                      const float *__restrict__ part, uint32_t part_ks,
+                                                     uint32_t part_pair,
                                                      const float *__restrict__ up,
                                                      const float *__restrict__ norm_w, float eps,
                                                      uint4 *__restrict__ xh, uint4 *__restrict__ xl,
@@ -453,6 +454,9 @@ __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict_
                           reinterpret_cast<uintptr_t>(part)) & 15u) == 0;  // 16-byte loads below
     // the product before this kernel may have left  x[t] += xscale[t] * (part[0][t] + part[1][t]
     // + ...)  to be done here (part: [part_ks][T][K], xscale[t] still that product's factor)
+    // With part_pair the partial sums are 2 K wide and hold a gate product in [0, K) and an up
+    // product in [K, 2 K): the gated activation is formed from their sums, x and up are not
+    // read (only for rows that fit the registers: the launcher sees to that).
     const float old_scale = part_ks ? xscale[t] : 0.f;
     if (part_ks && !cached) {
         for (uint32_t k = tid; k < K; k += PREP_THREADS) {
@@ -475,7 +479,27 @@ __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict_
             const uint32_t k0 = 8 * (tid + i * PREP_THREADS);
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[i][e] = 0.f;
-            if (k0 < K) {
+            if (k0 < K && part_ks && part_pair) {
+                const size_t wide = 2 * (size_t)K;
+                float g8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, u8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                for (uint32_t y = 0; y < part_ks; ++y) {
+                    const float4 *pg = reinterpret_cast<const float4 *>(part + ((size_t)y * T + t) * wide + k0);
+                    const float4 *pu = reinterpret_cast<const float4 *>(part + ((size_t)y * T + t) * wide + K + k0);
+                    const float4 g0 = pg[0], g1 = pg[1], u0 = pu[0], u1 = pu[1];
+                    const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+                    const float uv[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        g8[e] += gv[e];
+                        u8[e] += uv[e];
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float xv = g8[e] * old_scale;
+                    v[i][e] = (u8[e] * old_scale) * (xv / (1.0f + expf(-xv)));
+                }
+            } else if (k0 < K) {
                 float4 *xp = reinterpret_cast<float4 *>(xr + k0);
                 float4 a0 = xp[0], a1 = xp[1];
                 if (part_ks) {
@@ -936,11 +960,18 @@ int ensure_prefill_scratch(wgml_ctx *ctx, size_t xh_bytes) {
 int launch_prefill_prep(wgml_ctx *ctx, float *x, uint32_t x_stride, const float *up,
                         const float *norm_w, float eps, void *xh, float *xscale, uint32_t K,
                         uint32_t T) {
-    // partial sums a product with defer_reduce left for x (they are K wide: x is its output)
-    const uint32_t pending = ctx->gemm_pending_ks;
+    // partial sums a product with defer_reduce left: for x (K wide; x is its output), or for a
+    // gate / up pair (2 K wide; x and up are then not read)
+    const uint32_t pending = ctx->gemm_pending_ks, pair = ctx->gemm_pending_pair;
     ctx->gemm_pending_ks = 0;
+    ctx->gemm_pending_pair = 0;
+    if (pending && pair &&
+        !(up && K % 8 == 0 && x_stride % 4 == 0 && prefill_kpad(K) / 8 <= (uint32_t)(PREP_GROUPS * PREP_THREADS) &&
+          ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(up)) & 15u) == 0))
+        return set_error(WGML_E_INVALID, "prefill_prep: pending gate/up partial sums need a gated row of at "
+                                         "most %d columns", 8 * PREP_GROUPS * PREP_THREADS);
     prep_x_kernel<<<dim3(prefill_tpad(T)), dim3(PREP_THREADS), 0, ctx->stream>>>(
-        x, x_stride, pending ? ctx->gemm_part : nullptr, pending, up, norm_w, eps,
+        x, x_stride, pending ? ctx->gemm_part : nullptr, pending, pair, up, norm_w, eps,
         reinterpret_cast<uint4 *>(xh), ctx->gemm_precise ? reinterpret_cast<uint4 *>(ctx->prefill_xl) : nullptr,
         xscale, K, prefill_kpad(K), T);
     WGML_CHECK_LAUNCH();
@@ -1026,8 +1057,16 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
         WGML_TRY(ensure_gemm_partials(ctx, (size_t)a.ks * T * a.total_rows * sizeof(float)));
         a.part = ctx->gemm_part;
         // the caller's next kernel adds the partial sums up itself (one matrix, plain += only)
-        a.defer = defer_reduce && n == 1 && accumulate && !targets[0].bias;
-        if (a.defer) ctx->gemm_pending_ks = a.ks;
+        const bool residual = n == 1 && accumulate && !targets[0].bias;
+        // a gate / up pair whose next kernel is the gated launch_prefill_prep on (gate out, up out)
+        const bool pair = n == 2 && !accumulate && !targets[0].bias && !targets[1].bias &&
+                          targets[0].m->nrows == targets[1].m->nrows && targets[0].m->nrows % 8 == 0 &&
+                          targets[0].m->nrows <= 8u * 2 * 1024;
+        a.defer = defer_reduce && (residual || pair);
+        if (a.defer) {
+            ctx->gemm_pending_ks = a.ks;
+            ctx->gemm_pending_pair = pair ? 1 : 0;
+        }
     }
     switch (first->type) {
     case WGML_Q4_K: return launch_gemm_fmt<GemmQ4K>(ctx, a, tiles);
