@@ -283,11 +283,13 @@ WGML_API int wgml_llama2_decode_greedy_sync(wgml_llama2 *m, uint32_t first_token
  * start_pos + n_tokens - 1 of every layer and the logits of the last token (read
  * them with wgml_llama2_read_logits) -- with every matrix-vector product of the
  * step replaced by one product with up to 128 token vectors on the matrix cores
- * (wgml_gemm_quant; longer prompts go through in runs of 128).  Arithmetic: f16
- * operands, fp32 sums for the layer matrices; norms, RoPE, attention and the
- * output matrix in fp32 as in the step.  A product is within about 3e-4 of its
- * fp32 value; over a whole model that adds up (3e-3 of the logits' range on 2-layer
- * models, 6e-3 on the 32-layer 7B shape) rather than staying at fp32 rounding.  The layer matrices
+ * (wgml_gemm_quant; longer prompts go through in runs of 128).  The layer matrices
+ * are multiplied at the precision set with wgml_ctx_set_gemm_precision (default:
+ * to fp32 rounding); norms, RoPE, attention and the output matrix are fp32 as in
+ * the step, so with the default the logits agree with the step-by-step pass as two
+ * fp32 implementations do (2e-4 of their range is the bound the tests use); with
+ * level 0 a product is within about 3e-4 and a whole model adds that up (3e-3 of
+ * the logits' range on 2-layer models, 6e-3 on the 32-layer 7B shape).  The layer matrices
  * must be WGML_Q8_0, WGML_Q4_K or WGML_Q6_K (WGML_E_UNSUPPORTED otherwise).
  * Enqueues and returns. */
 WGML_API int wgml_llama2_prefill(wgml_llama2 *m, const uint32_t *tokens, uint32_t n_tokens,

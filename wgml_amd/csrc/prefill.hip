@@ -7,11 +7,14 @@
 //
 //   out[t][r] = sum_k W[r][k] * X[t][k]      W: Q4_K / Q6_K / Q8_0 as stored for the GEMV
 //
-// Weights are expanded to f16 in registers with the reference's dequantization
-// arithmetic (fp32, then rounded to f16), activations are f16 (scaled per token by a
-// power of two so that they stay in range), products accumulate in fp32 on
-// v_mfma_f32_16x16x32_f16.  With f16 inputs the results differ from the fp32 path
-// by about 3e-4 of a row's RMS (the tests bound it at 1e-3).
+// Weights are expanded in registers with the reference's dequantization arithmetic (fp32),
+// activations are scaled per token by a power of two so that they stay in f16 range, products
+// accumulate in fp32 on v_mfma_f32_16x16x32_f16.  Two precisions:
+//   split f16 (default)  each operand is a pair of f16 numbers, hi = f16(v) and
+//                        lo = f16((v - hi) * 2^11); the product is
+//                        W_hi X_hi + 2^-11 (W_hi X_lo + W_lo X_hi): three MFMAs per term group,
+//                        results to fp32 rounding (about 1e-6 of a row's magnitude);
+//   plain f16            both operands rounded to f16 once, one MFMA: about 3e-4 of a row's RMS.
 //
 // Tiling.  A workgroup (8 waves) owns 64 rows of one matrix -- four blocks of 16 -- and
 // a contiguous range of K, walked in iterations of two 64-element chunks.  Per iteration
