@@ -170,6 +170,8 @@ def test_gemm_rejects_bad_arguments(gpu):
     f = W.GpuQuantMatrix(gpu, W.F16, 8, 64, np.zeros(8 * 64 * 2, dtype=np.uint8))
     with pytest.raises(W.WgmlError):
         op.dispatch(out, f, x, 3)
+    with pytest.raises(W.WgmlError):
+        gpu.set_gemm_precision(2)
 
 
 # ---- the whole prompt pass against the oracle's token-by-token steps -----------------
