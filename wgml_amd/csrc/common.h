@@ -124,7 +124,14 @@ struct DynPos {
     const uint32_t *ptr;  // if non-null, *ptr is used
     uint32_t val;
 };
-__device__ __forceinline__ uint32_t dyn_pos(const DynPos &p) { return p.ptr ? *p.ptr : p.val; }
+// The value was written by an earlier launch and does not change while a kernel that reads
+// it runs, so it is read through the constant address space: a scalar load, which takes no
+// vector-memory slot and leaves the waits on the vector loads around it exact (behind a load
+// through a generic pointer the compiler waits for every outstanding vector load).
+__device__ __forceinline__ uint32_t dyn_pos(const DynPos &p) {
+    typedef const __attribute__((address_space(4))) uint32_t *const_u32_ptr;
+    return p.ptr ? *(const_u32_ptr)(uintptr_t)p.ptr : p.val;
+}
 
 // ---- internal launchers (async on ctx->stream, raw device pointers) --------
 struct GemvEpilogue {

@@ -24,6 +24,8 @@
 //   Q6_K: 64 elements {e, e+32, e+64, e+96 : e in 16-run} of one 128-half: 16
 //         bytes of ql, 16 of ql+32, 16 of qh, 8 scale bytes, d;
 //   Q8_0: one 32-element block: 32 bytes of qs + d.
+#include <type_traits>
+
 #include "common.h"
 #include "device_utils.h"
 
@@ -641,10 +643,10 @@ struct PlainPolicy {
                          bool ok) const {
         load_group<WF, R>(w, p, ok ? g : 0u, tile);
     }
-    // Lane n holds finished result n of the segment that starts at group g0:
-    // result n belongs to row (g0 + (n / R) * GW) * R + n % R.  The operands the
-    // epilogue of the first segment needs are fetched by prefetch() at kernel start:
-    // fetched at the end they would add a memory round trip to every wave's tail.
+    // Lane n holds finished result n of the wave, whose first group is g0: result n
+    // belongs to row (g0 + (n / R) * GW) * R + n % R.  The operands the epilogue needs
+    // are fetched by prefetch() at kernel start: fetched at the end they would add a
+    // memory round trip to every wave's tail.
     float *out;
     float pre_bias, pre_out;
     template <int R>
@@ -659,15 +661,12 @@ struct PlainPolicy {
         }
     }
     template <int R>
-    __device__ void finish(float mine, uint32_t n, uint32_t g0, uint32_t GW, uint32_t lane,
-                           bool first_segment) {
+    __device__ void finish(float mine, uint32_t n, uint32_t g0, uint32_t GW, uint32_t lane) {
         const uint32_t row = (g0 + (lane / R) * GW) * R + lane % R;
         if (lane < n && row < p.nrows) {
-            float v = mine;
-            v += first_segment ? pre_bias : (p.bias ? p.bias[row] : 0.f);
+            float v = mine + pre_bias;
             if (p.act == 1) v = gelu_tanh(v);
-            v += first_segment ? pre_out : (p.accumulate ? out[row] : 0.f);
-            out[row] = v;
+            out[row] = v + pre_out;
         }
     }
 };
@@ -747,11 +746,12 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     // tile to arrive from HBM.
     typename WF::Row w[D][R];
     uint32_t lg = first, lsub = 0, ls = 0;  // (group, pass, step) of the next load
-#pragma unroll
-    for (int d = 0; d < D; ++d) {
-        const uint32_t tile = ls * 64 + lane;
-        const bool ok = (uint32_t)d < n_it;
-        pol.template load<WF, R>(w[d], lg, lsub, ok && tile < ntiles ? tile : 0u, ok);
+    // A wave's finished row sums are parked one per lane (result n in lane n) until the
+    // policy's epilogue at the end, so a wave takes at most 64 results: the host sizes
+    // the grid accordingly (plan_groups).  The loads of the first D iterations go out
+    // here; with fewer than D iterations the other register sets take a dummy load and
+    // are never consumed.
+    auto advance_load_cursor = [&]() {
         if (++ls == nsteps) {
             ls = 0;
             if (++lsub == S) {
@@ -759,6 +759,13 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
                 lg += GW;
             }
         }
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        const uint32_t tile = ls * 64 + lane;
+        const bool ok = (uint32_t)d < n_it;
+        pol.template load<WF, R>(w[d], lg, lsub, ok && tile < ntiles ? tile : 0u, ok);
+        if (ok) advance_load_cursor();
     }
 
     // Stage x as 16-bit block fixed point (two int8 planes) + per-block scale and sum.
@@ -884,36 +891,28 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     }
     if (n_it == 0) return;
 
-    typename F::X xr;
+    // XREG: a lane without a tile (rows shorter than 64 tiles) keeps an all-zero tile of
+    // x, so that the row loop needs no condition on the lane
+    typename F::X xr{};
     if (XREG && lane < ntiles) F::load_x(xr, xq + lane, meta + (size_t)lane * MF);
-    uint32_t g = first, sub = 0, step = 0;  // (group, pass, step) being computed
+    uint32_t step = 0;  // step within the row being computed
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
-    // The iterations are cut into segments of whole groups, a multiple of D long (so
-    // that register set d always holds iteration d mod D) and with at most 64
-    // results; the policy's epilogue runs between segments, never inside the loop.
-    const uint32_t per_group = S * nsteps;
-    uint32_t unit = per_group;
-    while (unit % D) unit += per_group;
-    const uint32_t unit_groups = unit / per_group;
-    const uint32_t seg_len = ((64u / (S * R)) / unit_groups) * unit;
     uint32_t nres = 0;
     float mine = 0.f;
     // one iteration on a register set: the dot products of a tile, and the row
     // reduction when the row is complete (no memory operation, LDS aside)
     auto compute = [&](typename WF::Row(&wd)[R]) {
         const uint32_t tile = step * 64 + lane;
-        if (tile < ntiles) {
-            if (XREG) {
-                F::template accumulate<R>(wd, xr, tile, acc);
-            } else {
-                typename F::X xt;
-                F::load_x(xt, xq + (size_t)step * 2 * PCH * 64 + lane, meta + (size_t)tile * MF);
-                F::template accumulate<R>(wd, xt, tile, acc);
-            }
+        if (XREG) {
+            F::template accumulate<R>(wd, xr, lane, acc);
+        } else if (tile < ntiles) {
+            typename F::X xt;
+            F::load_x(xt, xq + (size_t)step * 2 * PCH * 64 + lane, meta + (size_t)tile * MF);
+            F::template accumulate<R>(wd, xt, tile, acc);
         }
-        if (++step == nsteps) {
+        if (XREG || ++step == nsteps) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const float t = wave_sum(acc[r]) * out_scale;
@@ -922,52 +921,52 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
                 acc[r] = 0.f;
             }
             step = 0;
-            if (++sub == S) {
-                sub = 0;
-                g += GW;
-            }
         }
     };
     // refills a register set with the next triple of the load cursor
     auto refill = [&](typename WF::Row(&wd)[R]) {
         const uint32_t tile_n = ls * 64 + lane;
         pol.template load<WF, R>(wd, lg, lsub, tile_n < ntiles ? tile_n : 0u, true);
-        if (++ls == nsteps) {
-            ls = 0;
-            if (++lsub == S) {
-                lsub = 0;
-                lg += GW;
-            }
+        advance_load_cursor();
+    };
+    // The last K < 2 D iterations as straight-line code: iteration i runs on
+    // register set i mod D and refills it only if iteration i + D exists.  No load sits
+    // under a run-time condition, so every wait is for exactly the tile that is needed.
+    auto tail = [&](auto kc) {
+        constexpr int K = decltype(kc)::value;
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            compute(w[i % D]);
+            if (i + D < K) refill(w[i % D]);
         }
     };
-    for (uint32_t it0 = 0; it0 < n_it; it0 += seg_len) {
-        const uint32_t seg_end = min(n_it, it0 + seg_len);
-        const uint32_t gseg = g;
-        nres = 0;
-        uint32_t base = it0;
-        // rounds of D iterations whose refills all exist: straight-line loads
-        for (; base < seg_end && base + 2 * D <= n_it; base += D) {
+    uint32_t left = n_it;
+    // rounds of D iterations whose refills all exist
+    for (; left >= 2u * D; left -= D) {
 #pragma unroll
-            for (int d = 0; d < D; ++d) {
-                compute(w[d]);
-                refill(w[d]);
-            }
+        for (int d = 0; d < D; ++d) {
+            compute(w[d]);
+            refill(w[d]);
         }
-        // the last rounds of the launch: refills only while iterations remain (a
-        // wave cannot end before a load it issued has returned)
-        for (; base < seg_end; base += D) {
-#pragma unroll
-            for (int d = 0; d < D; ++d) {
-                const uint32_t it = base + d;
-                if (it < seg_end) compute(w[d]);
-                if (it + D < n_it) refill(w[d]);
-            }
-        }
-        // Finished row sums are parked one per lane (result n in lane n) and handed
-        // to the policy here: its loads and stores (bias, RoPE table, accumulate)
-        // stay out of the weight stream.
-        pol.template finish<R>(mine, nres, gseg, GW, lane, it0 == 0);
     }
+    switch (left) {  // 1 .. 2 D - 1
+#define WGML_TAIL_CASE(K)                                                 \
+    case K:                                                               \
+        if constexpr (K < 2 * D) tail(std::integral_constant<int, K>{});  \
+        break;
+        WGML_TAIL_CASE(1)
+        WGML_TAIL_CASE(2)
+        WGML_TAIL_CASE(3)
+        WGML_TAIL_CASE(4)
+        WGML_TAIL_CASE(5)
+        WGML_TAIL_CASE(6)
+        WGML_TAIL_CASE(7)
+#undef WGML_TAIL_CASE
+    default: break;
+    }
+    // The policy's epilogue: its loads (bias, RoPE table, the value to accumulate into)
+    // were requested at kernel start, its stores come after the last weight tile.
+    pol.template finish<R>(mine, nres, first, GW, lane);
 }
 
 template <class F, int R, int D, int MAXT>
@@ -1021,34 +1020,35 @@ struct FusedParams {
     const float2 *rope_cs;  // optional: (cos, sin) of the current position per pair of a head
 };
 
-// A group is a pair of rows, done as two single-row passes of one wave:
+// A group is a pair of rows whose tiles a wave loads together and multiplies with one
+// read of its tile of x:
 //   PLAIN / ROPE  rows 2g and 2g+1 of the matrix
-//   SILU          row g of the gate matrix, then row g of the up matrix
+//   SILU          row g of the gate matrix and row g of the up matrix
 struct JobPolicy {
-    static constexpr int S = 2;
+    static constexpr int S = 1;
     const GemvJob &j;
     const GemvParams &pa, &pb;  // plane views of the two matrices
     uint32_t pos, head_size;
     float rope_base;
     const float2 *rope_cs;
     template <class WF, int R>
-    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t sub, uint32_t tile,
+    __device__ void load(typename WF::Row (&w)[R], uint32_t g, uint32_t, uint32_t tile,
                          bool ok) const {
-        static_assert(R == 1, "fused launches make single-row passes");
+        static_assert(R == 2, "fused launches work on row pairs");
         if (!ok) g = 0;
+        const bool silu = j.mode == JOB_SILU;
         // plane pointers are picked one by one (wave-uniform selects): choosing between
         // the two parameter blocks by reference would force them into memory
-        const bool second = j.mode == JOB_SILU && sub;
         GemvParams q{};
-        q.p0 = second ? pb.p0 : pa.p0;
-        q.p1 = second ? pb.p1 : pa.p1;
-        q.p2 = second ? pb.p2 : pa.p2;
-        q.p3 = second ? pb.p3 : pa.p3;
+        q.p0 = silu ? pb.p0 : pa.p0;
+        q.p1 = silu ? pb.p1 : pa.p1;
+        q.p2 = silu ? pb.p2 : pa.p2;
+        q.p3 = silu ? pb.p3 : pa.p3;
         q.ncols = pa.ncols;
-        const uint32_t row = j.mode == JOB_SILU ? g : min(2 * g + sub, j.nrows - 1);
-        WF::load(w[0], WF::row_base(q, row), tile);
+        WF::load(w[0], WF::row_base(pa, silu ? g : 2 * g), tile);
+        WF::load(w[1], WF::row_base(q, silu ? g : min(2 * g + 1, j.nrows - 1)), tile);
     }
-    // Lanes 2i and 2i+1 hold the two pass results of group g0 + i * GW.  prefetch()
+    // Lanes 2i and 2i+1 hold the two results of group g0 + i * GW.  prefetch()
     // fetches what the epilogue of the first segment needs at kernel start.
     float pre_bias, pre_out;
     float2 pre_cs;
@@ -1074,8 +1074,7 @@ struct JobPolicy {
         }
     }
     template <int R>
-    __device__ void finish(float mine, uint32_t n, uint32_t g0, uint32_t GW, uint32_t lane,
-                           bool first_segment) {
+    __device__ void finish(float mine, uint32_t n, uint32_t g0, uint32_t GW, uint32_t lane) {
         const uint32_t g = g0 + (lane >> 1) * GW, sub = lane & 1;
         const bool valid = lane < n;
         float *out = j.out + (size_t)pos * j.out_pos_stride;
@@ -1085,23 +1084,13 @@ struct JobPolicy {
             return;
         }
         const uint32_t row = 2 * g + sub;
-        const bool store = valid && row < j.nrows;
-        float t = mine, prev = 0.f;
-        float2 c = pre_cs;
-        if (first_segment) {
-            t += pre_bias;
-            prev = pre_out;
-        } else if (store) {
-            if (j.bias) t += j.bias[row];
-            if (j.accumulate) prev = out[row];
-            if (j.mode == JOB_ROPE) c = rope_entry(row);
-        }
+        float t = mine + pre_bias;
         if (j.mode == JOB_ROPE) {  // ROPE matrices have an even number of rows
             const float other = dpp_f32<0xB1>(t);
             // (x, y) = (even row, odd row):  x' = cs x - sn y,  y' = sn x + cs y
-            t = sub ? c.y * other + c.x * t : c.x * t - c.y * other;
+            t = sub ? pre_cs.y * other + pre_cs.x * t : pre_cs.x * t - pre_cs.y * other;
         }
-        if (store) out[row] = j.accumulate ? prev + t : t;
+        if (valid && row < j.nrows) out[row] = j.accumulate ? pre_out + t : t;
     }
 };
 
@@ -1121,10 +1110,10 @@ __device__ __forceinline__ void fused_job_body(const FusedParams &P, const GemvJ
     JobPolicy pol{j, pa, pb, dyn_pos(P.pos), P.head_size, P.rope_base, P.rope_cs, 0.f, 0.f, make_float2(1.f, 0.f)};
     const uint32_t ngroups = j.mode == JOB_SILU ? j.nrows : (j.nrows + 1) / 2;
     if (P.ncols <= 64 * F::TILE)
-        gemv_i8_body<F, 1, D, true>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves,
+        gemv_i8_body<F, 2, D, true>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves,
                                     ngroups);
     else
-        gemv_i8_body<F, 1, D, false>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves,
+        gemv_i8_body<F, 2, D, false>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves,
                                      ngroups);
 }
 
@@ -1260,13 +1249,18 @@ int launch_variant(wgml_ctx *ctx, const GemvParams &p, size_t lds) {
 // `max_waves` waves: every workgroup gets the same count c (the last one the
 // remainder), and the fewest waves are active that still give every wave at most
 // ceil(c / max_waves) groups, so that the waves of a workgroup finish together.
+// A wave parks one result per lane, so it takes at most `max_per_wave` groups (64 results
+// divided by the results of a group): very tall matrices get more workgroups than the
+// machine holds at once.
 struct WgPlan {
     uint32_t groups_per_wg, active_waves, wgs;
 };
-WgPlan plan_groups(uint32_t ngroups, uint32_t max_wgs, uint32_t max_waves, uint32_t min_c = 1) {
+WgPlan plan_groups(uint32_t ngroups, uint32_t max_wgs, uint32_t max_waves, uint32_t max_per_wave,
+                   uint32_t min_c = 1) {
     if (ngroups == 0) return {1, 1, 1};
     if (max_wgs < 1) max_wgs = 1;
     uint32_t c = (ngroups + max_wgs - 1) / max_wgs;
+    if (c > max_per_wave * max_waves) c = max_per_wave * max_waves;
     // small matrices: a few groups per workgroup rather than one wave per workgroup
     const uint32_t floor_c = max_waves < 4 ? max_waves : 4;
     if (c < floor_c) c = floor_c;
@@ -1299,7 +1293,7 @@ int launch_variant_i8(wgml_ctx *ctx, const GemvParams &p0, size_t lds) {
     int per_cu = cached_blocks;
     if (g_force_wg_per_cu > 0 && g_force_wg_per_cu < per_cu) per_cu = g_force_wg_per_cu;
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
-    const WgPlan plan = plan_groups((p0.nrows + R - 1) / R, cu * (uint32_t)per_cu, MAXT / 64);
+    const WgPlan plan = plan_groups((p0.nrows + R - 1) / R, cu * (uint32_t)per_cu, MAXT / 64, 64 / R);
     GemvParams p = p0;
     p.active_waves = plan.active_waves;
     gemv_quant_i8_kernel<F, R, D, MAXT><<<dim3(plan.wgs), dim3(MAXT), lds, ctx->stream>>>(p);
@@ -1341,8 +1335,8 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
         return set_error(WGML_E_UNSUPPORTED, "gemv_quant: %u columns are too many for the folded "
                                              "LayerNorm", p.ncols);
     if (R == 2) {
-        if (depth >= 3) return launch_rd_i8<F, 2, 3>(ctx, p, lds, waves);
-        return launch_rd_i8<F, 2, 2>(ctx, p, lds, waves);
+        if (depth >= 2) return launch_rd_i8<F, 2, 2>(ctx, p, lds, waves);
+        return launch_rd_i8<F, 2, 1>(ctx, p, lds, waves);
     }
     if (depth >= 4) return launch_rd_i8<F, 1, 4>(ctx, p, lds, waves);
     if (depth == 3) return launch_rd_i8<F, 1, 3>(ctx, p, lds, waves);
@@ -1596,7 +1590,7 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
     for (int i = 0; i < f.njobs; ++i) {
         uint32_t c = (uint32_t)(hi / bpg[i]);
         if (c < 1) c = 1;
-        const WgPlan plan = plan_groups(ngroups[i], (ngroups[i] + c - 1) / c, nwaves);
+        const WgPlan plan = plan_groups(ngroups[i], (ngroups[i] + c - 1) / c, nwaves, 32);
         P.jobs[i].wg_begin = begin;
         P.jobs[i].wg_count = plan.wgs;
         P.jobs[i].active_waves = plan.active_waves;
@@ -1611,7 +1605,6 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
 }
 
 int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
-    if (g_force_depth == 2) return launch_gemv_fused_variant<2, 1024, 1>(ctx, f);
     return launch_gemv_fused_variant<1, 1024, 1>(ctx, f);
 }
 
