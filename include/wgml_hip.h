@@ -191,6 +191,18 @@ typedef struct {
 WGML_API int wgml_attention(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
                             wgml_view key_cache, wgml_view value_cache, wgml_view att,
                             wgml_view xb);
+/* No counterpart in the reference.  wgml_attention without the `att` output, for callers
+ * that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the partial results of the position-split launches live
+ * in a fixed 2 MiB array inside the library (one copy per GPU, held until the process ends)
+ * instead of a workspace from hipMalloc, and the call allocates and frees nothing.  A shape
+ * whose partial results (n_heads * workgroups per head * (head_size rounded up to 64, + 2)
+ * floats; 1.06 MB for 32 heads of 128 at 8192 positions) exceed the array is refused with
+ * WGML_E_UNSUPPORTED.  Results equal
+ * wgml_attention's.  Every call on a GPU uses that GPU's one array: calls that overlap on
+ * one GPU (two contexts, two streams) race. */
+WGML_API int wgml_attention_noalloc(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
+                                    wgml_view key_cache, wgml_view value_cache, wgml_view xb);
 
 /* Silu::dispatch (ops/silu.rs:18-34): h1 = h2 * h1 / (1 + exp(-h1)). */
 WGML_API int wgml_silu(wgml_ctx *ctx, wgml_view h1, wgml_view h2);

@@ -119,6 +119,7 @@ PROTOTYPES = {
     "wgml_rope": (_i, [_P, _i, C.POINTER(RopeConfig), View, View]),
     "wgml_softmax": (_i, [_P, View, _u32, _u32, _u32]),
     "wgml_attention": (_i, [_P, C.POINTER(AttnParams), View, View, View, View, View]),
+    "wgml_attention_noalloc": (_i, [_P, C.POINTER(AttnParams), View, View, View, View]),
     "wgml_silu": (_i, [_P, View, View]),
     "wgml_unary_inplace": (_i, [_P, _i, View, _fp]),
     "wgml_op_assign": (_i, [_P, _i, View, View]),

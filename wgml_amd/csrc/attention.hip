@@ -472,6 +472,33 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
     }
 }
 
+// Scratch of the entry point that allocates nothing (wgml_attention_noalloc): the partial
+// results (max, sum, weighted V per workgroup and head) live in this fixed array instead of a
+// workspace from hipMalloc.  Every GPU the library runs on holds its own copy for the life of
+// the process.  In host code the array's name is only a handle for hipGetSymbolAddress: the
+// device address it returns, kept per device, is what kernels and copies are given.
+constexpr size_t kNoAllocScratchBytes = 2u << 20;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices];
+
+// The device address of `scratch` on the context's device (looked up once per device, with
+// that device current).
+int noalloc_scratch(wgml_ctx *ctx, float **ptr) {
+    if (ctx->device < 0 || ctx->device >= kMaxDevices)
+        return set_error(WGML_E_UNSUPPORTED, "wgml_attention_noalloc: device %d beyond %d",
+                         ctx->device, kMaxDevices);
+    if (!g_scratch_ptr[ctx->device]) {
+        WGML_CHECK_HIP(hipSetDevice(ctx->device));
+        void *p = nullptr;
+        WGML_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return set_error(WGML_E_HIP, "wgml_attention_noalloc: null scratch address");
+        g_scratch_ptr[ctx->device] = p;
+    }
+    *ptr = reinterpret_cast<float *>(g_scratch_ptr[ctx->device]);
+    return WGML_OK;
+}
+
 int ensure_ws(wgml_ctx *ctx, size_t bytes) {
     if (bytes <= ctx->attn_ws_bytes) return WGML_OK;
     // The old buffer is kept until the context goes: recorded launches (HIP graphs)
@@ -623,10 +650,27 @@ int reserve_attention_workspace(wgml_ctx *ctx, const wgml_attn_params &p, uint32
     return ensure_ws(ctx, bytes);
 }
 
+// `ext_ws` (optional): a caller-supplied partials workspace of `ext_ws_bytes` bytes that is
+// used instead of the context's own (which is grown with hipMalloc when it is too small);
+// a plan that needs more than it holds is refused.
 int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
                              uint32_t plan_positions, uint32_t cache_rows, const float *q,
-                             const float *kc, const float *vc, float *att, float *xb) {
+                             const float *kc, const float *vc, float *att, float *xb,
+                             float *ext_ws, size_t ext_ws_bytes) {
     AttnPlan pl;
+    auto workspace = [&](size_t bytes, float **ws) -> int {
+        if (ext_ws) {
+            if (bytes > ext_ws_bytes)
+                return set_error(WGML_E_UNSUPPORTED,
+                                 "attention: this shape needs %zu bytes of partial results, the "
+                                 "fixed scratch array holds %zu", bytes, ext_ws_bytes);
+            *ws = ext_ws;
+            return WGML_OK;
+        }
+        WGML_TRY(ensure_ws(ctx, bytes));
+        *ws = ctx->attn_ws;
+        return WGML_OK;
+    };
     const bool aligned = (((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) & 15u) == 0;
     if (fast_ok(p, aligned, att != nullptr)) {
         WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl));
@@ -645,8 +689,7 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
         a.spec_rows = cache_rows;
         const dim3 grid(pl.groups, pl.n_wg_y);
         if (pl.wide) return launch_fast<16>(ctx, a, pl.nv, pl.km, grid);
-        WGML_TRY(ensure_ws(ctx, (size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4));
-        a.ws = ctx->attn_ws;
+        WGML_TRY(workspace((size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4, &a.ws));
         WGML_TRY(launch_fast<WAVES>(ctx, a, pl.nv, pl.km, grid));
         if (pl.n_wg_y > 16)
             attn_merge_fast_kernel<64><<<dim3(p.n_heads), dim3(256), 0, ctx->stream>>>(a, pl.hsp);
@@ -678,10 +721,7 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
     a.direct = (n_wg_y == 1 && att == nullptr) ? 1 : 0;
     a.ws = nullptr;
     const uint32_t hsp = pl.hsp;
-    if (!a.direct) {
-        WGML_TRY(ensure_ws(ctx, (size_t)p.n_heads * n_wg_y * (2 + hsp) * 4));
-        a.ws = ctx->attn_ws;
-    }
+    if (!a.direct) WGML_TRY(workspace((size_t)p.n_heads * n_wg_y * (2 + hsp) * 4, &a.ws));
     const dim3 grid(groups, n_wg_y);
     switch (nv) {
     case 1: WGML_TRY(launch_nv<1>(ctx, a, km, grid)); break;
@@ -701,47 +741,65 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
 int launch_attention(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos, uint32_t cache_rows,
                      const float *q, const float *kc, const float *vc, float *att, float *xb) {
     return launch_attention_planned(ctx, p, pos, pos.ptr ? p.seq_len : pos.val + 1, cache_rows, q,
-                                    kc, vc, att, xb);
+                                    kc, vc, att, xb, nullptr, 0);
 }
 
 }  // namespace wgml
 
 extern "C" {
 
-int wgml_attention(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q, wgml_view key_cache,
-                   wgml_view value_cache, wgml_view att, wgml_view xb) {
-    WGML_REQUIRE(ctx && p, "wgml_attention: null argument");
-    WGML_TRY(check_view(q, "wgml_attention: q"));
-    WGML_TRY(check_view(key_cache, "wgml_attention: key_cache"));
-    WGML_TRY(check_view(value_cache, "wgml_attention: value_cache"));
-    WGML_TRY(check_view(xb, "wgml_attention: xb"));
+static int attention_entry(const char *name, wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
+                           wgml_view key_cache, wgml_view value_cache, wgml_view att, wgml_view xb,
+                           float *ext_ws, size_t ext_ws_bytes) {
+    WGML_REQUIRE(ctx && p, "%s: null argument", name);
+    WGML_TRY(check_view(q, "attention: q"));
+    WGML_TRY(check_view(key_cache, "attention: key_cache"));
+    WGML_TRY(check_view(value_cache, "attention: value_cache"));
+    WGML_TRY(check_view(xb, "attention: xb"));
     WGML_REQUIRE(p->n_heads > 0 && p->head_size > 0 && p->kv_mul > 0 &&
                      p->n_heads % p->kv_mul == 0,
-                 "wgml_attention: bad head configuration (%u heads, kv_mul %u)", p->n_heads,
-                 p->kv_mul);
+                 "%s: bad head configuration (%u heads, kv_mul %u)", name, p->n_heads, p->kv_mul);
     WGML_REQUIRE(p->kv_dim == p->n_heads / p->kv_mul * p->head_size,
-                 "wgml_attention: kv_dim %u != n_kv_heads * head_size", p->kv_dim);
-    WGML_REQUIRE(p->pos < p->seq_len, "wgml_attention: pos %u outside seq_len %u", p->pos,
-                 p->seq_len);
+                 "%s: kv_dim %u != n_kv_heads * head_size", name, p->kv_dim);
+    WGML_REQUIRE(p->pos < p->seq_len, "%s: pos %u outside seq_len %u", name, p->pos, p->seq_len);
     const uint64_t dim = (uint64_t)p->n_heads * p->head_size;
-    WGML_REQUIRE(q.len == dim && xb.len == dim, "wgml_attention: q/xb must have %llu elements",
+    WGML_REQUIRE(q.len == dim && xb.len == dim, "%s: q/xb must have %llu elements", name,
                  (unsigned long long)dim);
     const uint64_t need = (uint64_t)(p->pos + 1) * p->kv_dim;
     WGML_REQUIRE(key_cache.len >= need && value_cache.len >= need,
-                 "wgml_attention: KV cache views shorter than (pos+1)*kv_dim");
+                 "%s: KV cache views shorter than (pos+1)*kv_dim", name);
     float *att_ptr = nullptr;
     if (att.buf) {
-        WGML_TRY(check_view(att, "wgml_attention: att"));
+        WGML_TRY(check_view(att, "attention: att"));
         WGML_REQUIRE((uint64_t)att.len >= (uint64_t)p->n_heads * p->seq_len,
-                     "wgml_attention: att needs seq_len*n_heads elements");
+                     "%s: att needs seq_len*n_heads elements", name);
         att_ptr = view_ptr(att);
     }
     DynPos pos{nullptr, p->pos};
     const uint64_t rows = (key_cache.len < value_cache.len ? key_cache.len : value_cache.len) /
                           p->kv_dim;
-    return launch_attention(ctx, *p, pos, (uint32_t)(rows < p->seq_len ? rows : p->seq_len),
-                            view_ptr(q), view_ptr(key_cache), view_ptr(value_cache), att_ptr,
-                            view_ptr(xb));
+    return launch_attention_planned(ctx, *p, pos, p->pos + 1,
+                                    (uint32_t)(rows < p->seq_len ? rows : p->seq_len), view_ptr(q),
+                                    view_ptr(key_cache), view_ptr(value_cache), att_ptr,
+                                    view_ptr(xb), ext_ws, ext_ws_bytes);
+}
+
+int wgml_attention(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q, wgml_view key_cache,
+                   wgml_view value_cache, wgml_view att, wgml_view xb) {
+    return attention_entry("wgml_attention", ctx, p, q, key_cache, value_cache, att, xb, nullptr, 0);
+}
+
+// The same launches as wgml_attention with no `att` output, partial results in the library's
+// fixed scratch array: no hipMalloc / hipFree, no memset (every partial a merge reads is
+// written by the launch before it).  Calls that overlap on one GPU share the array and race.
+int wgml_attention_noalloc(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
+                           wgml_view key_cache, wgml_view value_cache, wgml_view xb) {
+    WGML_REQUIRE(ctx != nullptr, "wgml_attention_noalloc: null context");
+    float *ws = nullptr;
+    WGML_TRY(noalloc_scratch(ctx, &ws));
+    const wgml_view no_att{nullptr, 0, 0};
+    return attention_entry("wgml_attention_noalloc", ctx, p, q, key_cache, value_cache, no_att, xb,
+                           ws, kNoAllocScratchBytes);
 }
 
 }  // extern "C"

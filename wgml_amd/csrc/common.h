@@ -198,6 +198,13 @@ int launch_rope(wgml_ctx *ctx, int variant, uint32_t head_size, uint32_t kv_dim,
 int launch_softmax(wgml_ctx *ctx, float *mat, uint32_t nrows, uint32_t ncols, uint32_t col_stride);
 int launch_attention(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos, uint32_t cache_rows,
                      const float *q, const float *kc, const float *vc, float *att, float *xb);
+// The same with the grid planned for `plan_positions` positions (seq_len when the launch is
+// recorded and replayed at growing positions).  `ext_ws`: optional caller-supplied workspace
+// for the partial results (ext_ws_bytes bytes) instead of the context's own.
+int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
+                             uint32_t plan_positions, uint32_t cache_rows, const float *q,
+                             const float *kc, const float *vc, float *att, float *xb,
+                             float *ext_ws = nullptr, size_t ext_ws_bytes = 0);
 int launch_silu(wgml_ctx *ctx, float *h1, const float *h2, uint32_t n);
 int launch_unary(wgml_ctx *ctx, int op, float *x, uint32_t n, const float *args4);
 int launch_op_assign(wgml_ctx *ctx, int op, float *a, const float *b, uint32_t n);

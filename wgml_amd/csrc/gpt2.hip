@@ -9,9 +9,6 @@
 using namespace wgml;
 
 namespace wgml {
-int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
-                             uint32_t plan_positions, uint32_t cache_rows, const float *q,
-                             const float *kc, const float *vc, float *att, float *xb);
 int reserve_attention_workspace(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions);
 }
 

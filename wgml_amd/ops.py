@@ -324,6 +324,15 @@ class BatchedMultiqueryAttention(_Op):
     def dispatch_multi(self, params, q, key_cache, value_cache, xb) -> None:
         self.dispatch(params, q, key_cache, value_cache, None, xb)
 
+    def dispatch_noalloc(self, params: BatchedMultiqueryAttentionParams, q: GpuVector,
+                         key_cache: GpuVector, value_cache: GpuVector, xb: GpuVector) -> None:
+        """`dispatch_multi` through the entry point that allocates nothing: partial results go
+        to the library's fixed scratch array (no counterpart in the reference)."""
+        p = AttnParams(params.seq_len, params.kv_dim, params.kv_mul, params.n_heads,
+                       params.head_size, params.pos)
+        call("wgml_attention_noalloc", self.gpu.handle, C.byref(p), q.view(), key_cache.view(),
+             value_cache.view(), xb.view())
+
 
 class Silu(_Op):
     """ops/silu.rs:10-44"""
