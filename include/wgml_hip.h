@@ -77,6 +77,21 @@ typedef struct {
 WGML_API int wgml_ctx_create(int device, wgml_ctx **out);
 WGML_API int wgml_ctx_destroy(wgml_ctx *ctx);
 WGML_API int wgml_ctx_synchronize(wgml_ctx *ctx);
+/* Launch-shape overrides of one context, for kernel sweeps and for tests that must reach every
+ * kernel variant; value 0 restores the heuristic.  The reference has compile-time constants in
+ * this role (USE_OPTIMIZED, ops/gemv_quant.rs:15; USE_MATMUL_ATTN, models/llama2/transformer.rs:444).
+ * Results stay within the documented tolerances for every setting. */
+enum {
+    WGML_TUNE_GEMV_ROWS_PER_WAVE = 0,        /* 1 or 2 rows of a quantized GEMV per wave and step */
+    WGML_TUNE_GEMV_WAVES_PER_WG,             /* 4, 8 or 16 */
+    WGML_TUNE_GEMV_WG_PER_CU,                /* cap on resident workgroups per compute unit */
+    WGML_TUNE_GEMV_DEPTH,                    /* weight tiles in flight per wave, 1..4 */
+    WGML_TUNE_GEMV_F32_ACTIVATIONS,          /* 1: fp32 activations instead of 16-bit block fixed point */
+    WGML_TUNE_GEMM_K_SPLIT,                  /* 1..8 workgroups share the K range of a batched product */
+    WGML_TUNE_PREFILL_ATTENTION_PER_TOKEN,   /* 1: one workgroup per (head, token) in the prompt pass */
+    WGML_TUNE_COUNT
+};
+WGML_API int wgml_ctx_set_tuning(wgml_ctx *ctx, int key, int value);
 /* Device name and compute-unit count (diagnostics). */
 WGML_API int wgml_ctx_info(wgml_ctx *ctx, char *name, size_t name_len, int *n_cu);
 

@@ -25,11 +25,18 @@ def test_every_declared_symbol_is_exported():
     raw = C.CDLL(os.fspath(_lib.LIB_PATH))
     missing = [s for s in syms if not hasattr(raw, s)]
     assert not missing, missing
+    # and nothing is exported that the header does not declare
+    import subprocess
+
+    out = subprocess.run(["nm", "-D", "--defined-only", os.fspath(_lib.LIB_PATH)], capture_output=True,
+                         text=True, check=True).stdout
+    exported = {ln.split()[-1] for ln in out.splitlines() if " T " in ln and "wgml_" in ln}
+    assert exported == set(syms), exported ^ set(syms)
 
 
 def test_binding_covers_the_header():
     declared = set(header_symbols())
-    bound = {n for n in _lib.PROTOTYPES if not n.startswith("wgml_debug_")}
+    bound = set(_lib.PROTOTYPES)
     assert declared == bound, declared ^ bound
 
 

@@ -80,6 +80,24 @@ def test_malformed_input_is_refused(tmp_path):
     struct.pack_into("<Q", bad, 8, 1 << 40)  # absurd tensor count
     with pytest.raises(W.WgmlError):
         W.Gguf(bytes(bad))
+    # counts that are smaller than the file but larger than its remaining bytes could hold
+    # (13 bytes per metadata record, 24 per tensor record at the least)
+    for off in (8, 16):
+        bad = bytearray(raw)
+        struct.pack_into("<Q", bad, off, len(raw) // 2)
+        with pytest.raises(W.WgmlError, match="implausible"):
+            W.Gguf(bytes(bad))
+    # dimensions whose product wraps around 2^64 to a small number must not pass the
+    # "lies inside the file" check
+    g = W.Gguf(bytes(raw))
+    name, t = next((n, t) for n, t in g.tensors.items() if len(t.dimensions) >= 2)
+    g.close()
+    at = bytes(raw).index(name.encode() + struct.pack("<I", len(t.dimensions)))
+    dims_off = at + len(name) + 4
+    bad = bytearray(raw)
+    struct.pack_into("<QQ", bad, dims_off, 1 << 32, 1 << 32)
+    with pytest.raises(W.WgmlError, match="implausible"):
+        W.Gguf(bytes(bad))
     with pytest.raises(W.WgmlError, match="cannot open"):
         W.Gguf(str(tmp_path / "missing.gguf"))
 

@@ -23,10 +23,10 @@ MODES = {"int_dot": 5e-4, "f32_act": 1e-4}
 
 
 @pytest.fixture(params=list(MODES))
-def mode(request):
-    W._lib.lib.wgml_debug_set_gemv_f32_activations(1 if request.param == "f32_act" else 0)
+def mode(request, gpu):
+    gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 1 if request.param == "f32_act" else 0)
     yield request.param
-    W._lib.lib.wgml_debug_set_gemv_f32_activations(0)
+    gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 0)
 
 
 def close(got, ref):
@@ -75,16 +75,26 @@ def test_gemv_q8_0_unpaired_block_counts(gpu, mode, ncols):
 
 @pytest.mark.parametrize("qtype", QT)
 @pytest.mark.parametrize("r", [1, 2])
-def test_gemv_rows_per_wave_variants(gpu, mode, qtype, r):
+@pytest.mark.parametrize("depth", [0, 2])
+def test_gemv_rows_per_wave_variants(gpu, mode, qtype, r, depth):
     nrows, ncols = 1030, 1024  # not a multiple of rows-per-workgroup
     raw = weights(qtype, nrows, ncols, 8)
     x = W.rng_normal(9, ncols)
     _, ref = orc.gemv_quant(qtype, raw, nrows, ncols, x)
-    W._lib.call("wgml_debug_set_gemv_rows_per_wave", r)
+    gpu.set_tuning(gpu.TUNE_GEMV_ROWS_PER_WAVE, r)
+    gpu.set_tuning(gpu.TUNE_GEMV_DEPTH, depth)
     try:
         ok, e = close(gemv(gpu, qtype, raw, nrows, ncols, x), ref)
+        # tall and short: many rows per wave (pipelined rounds) and fewer rows than waves
+        for nr in (40000, 24):
+            raw2 = weights(qtype, nr, 256, 11)
+            x2 = W.rng_normal(12, 256)
+            _, ref2 = orc.gemv_quant(qtype, raw2, nr, 256, x2)
+            ok2, e2 = close(gemv(gpu, qtype, raw2, nr, 256, x2), ref2)
+            assert ok2, (nr, e2)
     finally:
-        W._lib.call("wgml_debug_set_gemv_rows_per_wave", 0)
+        gpu.set_tuning(gpu.TUNE_GEMV_ROWS_PER_WAVE, 0)
+        gpu.set_tuning(gpu.TUNE_GEMV_DEPTH, 0)
     assert ok, e
 
 

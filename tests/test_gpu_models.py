@@ -248,3 +248,29 @@ def test_gpt2_micro_greedy_with_norm_affine(gpu):
     assert np.array_equal(m.generate_greedy(prompt, p.n_seq), want)
     m.set_fusion(0)
     assert np.array_equal(m.generate_greedy(prompt, p.n_seq), want)
+
+
+def test_gpt2_matrix_replaced_after_a_recorded_run(gpu):
+    # the recorded step holds device pointers of the matrices: replacing one (and freeing the
+    # old one) must re-record, not replay launches that read freed memory
+    from wgml_amd.models import _rand_matrix
+
+    p = Gpt2Params(n_vocab=300, n_seq=40, n_embd=128, n_head=4, n_layer=2, ff_len=512, attn_b=384)
+    w = synth_gpt2(p, seed=13)
+    prompt = W.prompt_tokens(13, 5, p.n_vocab)
+    m = Gpt2(gpu, p).load(w)
+    want0, _ = orc.Gpt2(w).generate_greedy(prompt, p.n_seq)
+    assert np.array_equal(m.generate_greedy(prompt, p.n_seq), want0)  # records the step
+    for name, layer, shape in (("mlp_fc_w", 0, (p.ff_len, p.n_embd)), ("attn_w", 1, (p.attn_b, p.n_embd)),
+                               ("lm_head", 0, (p.n_vocab, p.n_embd))):
+        new = _rand_matrix(9000 + layer, shape[0], shape[1], W.Q8_0, std=0.05)
+        if name == "lm_head":
+            w.lm_head = new
+        else:
+            w.layers[layer][name] = new
+        m.set_matrix(name, layer, new)  # releases the matrix it replaces
+        import gc
+        gc.collect()
+        want, _ = orc.Gpt2(w).generate_greedy(prompt, p.n_seq)
+        assert np.array_equal(m.generate_greedy(prompt, p.n_seq), want), name
+    assert not np.array_equal(want, want0)

@@ -25,12 +25,12 @@ QT = [W.Q8_0, W.Q4_K, W.Q6_K]
 
 
 @pytest.fixture(params=[0, 1, 2, 3, 8], ids=["ksplit_auto", "ksplit1", "ksplit2", "ksplit3", "ksplit8"])
-def k_split(request):
+def k_split(request, gpu):
     # workgroups that share the K range of a product (their partial sums are added by a
     # second kernel): chosen by matrix shape, or forced
-    W._lib.lib.wgml_debug_set_gemm_k_split(request.param)
+    gpu.set_tuning(gpu.TUNE_GEMM_K_SPLIT, request.param)
     yield request.param
-    W._lib.lib.wgml_debug_set_gemm_k_split(0)
+    gpu.set_tuning(gpu.TUNE_GEMM_K_SPLIT, 0)
 
 
 TOL = {"prod_rel": 1e-4, "prod_rms": 2e-5, "model": 2e-4}
@@ -194,12 +194,12 @@ def spice(w, cfg, seed, biases):
 
 
 @pytest.fixture(params=[0, 1], ids=["attn16tok", "attn1tok"])
-def attn_mode(request):
+def attn_mode(request, gpu):
     # attention over a run: 16 tokens per workgroup on the fp32 matrix cores (head sizes that are
     # multiples of 16 up to 128), or one workgroup per (head, token) for every head size
-    W._lib.lib.wgml_debug_set_prefill_attention(request.param)
+    gpu.set_tuning(gpu.TUNE_PREFILL_ATTENTION_PER_TOKEN, request.param)
     yield request.param
-    W._lib.lib.wgml_debug_set_prefill_attention(0)
+    gpu.set_tuning(gpu.TUNE_PREFILL_ATTENTION_PER_TOKEN, 0)
 
 
 def assert_state_matches(m, ref, cfg, n_pos, want_logits, tol=None):

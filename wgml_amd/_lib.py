@@ -184,12 +184,7 @@ PROTOTYPES = {
     "wgml_rng_normal": (_i, [_u64, _P, _u64, _f, _f, _i]),
     "wgml_rng_uniform_f32": (_i, [_u64, _P, _u64]),
     "wgml_rng_uniform_u32": (_i, [_u64, _P, _u64, _u32]),
-    # debug knob, not part of the reference surface
-    "wgml_debug_set_gemv_rows_per_wave": (_i, [_i]),
-    "wgml_debug_set_gemv_config": (_i, [_i, _i, _i, _i]),
-    "wgml_debug_set_gemv_f32_activations": (_i, [_i]),
-    "wgml_debug_set_gemm_k_split": (_i, [_i]),
-    "wgml_debug_set_prefill_attention": (_i, [_i]),
+    "wgml_ctx_set_tuning": (_i, [_P, _i, _i]),
 }
 
 # calls whose return value is not a status code

@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "../../include/wgml_hip.h"
@@ -42,6 +43,14 @@ int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3
 }  // namespace wgml
 
 // ---- handles ----------------------------------------------------------------
+// What a context remembers about a kernel it launches with dynamic LDS: whether it has opted
+// in to more than 64 KB, and how many workgroups fit a CU at the LDS size last used.
+struct wgml_kernel_info {
+    bool opted_in = false;
+    size_t lds = ~size_t(0);
+    int blocks_per_cu = 0;
+};
+
 struct wgml_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -70,6 +79,9 @@ struct wgml_ctx {
     uint32_t gemm_pending_ks = 0;
     uint32_t gemm_pending_pair = 0;  // those sums are a gate / up pair for a gated launch_prefill_prep
     uint64_t launches = 0;  // kernels enqueued so far (diagnostics)
+    // launch-shape overrides for sweeps and tests (wgml_ctx_set_tuning), 0 = heuristic
+    int tuning[WGML_TUNE_COUNT] = {0};
+    std::unordered_map<const void *, wgml_kernel_info> kernel_info;
     // Buffers, matrices and models keep their context alive: the device objects
     // are torn down when the last reference goes, whatever order handles are
     // destroyed in.

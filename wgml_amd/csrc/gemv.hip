@@ -1195,31 +1195,34 @@ __global__ __launch_bounds__(256) void gemv_tr_f32_kernel(const float *__restric
     out[j] = acc;
 }
 
-int g_force_r = 0;      // rows per wave, 0 = heuristic
-int g_force_waves = 0;  // waves per workgroup, 0 = heuristic
-int g_force_depth = 0;  // pipeline depth, 0 = heuristic
-int g_force_wg_per_cu = 0;
-int g_f32_activations = 0;  // 1: fp32-activation kernels instead of the integer-dot path
 constexpr size_t kMaxLds = 128 * 1024;
 
-template <class KF, int R, int D, int MAXT>
-int launch_kernel(wgml_ctx *ctx, const GemvParams &p, size_t lds, const void *fn,
-                  void (*kern)(const GemvParams), bool &opted_in, size_t &cached_lds,
-                  int &cached_blocks) {
-    if (lds > 64 * 1024 && !opted_in) {
+// Workgroups of `fn` that fit a CU with `lds` bytes of dynamic LDS (opting in to more than
+// 64 KB first); remembered per context and kernel.
+int blocks_per_cu(wgml_ctx *ctx, const void *fn, int threads, size_t lds, int *blocks) {
+    wgml_kernel_info &ki = ctx->kernel_info[fn];
+    if (lds > 64 * 1024 && !ki.opted_in) {
         // gfx950 has 160 KB of LDS per CU; above 64 KB a kernel must opt in once.
         WGML_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)kMaxLds));
-        opted_in = true;
+        ki.opted_in = true;
     }
-    if (cached_lds != lds) {  // workgroups resident per CU for this variant and LDS size
+    if (ki.lds != lds) {
         int nb = 0;
-        WGML_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fn, MAXT, lds));
-        cached_blocks = nb > 0 ? nb : 1;
-        cached_lds = lds;
+        WGML_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fn, threads, lds));
+        ki.blocks_per_cu = nb > 0 ? nb : 1;
+        ki.lds = lds;
     }
-    int per_cu = cached_blocks;
-    if (g_force_wg_per_cu > 0 && g_force_wg_per_cu < per_cu) per_cu = g_force_wg_per_cu;
+    *blocks = ki.blocks_per_cu;
+    const int cap = ctx->tuning[WGML_TUNE_GEMV_WG_PER_CU];
+    if (cap > 0 && cap < *blocks) *blocks = cap;
+    return WGML_OK;
+}
+
+template <class F, int R, int D, int MAXT>
+int launch_variant(wgml_ctx *ctx, const GemvParams &p, size_t lds) {
+    int per_cu = 1;
+    WGML_TRY(blocks_per_cu(ctx, (const void *)gemv_quant_kernel<F, R, D, MAXT>, MAXT, lds, &per_cu));
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
     const uint32_t nwaves = MAXT / 64;
     const uint32_t ngroups = (p.nrows + R - 1) / R;
@@ -1228,21 +1231,10 @@ int launch_kernel(wgml_ctx *ctx, const GemvParams &p, size_t lds, const void *fn
     const uint32_t resident_waves = cu * (uint32_t)per_cu * nwaves;
     const uint32_t k = (ngroups + resident_waves - 1) / resident_waves;
     uint32_t grid = (ngroups + nwaves * k - 1) / (nwaves * k);
-    kern<<<dim3(grid), dim3(MAXT), lds, ctx->stream>>>(p);
+    gemv_quant_kernel<F, R, D, MAXT><<<dim3(grid), dim3(MAXT), lds, ctx->stream>>>(p);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
-}
-
-template <class F, int R, int D, int MAXT>
-int launch_variant(wgml_ctx *ctx, const GemvParams &p, size_t lds) {
-    static bool opted_in = false;
-    static size_t cached_lds = ~size_t(0);
-    static int cached_blocks = 0;
-    return launch_kernel<F, R, D, MAXT>(ctx, p, lds,
-                                        (const void *)gemv_quant_kernel<F, R, D, MAXT>,
-                                        gemv_quant_kernel<F, R, D, MAXT>, opted_in, cached_lds,
-                                        cached_blocks);
 }
 
 // Shares `ngroups` row-groups out over at most `max_wgs` workgroups of up to
@@ -1275,23 +1267,8 @@ WgPlan plan_groups(uint32_t ngroups, uint32_t max_wgs, uint32_t max_waves, uint3
 
 template <class F, int R, int D, int MAXT>
 int launch_variant_i8(wgml_ctx *ctx, const GemvParams &p0, size_t lds) {
-    static bool opted_in = false;
-    static size_t cached_lds = ~size_t(0);
-    static int cached_blocks = 0;
-    const void *fn = (const void *)gemv_quant_i8_kernel<F, R, D, MAXT>;
-    if (lds > 64 * 1024 && !opted_in) {
-        WGML_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)kMaxLds));
-        opted_in = true;
-    }
-    if (cached_lds != lds) {
-        int nb = 0;
-        WGML_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fn, MAXT, lds));
-        cached_blocks = nb > 0 ? nb : 1;
-        cached_lds = lds;
-    }
-    int per_cu = cached_blocks;
-    if (g_force_wg_per_cu > 0 && g_force_wg_per_cu < per_cu) per_cu = g_force_wg_per_cu;
+    int per_cu = 1;
+    WGML_TRY(blocks_per_cu(ctx, (const void *)gemv_quant_i8_kernel<F, R, D, MAXT>, MAXT, lds, &per_cu));
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
     const WgPlan plan = plan_groups((p0.nrows + R - 1) / R, cu * (uint32_t)per_cu, MAXT / 64, 64 / R);
     GemvParams p = p0;
@@ -1326,7 +1303,8 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
     // no register ring: with 16 waves per CU one tile in flight per wave already
     // exceeds what HBM needs to stay busy, and every deeper pipeline measured
     // slower, also with exact waits (11008x4096 Q4_K: 8.4 us at depth 1, 9.4 at 2).
-    int R = g_force_r, waves = g_force_waves, depth = g_force_depth;
+    int R = ctx->tuning[WGML_TUNE_GEMV_ROWS_PER_WAVE], waves = ctx->tuning[WGML_TUNE_GEMV_WAVES_PER_WG],
+        depth = ctx->tuning[WGML_TUNE_GEMV_DEPTH];
     const bool q8 = F::TILE == 32;
     if (!R) R = 1;
     if (!waves) waves = (q8 && p.ncols <= 1024) ? 8 : 16;  // short rows: less staging per row
@@ -1365,7 +1343,8 @@ int launch_fmt(wgml_ctx *ctx, const GemvParams &p) {
         return set_error(WGML_E_UNSUPPORTED,
                          "gemv_quant: %u columns need %zu bytes of LDS (limit %zu)", p.ncols, lds,
                          kMaxLds);
-    int R = g_force_r, waves = g_force_waves, depth = g_force_depth;
+    int R = ctx->tuning[WGML_TUNE_GEMV_ROWS_PER_WAVE], waves = ctx->tuning[WGML_TUNE_GEMV_WAVES_PER_WG],
+        depth = ctx->tuning[WGML_TUNE_GEMV_DEPTH];
     if (!R) R = 1;
     if (!waves) waves = 8;
     if (!depth) depth = 2;
@@ -1422,7 +1401,7 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
     p.ln_g = ep.ln_gamma;
     p.ln_b = ep.ln_beta;
     p.act = ep.act;
-    if ((p.ln_g || p.act) && (m->type == WGML_F32 || g_f32_activations))
+    if ((p.ln_g || p.act) && (m->type == WGML_F32 || ctx->tuning[WGML_TUNE_GEMV_F32_ACTIVATIONS]))
         return set_error(WGML_E_UNSUPPORTED,
                          "gemv_quant: LayerNorm / activation folding needs the integer-dot path");
     if (m->type == WGML_F32) {
@@ -1435,7 +1414,7 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
         ctx->launches++;
         return WGML_OK;
     }
-    if (!g_f32_activations) {
+    if (!ctx->tuning[WGML_TUNE_GEMV_F32_ACTIVATIONS]) {
         switch (m->type) {
         case WGML_Q4_K: return launch_fmt_i8<IFmtQ4K>(ctx, p);
         case WGML_Q6_K: return launch_fmt_i8<IFmtQ6K>(ctx, p);
@@ -1547,22 +1526,9 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
     case WGML_Q8_0: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q8_0>; slot = 3; break;
     default: break;
     }
-    const void *fn = (const void *)kern;
-    static bool opted_in[4] = {false, false, false, false};
-    if (lds > 64 * 1024 && !opted_in[slot]) {
-        WGML_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)kMaxLds));
-        opted_in[slot] = true;
-    }
-    static size_t cached_lds_s[4] = {~size_t(0), ~size_t(0), ~size_t(0), ~size_t(0)};
-    static int cached_blocks_s[4] = {0, 0, 0, 0};
-    if (cached_lds_s[slot] != lds) {
-        int nb = 0;
-        WGML_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fn, MAXT, lds));
-        cached_blocks_s[slot] = nb > 0 ? nb : 1;
-        cached_lds_s[slot] = lds;
-    }
-    const int cached_blocks = cached_blocks_s[slot];
+    (void)slot;
+    int cached_blocks = 1;
+    WGML_TRY(blocks_per_cu(ctx, (const void *)kern, MAXT, lds, &cached_blocks));
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
     const uint32_t resident = cu * (uint32_t)cached_blocks;
     // Every workgroup streams about the same number of bytes: the smallest per-
@@ -1611,35 +1577,6 @@ int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
 }  // namespace wgml
 
 extern "C" {
-
-// Debug knobs for kernel sweeps (0 = heuristic): rows per wave, waves per
-// workgroup and a cap on resident workgroups per CU of the quantized GEMV.
-WGML_API int wgml_debug_set_gemv_rows_per_wave(int r) {
-    WGML_REQUIRE(r == 0 || r == 1 || r == 2,
-                 "wgml_debug_set_gemv_rows_per_wave: %d not in {0,1,2}", r);
-    g_force_r = r;
-    return WGML_OK;
-}
-// 1 selects the fp32-activation GEMV kernels, 0 (default) the integer-dot path.
-WGML_API int wgml_debug_set_gemv_f32_activations(int on) {
-    g_f32_activations = on ? 1 : 0;
-    return WGML_OK;
-}
-WGML_API int wgml_debug_set_gemv_config(int rows_per_wave, int waves_per_wg, int wg_per_cu,
-                                        int depth) {
-    WGML_REQUIRE(rows_per_wave == 0 || rows_per_wave == 1 || rows_per_wave == 2,
-                 "wgml_debug_set_gemv_config: rows_per_wave %d not in {0,1,2}", rows_per_wave);
-    WGML_REQUIRE(depth >= 0 && depth <= 4,
-                 "wgml_debug_set_gemv_config: depth %d not in 0..4", depth);
-    g_force_depth = depth;
-    WGML_REQUIRE(waves_per_wg == 0 || waves_per_wg == 4 || waves_per_wg == 8 || waves_per_wg == 16,
-                 "wgml_debug_set_gemv_config: waves_per_wg %d not in {0,4,8,16}", waves_per_wg);
-    WGML_REQUIRE(wg_per_cu >= 0, "wgml_debug_set_gemv_config: negative wg_per_cu");
-    g_force_r = rows_per_wave;
-    g_force_waves = waves_per_wg;
-    g_force_wg_per_cu = wg_per_cu;
-    return WGML_OK;
-}
 
 int wgml_gemv_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, wgml_view v) {
     WGML_REQUIRE(ctx && m, "wgml_gemv_quant: null argument");

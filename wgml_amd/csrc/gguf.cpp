@@ -14,6 +14,9 @@
 #include <unordered_map>
 #include <vector>
 
+#include <exception>
+#include <new>
+
 #include "common.h"
 
 using namespace wgml;
@@ -174,7 +177,11 @@ int parse(wgml_gguf *g) {
     const uint64_t n_tensors = c.pod<uint64_t>();
     const uint64_t n_meta = c.pod<uint64_t>();
     if (!c.ok) return set_error(WGML_E_INVALID, "gguf: truncated header");
-    if (n_meta > g->size || n_tensors > g->size)
+    // a metadata record takes at least 13 bytes of the file (key length, type, one value
+    // byte), a tensor record at least 24 (name length, ndims, type, offset): counts beyond
+    // what the remaining bytes can hold are refused before anything is reserved for them
+    const uint64_t remaining = g->size - c.off;
+    if (n_meta > remaining / 13 || n_tensors > remaining / 24)
         return set_error(WGML_E_INVALID, "gguf: implausible counts in the header");
     g->meta.reserve((size_t)n_meta);
     for (uint64_t i = 0; i < n_meta; ++i) {
@@ -216,8 +223,15 @@ int parse(wgml_gguf *g) {
     const uint64_t a = g->alignment;
     const uint64_t data_start = c.off + (a - c.off % a) % a;
     for (Tensor &t : g->tensors) {
+        // element count with overflow checks: a wrapped product would pass the bounds check
+        // below with dims that describe a far larger tensor
+        uint64_t n = 1;
+        bool wrapped = false;
+        for (int d = 0; d < 4; ++d) wrapped = wrapped || __builtin_mul_overflow(n, t.dims[d], &n);
+        if (wrapped || n > (uint64_t)1 << 48 || t.offset > g->size)
+            return set_error(WGML_E_INVALID, "gguf: tensor '%s' has implausible dimensions or offset",
+                             t.name.c_str());
         t.offset += data_start;
-        const uint64_t n = t.dims[0] * t.dims[1] * t.dims[2] * t.dims[3];
         t.nbytes = tensor_bytes(t.type, n);
         if (t.offset > g->size || t.nbytes > g->size - t.offset)
             return set_error(WGML_E_INVALID, "gguf: tensor '%s' lies outside the file",
@@ -233,10 +247,20 @@ extern "C" {
 int wgml_gguf_open_bytes(const void *bytes, uint64_t size, wgml_gguf **out) {
     WGML_REQUIRE(bytes && out, "wgml_gguf_open_bytes: null argument");
     *out = nullptr;
-    wgml_gguf *g = new wgml_gguf();
-    g->bytes = static_cast<const uint8_t *>(bytes);
-    g->size = size;
-    const int rc = parse(g);
+    // no C++ exception may cross the C boundary: a file that makes the tables run out of
+    // memory is reported like any other unreadable file
+    wgml_gguf *g = nullptr;
+    int rc;
+    try {
+        g = new wgml_gguf();
+        g->bytes = static_cast<const uint8_t *>(bytes);
+        g->size = size;
+        rc = parse(g);
+    } catch (const std::bad_alloc &) {
+        rc = set_error(WGML_E_OOM, "wgml_gguf_open: out of memory while reading the tables");
+    } catch (const std::exception &e) {
+        rc = set_error(WGML_E_INVALID, "wgml_gguf_open: %s", e.what());
+    }
     if (rc != WGML_OK) {
         delete g;
         return rc;

@@ -67,6 +67,10 @@ int check_ready(const wgml_gpt2 *m) {
 
 }  // namespace
 
+namespace {
+void drop_graph(wgml_gpt2 *m);  // recorded launches hold device pointers
+}
+
 extern "C" {
 
 int wgml_gpt2_create(wgml_ctx *ctx, const wgml_gpt2_params *p, wgml_gpt2 **out) {
@@ -144,6 +148,7 @@ int wgml_gpt2_set_matrix(wgml_gpt2 *m, int which, uint32_t layer, const wgml_qma
     WGML_REQUIRE(mat->nrows == er && mat->ncols == ec,
                  "wgml_gpt2_set_matrix: matrix %d is %ux%u, expected %ux%u", which, mat->nrows,
                  mat->ncols, er, ec);
+    drop_graph(m);  // a recorded step holds the plane pointers of the matrix it replaces
     if (which == WGML_GPT2_LM_HEAD) {
         m->lm_head = mat;
         return WGML_OK;
@@ -184,7 +189,10 @@ int wgml_gpt2_set_vector(wgml_gpt2 *m, int which, uint32_t layer, const float *h
     }
     WGML_REQUIRE(len == expect, "wgml_gpt2_set_vector: vector %d has %u elements, expected %u",
                  which, len, expect);
-    if (!*slot) WGML_TRY(dev_alloc(m, slot, len, false));
+    if (!*slot) {
+        WGML_TRY(dev_alloc(m, slot, len, false));
+        drop_graph(m);  // a step recorded without this vector (optional biases) is stale
+    }
     WGML_CHECK_HIP(hipMemcpyAsync(*slot, host, (size_t)len * 4, hipMemcpyHostToDevice,
                                   m->ctx->stream));
     WGML_CHECK_HIP(hipStreamSynchronize(m->ctx->stream));
@@ -194,6 +202,7 @@ int wgml_gpt2_set_vector(wgml_gpt2 *m, int which, uint32_t layer, const float *h
 int wgml_gpt2_set_embeddings(wgml_gpt2 *m, const float *wte, const float *wpe) {
     WGML_REQUIRE(m && wte && wpe, "wgml_gpt2_set_embeddings: null argument");
     const uint64_t nt = (uint64_t)m->p.n_embd * m->p.n_vocab, np = (uint64_t)m->p.n_embd * m->p.n_seq;
+    if (!m->wte || !m->wpe) drop_graph(m);
     if (!m->wte) WGML_TRY(dev_alloc(m, &m->wte, nt, false));
     if (!m->wpe) WGML_TRY(dev_alloc(m, &m->wpe, np, false));
     WGML_CHECK_HIP(hipMemcpyAsync(m->wte, wte, nt * 4, hipMemcpyHostToDevice, m->ctx->stream));

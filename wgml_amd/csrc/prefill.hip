@@ -870,8 +870,6 @@ __global__ __launch_bounds__(256) void attn_block_kernel(const AttnRowsArgs a, u
     }
 }
 
-int g_attn_rows_per_token = 0;  // 1: one workgroup per (head, token) for every head size (tests)
-int g_force_k_split = 0;  // 0: by matrix shape; 1..8: forced (tests)
 
 // How many workgroups split K (a power of two, at least 8 iterations each).
 //   plain f16: two workgroups fit a compute unit; split while tiles x ks stays within 1.5 per unit.
@@ -880,7 +878,8 @@ int g_force_k_split = 0;  // 0: by matrix shape; 1..8: forced (tests)
 //   doubling for the partial sums it adds.
 uint32_t gemm_k_split(const wgml_ctx *ctx, uint32_t tiles, uint32_t kpad, bool split) {
     const uint32_t nchunks = kpad / KC;
-    if (g_force_k_split) return min((uint32_t)g_force_k_split, max(nchunks, 1u));
+    const int forced = ctx->tuning[WGML_TUNE_GEMM_K_SPLIT];  // 0: by matrix shape
+    if (forced) return min((uint32_t)forced, max(nchunks, 1u));
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
     if (!split) {
         uint32_t ks = 1;
@@ -902,12 +901,12 @@ uint32_t gemm_k_split(const wgml_ctx *ctx, uint32_t tiles, uint32_t kpad, bool s
 template <class F, int NT, bool SPLIT>
 int launch_gemm_kernel(wgml_ctx *ctx, const GemmArgs &a, dim3 grid) {
     const size_t lds = (size_t)NT * 8192 * (SPLIT ? 2 : 1);  // 2 buffers x 2 chunks x NT x 2 KiB (x 2 parts)
-    static bool opted_in = false;
-    if (lds > 64 * 1024 && !opted_in) {
+    wgml_kernel_info &ki = ctx->kernel_info[(const void *)gemm_lds_kernel<F, NT, SPLIT>];
+    if (lds > 64 * 1024 && !ki.opted_in) {
         // gfx950 has 160 KB of LDS per CU; above 64 KB a kernel must opt in once
         WGML_CHECK_HIP(hipFuncSetAttribute((const void *)gemm_lds_kernel<F, NT, SPLIT>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        opted_in = true;
+        ki.opted_in = true;
     }
     gemm_lds_kernel<F, NT, SPLIT><<<grid, dim3(KWAVES * 64), lds, ctx->stream>>>(a);
     WGML_CHECK_LAUNCH();
@@ -1117,7 +1116,7 @@ int launch_attention_rows(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pos
                          "attention over a run of tokens: head_size %u (multiple of 4, <= 256)",
                          p.head_size);
     AttnRowsArgs a{q, kc, vc, xb, q_stride, xb_stride, p.kv_dim, p.kv_mul, p.head_size, pos0};
-    if (p.head_size % 16 == 0 && p.head_size <= 128 && !g_attn_rows_per_token) {
+    if (p.head_size % 16 == 0 && p.head_size <= 128 && !ctx->tuning[WGML_TUNE_PREFILL_ATTENTION_PER_TOKEN]) {
         // 16 tokens per workgroup on the fp32 matrix cores
         const dim3 bgrid(p.n_heads, (T + 15) / 16), bblock(256);
         switch (p.head_size / 16) {
@@ -1150,18 +1149,6 @@ int launch_attention_rows(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pos
 
 extern "C" {
 
-// Test hook: 1 = the attention of a run uses one workgroup per (head, token) for every head
-// size, 0 = 16 tokens per workgroup where the head size allows it.
-WGML_API int wgml_debug_set_prefill_attention(int per_token) {
-    g_attn_rows_per_token = per_token ? 1 : 0;
-    return WGML_OK;
-}
-// Test hook: 0 = choose by matrix shape how many workgroups split K, 1..8 = that many.
-WGML_API int wgml_debug_set_gemm_k_split(int n) {
-    g_force_k_split = n >= 1 && n <= 8 ? n : 0;
-    return WGML_OK;
-}
-
 // 1 (default): products of the batched path take both operands as pairs of f16 numbers (error
 // about 2^-22 per term, three MFMAs per sub-block); 0: plain f16 operands (2^-11, one MFMA).
 int wgml_ctx_set_gemm_precision(wgml_ctx *ctx, int level) {
@@ -1187,6 +1174,10 @@ int wgml_gemm_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, wgml_view 
                  n_tokens, m->nrows);
     const size_t xh_bytes = (size_t)kPrefillMaxTokens * prefill_kpad(m->ncols) * 2;
     WGML_TRY(ensure_prefill_scratch(ctx, xh_bytes));
+    // a prompt pass that failed half way may have left partial sums owed to its next packing
+    // kernel: they are not this product's (the packing kernel would add them to x)
+    ctx->gemm_pending_ks = 0;
+    ctx->gemm_pending_pair = 0;
     WGML_TRY(launch_prefill_prep(ctx, view_ptr(x), m->ncols, nullptr, nullptr, 0.f, ctx->prefill_xh,
                                  ctx->prefill_xscale, m->ncols, n_tokens));
     return launch_gemm_quant(ctx, view_ptr(out), m->nrows, m, ctx->prefill_xh, ctx->prefill_xscale,

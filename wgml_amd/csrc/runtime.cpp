@@ -99,6 +99,26 @@ int wgml_ctx_destroy(wgml_ctx *ctx) {
     return WGML_OK;
 }
 
+// Launch-shape overrides of one context, for kernel sweeps and for tests that must reach
+// every kernel variant.  0 restores the heuristic.
+int wgml_ctx_set_tuning(wgml_ctx *ctx, int key, int value) {
+    WGML_REQUIRE(ctx != nullptr, "wgml_ctx_set_tuning: null context");
+    WGML_REQUIRE(key >= 0 && key < WGML_TUNE_COUNT, "wgml_ctx_set_tuning: unknown key %d", key);
+    bool ok = value >= 0;
+    switch (key) {
+    case WGML_TUNE_GEMV_ROWS_PER_WAVE: ok = value >= 0 && value <= 2; break;
+    case WGML_TUNE_GEMV_WAVES_PER_WG: ok = value == 0 || value == 4 || value == 8 || value == 16; break;
+    case WGML_TUNE_GEMV_DEPTH: ok = value >= 0 && value <= 4; break;
+    case WGML_TUNE_GEMV_F32_ACTIVATIONS:
+    case WGML_TUNE_PREFILL_ATTENTION_PER_TOKEN: ok = value == 0 || value == 1; break;
+    case WGML_TUNE_GEMM_K_SPLIT: ok = value >= 0 && value <= 8; break;
+    default: break;
+    }
+    WGML_REQUIRE(ok, "wgml_ctx_set_tuning: value %d is not valid for key %d", value, key);
+    ctx->tuning[key] = value;
+    return WGML_OK;
+}
+
 int wgml_ctx_synchronize(wgml_ctx *ctx) {
     WGML_REQUIRE(ctx != nullptr, "wgml_ctx_synchronize: null context");
     WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));

@@ -271,21 +271,17 @@ class Gpt2:
         call("wgml_gpt2_create", gpu.handle, C.byref(p), C.byref(h))
         self._h = h
         self._mats: List[GpuQuantMatrix] = []
+        self._slots: Dict[Tuple[str, int], GpuQuantMatrix] = {}
 
     def load(self, w: Gpt2HostWeights) -> "Gpt2":
         for l, layer in enumerate(w.layers):
             for name, v in layer.items():
                 if isinstance(v, HostMatrix):
-                    qm = GpuQuantMatrix(self.gpu, v.qtype, v.nrows, v.ncols, v.data)
-                    self._mats.append(qm)
-                    call("wgml_gpt2_set_matrix", self._h, _GPT2_MAT_ID[name], l, qm.handle)
+                    self.set_matrix(name, l, v)
                 else:
                     a = np.ascontiguousarray(v, dtype=np.float32)
                     call("wgml_gpt2_set_vector", self._h, _GPT2_VEC_ID[name], l, _ptr(a), a.size)
-        qm = GpuQuantMatrix(self.gpu, w.lm_head.qtype, w.lm_head.nrows, w.lm_head.ncols,
-                            w.lm_head.data)
-        self._mats.append(qm)
-        call("wgml_gpt2_set_matrix", self._h, _GPT2_LM_HEAD, 0, qm.handle)
+        self.set_matrix("lm_head", 0, w.lm_head)
         for which, v in ((_GPT2_LN_F_G, w.ln_f_g), (_GPT2_LN_F_B, w.ln_f_b)):
             a = np.ascontiguousarray(v, dtype=np.float32)
             call("wgml_gpt2_set_vector", self._h, which, 0, _ptr(a), a.size)
@@ -293,6 +289,18 @@ class Gpt2:
         wpe = np.ascontiguousarray(w.wpe, dtype=np.float32)
         call("wgml_gpt2_set_embeddings", self._h, _ptr(wte), _ptr(wpe))
         return self
+
+    def set_matrix(self, name: str, layer: int, hm: HostMatrix) -> None:
+        """Sets or replaces one matrix ("lm_head" or a per-layer name of GPT2_MATS); a matrix
+        it replaces is released."""
+        qm = GpuQuantMatrix(self.gpu, hm.qtype, hm.nrows, hm.ncols, hm.data)
+        which = _GPT2_LM_HEAD if name == "lm_head" else _GPT2_MAT_ID[name]
+        call("wgml_gpt2_set_matrix", self._h, which, layer, qm.handle)
+        old = self._slots.get((name, layer))
+        self._slots[(name, layer)] = qm
+        self._mats.append(qm)
+        if old is not None:
+            self._mats.remove(old)
 
     @classmethod
     def from_gguf(cls, gpu: GpuInstance, gguf) -> "Gpt2":

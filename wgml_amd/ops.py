@@ -45,6 +45,14 @@ class GpuInstance:
     def synchronize(self) -> None:
         call("wgml_ctx_synchronize", self._h)
 
+    # keys of set_tuning (enum WGML_TUNE_* of the C header, same order)
+    (TUNE_GEMV_ROWS_PER_WAVE, TUNE_GEMV_WAVES_PER_WG, TUNE_GEMV_WG_PER_CU, TUNE_GEMV_DEPTH,
+     TUNE_GEMV_F32_ACTIVATIONS, TUNE_GEMM_K_SPLIT, TUNE_PREFILL_ATTENTION_PER_TOKEN) = range(7)
+
+    def set_tuning(self, key: int, value: int) -> None:
+        """Launch-shape override of this context (0 = heuristic); for sweeps and tests."""
+        call("wgml_ctx_set_tuning", self._h, key, value)
+
     def set_gemm_precision(self, level: int) -> None:
         """Batched products (GemmQuant, Llama2.prefill): 1 = split-f16 operands, results to fp32
         rounding (default); 0 = plain f16 operands, faster, about 3e-4 of a row's magnitude."""
