@@ -4,20 +4,27 @@
 Workload (default): Llama-2-7B shape (dim 4096, 32 layers, 32 heads, FFN 11008,
 vocab 32000), weights seeded N(0, 0.02) quantized with the ggml reference
 quantizers in a Q4_K_M-style mix (Q4_K; Q6_K for attn_v, output and the
-ffn_down layers picked by use_more_bits), embedding f32, activations and KV
-cache f32.  `--warmup` prompt tokens are pushed through the decoder one at a
-time (untimed), then exactly `--steps` greedy decode steps are timed: one step =
-one token = one pass over every weight.
+ffn_down layers picked by use_more_bits), embedding f32, KV cache f32.  The
+128-token prompt always goes through the batched prompt pass (untimed here,
+timed on its own below), then `--warmup` greedy decode steps run untimed from
+position 128, then exactly `--steps` greedy decode steps are timed: one step =
+one token = one pass over every weight.  The flags never change the workload's
+shape, only how many steps of it are timed.
 
-Prints ONE JSON line: decode tok/s, the HBM roofline of the dominant kernel
-(gemv_fused_kernel as launched for the gate/up projections: two Q4_K 11008x4096
-matrices, RMSNorm folded into the staging of x, SiLU gating in the epilogue)
-measured with HIP events on the library's own stream over the model's 32
-layers, a GEMV sweep over the model's four matrix shapes for the three formats,
-and the CPU baseline (the single-threaded C restatement of the reference's CPU
-transformer) timed on this host on a bounded sample.
+Prints ONE JSON line: decode tok/s; what arithmetic ran (`dtype`: the GEMVs
+multiply the quantized weights with activations rounded to 16-bit block fixed
+point on the integer dot-product units and accumulate in i32 / f32) with the
+same decode on fp32 activations beside it; the logit error of the GPU step
+against the CPU oracle on the positions the CPU baseline runs; the HBM roofline
+of the dominant kernel (gemv_fused_kernel as launched for the gate/up
+projections) measured with HIP events on the library's own stream, launch by
+launch as rocprofv3 sees it, and inside a recorded graph as the decode loop
+runs it; a GEMV sweep over the model's four matrix shapes for the three
+formats, on the GPU (both activation modes) and on the host cores; and the CPU
+baseline (the C restatement of the reference's CPU transformer) on a bounded
+sample, single-threaded as the reference and on all host cores.
 
-    python bench.py [--gpus 1] [--steps 256] [--warmup 128] [--model 7b|tiny]
+    python bench.py [--gpus 1] [--steps 256] [--warmup 8] [--model 7b|tiny]
 
 Two further workloads print a JSON line of the same shape (no roofline / CPU
 legs): `--model gpt2` (GPT-2 124M, every matrix Q8_0: a 32-token prompt, then
@@ -47,6 +54,25 @@ def log(*a):
 def gemv_bytes(qtype_bytes_per_matrix: int, nrows: int, ncols: int) -> int:
     """Algorithmic bytes of one GEMV: GGUF bytes of W + x (f32) + y (f32)."""
     return qtype_bytes_per_matrix + 4 * ncols + 4 * nrows
+
+
+DTYPE = ("quantized weights (q4_k/q6_k/q8_0 ints) x 16-bit block-fixed-point activations on "
+         "v_dot4 i8, i32 sub-block sums, f32 scales and accumulation; norms/RoPE/attention f32")
+
+
+class eager_launches:
+    """Inside: recorded launch sequences are enqueued launch by launch instead of replayed as
+    HIP graphs (what rocprofv3's kernel trace can see)."""
+
+    def __enter__(self):
+        self.old = os.environ.get("WGML_DISABLE_GRAPHS")
+        os.environ["WGML_DISABLE_GRAPHS"] = "1"
+
+    def __exit__(self, *a):
+        if self.old is None:
+            del os.environ["WGML_DISABLE_GRAPHS"]
+        else:
+            os.environ["WGML_DISABLE_GRAPHS"] = self.old
 
 
 def time_gemv(W, gpu, mats, nrows, ncols, iters):
@@ -98,43 +124,90 @@ def time_gate_up(W, gpu, cfg, weights):
     return best, nbytes
 
 
-def gemv_sweep(W, gpu, nrows, ncols, min_total_bytes=640 << 20):
-    """One matrix shape for Q8_0 / Q4_K / Q6_K: GB/s and fraction of HBM peak."""
+def gemv_sweep(W, gpu, nrows, ncols, cpu_threads, min_total_bytes=640 << 20):
+    """One matrix shape for Q8_0 / Q4_K / Q6_K: GB/s and fraction of HBM peak on the GPU (the
+    default integer-dot kernels and the fp32-activation kernels), and the CPU oracle's
+    dequantize-and-dot over the same bytes on one core and on `cpu_threads` cores."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle as orc
+
     res = {}
     vals = W.rng_normal(4242, nrows * ncols, 0.0, 0.02)
+    xcpu = W.rng_normal(99, ncols)
     for qtype, name in ((W.Q8_0, "q8_0"), (W.Q4_K, "q4_k"), (W.Q6_K, "q6_k")):
         raw = W.quantize(qtype, vals)
         n_copies = max(2, -(-min_total_bytes // raw.nbytes))
         mats = [W.GpuQuantMatrix(gpu, qtype, nrows, ncols, raw) for _ in range(n_copies)]
         us = time_gemv(W, gpu, mats, nrows, ncols, iters=4 * n_copies)
+        gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 1)
+        us32 = time_gemv(W, gpu, mats, nrows, ncols, iters=4 * n_copies)
+        gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 0)
         b = gemv_bytes(raw.nbytes, nrows, ncols)
         gbs = b / us * 1e-3
+        cpu = {}
+        for threads in sorted({1, cpu_threads}):
+            orc.set_threads(threads)
+            t0 = time.perf_counter()
+            orc.gemv_quant(qtype, raw, nrows, ncols, xcpu)
+            cpu[f"GB/s_{threads}_cores"] = round(b / (time.perf_counter() - t0) * 1e-9, 3)
+        orc.set_threads(1)
         res[name] = {"us": round(us, 3), "GB/s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
-                     "bytes": b, "copies": n_copies}
+                     "bytes": b, "copies": n_copies,
+                     "fp32_activations": {"us": round(us32, 3), "GB/s": round(b / us32 * 1e-3, 1)},
+                     "cpu_oracle": cpu}
         log(f"  gemv {name} {nrows}x{ncols}: {us:.2f} us  {gbs:.0f} GB/s  "
-            f"({100 * gbs / HBM_PEAK_GBS:.1f}% of HBM peak)")
+            f"({100 * gbs / HBM_PEAK_GBS:.1f}% of HBM peak); fp32 activations {us32:.2f} us; cpu {cpu}")
         del mats
     return res
 
 
-def cpu_baseline(weights, prompt, n_steps):
-    """Times the CPU oracle (port of the reference's single-threaded CPU
-    transformer, weights expanded to f32 at load as the reference does) on the
-    first `n_steps` positions of the same model and prompt."""
+def cpu_baseline(weights, prompt, n_steps, threads_all):
+    """Times the CPU oracle (port of the reference's CPU transformer, weights expanded to f32
+    at load as the reference does) on the first `n_steps` positions of the same model and
+    prompt: single-threaded as the reference is, and once more with the rows of every
+    matrix-vector product shared out over `threads_all` host cores.  Returns the JSON object
+    and the oracle's logits per position."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle as orc
 
     t0 = time.perf_counter()
     m = orc.Llama2(weights, predequantize=True)
     t_load = time.perf_counter() - t0
+    logits = []
+    orc.set_threads(1)
     t0 = time.perf_counter()
     for pos in range(n_steps):
-        m.forward(int(prompt[pos]), pos)
+        logits.append(m.forward(int(prompt[pos]), pos))
     dt = time.perf_counter() - t0
-    log(f"  cpu oracle: load (dequantize) {t_load:.1f}s, {n_steps} steps in {dt:.1f}s")
-    return {"value": round(n_steps / dt, 4), "unit": "tok/s", "cores": 1, "kind": "port",
-            "sample": f"{n_steps} decode steps (positions 0..{n_steps - 1}) of the same model, "
-                      f"f32 weights dequantized at load, single thread"}
+    m2 = orc.Llama2(weights, predequantize=True) if threads_all > 1 else None
+    dt_all = None
+    if m2 is not None:
+        orc.set_threads(threads_all)
+        t0 = time.perf_counter()
+        for pos in range(n_steps):
+            m2.forward(int(prompt[pos]), pos)
+        dt_all = time.perf_counter() - t0
+        orc.set_threads(1)
+    log(f"  cpu oracle: load (dequantize) {t_load:.1f}s, {n_steps} steps in {dt:.1f}s on 1 core"
+        + (f", {dt_all:.1f}s on {threads_all} cores" if dt_all else ""))
+    out = {"value": round(n_steps / dt, 4), "unit": "tok/s", "cores": 1, "kind": "port",
+           "sample": f"{n_steps} decode steps (positions 0..{n_steps - 1}) of the same model and "
+                     f"prompt, f32 weights dequantized at load, single thread as the reference",
+           "all_cores": None}
+    if dt_all:
+        out["all_cores"] = {"value": round(n_steps / dt_all, 4), "unit": "tok/s", "cores": threads_all,
+                            "sample": "the same steps, rows of every matrix-vector product shared "
+                                      "out over the host cores (OpenMP); identical results"}
+    return out, logits
+
+
+def host_cores():
+    """Cores this process may use (the box's CPU share, not the machine's core count)."""
+    n = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit() and int(env) > 0:
+        n = min(n, int(env))
+    return max(1, n)
 
 
 def bench_gpt2(args, W, gpu):
@@ -165,7 +238,7 @@ def bench_gpt2(args, W, gpu):
         f"{m.launches_per_token()} launches/token")
     return {"metric": "decode tok/s bs1 GPT-2 124M Q8_0", "value": round(n / dt, 1), "unit": "tok/s",
             "n_gpus": 1, "steps": n, "warmup": min(64, n), "ms_per_step": round(dt * 1e3 / n, 4),
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": DTYPE,
             "data": "synthetic",
             "config": {"workload": f"gpt2-124m q8_0 bs1 greedy: 32-token prompt, positions 0..{n - 1}",
                        "launches_per_token": launches,
@@ -202,7 +275,7 @@ def bench_8b_gqa(args, W, gpu):
         f"tok/s; {(wb + kvb) / (dt / n) / 1e12:.2f} TB/s over weights + KV")
     return {"metric": "decode tok/s bs1 Llama-3-8B-shape Q6_K at position 8192", "value": round(n / dt, 2),
             "unit": "tok/s", "n_gpus": 1, "steps": n, "warmup": 4, "ms_per_step": round(dt * 1e3 / n, 4),
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": DTYPE,
             "data": "synthetic",
             "config": {"workload": f"llama3-8b-shape q6_k bs1 greedy decode, KV caches N(0,1) up to "
                                    f"position 8191, {n} timed steps from position 8192",
@@ -217,27 +290,26 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None,
-                    help="timed decode steps (default 256; 128 for --model tiny)")
-    ap.add_argument("--warmup", type=int, default=None,
-                    help="prompt tokens before the timed steps (default 128; 16 for --model tiny)")
+                    help="timed decode steps (default 256; 112 for --model tiny)")
+    ap.add_argument("--warmup", type=int, default=8,
+                    help="untimed decode steps between the prompt and the timed steps (default 8)")
     ap.add_argument("--model", default="7b", choices=["7b", "tiny", "gpt2", "8b-gqa"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--cpu-steps", type=int, default=0, help="CPU baseline steps (0 = auto)")
     ap.add_argument("--roofline-only", action="store_true",
-                    help="only the dominant-kernel measurement (for profiler runs): the fused "
-                         "gate/up launches, then three plain copies of 256 MiB (op_assign Copy) "
-                         "as the known-size kernel that calibrates the HBM byte counters")
+                    help="only the dominant-kernel measurement, launch by launch (for profiler "
+                         "runs): the fused gate/up launches, then three plain copies of 256 MiB "
+                         "(op_assign Copy) as the known-size kernel that calibrates the HBM byte "
+                         "counters")
+    ap.add_argument("--sweep-only", action="store_true",
+                    help="only the GEMV sweep, launch by launch (for profiler runs)")
     ap.add_argument("--prefill-only", action="store_true",
-                    help="only the batched prompt pass over a --warmup-token prompt, 1 untimed + "
-                         "3 timed calls (for profiler runs)")
+                    help="only the batched prompt pass over the prompt, 1 untimed + 3 timed calls "
+                         "(for profiler runs)")
     ap.add_argument("--gemm-precision", type=int, default=1, choices=[0, 1],
                     help="with --prefill-only: 1 = split-f16 operands (default), 0 = plain f16")
     args = ap.parse_args()
-    if args.steps is None:
-        args.steps = 128 if args.model == "tiny" else 256
-    if args.warmup is None:
-        args.warmup = 16 if args.model == "tiny" else 128
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every kernel uses a single device; "
                  "no collectives are built). Use --gpus 1.")
@@ -249,17 +321,32 @@ def main():
 
     gpu = W.GpuInstance(0)
     name, n_cu = gpu.info()
-    log(f"device: {name}, {n_cu} CUs")
+    cores = host_cores()
+    log(f"device: {name}, {n_cu} CUs; host cores for the CPU legs: {cores}")
     if args.model in ("gpt2", "8b-gqa"):
+        if args.steps is None:
+            args.steps = 256
         line = bench_gpt2(args, W, gpu) if args.model == "gpt2" else bench_8b_gqa(args, W, gpu)
         print(json.dumps(line), flush=True)
         return
 
+    # The workload's shape is fixed: the flags only say how many of its decode steps are
+    # warm-up and how many are timed.
     if args.model == "7b":
-        cfg, scheme, label = LLAMA2_7B, "q4_k_m", "llama2-7b-shape q4_k_m"
+        cfg, scheme, label, n_prompt = LLAMA2_7B, "q4_k_m", "llama2-7b-shape q4_k_m", 128
     else:
-        cfg, scheme, label = TINY_LLAMA, "q8_0", "tiny-llama2 q8_0"
-    assert args.warmup >= 1 and args.warmup + args.steps <= cfg.seq_len, "positions exceed seq_len"
+        cfg, scheme, label, n_prompt = TINY_LLAMA, "q8_0", "tiny-llama2 q8_0", 16
+    if args.steps is None:
+        args.steps = 256 if args.model == "7b" else 112
+    if args.warmup < 1 or n_prompt + args.warmup + args.steps > cfg.seq_len:
+        sys.exit(f"bench.py: {n_prompt} prompt positions + {args.warmup} warm-up + {args.steps} timed "
+                 f"steps must fit the model's {cfg.seq_len} positions (and --warmup >= 1)")
+
+    if args.sweep_only:
+        with eager_launches():
+            for nrows, ncols in ((4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)):
+                gemv_sweep(W, gpu, nrows, ncols, 1)
+        return
 
     t0 = time.perf_counter()
     weights = synth_llama(cfg, seed=4, scheme=scheme,
@@ -269,7 +356,8 @@ def main():
     log(f"weights built in {time.perf_counter() - t0:.0f}s "
         f"({weights.weight_bytes_per_token() / 1e9:.3f} GB per token)")
     if args.roofline_only:
-        us, b = time_gate_up(W, gpu, cfg, weights)
+        with eager_launches():
+            us, b = time_gate_up(W, gpu, cfg, weights)
         n = 64 << 20
         src = W.GpuVector.init(gpu, np.zeros(n, np.float32))
         dst = W.GpuVector.uninit(gpu, n)
@@ -282,7 +370,7 @@ def main():
                                          "268435456 B written per launch"}), flush=True)
         return
     model = Llama2(gpu, cfg).load(weights)
-    prompt = W.prompt_tokens(4, args.warmup, cfg.vocab_size)
+    prompt = W.prompt_tokens(4, n_prompt, cfg.vocab_size)
     if args.prefill_only:
         gpu.set_gemm_precision(args.gemm_precision)
         model.prefill(prompt)
@@ -292,88 +380,113 @@ def main():
             model.prefill(prompt)
         gpu.synchronize()
         pdt = (time.perf_counter() - t0) / 3
-        print(json.dumps({"prefill_tokens": args.warmup, "gemm_precision": args.gemm_precision,
+        print(json.dumps({"prefill_tokens": n_prompt, "gemm_precision": args.gemm_precision,
                           "ms": round(pdt * 1e3, 3),
-                          "tok_s": round(args.warmup / pdt, 1),
+                          "tok_s": round(n_prompt / pdt, 1),
                           "launches": model.launches_per_token()}), flush=True)
         return
 
-    # warm-up: the prompt, one token at a time (the reference has no batched prefill)
-    out = model.generate_greedy(prompt, args.warmup)
-    gpu.synchronize()
-    first = int(out[-1])
+    # the prompt: one batched pass (timed on its own further down); its last logits give the
+    # first generated token
+    model.prefill(prompt)
+    first = int(np.argmax(model.logits()))
+    p0 = n_prompt  # position of the first decode step
 
     # the same steps with a blocking read-back of every sampled token, as the reference's
-    # chat loop does (reported beside the headline figure, and it warms the recorded step)
+    # chat loop does (reported beside the headline figure; part of the warm-up)
     n_sync = min(args.steps, 64)
     gpu.synchronize()
     t0 = time.perf_counter()
-    toks_sync = model.decode_greedy_sync(first, args.warmup, n_sync)
+    toks_sync = model.decode_greedy_sync(first, p0, args.warmup + n_sync)
     gpu.synchronize()
-    tok_s_sync = n_sync / (time.perf_counter() - t0)
-    model.decode_greedy(first, args.warmup, 2)  # records the step (graph capture), untimed
+    tok_s_sync = (args.warmup + n_sync) / (time.perf_counter() - t0)
+
+    # warm-up: `--warmup` recorded steps (the first call captures the step as a graph)
+    wtoks = model.decode_greedy(first, p0, args.warmup)
+    gpu.synchronize()
 
     # timed region: exactly `steps` greedy decode steps.  Sampling (arg-max) and the loop
     # bookkeeping run on the device; the host enqueues one recorded step per token and
     # synchronises at the end, when the token ids are copied back.
-    gpu.synchronize()
     t0 = time.perf_counter()
-    toks = model.decode_greedy(first, args.warmup, args.steps)
+    toks = model.decode_greedy(int(wtoks[-1]), p0 + args.warmup, args.steps)
     gpu.synchronize()
     dt = time.perf_counter() - t0
     tok_s = args.steps / dt
-    assert np.array_equal(toks[:n_sync], toks_sync), "recorded and synchronous loops disagree"
+    assert np.array_equal(np.concatenate([wtoks, toks])[:args.warmup + n_sync], toks_sync), \
+        "recorded and synchronous loops disagree"
     launches_per_token = model.launches_per_token()
     wbytes = weights.weight_bytes_per_token()
-    kv_bytes_mid = 2 * cfg.n_layers * cfg.kv_dim * 4 * (args.warmup + args.steps // 2)
+    kv_bytes_mid = 2 * cfg.n_layers * cfg.kv_dim * 4 * (p0 + args.warmup + args.steps // 2)
     roof_tok_s = HBM_PEAK_GBS * 1e9 / wbytes
     log(f"decode: {args.steps} steps in {dt * 1e3:.1f} ms -> {tok_s:.1f} tok/s "
         f"({100 * tok_s / roof_tok_s:.1f}% of the weight-bytes roofline {roof_tok_s:.0f} tok/s); "
         f"{launches_per_token} launches/token; with a host read-back per token: "
         f"{tok_s_sync:.1f} tok/s")
 
-    # the batched prompt pass over the same prompt (f16 MFMA products, 128 tokens per run);
-    # untimed first call allocates its buffers.  It rewrites KV rows 0..warmup-1 with values
-    # that agree with the step-by-step ones to ~1e-3, which nothing after this point reads.
-    prefill = None
-    if args.warmup >= 2:
-        layer_elems = cfg.n_layers * (2 * cfg.dim * cfg.dim + 2 * cfg.kv_dim * cfg.dim +
-                                      3 * cfg.dim * cfg.hidden_dim)
-        flops = 2.0 * layer_elems * args.warmup
-        stepwise_logits = None
-        prefill = {"tokens": args.warmup,
-                   "ms_step_by_step_at_decode_rate": round(args.warmup / tok_s * 1e3, 1)}
-        # level 1 (default): split-f16 operands, results to fp32 rounding; level 0: plain f16
-        for level, key in ((1, "split_f16"), (0, "plain_f16")):
-            gpu.set_gemm_precision(level)
+    # the same decode with fp32 activations in every GEMV (no 16-bit rounding of x): the
+    # fused launches exist for the integer-dot kernels only, so this is the level with one
+    # launch per matrix (norms still folded into the staging of x)
+    gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 1)
+    model.set_fusion(2)
+    n32 = min(args.steps, 64)
+    model.decode_greedy(first, p0, 2)
+    gpu.synchronize()
+    t0 = time.perf_counter()
+    toks32 = model.decode_greedy(first, p0, n32)
+    gpu.synchronize()
+    dt32 = time.perf_counter() - t0
+    fp32_act = {"tok_s": round(n32 / dt32, 2), "steps": n32, "launches_per_token": model.launches_per_token(),
+                "same_tokens_as_default": bool(np.array_equal(toks32, np.concatenate([wtoks, toks])[:n32])),
+                "note": "one launch per matrix (fusion level 2), fp32 activations staged in LDS"}
+    gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 0)
+    model.set_fusion(3)
+    log(f"decode with fp32 activations: {n32 / dt32:.1f} tok/s ({fp32_act['launches_per_token']} launches/token), "
+        f"same tokens: {fp32_act['same_tokens_as_default']}")
+
+    # the batched prompt pass over the prompt (MFMA products, 128 tokens per run).  It
+    # rewrites KV rows 0..n_prompt-1 with the values they already hold.
+    layer_elems = cfg.n_layers * (2 * cfg.dim * cfg.dim + 2 * cfg.kv_dim * cfg.dim +
+                                  3 * cfg.dim * cfg.hidden_dim)
+    flops = 2.0 * layer_elems * n_prompt
+    prefill = {"tokens": n_prompt, "ms_step_by_step_at_decode_rate": round(n_prompt / tok_s * 1e3, 1)}
+    # level 1 (default): split-f16 operands, results to fp32 rounding; level 0: plain f16
+    for level, key in ((1, "split_f16"), (0, "plain_f16")):
+        gpu.set_gemm_precision(level)
+        model.prefill(prompt)
+        gpu.synchronize()
+        reps = 3
+        t0 = time.perf_counter()
+        for _ in range(reps):
             model.prefill(prompt)
-            gpu.synchronize()
-            reps = 3
-            t0 = time.perf_counter()
-            for _ in range(reps):
-                model.prefill(prompt)
-            gpu.synchronize()
-            pdt = (time.perf_counter() - t0) / reps
-            prefill[key] = {"ms": round(pdt * 1e3, 3), "tok_s": round(args.warmup / pdt, 1),
-                            "model_TFLOP/s": round(flops / pdt * 1e-12, 1),
-                            "first_token_matches_step_by_step": int(np.argmax(model.logits())) == first,
-                            "launches": model.launches_per_token()}
-            log(f"prefill ({key}): {args.warmup} tokens in {pdt * 1e3:.2f} ms -> {args.warmup / pdt:.0f} "
-                f"tok/s, {flops / pdt * 1e-12:.1f} model TFLOP/s (step by step: "
-                f"{args.warmup / tok_s * 1e3:.0f} ms); first token matches: "
-                f"{prefill[key]['first_token_matches_step_by_step']}")
-        gpu.set_gemm_precision(1)
+        gpu.synchronize()
+        pdt = (time.perf_counter() - t0) / reps
+        prefill[key] = {"ms": round(pdt * 1e3, 3), "tok_s": round(n_prompt / pdt, 1),
+                        "model_TFLOP/s": round(flops / pdt * 1e-12, 1),
+                        "first_token_matches_default": int(np.argmax(model.logits())) == first,
+                        "launches": model.launches_per_token()}
+        log(f"prefill ({key}): {n_prompt} tokens in {pdt * 1e3:.2f} ms -> {n_prompt / pdt:.0f} "
+            f"tok/s, {flops / pdt * 1e-12:.1f} model TFLOP/s (step by step: "
+            f"{n_prompt / tok_s * 1e3:.0f} ms); first token matches: "
+            f"{prefill[key]['first_token_matches_default']}")
+    gpu.set_gemm_precision(1)
 
     # dominant kernel: the fused gate/up launch (27% of a step), timed live over the model's
-    # own per-layer matrices; the plain single-matrix Q4_K GEMV of the same shape beside it
+    # own per-layer matrices.  `achieved` / `frac` come from launch-by-launch timing, the way
+    # rocprofv3's kernel trace sees the same command (profiles/); the figure inside a recorded
+    # graph, as the decode loop runs it, is carried beside it.
     roofline = None
     if args.model == "7b":
-        us, b = time_gate_up(W, gpu, cfg, weights)
-        gbs = b / us * 1e-3
-        traffic = None
+        with eager_launches():
+            us_eager, b = time_gate_up(W, gpu, cfg, weights)
+        us_graph, _ = time_gate_up(W, gpu, cfg, weights)
+        gbs = b / us_eager * 1e-3
+        traffic, traffic_src = None, None
         tpath = os.path.join(ROOT, "profiles", "traffic.json")
         if os.path.exists(tpath):
-            traffic = json.load(open(tpath)).get("gemv_fused_gate_up_bytes_per_launch")
+            tj = json.load(open(tpath))
+            traffic = tj.get("gemv_fused_gate_up_bytes_per_launch")
+            traffic_src = tj.get("source")
         gate = [W.GpuQuantMatrix(gpu, W.Q4_K, cfg.hidden_dim, cfg.dim, l["ffn_gate"].data)
                 for l in weights.layers[:24]]
         us1 = time_gemv(W, gpu, gate, cfg.hidden_dim, cfg.dim, iters=4 * len(gate))
@@ -381,45 +494,64 @@ def main():
         del gate
         roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                    "traffic_source": traffic_src,
                     "kernel": "gemv_fused_kernel, gate+up launch: 2 x Q4_K 11008x4096, RMSNorm "
                               "folded into staging, SiLU epilogue",
-                    "bytes_per_launch": b, "us_per_launch": round(us, 3),
-                    "plain_gemv_q4_k_11008x4096": {"us_per_launch": round(us1, 3),
-                                                   "bytes_per_launch": b1,
-                                                   "GB/s": round(b1 / us1 * 1e-3, 1)}}
-        log(f"dominant kernel gemv_fused_kernel gate+up: {us:.2f} us, {gbs:.0f} GB/s; "
-            f"plain Q4_K gemv 11008x4096: {us1:.2f} us, {b1 / us1 * 1e-3:.0f} GB/s")
+                    "bytes_per_launch": b, "us_per_launch": round(us_eager, 3),
+                    "timing": "HIP events around back-to-back launches on the library's stream, "
+                              "launch by launch (no graph)",
+                    "in_recorded_graph": {"us_per_launch": round(us_graph, 3),
+                                          "GB/s": round(b / us_graph * 1e-3, 1),
+                                          "frac": round(b / us_graph * 1e-3 / HBM_PEAK_GBS, 4)},
+                    "plain_gemv_q4_k_11008x4096_in_graph": {"us_per_launch": round(us1, 3),
+                                                            "bytes_per_launch": b1,
+                                                            "GB/s": round(b1 / us1 * 1e-3, 1)}}
+        log(f"dominant kernel gemv_fused_kernel gate+up: {us_eager:.2f} us launch by launch "
+            f"({gbs:.0f} GB/s), {us_graph:.2f} us in a graph; plain Q4_K gemv 11008x4096: "
+            f"{us1:.2f} us, {b1 / us1 * 1e-3:.0f} GB/s")
 
     sweep = None
     if not args.no_sweep and args.model == "7b":
-        # the four GEMV shapes of the 7B model, three formats each; every timing rotates
+        # the four GEMV shapes of the 7B model, three formats each; every GPU timing rotates
         # through enough distinct copies (> 640 MB) that nothing is served from a cache
         sweep = {}
         for nrows, ncols in ((4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)):
-            sweep[f"{nrows}x{ncols}"] = gemv_sweep(W, gpu, nrows, ncols)
+            sweep[f"{nrows}x{ncols}"] = gemv_sweep(W, gpu, nrows, ncols, cores)
 
-    cpu = None
+    cpu, parity = None, None
     if not args.no_cpu_baseline:
-        n = args.cpu_steps or (2 if args.model == "7b" else 32)
-        cpu = cpu_baseline(weights, prompt, min(n, args.warmup))
+        n = args.cpu_steps or (2 if args.model == "7b" else 16)
+        n = min(n, n_prompt)
+        cpu, ref_logits = cpu_baseline(weights, prompt, n, cores)
+        # the GPU step on the same positions against the oracle's logits
+        worst = 0.0
+        for pos in range(n):
+            got = model.forward_logits(pos, int(prompt[pos])).astype(np.float64)
+            worst = max(worst, float(np.abs(got - ref_logits[pos]).max() / np.abs(ref_logits[pos]).max()))
+        parity = {"max_logit_err_over_max_logit": float(f"{worst:.3e}"), "positions": n, "budget": 1e-3,
+                  "against": "CPU oracle, same weights and tokens (the steps of cpu_baseline)"}
+        log(f"  GPU step vs oracle logits on positions 0..{n - 1}: {worst:.2e} of max|logit| (budget 1e-3)")
 
     line = {
         "metric": "decode tok/s bs1 Llama-2-7B-shape Q4_K" if args.model == "7b"
         else "decode tok/s bs1 tiny Llama-2 Q8_0",
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(dt * 1e3 / args.steps, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": DTYPE,
         "data": "synthetic",
-        "config": {"workload": f"{label} bs1 greedy decode: {args.warmup}-token prompt "
-                               f"(one token per step), then {args.steps} timed steps",
-                   "weights": "seeded N(0,0.02), ggml reference quantizers; embedding/activations/KV f32",
+        "config": {"workload": f"{label} bs1 greedy decode: {n_prompt}-token prompt (batched prompt "
+                               f"pass), {args.warmup} untimed steps from position {p0}, then "
+                               f"{args.steps} timed steps from position {p0 + args.warmup}",
+                   "weights": "seeded N(0,0.02), ggml reference quantizers; embedding/KV f32",
                    "weight_bytes_per_token": wbytes, "kv_bytes_per_token_mid_run": kv_bytes_mid,
                    "roofline_tok_s_at_8TBs": round(roof_tok_s, 1),
                    "frac_of_weight_roofline": round(tok_s / roof_tok_s, 4),
                    "launches_per_token": launches_per_token,
                    "tok_s_with_per_token_host_sync": round(tok_s_sync, 2),
+                   "fp32_activations": fp32_act,
                    "last_token": int(toks[-1])},
-        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "gemv_sweep": sweep,
+        "roofline": roofline, "cpu_baseline": cpu, "parity": parity, "prefill": prefill,
+        "gemv_sweep": sweep,
     }
     print(json.dumps(line), flush=True)
 

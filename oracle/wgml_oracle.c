@@ -1,7 +1,8 @@
 /*
  * wgml_oracle — TEST INFRASTRUCTURE ONLY (see wgml_oracle.h).
  *
- * Single-threaded C restatement of the reference's CPU arithmetic.  Compile
+ * C restatement of the reference's CPU arithmetic, single-threaded unless orc_set_threads
+ * asks otherwise (a timing mode with identical results).  Compile
  * with -ffp-contract=off so that no multiply-add is fused: the reference is
  * Rust, which never contracts a*b+c.
  */
@@ -330,7 +331,16 @@ static float dot8(const float *a, const float *b, int n) {
 
 /* models/llama2/cpu.rs:373: out.gemv(1.0, w, x, 0.0) — one axpy per column, so
  * out[i] = (..((x0*w[i][0]) + x1*w[i][1]) + ..), each product rounded. */
+/* Timing mode only (the benchmark's all-cores CPU baseline): rows of a matrix-vector
+ * product are shared out over n threads.  Every row's sum keeps its sequential order, so
+ * results are identical to the single-threaded ones; the reference itself has no threading
+ * (models/llama2/cpu.rs), so 1 is the faithful setting and the default. */
+static int g_threads = 1;
+void orc_set_threads(int n) { g_threads = n > 1 ? n : 1; }
+int orc_get_threads(void) { return g_threads; }
+
 void orc_gemv_f32(float *out, const float *w, const float *x, int nrows, int ncols) {
+#pragma omp parallel for num_threads(g_threads) if (g_threads > 1 && nrows >= 64) schedule(static)
     for (int i = 0; i < nrows; ++i) {
         const float *row = w + (size_t)i * ncols;
         float acc = (1.0f * x[0]) * row[0];
@@ -365,15 +375,25 @@ int orc_gemv_quant(int type, const void *blocks, int nrows, int ncols, const flo
     size_t be = orc_block_elems(type), bb = orc_block_bytes(type);
     if (!be || ncols % (int)be) return -1;
     size_t row_bytes = (size_t)ncols / be * bb;
-    float *row = (float *)malloc((size_t)ncols * sizeof(float));
-    if (!row) return -2;
-    for (int i = 0; i < nrows; ++i) {
-        orc_dequantize(type, (const uint8_t *)blocks + (size_t)i * row_bytes, (size_t)ncols, row);
-        if (out_f32) orc_gemv_f32(out_f32 + i, row, x, 1, ncols);
-        if (out_f64) orc_gemv_f64(out_f64 + i, row, x, 1, ncols);
+    int failed = 0;
+#pragma omp parallel num_threads(g_threads) if (g_threads > 1 && nrows >= 64)
+    {
+        float *row = (float *)malloc((size_t)ncols * sizeof(float));
+        if (!row) {
+#pragma omp atomic write
+            failed = 1;
+        } else {
+#pragma omp for schedule(static)
+            for (int i = 0; i < nrows; ++i) {
+                orc_dequantize(type, (const uint8_t *)blocks + (size_t)i * row_bytes, (size_t)ncols,
+                               row);
+                if (out_f32) orc_gemv_f32(out_f32 + i, row, x, 1, ncols);
+                if (out_f64) orc_gemv_f64(out_f64 + i, row, x, 1, ncols);
+            }
+            free(row);
+        }
     }
-    free(row);
-    return 0;
+    return failed ? -2 : 0;
 }
 
 /* ------------------------------------------------------------------ ops -- */

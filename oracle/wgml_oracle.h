@@ -87,6 +87,9 @@ int orc_dequantize(int type, const void *blocks, size_t nelems, float *out);
  * matrix: every out[i] is the f32 sum over columns j = 0..n in order, each
  * term a separately rounded product (no fused multiply-add).  `w` is row-major
  * nrows x ncols. */
+/* threads for the rows of matrix-vector products (1 = as the reference; results do not depend on it) */
+void orc_set_threads(int n);
+int orc_get_threads(void);
 void orc_gemv_f32(float *out, const float *w, const float *x, int nrows, int ncols);
 /* Same product accumulated in double: the tolerance anchor for GPU GEMVs. */
 void orc_gemv_f64(double *out, const float *w, const float *x, int nrows, int ncols);

@@ -76,6 +76,17 @@ lib.orc_dequantize.argtypes = [_i, _P, C.c_size_t, _P]
 lib.orc_gemv_f32.argtypes = [_P, _P, _P, _i, _i]
 lib.orc_gemv_f32_colmajor.argtypes = [_P, _P, _P, _i, _i]
 lib.orc_gemv_f64.argtypes = [_P, _P, _P, _i, _i]
+lib.orc_set_threads.restype = None
+lib.orc_set_threads.argtypes = [_i]
+lib.orc_get_threads.restype = _i
+
+
+def set_threads(n: int) -> None:
+    """Threads for the rows of matrix-vector products (timing mode of the benchmark's CPU
+    baseline; 1 = single-threaded as the reference, results do not depend on it)."""
+    lib.orc_set_threads(int(n))
+
+
 lib.orc_gemv_quant.restype = _i
 lib.orc_gemv_quant.argtypes = [_i, _P, _i, _i, _P, _P, _P]
 lib.orc_rms_norm.argtypes = [_P, _P, _P, _i, _f]

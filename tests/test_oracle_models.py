@@ -74,3 +74,28 @@ def test_greedy_loop_contract():
     longer = np.concatenate([prompt, out[3:6]])
     out2, _ = m2.generate_greedy(longer, 10)
     assert np.array_equal(out, out2)
+
+
+def test_thread_count_of_the_timing_mode_does_not_change_results():
+    from wgml_amd.models import Llama2Config, synth_llama
+
+    cfg = Llama2Config(dim=256, hidden_dim=512, n_layers=2, n_q_heads=4, n_kv_heads=2,
+                       vocab_size=320, seq_len=16)
+    w = synth_llama(cfg, seed=3, scheme="q4_k_m")
+    a = orc.Llama2(w, predequantize=True)
+    b = orc.Llama2(w)
+    try:
+        for pos, t in enumerate([5, 17, 300]):
+            orc.set_threads(1)
+            want = a.forward(t, pos)
+            orc.set_threads(4)
+            assert np.array_equal(b.forward(t, pos), want)
+            raw = w.layers[0]["ffn_gate"]
+            x = W.rng_normal(pos, cfg.dim)
+            orc.set_threads(1)
+            r1 = orc.gemv_quant(raw.qtype, raw.data, raw.nrows, raw.ncols, x)
+            orc.set_threads(4)
+            r4 = orc.gemv_quant(raw.qtype, raw.data, raw.nrows, raw.ncols, x)
+            assert np.array_equal(r1[0], r4[0]) and np.array_equal(r1[1], r4[1])
+    finally:
+        orc.set_threads(1)

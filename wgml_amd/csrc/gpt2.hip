@@ -36,7 +36,8 @@ struct wgml_gpt2 {
     hipGraphExec_t graph_exec = nullptr;
     int fusion = 1;  // 0: one launch per op group as before; 1: folded launches
     int graph_fusion = -1;
-    uint64_t launches_last = 0;
+    uint64_t launches_last = 0;   // launches of the last step that ran
+    uint64_t graph_launches = 0;  // launches of the recorded step
 };
 
 namespace {
@@ -372,7 +373,7 @@ int build_graph(wgml_gpt2 *m) {
     int rc = enqueue_step(m, true, 0, 0);
     if (rc == WGML_OK)
         rc = launch_argmax_next(ctx, m->curr_vocab, p.n_vocab, m->dyn, m->d_prompt, m->d_tokens);
-    m->launches_last = ctx->launches - launches0;
+    m->graph_launches = ctx->launches - launches0;
     hipError_t e = hipStreamEndCapture(ctx->stream, &m->graph);
     if (rc == WGML_OK && e != hipSuccess)
         rc = set_error(WGML_E_HIP, "wgml_gpt2: graph capture failed: %s", hipGetErrorString(e));
@@ -470,6 +471,7 @@ int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_p
     for (uint32_t i = 0; i < n_total; ++i) {
         if (use_graph) {
             WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec, ctx->stream));
+            m->launches_last = m->graph_launches;
         } else {
             const uint64_t l0 = ctx->launches;
             WGML_TRY(enqueue_step(m, true, 0, 0));

@@ -50,7 +50,8 @@ struct wgml_llama2 {
     float *pf_x = nullptr, *pf_xb = nullptr, *pf_q = nullptr, *pf_hb = nullptr, *pf_hb2 = nullptr;
     uint32_t *pf_tokens = nullptr;
     std::vector<void *> allocs;
-    uint64_t launches_last = 0;
+    uint64_t launches_last = 0;   // launches of the last step that ran
+    uint64_t graph_launches = 0;  // launches of the recorded step
 };
 
 namespace {
@@ -290,7 +291,7 @@ int build_graph(wgml_llama2 *m) {
     int rc = enqueue_step(m, true, 0, 0);
     if (rc == WGML_OK)
         rc = launch_argmax_next(ctx, m->logits, c.vocab_size, m->dyn, m->d_prompt, m->d_tokens);
-    m->launches_last = ctx->launches - launches0;
+    m->graph_launches = ctx->launches - launches0;
     hipError_t e = hipStreamEndCapture(ctx->stream, &m->graph);
     if (rc != WGML_OK) {
         drop_graph(m);
@@ -333,6 +334,7 @@ int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint3
     for (uint32_t i = 0; i < n_steps; ++i) {
         if (use_graph) {
             WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec, ctx->stream));
+            m->launches_last = m->graph_launches;
         } else {
             // the same launches, enqueued one by one (no host synchronisation either)
             const uint64_t launches0 = ctx->launches;
