@@ -115,14 +115,15 @@ WGML_API int wgml_buf_zero(wgml_buf *buf);
 /* ---- quantized matrices: GpuQuantMatrix (quantized_matrix.rs:9-75) and
  *      GgufTensorData::to_gpu_matrix (gguf.rs:131-184) ---------------------- *
  * `gguf_bytes` is the tensor exactly as stored in a GGUF file: row-major,
- * nrows rows of ncols/elems_per_block blocks.  WGML_Q8_0, WGML_Q4_K and WGML_Q6_K
- * stay quantized (re-laid out on the device, see the layout notes in
- * csrc/common.h; the values are unchanged).  WGML_F16, WGML_Q4_0, WGML_Q4_1,
- * WGML_Q5_0, WGML_Q5_1, WGML_Q5_K and WGML_Q8_K are expanded to f32 on the device
- * at creation, as to_gpu_matrix does for every format its GEMV cannot read; the
- * matrix then reports WGML_F32.  Other tags give WGML_E_UNSUPPORTED.  Unlike the
- * reference there is no pairing rule (ncols % 64 / % 512) for the quantized
- * formats: any ncols that is a multiple of the block length stays quantized. */
+ * nrows rows of ncols/elems_per_block blocks.  Every block format the reference keeps
+ * quantized on the GPU (gguf.rs:172-182) stays quantized here: WGML_Q8_0 and WGML_Q6_K are
+ * re-laid out into aligned planes on the device (same bytes in total, see the layout
+ * notes in csrc/common.h), WGML_Q4_K, WGML_Q4_0, WGML_Q4_1, WGML_Q5_0, WGML_Q5_1,
+ * WGML_Q5_K and WGML_Q8_K keep the GGUF bytes unchanged; the values are those of
+ * Block*::dequantize in every case.  WGML_F16 is expanded to f32 on the device at
+ * creation, as to_gpu_matrix does (the matrix then reports WGML_F32).  Other tags give
+ * WGML_E_UNSUPPORTED.  Unlike the reference there is no pairing rule (ncols % 64 /
+ * % 512): any ncols that is a multiple of the block length stays quantized. */
 WGML_API int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t ncols,
                                       const void *gguf_bytes, wgml_qmat **out);
 WGML_API int wgml_quant_matrix_destroy(wgml_qmat *m);
@@ -316,8 +317,9 @@ WGML_API int wgml_llama2_decode_greedy_sync(wgml_llama2 *m, uint32_t first_token
  * the step, so with the default the logits agree with the step-by-step pass as two
  * fp32 implementations do (2e-4 of their range is the bound the tests use); with
  * level 0 a product is within about 3e-4 and a whole model adds that up (3e-3 of
- * the logits' range on 2-layer models, 6e-3 on the 32-layer 7B shape).  The layer matrices
- * must be WGML_Q8_0, WGML_Q4_K or WGML_Q6_K (WGML_E_UNSUPPORTED otherwise).
+ * the logits' range on 2-layer models, 6e-3 on the 32-layer 7B shape).  The batched
+ * products exist for WGML_Q8_0, WGML_Q4_K and WGML_Q6_K: a model with a layer matrix in
+ * another format takes the prompt one step per token, as the reference does.
  * Enqueues and returns. */
 WGML_API int wgml_llama2_prefill(wgml_llama2 *m, const uint32_t *tokens, uint32_t n_tokens,
                                  uint32_t start_pos);

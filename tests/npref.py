@@ -173,6 +173,90 @@ def random_blocks(qtype: int, nblocks: int, seed: int) -> np.ndarray:
     return raw.reshape(-1)
 
 
+# ---- simple encoders for the formats the library's quantizer does not write -------------
+# (test inputs only: any valid block is a fair input, parity always compares both sides on
+# identical bytes; these round to nearest with the obvious scales, nothing more)
+
+def _f16(a):
+    return np.asarray(a, dtype=np.float32).astype(np.float16)
+
+
+def encode_simple(qtype: int, x) -> np.ndarray:
+    """x (float32, length a multiple of the block) -> GGUF block bytes of Q4_0 / Q4_1 / Q5_0 /
+    Q5_1 / Q5_K / Q8_K."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    if qtype in (2, 3, 6, 7):
+        xb = x.reshape(-1, 32)
+        nb = xb.shape[0]
+        five = qtype in (6, 7)
+        levels = 31 if five else 15
+        if qtype in (3, 7):  # d q + m
+            mn = xb.min(axis=1)
+            d = _f16((xb.max(axis=1) - mn) / levels)
+            m = _f16(mn)
+            df = np.where(d.astype(np.float32) == 0, 1, d.astype(np.float32))
+            q = np.clip(np.rint((xb - m.astype(np.float32)[:, None]) / df[:, None]), 0, levels).astype(np.uint8)
+            head = np.concatenate([d.view(np.uint8).reshape(nb, 2), m.view(np.uint8).reshape(nb, 2)], axis=1)
+        else:  # d (q - 8) or d (q - 16)
+            off = 16 if five else 8
+            d = _f16(np.abs(xb).max(axis=1) / (off - 1))
+            df = np.where(d.astype(np.float32) == 0, 1, d.astype(np.float32))
+            q = np.clip(np.rint(xb / df[:, None]) + off, 0, levels).astype(np.uint8)
+            head = d.view(np.uint8).reshape(nb, 2)
+        qs = (q[:, :16] & 15) | ((q[:, 16:] & 15) << 4)
+        parts = [head]
+        if five:
+            bits = (q >> 4).astype(np.uint32)
+            qh = (bits << np.arange(32, dtype=np.uint32)[None, :]).sum(axis=1).astype(np.uint32)
+            parts.append(qh.view(np.uint8).reshape(nb, 4))
+        parts.append(qs.astype(np.uint8))
+        return np.ascontiguousarray(np.concatenate(parts, axis=1)).reshape(-1)
+    if qtype == 15:
+        xb = x.reshape(-1, 256)
+        nb = xb.shape[0]
+        d = (np.abs(xb).max(axis=1) / 127).astype(np.float32)
+        df = np.where(d == 0, 1, d)
+        q = np.clip(np.rint(xb / df[:, None]), -127, 127).astype(np.int8)
+        bsums = q.reshape(nb, 16, 16).astype(np.int16).sum(axis=2).astype(np.int16)
+        return np.ascontiguousarray(np.concatenate(
+            [d.view(np.uint8).reshape(nb, 4), q.view(np.uint8), bsums.view(np.uint8).reshape(nb, 32)],
+            axis=1)).reshape(-1)
+    if qtype == 13:
+        xb = x.reshape(-1, 8, 32)
+        nb = xb.shape[0]
+        mn = np.maximum(0, -xb.min(axis=2))                    # (nb, 8) minima, as positive offsets
+        sc = (xb.max(axis=2) + mn) / 31
+        d = _f16(sc.max(axis=1) / 63)
+        dmin = _f16(mn.max(axis=1) / 63)
+        df = np.where(d.astype(np.float32) == 0, 1, d.astype(np.float32))[:, None]
+        mf = np.where(dmin.astype(np.float32) == 0, 1, dmin.astype(np.float32))[:, None]
+        ls = np.clip(np.rint(sc / df), 0, 63).astype(np.uint8)
+        lm = np.clip(np.rint(mn / mf), 0, 63).astype(np.uint8)
+        step = (d.astype(np.float32)[:, None] * ls.astype(np.float32))
+        step = np.where(step == 0, 1, step)
+        q = np.clip(np.rint((xb + (dmin.astype(np.float32)[:, None] * lm)[:, :, None]) / step[:, :, None]),
+                    0, 31).astype(np.uint8)
+        scales = np.zeros((nb, 12), dtype=np.uint8)
+        for j in range(8):  # the packing get_scale_min_k4 reads (quantization.rs:381-389)
+            if j < 4:
+                scales[:, j] |= ls[:, j]
+                scales[:, j + 4] |= lm[:, j]
+            else:
+                scales[:, j + 4] |= (ls[:, j] & 15) | ((lm[:, j] & 15) << 4)
+                scales[:, j - 4] |= (ls[:, j] >> 4) << 6
+                scales[:, j] |= (lm[:, j] >> 4) << 6
+        qh = np.zeros((nb, 32), dtype=np.uint8)
+        for s_ in range(8):
+            qh |= ((q[:, s_, :] >> 4) << s_).astype(np.uint8)
+        qs = np.empty((nb, 4, 32), dtype=np.uint8)
+        for g in range(4):
+            qs[:, g, :] = (q[:, 2 * g, :] & 15) | ((q[:, 2 * g + 1, :] & 15) << 4)
+        return np.ascontiguousarray(np.concatenate(
+            [d.view(np.uint8).reshape(nb, 2), dmin.view(np.uint8).reshape(nb, 2), scales, qh,
+             qs.reshape(nb, 128)], axis=1)).reshape(-1)
+    raise ValueError(f"no simple encoder for type {qtype}")
+
+
 # ---- float64 model forwards (composition check for the oracle) ---------------
 
 def llama_forward_f64(w, tokens, rope_variant: int = 0):

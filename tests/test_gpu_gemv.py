@@ -233,3 +233,34 @@ def test_fused_gate_up_silu_launch(gpu, nrows, ncols):
     ref = u * (g / (1.0 + np.exp(-g)))
     ok, e = close(out.read(), ref)
     assert ok, e
+
+
+OTHER = [W.Q4_0, W.Q4_1, W.Q5_0, W.Q5_1, W.Q5_K, W.Q8_K]
+
+
+@pytest.mark.parametrize("qtype", OTHER)
+@pytest.mark.parametrize("nrows,ncols", [(4, 256), (1, 512), (37, 768), (33, 4096), (260, 11008),
+                                         (4096, 4096), (7, 14336)])
+def test_gemv_remaining_block_formats(gpu, qtype, nrows, ncols):
+    # the formats the reference's to_gpu_matrix also keeps quantized (gguf.rs:172-182), random
+    # block bits with finite scales: result against the float64 dot product of the bit-exact
+    # dequantized weights
+    be = npref.BLOCK_ELEMS[qtype]
+    raw = npref.random_blocks(qtype, nrows * ncols // be, seed=3000 + qtype + nrows)
+    x = W.rng_normal(4000 + ncols, ncols)
+    _, ref = orc.gemv_quant(qtype, raw, nrows, ncols, x)
+    ok, e = close(gemv(gpu, qtype, raw, nrows, ncols, x), ref)
+    assert ok, e
+
+
+@pytest.mark.parametrize("qtype", OTHER)
+def test_gemv_remaining_formats_all_ones_vector_sums_rows(gpu, qtype):
+    # x = 1 is exact in the block fixed-point staging, so the result is the row sum of the
+    # dequantized weights up to fp32 rounding of the per-block scaling
+    be = npref.BLOCK_ELEMS[qtype]
+    nrows, ncols = 8, 1024
+    raw = npref.random_blocks(qtype, nrows * ncols // be, seed=77)
+    w = orc.dequantize(qtype, raw, nrows * ncols).reshape(nrows, ncols).astype(np.float64)
+    x = np.ones(ncols, np.float32)
+    got = gemv(gpu, qtype, raw, nrows, ncols, x)
+    np.testing.assert_allclose(got, w.sum(axis=1), rtol=2e-5, atol=2e-5 * np.abs(w).sum(axis=1).max())

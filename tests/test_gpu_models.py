@@ -274,3 +274,37 @@ def test_gpt2_matrix_replaced_after_a_recorded_run(gpu):
         want, _ = orc.Gpt2(w).generate_greedy(prompt, p.n_seq)
         assert np.array_equal(m.generate_greedy(prompt, p.n_seq), want), name
     assert not np.array_equal(want, want0)
+
+
+@pytest.mark.parametrize("qtype", [W.Q4_0, W.Q4_1, W.Q5_0, W.Q5_1, W.Q5_K, W.Q8_K])
+def test_llama_micro_in_the_remaining_block_formats(gpu, qtype):
+    # a model whose matrices are all in one of the formats beside Q8_0 / Q4_K / Q6_K: they
+    # stay quantized on the device (one launch per matrix, no fused launches), the prompt pass
+    # falls back to one step per token; logits, KV rows and greedy tokens against the oracle
+    import npref
+
+    w = synth_llama(MICRO, seed=61, scheme="f32")
+    for layer in w.layers:
+        for name, v in list(layer.items()):
+            if isinstance(v, HostMatrix):
+                vals = v.data.view(np.float32)
+                layer[name] = HostMatrix(qtype, v.nrows, v.ncols, npref.encode_simple(qtype, vals))
+    w.output = HostMatrix(qtype, w.output.nrows, w.output.ncols,
+                          npref.encode_simple(qtype, w.output.data.view(np.float32)))
+    spice(w, MICRO, 9, biases=False)
+    ref = orc.Llama2(w)
+    m = Llama2(gpu, MICRO).load(w)
+    toks = [3, 300, 17, 250, 9, 1]
+    for pos, t in enumerate(toks):
+        ok, e = logits_close(m.forward_logits(pos, t), ref.forward(t, pos))
+        assert ok, (pos, e)
+    want_k = ref.key_cache(1)[:len(toks)].copy()
+    np.testing.assert_allclose(m.kv_download(1, 0, 0, len(toks)), want_k, rtol=0,
+                               atol=1e-3 * np.abs(want_k).max())
+    m2 = Llama2(gpu, MICRO).load(w)
+    m2.prefill(toks)  # no batched product for these formats: steps through the prompt
+    ok, e = logits_close(m2.logits(), ref.forward(toks[-1], len(toks) - 1))
+    assert ok, e
+    prompt = W.prompt_tokens(61, 4, MICRO.vocab_size)
+    want, _ = orc.Llama2(w).generate_greedy(prompt, 20)
+    assert np.array_equal(Llama2(gpu, MICRO).load(w).generate_greedy(prompt, 20), want)

@@ -59,18 +59,19 @@ def test_dequant_random_bits_bit_exact(gpu, qtype, nrows, nblk_per_row):
     assert np.array_equal(bits(got), bits(want))
 
 
-EXPANDED = [("q4_0", W.Q4_0), ("q4_1", W.Q4_1), ("q5_0", W.Q5_0), ("q5_1", W.Q5_1),
-            ("q5_k", W.Q5_K), ("q8_k", W.Q8_K)]
+OTHER = [("q4_0", W.Q4_0), ("q4_1", W.Q4_1), ("q5_0", W.Q5_0), ("q5_1", W.Q5_1),
+         ("q5_k", W.Q5_K), ("q8_k", W.Q8_K)]
 
 
-@pytest.mark.parametrize("name,qtype", EXPANDED)
-def test_formats_expanded_to_f32_at_load(gpu, name, qtype):
-    # GgufTensorData::to_gpu_matrix dequantizes these to an f32 matrix (gguf.rs:131-184); here the
-    # expansion runs on the device.  Reference fixture blocks, then random bits; bit-exact.
+@pytest.mark.parametrize("name,qtype", OTHER)
+def test_remaining_block_formats_stay_quantized(gpu, name, qtype):
+    # GgufTensorData::to_gpu_matrix keeps these quantized on the GPU too (gguf.rs:172-182); the
+    # matrix holds the GGUF bytes unchanged.  Reference fixture blocks, then random bits; the
+    # dequantization kernel is bit-exact, the GEMV within the GEMV tolerance.
     raw, want = GOLD[f"{name}_raw"], GOLD[f"{name}_expected"]
     be = npref.BLOCK_ELEMS[qtype]
     m = W.GpuQuantMatrix(gpu, qtype, 2, 8 * be, raw)
-    assert m.shape() == (W.F32, 2, 8 * be) and m.gguf_bytes() == 2 * 8 * be * 4
+    assert m.shape() == (qtype, 2, 8 * be) and m.gguf_bytes() == raw.size
     assert np.array_equal(bits(gpu_dequant(gpu, qtype, raw, 2, 8 * be)), bits(want))
     nrows, nblk = 5, 7
     rnd = npref.random_blocks(qtype, nrows * nblk, seed=500 + qtype)
@@ -78,13 +79,16 @@ def test_formats_expanded_to_f32_at_load(gpu, name, qtype):
     assert np.array_equal(bits(gpu_dequant(gpu, qtype, rnd, nrows, nblk * be)), bits(want))
     # host dequantizer, same values
     assert np.array_equal(bits(W.dequantize_host(qtype, rnd, want.size)), bits(want))
-    # and the matrix is usable by the GEMV (f32 path)
-    x = W.rng_normal(5, nblk * be)
-    out = W.GpuVector.uninit(gpu, nrows)
-    W.GemvQuant.from_device(gpu).dispatch(out, W.GpuQuantMatrix(gpu, qtype, nrows, nblk * be, rnd),
-                                          W.GpuVector.init(gpu, x))
-    ref = want.reshape(nrows, -1).astype(np.float64) @ x.astype(np.float64)
-    np.testing.assert_allclose(out.read(), ref, rtol=0, atol=1e-4 * np.abs(ref).max())
+    # the fixture blocks through the GEMV: one-hot vectors return dequantized columns
+    ncols = 8 * be
+    gm = W.GemvQuant.from_device(gpu)
+    ref = GOLD[f"{name}_expected"].reshape(2, ncols)
+    for col in (0, 1, 15, 16, 31, ncols - 1, ncols // 2 + 3):
+        x = np.zeros(ncols, np.float32)
+        x[col] = 1.0
+        out = W.GpuVector.uninit(gpu, 2)
+        gm.dispatch(out, m, W.GpuVector.init(gpu, x))
+        np.testing.assert_allclose(out.read(), ref[:, col], rtol=1e-6, atol=0)
 
 
 def test_f16_matrix_expanded_at_load(gpu):

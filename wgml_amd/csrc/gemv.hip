@@ -274,6 +274,86 @@ struct FmtQ8_0 {
     }
 };
 
+// ----------------------------------------- the 32-element GGUF blocks ----
+// Q4_0 (18 B: d, 16 B of nibbles), Q4_1 (20 B: d, m, nibbles), Q5_0 (22 B: d, 32 fifth
+// bits, nibbles), Q5_1 (24 B: d, m, fifth bits, nibbles); quantization.rs:47-162 of the
+// reference.  The bytes stay as in the GGUF file (blocks are only 2-byte aligned: the loads
+// below are unaligned 16-byte loads, which gfx950 serves).  A tile is one block: element k
+// of a block is the low nibble of qs[k] for k < 16, the high nibble of qs[k-16] otherwise,
+// plus bit k of qh as its fifth bit.  Integer-dot kernels only.
+template <int BYTES, bool HAS_M, bool HAS_QH>
+struct FmtLegacy {
+    struct Row {
+        uint4 q;
+        uint32_t qh;
+        uint16_t d, m;
+    };
+    struct RowBase {
+        const uint8_t *blocks;
+    };
+    __device__ static RowBase row_base(const GemvParams &p, uint32_t row) {
+        return {p.p0 + (size_t)row * (p.ncols / 32) * BYTES};
+    }
+    __device__ static void load(Row &w, const RowBase &rb, uint32_t tile) {
+        const uint8_t *b = rb.blocks + (size_t)tile * BYTES;
+        __builtin_memcpy(&w.d, b, 2);
+        w.m = 0;
+        w.qh = 0;
+        if (HAS_M) __builtin_memcpy(&w.m, b + 2, 2);
+        if (HAS_QH) __builtin_memcpy(&w.qh, b + 2 + (HAS_M ? 2 : 0), 4);
+        __builtin_memcpy(&w.q, b + 2 + (HAS_M ? 2 : 0) + (HAS_QH ? 4 : 0), 16);
+    }
+};
+using FmtQ4_0 = FmtLegacy<18, false, false>;
+using FmtQ4_1 = FmtLegacy<20, true, false>;
+using FmtQ5_0 = FmtLegacy<22, false, true>;
+using FmtQ5_1 = FmtLegacy<24, true, true>;
+
+// Q8_K (292 B: f32 d, 256 int8, 16 block sums that dequantization does not use;
+// quantization.rs:170-199).  A tile is 32 of the 256 quants.
+struct FmtQ8K {
+    struct Row {
+        uint4 a, b;
+        float d;
+    };
+    struct RowBase {
+        const uint8_t *blocks;
+    };
+    __device__ static RowBase row_base(const GemvParams &p, uint32_t row) {
+        return {p.p0 + (size_t)row * (p.ncols / 256) * 292};
+    }
+    __device__ static void load(Row &w, const RowBase &rb, uint32_t tile) {
+        const uint8_t *b = rb.blocks + (size_t)(tile >> 3) * 292;
+        __builtin_memcpy(&w.d, b, 4);
+        __builtin_memcpy(&w.a, b + 4 + (tile & 7) * 32, 16);
+        __builtin_memcpy(&w.b, b + 4 + (tile & 7) * 32 + 16, 16);
+    }
+};
+
+// Q5_K (176 B: d, dmin, scales[12] as Q4_K, 32 bytes of fifth bits, 128 bytes of nibbles;
+// quantization.rs:249-317).  A tile is a 64-element group as for Q4_K: sub-blocks 2j (low
+// nibbles) and 2j+1 (high nibbles), whose fifth bits are bits 2j and 2j+1 of qh[l].
+struct FmtQ5K {
+    struct Row {
+        uint4 hdr, qa, qb, ha, hb;
+    };
+    struct RowBase {
+        const uint8_t *blocks;
+    };
+    __device__ static RowBase row_base(const GemvParams &p, uint32_t row) {
+        return {p.p0 + (size_t)row * (p.ncols / 256) * 176};
+    }
+    __device__ static void load(Row &w, const RowBase &rb, uint32_t tile) {
+        const uint8_t *blk = rb.blocks + (size_t)(tile >> 2) * 176;
+        w.hdr = *reinterpret_cast<const uint4 *>(blk);
+        w.ha = *reinterpret_cast<const uint4 *>(blk + 16);
+        w.hb = *reinterpret_cast<const uint4 *>(blk + 32);
+        const uint4 *q = reinterpret_cast<const uint4 *>(blk + 48 + (tile & 3) * 32);
+        w.qa = q[0];
+        w.qb = q[1];
+    }
+};
+
 // LDS layout: x as float4 xs[step][chunk][lane]; then sums[sum][tile_padded].
 template <class F>
 __device__ __forceinline__ uint32_t lds_slot(uint32_t tile, uint32_t chunk) {
@@ -628,6 +708,150 @@ struct IFmtQ8_0 {
                 l = sdot4(q, (&xl[k >> 2].x)[k & 3], l);
             }
             acc[r] = fmaf(f16_bits_to_f32(w[r].d) * s0, (float)((h << 8) + l), acc[r]);
+        }
+    }
+};
+
+// Bits 0..3 of b moved to bit 4 of bytes 0..3 (the fifth bits of four 5-bit quants).
+__device__ __forceinline__ uint32_t spread_bit4(uint32_t b) {
+    return ((b * 0x00204081u) & 0x01010101u) << 4;
+}
+
+template <int BYTES, bool HAS_M, bool HAS_QH>
+struct IFmtLegacy {
+    using W = FmtLegacy<BYTES, HAS_M, HAS_QH>;
+    static constexpr int TILE = 32, XB = 32, NXB = 1, NSUM = 1;
+    __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
+        tile = e >> 5;
+        local = e & 31;
+        xb = 0;
+    }
+    struct X {
+        uint4 xh[2], xl[2];
+        float s0, S0;  // scale of the block's fixed-point activations, sum of the rounded values
+    };
+    __device__ static void load_x(X &x, const uint4 *xq, const float *meta) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            x.xh[c] = xq[c * 64];
+            x.xl[c] = xq[(2 + c) * 64];
+        }
+        x.s0 = meta[0];
+        x.S0 = meta[1];
+    }
+    template <int R>
+    __device__ static void accumulate(const typename W::Row (&w)[R], const X &x, uint32_t,
+                                      float (&acc)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int h = 0, l = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t q = (&w[r].q.x)[k];
+                uint32_t lo = q & 0x0f0f0f0fu, hi = (q >> 4) & 0x0f0f0f0fu;
+                if (HAS_QH) {
+                    lo |= spread_bit4((w[r].qh >> (4 * k)) & 15u);
+                    hi |= spread_bit4((w[r].qh >> (16 + 4 * k)) & 15u);
+                }
+                h = sdot4(lo, (&x.xh[0].x)[k], h);
+                l = sdot4(lo, (&x.xl[0].x)[k], l);
+                h = sdot4(hi, (&x.xh[1].x)[k], h);
+                l = sdot4(hi, (&x.xl[1].x)[k], l);
+            }
+            const float dot = (float)((h << 8) + l) * x.s0;  // sum of quant * x over the block
+            const float d = f16_bits_to_f32(w[r].d);
+            if (HAS_M)  // y = d q + m   (quantization.rs:93-96, 160-165)
+                acc[r] += fmaf(d, dot, f16_bits_to_f32(w[r].m) * x.S0);
+            else  // y = d (q - 8) or d (q - 16)   (quantization.rs:62-66, 123-129)
+                acc[r] = fmaf(d, fmaf(HAS_QH ? -16.f : -8.f, x.S0, dot), acc[r]);
+        }
+    }
+};
+using IFmtQ4_0 = IFmtLegacy<18, false, false>;
+using IFmtQ4_1 = IFmtLegacy<20, true, false>;
+using IFmtQ5_0 = IFmtLegacy<22, false, true>;
+using IFmtQ5_1 = IFmtLegacy<24, true, true>;
+
+struct IFmtQ8K {
+    using W = FmtQ8K;
+    static constexpr int TILE = 32, XB = 32, NXB = 1, NSUM = 0;
+    __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
+        tile = e >> 5;
+        local = e & 31;
+        xb = 0;
+    }
+    using X = IFmtQ8_0::X;
+    __device__ static void load_x(X &x, const uint4 *xq, const float *meta) {
+        IFmtQ8_0::load_x(x, xq, meta);
+    }
+    template <int R>
+    __device__ static void accumulate(const W::Row (&w)[R], const X &x, uint32_t,
+                                      float (&acc)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int h = 0, l = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t q = k < 4 ? (&w[r].a.x)[k] : (&w[r].b.x)[k - 4];
+                h = sdot4(q, (&x.xh[k >> 2].x)[k & 3], h);
+                l = sdot4(q, (&x.xl[k >> 2].x)[k & 3], l);
+            }
+            acc[r] = fmaf(w[r].d * x.s0, (float)((h << 8) + l), acc[r]);
+        }
+    }
+};
+
+struct IFmtQ5K {
+    using W = FmtQ5K;
+    static constexpr int TILE = 64, XB = 32, NXB = 2, NSUM = 2;
+    __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
+        IFmtQ4K::locate(e, tile, local, xb);
+    }
+    using X = IFmtQ4K::X;
+    __device__ static void load_x(X &x, const uint4 *xq, const float *meta) {
+        IFmtQ4K::load_x(x, xq, meta);
+    }
+    template <int R>
+    __device__ static void accumulate(const W::Row (&w)[R], const X &x, uint32_t tile,
+                                      float (&acc)[R]) {
+        const uint4(&xh)[4] = x.xh;
+        const uint4(&xl)[4] = x.xl;
+        const float4 mt = x.mt;
+        const uint32_t j = tile & 3;
+        const uint32_t sh = (j & 1u) * 16u;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int hlo = 0, llo = 0, hhi = 0, lhi = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t q = k < 4 ? (&w[r].qa.x)[k] : (&w[r].qb.x)[k - 4];
+                const uint32_t H = (k < 4 ? (&w[r].ha.x)[k] : (&w[r].hb.x)[k - 4]) >> (2 * j);
+                const uint32_t lo = (q & 0x0f0f0f0fu) | ((H & 0x01010101u) << 4);
+                const uint32_t hi = ((q >> 4) & 0x0f0f0f0fu) | (((H >> 1) & 0x01010101u) << 4);
+                hlo = sdot4(lo, (&xh[k >> 2].x)[k & 3], hlo);
+                llo = sdot4(lo, (&xl[k >> 2].x)[k & 3], llo);
+                hhi = sdot4(hi, (&xh[2 + (k >> 2)].x)[k & 3], hhi);
+                lhi = sdot4(hi, (&xl[2 + (k >> 2)].x)[k & 3], lhi);
+            }
+            const float flo = (float)((hlo << 8) + llo) * mt.x;
+            const float fhi = (float)((hhi << 8) + lhi) * mt.y;
+            const float d = f16_bits_to_f32((uint16_t)(w[r].hdr.x & 0xffffu));
+            const float dmin = f16_bits_to_f32((uint16_t)(w[r].hdr.x >> 16));
+            // 6-bit scale / min pairs of sub-blocks 2j and 2j+1 (get_scale_min_k4)
+            const uint32_t a = (w[r].hdr.y >> sh) & 0xffffu, b = (w[r].hdr.z >> sh) & 0xffffu,
+                           c = (w[r].hdr.w >> sh) & 0xffffu;
+            uint32_t sc2, m2;
+            if (j < 2) {
+                sc2 = a & 0x3f3fu;
+                m2 = b & 0x3f3fu;
+            } else {
+                sc2 = (c & 0x0f0fu) | ((a >> 2) & 0x3030u);
+                m2 = ((c >> 4) & 0x0f0fu) | ((b >> 2) & 0x3030u);
+            }
+            float v = (d * ub0(sc2)) * flo;
+            v = fmaf(d * ub1(sc2), fhi, v);
+            v = fmaf(-dmin, fmaf(ub0(m2), mt.z, ub1(m2) * mt.w), v);
+            acc[r] += v;
         }
     }
 };
@@ -1288,7 +1512,9 @@ int launch_rd_i8(wgml_ctx *ctx, const GemvParams &p, size_t lds, int waves) {
     }
 }
 
-template <class F>
+// SWEEP: the variants the tuning keys select (rows per wave, waves per workgroup, depth) exist
+// for this format; otherwise only the default one.
+template <class F, bool SWEEP = true>
 int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
     constexpr int PCH = F::TILE / 16, MF = F::NXB + F::NSUM;
     const uint32_t ntiles = p.ncols / F::TILE;
@@ -1312,14 +1538,21 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
     if (p.ln_g && (p.ncols >> 2) > 3u * (uint32_t)waves * 64u)  // XP float4 per thread
         return set_error(WGML_E_UNSUPPORTED, "gemv_quant: %u columns are too many for the folded "
                                              "LayerNorm", p.ncols);
-    if (R == 2) {
-        if (depth >= 2) return launch_rd_i8<F, 2, 2>(ctx, p, lds, waves);
-        return launch_rd_i8<F, 2, 1>(ctx, p, lds, waves);
+    if constexpr (SWEEP) {
+        if (R == 2) {
+            if (depth >= 2) return launch_rd_i8<F, 2, 2>(ctx, p, lds, waves);
+            return launch_rd_i8<F, 2, 1>(ctx, p, lds, waves);
+        }
+        if (depth >= 4) return launch_rd_i8<F, 1, 4>(ctx, p, lds, waves);
+        if (depth == 3) return launch_rd_i8<F, 1, 3>(ctx, p, lds, waves);
+        if (depth == 2) return launch_rd_i8<F, 1, 2>(ctx, p, lds, waves);
+        return launch_rd_i8<F, 1, 1>(ctx, p, lds, waves);
+    } else {
+        if (p.ln_g && (p.ncols >> 2) > 3u * 1024u)
+            return set_error(WGML_E_UNSUPPORTED, "gemv_quant: %u columns are too many for the "
+                                                 "folded LayerNorm", p.ncols);
+        return launch_variant_i8<F, 1, 1, 1024>(ctx, p, lds);
     }
-    if (depth >= 4) return launch_rd_i8<F, 1, 4>(ctx, p, lds, waves);
-    if (depth == 3) return launch_rd_i8<F, 1, 3>(ctx, p, lds, waves);
-    if (depth == 2) return launch_rd_i8<F, 1, 2>(ctx, p, lds, waves);
-    return launch_rd_i8<F, 1, 1>(ctx, p, lds, waves);
 }
 
 // fp32-activation path: one configuration per format
@@ -1363,8 +1596,10 @@ int launch_gemv_f32(wgml_ctx *ctx, float *out, const float *a, uint32_t nrows, u
                                                                                      nrows, ncols);
     } else {
         const size_t lds = (((size_t)ncols + 3) / 4) * 16;
-        if (lds > 64 * 1024)
+        if (lds > kMaxLds)
             return set_error(WGML_E_UNSUPPORTED, "gemv_f32: %u columns exceed the LDS limit", ncols);
+        int unused = 0;  // opts in to more than 64 KB of LDS when the row needs it
+        WGML_TRY(blocks_per_cu(ctx, (const void *)gemv_f32_kernel, 256, lds, &unused));
         const int vec4 = (ncols % 4 == 0) && ((uintptr_t)a % 16 == 0);
         GemvParams p{};
         p.p0 = reinterpret_cast<const uint8_t *>(a);
@@ -1401,18 +1636,31 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
     p.ln_g = ep.ln_gamma;
     p.ln_b = ep.ln_beta;
     p.act = ep.act;
-    if ((p.ln_g || p.act) && (m->type == WGML_F32 || ctx->tuning[WGML_TUNE_GEMV_F32_ACTIVATIONS]))
+    const bool main_fmt = m->type == WGML_Q4_K || m->type == WGML_Q6_K || m->type == WGML_Q8_0;
+    if ((p.ln_g || p.act) &&
+        (m->type == WGML_F32 || (main_fmt && ctx->tuning[WGML_TUNE_GEMV_F32_ACTIVATIONS])))
         return set_error(WGML_E_UNSUPPORTED,
                          "gemv_quant: LayerNorm / activation folding needs the integer-dot path");
     if (m->type == WGML_F32) {
         const size_t lds = (size_t)m->ncols * 4;
-        if (lds > 64 * 1024)
+        if (lds > kMaxLds)
             return set_error(WGML_E_UNSUPPORTED, "gemv_f32: %u columns exceed the LDS limit",
                              m->ncols);
+        int unused = 0;  // opts in to more than 64 KB of LDS when the row needs it
+        WGML_TRY(blocks_per_cu(ctx, (const void *)gemv_f32_kernel, 256, lds, &unused));
         gemv_f32_kernel<<<dim3((m->nrows + 3) / 4), dim3(256), lds, ctx->stream>>>(p, 1);
         WGML_CHECK_LAUNCH();
         ctx->launches++;
         return WGML_OK;
+    }
+    switch (m->type) {  // formats that exist as integer-dot kernels only
+    case WGML_Q4_0: return launch_fmt_i8<IFmtQ4_0, false>(ctx, p);
+    case WGML_Q4_1: return launch_fmt_i8<IFmtQ4_1, false>(ctx, p);
+    case WGML_Q5_0: return launch_fmt_i8<IFmtQ5_0, false>(ctx, p);
+    case WGML_Q5_1: return launch_fmt_i8<IFmtQ5_1, false>(ctx, p);
+    case WGML_Q5_K: return launch_fmt_i8<IFmtQ5K, false>(ctx, p);
+    case WGML_Q8_K: return launch_fmt_i8<IFmtQ8K, false>(ctx, p);
+    default: break;
     }
     if (!ctx->tuning[WGML_TUNE_GEMV_F32_ACTIVATIONS]) {
         switch (m->type) {

@@ -614,14 +614,21 @@ int wgml_llama2_prefill(wgml_llama2 *m, const uint32_t *tokens, uint32_t n_token
     for (uint32_t i = 0; i < n_tokens; ++i)
         WGML_REQUIRE(tokens[i] < c.vocab_size,
                      "wgml_llama2_prefill: token %u outside vocabulary %u", tokens[i], c.vocab_size);
+    wgml_ctx *ctx = m->ctx;
+    bool batched = true;
     for (const LlamaLayer &w : m->layers)
         for (const wgml_qmat *q : {w.attn_q, w.attn_k, w.attn_v, w.attn_output, w.ffn_gate, w.ffn_up,
                                    w.ffn_down})
-            if (!gemm_supported(q))
-                return set_error(WGML_E_UNSUPPORTED,
-                                 "wgml_llama2_prefill: layer matrices must be Q8_0, Q4_K or Q6_K "
-                                 "(found type %d)", q->type);
-    wgml_ctx *ctx = m->ctx;
+            if (!gemm_supported(q)) batched = false;
+    if (!batched) {
+        // The batched products exist for Q8_0, Q4_K and Q6_K.  A model with a matrix in another
+        // format takes the prompt the way the reference does: one step per token
+        // (chat_llama2.rs:155-228), which leaves the same state.
+        const uint64_t launches0 = ctx->launches;
+        for (uint32_t i = 0; i < n_tokens; ++i) WGML_TRY(enqueue_step(m, false, tokens[i], start_pos + i));
+        m->launches_last = ctx->launches - launches0;
+        return WGML_OK;
+    }
     if (!m->pf_x) {
         int rc = WGML_OK;
         auto A = [&](float **p, uint64_t n) {

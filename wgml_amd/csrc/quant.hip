@@ -170,10 +170,14 @@ __global__ void dequant_raw_kernel(const uint8_t *__restrict__ raw, float *__res
     }
 }
 
-// True for the formats expanded to f32 at load.
-bool expands_to_f32(int type) {
-    return type == WGML_F16 || type == WGML_Q4_0 || type == WGML_Q4_1 || type == WGML_Q5_0 ||
-           type == WGML_Q5_1 || type == WGML_Q5_K || type == WGML_Q8_K;
+// True for the formats expanded to f32 at load: F16 only, as GgufTensorData::to_gpu_matrix
+// does (gguf.rs:131-184: every block format stays quantized on the GPU).
+bool expands_to_f32(int type) { return type == WGML_F16; }
+
+// Block formats whose bytes stay exactly as in the GGUF file (no re-layout).
+bool kept_raw(int type) {
+    return type == WGML_F32 || type == WGML_Q4_K || type == WGML_Q4_0 || type == WGML_Q4_1 ||
+           type == WGML_Q5_0 || type == WGML_Q5_1 || type == WGML_Q5_K || type == WGML_Q8_K;
 }
 
 uint32_t block_elems(int type) {
@@ -230,6 +234,18 @@ int launch_dequantize(wgml_ctx *ctx, float *out, const wgml_qmat *m) {
             m->p0, m->p1, (const int8_t *)m->p2, (const uint16_t *)m->p3, out, nb);
         break;
     }
+    case WGML_Q4_0: case WGML_Q4_1: case WGML_Q5_0: case WGML_Q5_1: case WGML_Q5_K: case WGML_Q8_K: {
+        const dim3 g((unsigned)((n + T - 1) / T)), b(T);
+        switch (m->type) {
+        case WGML_Q4_0: dequant_raw_kernel<WGML_Q4_0><<<g, b, 0, ctx->stream>>>(m->p0, out, n); break;
+        case WGML_Q4_1: dequant_raw_kernel<WGML_Q4_1><<<g, b, 0, ctx->stream>>>(m->p0, out, n); break;
+        case WGML_Q5_0: dequant_raw_kernel<WGML_Q5_0><<<g, b, 0, ctx->stream>>>(m->p0, out, n); break;
+        case WGML_Q5_1: dequant_raw_kernel<WGML_Q5_1><<<g, b, 0, ctx->stream>>>(m->p0, out, n); break;
+        case WGML_Q5_K: dequant_raw_kernel<WGML_Q5_K><<<g, b, 0, ctx->stream>>>(m->p0, out, n); break;
+        default: dequant_raw_kernel<WGML_Q8_K><<<g, b, 0, ctx->stream>>>(m->p0, out, n); break;
+        }
+        break;
+    }
     default: return set_error(WGML_E_UNSUPPORTED, "dequantize: unsupported type %d", m->type);
     }
     WGML_CHECK_LAUNCH();
@@ -257,8 +273,8 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
     if (!be)
         return set_error(WGML_E_UNSUPPORTED,
                          "wgml_quant_matrix_create: quantization type %d is not supported "
-                         "(quantized: Q8_0, Q4_K, Q6_K; expanded to f32: F32, F16, Q4_0, Q4_1, "
-                         "Q5_0, Q5_1, Q5_K, Q8_K)",
+                         "(F32, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, Q4_K, Q5_K, Q6_K, Q8_K; F16 is "
+                         "expanded to f32)",
                          type);
     WGML_REQUIRE(nrows > 0 && ncols > 0, "wgml_quant_matrix_create: empty matrix %ux%u", nrows,
                  ncols);
@@ -284,8 +300,10 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
     uint64_t o1 = 0, o2 = 0, o3 = 0, total = 0;
     if (expand) total = align256(nelem * 4);
     switch (expand ? -1 : type) {
-    case WGML_F32:
-    case WGML_Q4_K: total = align256(gguf); break;
+    case WGML_F32: case WGML_Q4_K: case WGML_Q4_0: case WGML_Q4_1: case WGML_Q5_0: case WGML_Q5_1:
+    case WGML_Q5_K: case WGML_Q8_K:
+        total = align256(gguf);
+        break;
     case WGML_Q8_0:
         o1 = align256(nblocks * 32);
         total = o1 + align256(nblocks * 2);
@@ -321,7 +339,7 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
                          hipGetErrorString(err));
     };
 
-    if (type == WGML_F32 || type == WGML_Q4_K) {
+    if (kept_raw(type)) {
         e = hipMemcpyAsync(m->base, gguf_bytes, gguf, hipMemcpyHostToDevice, ctx->stream);
         if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) return fail(e, "upload");
@@ -335,18 +353,9 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
             if (type == WGML_Q8_0) {
                 repack_q8_0<<<dim3((unsigned)((nblocks + T - 1) / T)), dim3(T), 0, ctx->stream>>>(
                     (const uint16_t *)raw, (uint32_t *)m->p0, (uint16_t *)m->p1, nblocks);
-            } else if (expand) {
-                const dim3 g((unsigned)((nelem + T - 1) / T)), b(T);
-                float *o = reinterpret_cast<float *>(m->p0);
-                switch (type) {
-                case WGML_F16: dequant_raw_kernel<WGML_F16><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
-                case WGML_Q4_0: dequant_raw_kernel<WGML_Q4_0><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
-                case WGML_Q4_1: dequant_raw_kernel<WGML_Q4_1><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
-                case WGML_Q5_0: dequant_raw_kernel<WGML_Q5_0><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
-                case WGML_Q5_1: dequant_raw_kernel<WGML_Q5_1><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
-                case WGML_Q5_K: dequant_raw_kernel<WGML_Q5_K><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
-                default: dequant_raw_kernel<WGML_Q8_K><<<g, b, 0, ctx->stream>>>(raw, o, nelem); break;
-                }
+            } else if (expand) {  // F16
+                dequant_raw_kernel<WGML_F16><<<dim3((unsigned)((nelem + T - 1) / T)), dim3(T), 0,
+                                               ctx->stream>>>(raw, reinterpret_cast<float *>(m->p0), nelem);
             } else {
                 uint64_t nt = nblocks * 105;
                 repack_q6_k<<<dim3((unsigned)((nt + T - 1) / T)), dim3(T), 0, ctx->stream>>>(
