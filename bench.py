@@ -124,7 +124,7 @@ def time_gate_up(W, gpu, cfg, weights):
     return best, nbytes
 
 
-def gemv_sweep(W, gpu, nrows, ncols, cpu_threads, min_total_bytes=640 << 20):
+def gemv_sweep(W, gpu, nrows, ncols, cpu_threads, min_total_bytes=640 << 20, formats=None):
     """One matrix shape for Q8_0 / Q4_K / Q6_K: GB/s and fraction of HBM peak on the GPU (the
     default integer-dot kernels and the fp32-activation kernels), and the CPU oracle's
     dequantize-and-dot over the same bytes on one core and on `cpu_threads` cores."""
@@ -135,6 +135,8 @@ def gemv_sweep(W, gpu, nrows, ncols, cpu_threads, min_total_bytes=640 << 20):
     vals = W.rng_normal(4242, nrows * ncols, 0.0, 0.02)
     xcpu = W.rng_normal(99, ncols)
     for qtype, name in ((W.Q8_0, "q8_0"), (W.Q4_K, "q4_k"), (W.Q6_K, "q6_k")):
+        if formats and name not in formats:
+            continue
         raw = W.quantize(qtype, vals)
         n_copies = max(2, -(-min_total_bytes // raw.nbytes))
         mats = [W.GpuQuantMatrix(gpu, qtype, nrows, ncols, raw) for _ in range(n_copies)]
@@ -145,7 +147,7 @@ def gemv_sweep(W, gpu, nrows, ncols, cpu_threads, min_total_bytes=640 << 20):
         b = gemv_bytes(raw.nbytes, nrows, ncols)
         gbs = b / us * 1e-3
         cpu = {}
-        for threads in sorted({1, cpu_threads}):
+        for threads in sorted({1, cpu_threads} if cpu_threads else ()):
             orc.set_threads(threads)
             t0 = time.perf_counter()
             orc.gemv_quant(qtype, raw, nrows, ncols, xcpu)
@@ -304,6 +306,10 @@ def main():
                          "counters")
     ap.add_argument("--sweep-only", action="store_true",
                     help="only the GEMV sweep, launch by launch (for profiler runs)")
+    ap.add_argument("--sweep-shape", default=None,
+                    help="with --sweep-only: one shape, ROWSxCOLS (e.g. 4096x11008), default all four")
+    ap.add_argument("--sweep-format", default=None,
+                    help="with --sweep-only: one of q8_0, q4_k, q6_k (default all three)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only the batched prompt pass over the prompt, 1 untimed + 3 timed calls "
                          "(for profiler runs)")
@@ -343,9 +349,13 @@ def main():
                  f"steps must fit the model's {cfg.seq_len} positions (and --warmup >= 1)")
 
     if args.sweep_only:
+        shapes = ((4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096))
+        if args.sweep_shape:
+            shapes = (tuple(int(v) for v in args.sweep_shape.split("x")),)
         with eager_launches():
-            for nrows, ncols in ((4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)):
-                gemv_sweep(W, gpu, nrows, ncols, 1)
+            for nrows, ncols in shapes:
+                gemv_sweep(W, gpu, nrows, ncols, 0,
+                           formats=(args.sweep_format,) if args.sweep_format else None)
         return
 
     t0 = time.perf_counter()
