@@ -310,6 +310,9 @@ def main():
                     help="with --sweep-only: one shape, ROWSxCOLS (e.g. 4096x11008), default all four")
     ap.add_argument("--sweep-format", default=None,
                     help="with --sweep-only: one of q8_0, q4_k, q6_k (default all three)")
+    ap.add_argument("--decode-only", action="store_true",
+                    help="only the prompt pass, the warm-up and the timed decode steps (for profiler "
+                         "runs: the kernel trace then holds the decode step and little else)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only the batched prompt pass over the prompt, 1 untimed + 3 timed calls "
                          "(for profiler runs)")
@@ -401,6 +404,18 @@ def main():
     model.prefill(prompt)
     first = int(np.argmax(model.logits()))
     p0 = n_prompt  # position of the first decode step
+
+    if args.decode_only:
+        wtoks = model.decode_greedy(first, p0, args.warmup)
+        gpu.synchronize()
+        t0 = time.perf_counter()
+        model.decode_greedy(int(wtoks[-1]), p0 + args.warmup, args.steps)
+        gpu.synchronize()
+        dt = time.perf_counter() - t0
+        print(json.dumps({"decode_steps": args.steps, "from_position": p0 + args.warmup,
+                          "tok_s": round(args.steps / dt, 2),
+                          "launches_per_token": model.launches_per_token()}), flush=True)
+        return
 
     # the same steps with a blocking read-back of every sampled token, as the reference's
     # chat loop does (reported beside the headline figure; part of the warm-up)

@@ -89,6 +89,9 @@ enum {
     WGML_TUNE_GEMV_F32_ACTIVATIONS,          /* 1: fp32 activations instead of 16-bit block fixed point */
     WGML_TUNE_GEMM_K_SPLIT,                  /* 1..8 workgroups share the K range of a batched product */
     WGML_TUNE_PREFILL_ATTENTION_PER_TOKEN,   /* 1: one workgroup per (head, token) in the prompt pass */
+    WGML_TUNE_ATTN_WIDE_POSITIONS,           /* decode attention planned for up to this many positions runs
+                                                as one workgroup per head group, without partial results */
+    WGML_TUNE_ATTN_SPLITS,                   /* workgroups that share the positions of a head group, 2..64 */
     WGML_TUNE_COUNT
 };
 WGML_API int wgml_ctx_set_tuning(wgml_ctx *ctx, int key, int value);
@@ -410,6 +413,16 @@ WGML_API int wgml_bench_gemv_fused(wgml_ctx *ctx, const wgml_qmat *const *a,
                                    const wgml_qmat *const *b, const int *modes, uint32_t njobs,
                                    uint32_t nsets, wgml_view out, uint32_t stride, wgml_view v,
                                    const wgml_view *norm_w, uint32_t iters, float *total_ms);
+
+/* The same loop for the decode attention of one layer (BatchedMultiqueryAttention::dispatch,
+ * ops/batched_multiquery_attention.rs:99-136): launch i reads the KV caches of set i % n_sets
+ * (seq_len x kv_dim each), the position p->pos comes from device memory as in a recorded decode
+ * step, and the launch grid is the one a recorded step planned for `plan_positions` positions
+ * (p->pos < plan_positions <= p->seq_len) would use. */
+WGML_API int wgml_bench_attention(wgml_ctx *ctx, const wgml_attn_params *p, uint32_t plan_positions,
+                                  wgml_view q, const wgml_view *key_caches,
+                                  const wgml_view *value_caches, uint32_t n_sets, wgml_view xb,
+                                  uint32_t iters, float *total_ms);
 
 /* ---- tokenizers (host only) ------------------------------------------------ *
  * The vocabulary is handed over as one block of UTF-8 bytes plus n + 1 offsets

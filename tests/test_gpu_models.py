@@ -230,6 +230,53 @@ def test_gpt2_124m_greedy_prefix(gpu):
     assert np.array_equal(m.generate_greedy(prompt, n_total), want)
 
 
+def _same_where_decided(got, want, margins, scale):
+    # the oracle's arg-max is only binding where its top-2 margin is wider than the logit
+    # error the kernels may have (1e-3 of the logit scale, twice)
+    decided = margins > 2e-3 * scale
+    assert decided.mean() > 0.5
+    assert np.array_equal(got[decided], want[decided]), np.nonzero(got != want)[0]
+
+
+def test_gpt2_124m_long_prompt_across_recorded_ranges(gpu):
+    # the recorded step is captured once per range of positions (attention planned for 256,
+    # 512, 1024 positions): a forced 540-token prompt + 8 generated tokens walk through all three
+    p = GPT2_124M
+    w = synth_gpt2(p, seed=3)
+    n_prompt, n_total = 540, 548
+    prompt = W.prompt_tokens(5, n_prompt, p.n_vocab)
+    orc.set_threads(8)
+    try:
+        ref = orc.Gpt2(w, predequantize=True)
+        want, margins = ref.generate_greedy(prompt, n_total)
+        scale = float(np.abs(ref.forward(int(prompt[0]), 0)).max())
+    finally:
+        orc.set_threads(1)
+    m = Gpt2(gpu, p).load(w)
+    got = m.generate_greedy(prompt, n_total)
+    _same_where_decided(got, want, margins, scale)
+    assert np.array_equal(m.generate_greedy(prompt, n_total), got)  # replayable
+
+
+def test_llama_micro_long_prompt_across_recorded_ranges(gpu):
+    cfg = Llama2Config(dim=256, hidden_dim=512, n_layers=2, n_q_heads=4, n_kv_heads=2, vocab_size=500,
+                       seq_len=1100, rope_base_freq=10000.0, rms_norm_eps=1.0e-5)
+    w = synth_llama(cfg, seed=21, scheme="q4_k_m")
+    n_prompt, n_total = 1050, 1060
+    prompt = W.prompt_tokens(6, n_prompt, cfg.vocab_size)
+    ref = orc.Llama2(w)
+    want, margins = ref.generate_greedy(prompt, n_total)
+    scale = float(np.abs(ref.forward(int(prompt[0]), 0)).max())
+    m = Llama2(gpu, cfg).load(w)
+    got = m.generate_greedy(prompt, n_total)
+    _same_where_decided(got, want, margins, scale)
+    # a second run that starts inside the second range, from the KV cache the first one left
+    # (only its first step sees the forced prompt's context and nothing else)
+    tail = m.decode_greedy(int(prompt[300]), 300, 4)
+    if margins[300] > 2e-3 * scale:
+        assert int(tail[0]) == int(want[300])
+
+
 def test_gpt2_micro_greedy_with_norm_affine(gpu):
     # non-trivial LayerNorm gains / shifts and biases through the folded, recorded loop
     p = Gpt2Params(n_vocab=300, n_seq=48, n_embd=128, n_head=4, n_layer=3, ff_len=512, attn_b=384)

@@ -153,6 +153,8 @@ PROTOTYPES = {
     "wgml_bench_gemv_quant": (_i, [_P, _PP, _u32, View, View, _u32, _i, _fp]),
     "wgml_bench_gemv_fused": (_i, [_P, _PP, _PP, C.POINTER(C.c_int), _u32, _u32, View, _u32, View,
                                    C.POINTER(View), _u32, _fp]),
+    "wgml_bench_attention": (_i, [_P, C.POINTER(AttnParams), _u32, View, C.POINTER(View), C.POINTER(View),
+                                  _u32, View, _u32, _fp]),
     "wgml_sample": (_i, [_P, _u32, _f, _f, _f, _u32p]),
     "wgml_llama2_generate_sampled": (_i, [_P, _P, _u32, _u32, _f, _f, _u64, _P]),
     "wgml_gguf_open": (_i, [C.c_char_p, _PP]),

@@ -581,13 +581,15 @@ static bool fast_ok(const wgml_attn_params &p, bool aligned, bool wants_scores) 
            p.head_size <= 256;
 }
 
-constexpr uint32_t kWidePositions = 128;  // up to here one workgroup per head group
+constexpr uint32_t kWidePositions = 256;  // up to here one workgroup per head group
 
 static int make_fast_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions,
                           AttnPlan &pl) {
     const uint32_t hs = p.head_size;
     pl.nv = (int)((hs + 63) / 64);  // float4 per lane: 16 lanes x 4 floats x nv
-    pl.wide = (plan_positions <= kWidePositions && pl.nv <= 2) ? 1 : 0;
+    const int wide_tune = ctx->tuning[WGML_TUNE_ATTN_WIDE_POSITIONS];
+    const uint32_t wide_limit = wide_tune > 0 ? (uint32_t)wide_tune : kWidePositions;
+    pl.wide = (plan_positions <= wide_limit && pl.nv <= 2) ? 1 : 0;
     pl.km = 1;
     if (p.kv_mul == 2 || p.kv_mul == 4) pl.km = (int)p.kv_mul;
     if (p.kv_mul == 8) pl.km = 4;
@@ -603,11 +605,14 @@ static int make_fast_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pla
         return WGML_OK;
     }
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
-    // about two workgroups per CU, each with at least 16 positions at full length
+    // about two workgroups per CU, each with at least 64 positions at full length (four
+    // quads per wave; measured on 32 x 128 and 12 x 64 heads, shorter shares only add
+    // partial results for the merge to read)
     uint32_t n_wg_y = (2 * cu + pl.groups - 1) / pl.groups;
-    const uint32_t max_y = (plan_positions + 4 * WAVES - 1) / (4 * WAVES);
+    const uint32_t max_y = (plan_positions + 16 * WAVES - 1) / (16 * WAVES);
     if (n_wg_y > max_y) n_wg_y = max_y;
     if (n_wg_y > (uint32_t)MERGE_MAX_Y) n_wg_y = MERGE_MAX_Y;  // what the merge takes in one go
+    if (ctx->tuning[WGML_TUNE_ATTN_SPLITS] > 0) n_wg_y = (uint32_t)ctx->tuning[WGML_TUNE_ATTN_SPLITS];
     if (n_wg_y < 2) n_wg_y = 2;
     pl.n_wg_y = n_wg_y;
     return WGML_OK;

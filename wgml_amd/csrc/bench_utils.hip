@@ -129,4 +129,71 @@ int wgml_bench_gemv_fused(wgml_ctx *ctx, const wgml_qmat *const *a,
     return WGML_OK;
 }
 
+int wgml_bench_attention(wgml_ctx *ctx, const wgml_attn_params *p, uint32_t plan_positions,
+                         wgml_view q, const wgml_view *key_caches, const wgml_view *value_caches,
+                         uint32_t n_sets, wgml_view xb, uint32_t iters, float *total_ms) {
+    WGML_REQUIRE(ctx && p && key_caches && value_caches && total_ms && n_sets > 0 && iters > 0,
+                 "wgml_bench_attention: bad argument");
+    WGML_REQUIRE(p->n_heads > 0 && p->kv_mul > 0 && p->head_size > 0 && p->pos < p->seq_len &&
+                     plan_positions > p->pos && plan_positions <= p->seq_len &&
+                     p->kv_dim == p->n_heads / p->kv_mul * p->head_size,
+                 "wgml_bench_attention: inconsistent parameters");
+    WGML_TRY(check_view(q, "wgml_bench_attention: q"));
+    WGML_TRY(check_view(xb, "wgml_bench_attention: xb"));
+    const uint64_t dim = (uint64_t)p->n_heads * p->head_size;
+    WGML_REQUIRE(q.len >= dim && xb.len >= dim, "wgml_bench_attention: q / xb too short");
+    for (uint32_t s = 0; s < n_sets; ++s) {
+        WGML_TRY(check_view(key_caches[s], "wgml_bench_attention: key cache"));
+        WGML_TRY(check_view(value_caches[s], "wgml_bench_attention: value cache"));
+        WGML_REQUIRE(key_caches[s].len >= (uint64_t)p->seq_len * p->kv_dim &&
+                         value_caches[s].len >= (uint64_t)p->seq_len * p->kv_dim,
+                     "wgml_bench_attention: cache %u shorter than seq_len x kv_dim", s);
+    }
+    // the position comes from device memory, as in a recorded decode step
+    DynState *dyn = nullptr;
+    WGML_CHECK_HIP(hipMalloc(&dyn, sizeof(DynState)));
+    const DynState init{p->pos, 0, 0, 0};
+    hipError_t e = hipMemcpy(dyn, &init, sizeof(init), hipMemcpyHostToDevice);
+    DynPos dpos{};
+    dpos.ptr = &dyn->pos;
+    auto launch = [&](uint32_t i) {
+        return launch_attention_planned(ctx, *p, dpos, plan_positions, p->seq_len, view_ptr(q),
+                                        view_ptr(key_caches[i % n_sets]),
+                                        view_ptr(value_caches[i % n_sets]), nullptr, view_ptr(xb));
+    };
+    int rc = e == hipSuccess ? reserve_attention_workspace(ctx, *p, plan_positions) : WGML_E_HIP;
+    for (uint32_t s = 0; s < n_sets && s < iters && rc == WGML_OK; ++s) rc = launch(s);
+    if (rc == WGML_OK && hipStreamSynchronize(ctx->stream) != hipSuccess) rc = WGML_E_HIP;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    if (rc == WGML_OK) {
+        const bool eager = graphs_disabled();
+        if (!eager) {
+            e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+            for (uint32_t i = 0; i < iters && rc == WGML_OK && e == hipSuccess; ++i) rc = launch(i);
+            if (e == hipSuccess) e = hipStreamEndCapture(ctx->stream, &graph);
+            if (e == hipSuccess && rc == WGML_OK) e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+            if (e == hipSuccess && rc == WGML_OK) e = hipGraphLaunch(exec, ctx->stream);
+            if (e == hipSuccess && rc == WGML_OK) e = hipStreamSynchronize(ctx->stream);
+        }
+        if (e == hipSuccess && rc == WGML_OK) e = hipEventRecord(ctx->ev_start, ctx->stream);
+        if (e == hipSuccess && rc == WGML_OK) {
+            if (eager)
+                for (uint32_t i = 0; i < iters && rc == WGML_OK; ++i) rc = launch(i);
+            else
+                e = hipGraphLaunch(exec, ctx->stream);
+        }
+        if (e == hipSuccess && rc == WGML_OK) e = hipEventRecord(ctx->ev_stop, ctx->stream);
+        if (e == hipSuccess && rc == WGML_OK) e = hipEventSynchronize(ctx->ev_stop);
+        if (e == hipSuccess && rc == WGML_OK) e = hipEventElapsedTime(total_ms, ctx->ev_start, ctx->ev_stop);
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    (void)hipFree(dyn);
+    if (rc != WGML_OK) return rc;
+    if (e != hipSuccess) return set_error(WGML_E_HIP, "wgml_bench_attention: %s", hipGetErrorString(e));
+    return WGML_OK;
+}
+
 }  // extern "C"

@@ -213,6 +213,23 @@ int launch_attention(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos, uint3
 // The same with the grid planned for `plan_positions` positions (seq_len when the launch is
 // recorded and replayed at growing positions).  `ext_ws`: optional caller-supplied workspace
 // for the partial results (ext_ws_bytes bytes) instead of the context's own.
+// A recorded decode step is captured once per range of positions ("bucket"): the attention
+// launch of a step is planned for the bucket's upper limit rather than for seq_len, so that
+// short contexts run the grid that suits them (one workgroup per head group and no partial
+// results up to 256 positions, few partials per head after that).  Limits: 256, 512, 1024, ...
+// doubling, the last one seq_len.
+constexpr int kMaxPlanBuckets = 24;
+inline uint32_t plan_bucket(uint32_t pos, uint32_t seq_len, int *index) {
+    uint32_t limit = 256;
+    int i = 0;
+    while (pos >= limit && limit < seq_len && i + 1 < kMaxPlanBuckets) {
+        limit <<= 1;
+        ++i;
+    }
+    if (index) *index = i;
+    return limit < seq_len ? limit : seq_len;
+}
+int reserve_attention_workspace(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions);
 int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
                              uint32_t plan_positions, uint32_t cache_rows, const float *q,
                              const float *kc, const float *vc, float *att, float *xb,

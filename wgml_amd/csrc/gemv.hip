@@ -962,51 +962,20 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
         }
     }
 
-    // The weight loads below and in the main loop are issued unconditionally (a lane
-    // without a tile re-reads tile 0, a wave without work row-group 0).  Only then
-    // can the compiler count the loads in flight and wait for exactly the one it
-    // needs: with a load under a condition it falls back to waiting for all of
-    // them, and the staging of x, a cache hit, would wait for the first weight
-    // tile to arrive from HBM.
-    typename WF::Row w[D][R];
-    uint32_t lg = first, lsub = 0, ls = 0;  // (group, pass, step) of the next load
-    // A wave's finished row sums are parked one per lane (result n in lane n) until the
-    // policy's epilogue at the end, so a wave takes at most 64 results: the host sizes
-    // the grid accordingly (plan_groups).  The loads of the first D iterations go out
-    // here; with fewer than D iterations the other register sets take a dummy load and
-    // are never consumed.
-    auto advance_load_cursor = [&]() {
-        if (++ls == nsteps) {
-            ls = 0;
-            if (++lsub == S) {
-                lsub = 0;
-                lg += GW;
-            }
-        }
-    };
-#pragma unroll
-    for (int d = 0; d < D; ++d) {
-        const uint32_t tile = ls * 64 + lane;
-        const bool ok = (uint32_t)d < n_it;
-        pol.template load<WF, R>(w[d], lg, lsub, ok && tile < ntiles ? tile : 0u, ok);
-        if (ok) advance_load_cursor();
-    }
-
     // Stage x as 16-bit block fixed point (two int8 planes) + per-block scale and sum.
     // A fused RMSNorm costs no extra pass and no extra barrier: the normalisation
     // factor rsqrt(mean(x^2) + eps) is one scalar for the whole vector, so x * w is
     // staged, the sum of squares is gathered on the way and the factor multiplies
     // the finished dot products instead.
-    __shared__ float red[16];
-    float out_scale = 1.f;
-    {
+    __shared__ float red[16], red_a[16], red_b[16];
+    auto stage_x = [&]() -> float {
+        float out_scale = 1.f;
         uint32_t *xq32 = reinterpret_cast<uint32_t *>(xq);
         float ss = 0.f;
         if (p.ln_g) {
             // LayerNorm folded in (host guarantees that the XP float4 per thread cover
             // x): mean, then variance about the mean (two exact passes over registers,
             // ops/layernorm.rs:46-53), then x <- (x - mean) * rstd * gamma + beta.
-            __shared__ float red_a[16], red_b[16];
             auto block_total = [&](float v, float *buf) {
                 v = wave_sum(v);
                 if (lane == 0) buf[wave] = v;
@@ -1112,7 +1081,43 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
             const float total = readlane_f32(row16_sum(part), 0);
             out_scale = 1.0f / sqrtf(total / (float)p.ncols + p.norm_eps);
         }
+        return out_scale;
+    };
+
+    // The weight loads below and in the main loop are issued unconditionally (a lane
+    // without a tile re-reads tile 0; a register set beyond the wave's last iteration
+    // re-reads the wave's own first tile, a cache hit).  Only then can the compiler
+    // count the loads in flight and wait for exactly the one it needs: with a load
+    // under a condition it falls back to waiting for all of them, and the staging of
+    // x, a cache hit, would wait for the first weight tile to arrive from HBM.
+    // A wave without any row re-reads row-group 0: the host sizes the workgroups so that
+    // only the last one can have such waves (thousands of idle waves asking for one and
+    // the same tile would queue up on a single cache line).
+    typename WF::Row w[D][R];
+    uint32_t lg = first, lsub = 0, ls = 0;  // (group, pass, step) of the next load
+    // A wave's finished row sums are parked one per lane (result n in lane n) until the
+    // policy's epilogue at the end, so a wave takes at most 64 results: the host sizes
+    // the grid accordingly (plan_groups).  The loads of the first D iterations go out
+    // here; with fewer than D iterations the other register sets take a dummy load and
+    // are never consumed.
+    auto advance_load_cursor = [&]() {
+        if (++ls == nsteps) {
+            ls = 0;
+            if (++lsub == S) {
+                lsub = 0;
+                lg += GW;
+            }
+        }
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        const bool ok = (uint32_t)d < n_it;
+        const uint32_t tile = ok ? ls * 64 + lane : lane;
+        pol.template load<WF, R>(w[d], ok ? lg : (n_it ? first : 0u), ok ? lsub : 0u, tile < ntiles ? tile : 0u, true);
+        if (ok) advance_load_cursor();
     }
+
+    const float out_scale = stage_x();
     if (n_it == 0) return;
 
     // XREG: a lane without a tile (rows shorter than 64 tiles) keeps an all-zero tile of
@@ -1193,8 +1198,11 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     pol.template finish<R>(mine, nres, first, GW, lane);
 }
 
-template <class F, int R, int D, int MAXT>
-__global__ __launch_bounds__(MAXT) void gemv_quant_i8_kernel(const GemvParams p) {
+// MINW: waves per SIMD the register allocation must leave room for (MAXT / 256 = one
+// workgroup per CU; twice that caps the kernel at 64 vector registers, so that two
+// 1024-thread workgroups share a CU).
+template <class F, int R, int D, int MAXT, int MINW = MAXT / 256>
+__global__ __launch_bounds__(MAXT, MINW) void gemv_quant_i8_kernel(const GemvParams p) {
     PlainPolicy pol{p, nullptr, 0.f, 0.f};
     const uint32_t ngroups = (p.nrows + R - 1) / R;
     if (p.ncols <= 64 * F::TILE)
@@ -1489,15 +1497,19 @@ WgPlan plan_groups(uint32_t ngroups, uint32_t max_wgs, uint32_t max_waves, uint3
     return {c, nw, wgs};
 }
 
-template <class F, int R, int D, int MAXT>
+template <class F, int R, int D, int MAXT, int MINW = MAXT / 256>
 int launch_variant_i8(wgml_ctx *ctx, const GemvParams &p0, size_t lds) {
     int per_cu = 1;
-    WGML_TRY(blocks_per_cu(ctx, (const void *)gemv_quant_i8_kernel<F, R, D, MAXT>, MAXT, lds, &per_cu));
+    WGML_TRY(blocks_per_cu(ctx, (const void *)gemv_quant_i8_kernel<F, R, D, MAXT, MINW>, MAXT, lds,
+                           &per_cu));
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
-    const WgPlan plan = plan_groups((p0.nrows + R - 1) / R, cu * (uint32_t)per_cu, MAXT / 64, 64 / R);
+    // every workgroup with all its waves at work (min_c): a workgroup with idle waves
+    // stages x for nothing, and idle waves re-read row-group 0
+    const WgPlan plan = plan_groups((p0.nrows + R - 1) / R, cu * (uint32_t)per_cu, MAXT / 64, 64 / R,
+                                    MAXT / 64);
     GemvParams p = p0;
     p.active_waves = plan.active_waves;
-    gemv_quant_i8_kernel<F, R, D, MAXT><<<dim3(plan.wgs), dim3(MAXT), lds, ctx->stream>>>(p);
+    gemv_quant_i8_kernel<F, R, D, MAXT, MINW><<<dim3(plan.wgs), dim3(MAXT), lds, ctx->stream>>>(p);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
@@ -1546,6 +1558,10 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
         if (depth >= 4) return launch_rd_i8<F, 1, 4>(ctx, p, lds, waves);
         if (depth == 3) return launch_rd_i8<F, 1, 3>(ctx, p, lds, waves);
         if (depth == 2) return launch_rd_i8<F, 1, 2>(ctx, p, lds, waves);
+        if constexpr (std::is_same_v<F, IFmtQ4K> || std::is_same_v<F, IFmtQ8_0>) {
+            // these fit 64 vector registers without spilling: two workgroups per CU
+            if (waves == 16) return launch_variant_i8<F, 1, 1, 1024, 8>(ctx, p, lds);
+        }
         return launch_rd_i8<F, 1, 1>(ctx, p, lds, waves);
     } else {
         if (p.ln_g && (p.ncols >> 2) > 3u * 1024u)

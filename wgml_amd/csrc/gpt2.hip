@@ -32,12 +32,13 @@ struct wgml_gpt2 {
     // recorded token loop: position / token / output cursor on the device
     DynState *dyn = nullptr;
     uint32_t *d_prompt = nullptr, *d_tokens = nullptr;
-    hipGraph_t graph = nullptr;
-    hipGraphExec_t graph_exec = nullptr;
+    // the recorded step, one capture per bucket of positions (plan_bucket)
+    hipGraph_t graph[kMaxPlanBuckets] = {};
+    hipGraphExec_t graph_exec[kMaxPlanBuckets] = {};
+    uint64_t graph_launches[kMaxPlanBuckets] = {};  // launches of the recorded step
     int fusion = 1;  // 0: one launch per op group as before; 1: folded launches
     int graph_fusion = -1;
     uint64_t launches_last = 0;   // launches of the last step that ran
-    uint64_t graph_launches = 0;  // launches of the recorded step
 };
 
 namespace {
@@ -126,8 +127,7 @@ int wgml_gpt2_create(wgml_ctx *ctx, const wgml_gpt2_params *p, wgml_gpt2 **out) 
 int wgml_gpt2_destroy(wgml_gpt2 *m) {
     if (!m) return WGML_OK;
     if (m->ctx && m->ctx->stream) (void)hipStreamSynchronize(m->ctx->stream);
-    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
-    if (m->graph) (void)hipGraphDestroy(m->graph);
+    drop_graph(m);
     for (void *p : m->allocs) (void)hipFree(p);
     ctx_release(m->ctx);
     delete m;
@@ -235,14 +235,15 @@ bool can_fold(const wgml_gpt2 *m) {
     return true;
 }
 
-int enqueue_step(wgml_gpt2 *m, bool dynamic, uint32_t token, uint32_t pos) {
+int enqueue_step(wgml_gpt2 *m, bool dynamic, uint32_t token, uint32_t pos,
+                 uint32_t plan_positions = 0) {
     const wgml_gpt2_params &p = m->p;
     wgml_ctx *ctx = m->ctx;
     const uint32_t n = p.n_embd;
     const DynPos dpos = dynamic ? DynPos{&m->dyn->pos, 0} : DynPos{nullptr, pos};
     const DynPos dtok = dynamic ? DynPos{&m->dyn->token, 0} : DynPos{nullptr, token};
     const wgml_attn_params ap{p.n_seq, n, 1u, p.n_head, n / p.n_head, pos};
-    const uint32_t plan = dynamic ? p.n_seq : pos + 1;
+    const uint32_t plan = dynamic ? (plan_positions ? plan_positions : p.n_seq) : pos + 1;
     const bool fold = m->fusion >= 1 && can_fold(m);
     if (dynamic && !fold)
         return set_error(WGML_E_UNSUPPORTED, "wgml_gpt2: the recorded step needs fusion 1");
@@ -324,22 +325,40 @@ int enqueue_step(wgml_gpt2 *m, bool dynamic, uint32_t token, uint32_t pos) {
 }
 
 void drop_graph(wgml_gpt2 *m) {
-    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
-    if (m->graph) (void)hipGraphDestroy(m->graph);
-    m->graph_exec = nullptr;
-    m->graph = nullptr;
+    for (int b = 0; b < kMaxPlanBuckets; ++b) {
+        if (m->graph_exec[b]) (void)hipGraphExecDestroy(m->graph_exec[b]);
+        if (m->graph[b]) (void)hipGraphDestroy(m->graph[b]);
+        m->graph_exec[b] = nullptr;
+        m->graph[b] = nullptr;
+    }
     m->graph_fusion = -1;
 }
 
-// Records one step (+ greedy sampling and bookkeeping) into a HIP graph.
-int build_graph(wgml_gpt2 *m) {
-    if (m->graph_exec && m->graph_fusion == m->fusion) return WGML_OK;
-    drop_graph(m);
+// The attention workspace for the largest plan of any bucket (recorded launches hold its
+// address, so it must not grow between captures).
+int reserve_all_plans(wgml_gpt2 *m) {
+    const wgml_gpt2_params &p = m->p;
+    const wgml_attn_params ap{p.n_seq, p.n_embd, 1u, p.n_head, p.n_embd / p.n_head, 0};
+    for (uint32_t pos = 0;;) {
+        const uint32_t limit = plan_bucket(pos, p.n_seq, nullptr);
+        WGML_TRY(reserve_attention_workspace(m->ctx, ap, limit));
+        if (limit >= p.n_seq) break;
+        pos = limit;
+    }
+    return WGML_OK;
+}
+
+// Records one step (+ greedy sampling and bookkeeping) into a HIP graph, for the bucket of
+// positions that `pos` lies in.
+int build_graph(wgml_gpt2 *m, uint32_t pos) {
     wgml_ctx *ctx = m->ctx;
     const wgml_gpt2_params &p = m->p;
     const uint32_t n = p.n_embd;
-    const wgml_attn_params ap{p.n_seq, n, 1u, p.n_head, n / p.n_head, 0};
-    WGML_TRY(reserve_attention_workspace(ctx, ap, p.n_seq));
+    if (m->graph_fusion != m->fusion) drop_graph(m);
+    int b = 0;
+    const uint32_t plan = plan_bucket(pos, p.n_seq, &b);
+    if (m->graph_exec[b]) return WGML_OK;
+    WGML_TRY(reserve_all_plans(m));
     // An eager step first (function attributes, lazy loading); it runs at position 0
     // and would overwrite that column of every cache: keep a copy and put it back.
     const size_t col = (size_t)n * 4;
@@ -353,7 +372,7 @@ int build_graph(wgml_gpt2 *m) {
     }
     const DynState init{0, 0, 0, 0};
     hipError_t ew = hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream);
-    int rcw = ew == hipSuccess ? enqueue_step(m, true, 0, 0) : WGML_E_HIP;
+    int rcw = ew == hipSuccess ? enqueue_step(m, true, 0, 0, plan) : WGML_E_HIP;
     if (rcw == WGML_OK)
         rcw = launch_argmax_next(ctx, m->curr_vocab, p.n_vocab, m->dyn, m->d_prompt, m->d_tokens);
     for (uint32_t l = 0; l < p.n_layer; ++l) {
@@ -370,15 +389,15 @@ int build_graph(wgml_gpt2 *m) {
 
     WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     const uint64_t launches0 = ctx->launches;
-    int rc = enqueue_step(m, true, 0, 0);
+    int rc = enqueue_step(m, true, 0, 0, plan);
     if (rc == WGML_OK)
         rc = launch_argmax_next(ctx, m->curr_vocab, p.n_vocab, m->dyn, m->d_prompt, m->d_tokens);
-    m->graph_launches = ctx->launches - launches0;
-    hipError_t e = hipStreamEndCapture(ctx->stream, &m->graph);
+    m->graph_launches[b] = ctx->launches - launches0;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &m->graph[b]);
     if (rc == WGML_OK && e != hipSuccess)
         rc = set_error(WGML_E_HIP, "wgml_gpt2: graph capture failed: %s", hipGetErrorString(e));
     if (rc == WGML_OK) {
-        e = hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0);
+        e = hipGraphInstantiate(&m->graph_exec[b], m->graph[b], nullptr, nullptr, 0);
         if (e != hipSuccess)
             rc = set_error(WGML_E_HIP, "wgml_gpt2: graph instantiate failed: %s",
                            hipGetErrorString(e));
@@ -457,11 +476,15 @@ int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_p
     // one synchronisation at the end.
     const bool use_graph = !graphs_disabled();
     if (use_graph) {
-        WGML_TRY(build_graph(m));
+        // every bucket this run passes through, before the first launch
+        for (uint32_t pos = 0; n_total > 0;) {
+            WGML_TRY(build_graph(m, pos));
+            const uint32_t limit = plan_bucket(pos, m->p.n_seq, nullptr);
+            if (limit >= n_total || limit >= m->p.n_seq) break;
+            pos = limit;
+        }
     } else {
-        const wgml_attn_params ap{m->p.n_seq, m->p.n_embd, 1u, m->p.n_head,
-                                  m->p.n_embd / m->p.n_head, 0};
-        WGML_TRY(reserve_attention_workspace(ctx, ap, m->p.n_seq));
+        WGML_TRY(reserve_all_plans(m));
     }
     const uint32_t np = n_prompt < n_total ? n_prompt : n_total;
     WGML_CHECK_HIP(hipMemcpyAsync(m->d_prompt, prompt, (size_t)np * 4, hipMemcpyHostToDevice,
@@ -469,12 +492,14 @@ int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_p
     const DynState init{0, prompt[0], 0, np};
     WGML_CHECK_HIP(hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream));
     for (uint32_t i = 0; i < n_total; ++i) {
+        int b = 0;
+        const uint32_t plan = plan_bucket(i, m->p.n_seq, &b);
         if (use_graph) {
-            WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec, ctx->stream));
-            m->launches_last = m->graph_launches;
+            WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec[b], ctx->stream));
+            m->launches_last = m->graph_launches[b];
         } else {
             const uint64_t l0 = ctx->launches;
-            WGML_TRY(enqueue_step(m, true, 0, 0));
+            WGML_TRY(enqueue_step(m, true, 0, 0, plan));
             WGML_TRY(launch_argmax_next(ctx, m->curr_vocab, m->p.n_vocab, m->dyn, m->d_prompt,
                                         m->d_tokens));
             m->launches_last = ctx->launches - l0;

@@ -42,8 +42,10 @@ struct wgml_llama2 {
     // token-loop state on the device
     DynState *dyn = nullptr;
     uint32_t *d_prompt = nullptr, *d_tokens = nullptr;  // seq_len entries each
-    hipGraph_t graph = nullptr;
-    hipGraphExec_t graph_exec = nullptr;
+    // the recorded step, one capture per bucket of positions (plan_bucket)
+    hipGraph_t graph[kMaxPlanBuckets] = {};
+    hipGraphExec_t graph_exec[kMaxPlanBuckets] = {};
+    uint64_t graph_launches[kMaxPlanBuckets] = {};  // launches of the recorded step
     int graph_fusion = -1;
     // state of the batched prompt pass, allocated at its first use: one row per token
     // of a run (up to kPrefillMaxTokens)
@@ -51,7 +53,6 @@ struct wgml_llama2 {
     uint32_t *pf_tokens = nullptr;
     std::vector<void *> allocs;
     uint64_t launches_last = 0;   // launches of the last step that ran
-    uint64_t graph_launches = 0;  // launches of the recorded step
 };
 
 namespace {
@@ -85,10 +86,12 @@ int check_ready(const wgml_llama2 *m) {
 }
 
 void drop_graph(wgml_llama2 *m) {
-    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
-    if (m->graph) (void)hipGraphDestroy(m->graph);
-    m->graph_exec = nullptr;
-    m->graph = nullptr;
+    for (int b = 0; b < kMaxPlanBuckets; ++b) {
+        if (m->graph_exec[b]) (void)hipGraphExecDestroy(m->graph_exec[b]);
+        if (m->graph[b]) (void)hipGraphDestroy(m->graph[b]);
+        m->graph_exec[b] = nullptr;
+        m->graph[b] = nullptr;
+    }
     m->graph_fusion = -1;
 }
 
@@ -96,11 +99,12 @@ void drop_graph(wgml_llama2 *m) {
 // preceded by the embedding copy of chat_llama2.rs:185-187).
 //   dynamic == false: token/pos are the given host values;
 //   dynamic == true : they are read from m->dyn on the device, the attention
-//                     grid is planned for seq_len positions.
+//                     grid is planned for `plan_positions` positions (0: seq_len).
 // fusion 0: one launch per reference op.  1: bias and residual adds folded into
 // the GEMV epilogues.  2: additionally every RMSNorm folded into the staging of
 // the GEMVs that consume it.
-int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos) {
+int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos,
+                 uint32_t plan_positions = 0) {
     const wgml_llama2_config &c = m->cfg;
     wgml_ctx *ctx = m->ctx;
     const uint32_t dim = c.dim, kv_dim = m->kv_dim;
@@ -109,7 +113,7 @@ int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos) {
     const int variant = m->model_type == WGML_MODEL_QWEN2 ? WGML_ROPE_NEOX : WGML_ROPE_ORIGINAL;
     const wgml_attn_params ap{c.seq_len, kv_dim, m->kv_mul, c.n_q_heads, m->head_size, pos};
     const int fusion = m->fusion;
-    const uint32_t plan = dynamic ? c.seq_len : pos + 1;
+    const uint32_t plan = dynamic ? (plan_positions ? plan_positions : c.seq_len) : pos + 1;
 
     // dim >= head_size / 2, so the embedding launch also covers the RoPE table
     WGML_TRY(launch_embed(ctx, m->x, m->token_embd, dim, dtok, m->rope_cs, m->head_size,
@@ -248,16 +252,32 @@ int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos) {
     return WGML_OK;
 }
 
-// Records one step (+ greedy sampling and bookkeeping) into a HIP graph.
-int build_graph(wgml_llama2 *m) {
-    if (m->graph_exec && m->graph_fusion == m->fusion) return WGML_OK;
-    drop_graph(m);
+// The attention workspace for the largest plan of any bucket (recorded launches hold its
+// address, so it must not grow between captures).
+int reserve_all_plans(wgml_llama2 *m) {
+    const wgml_llama2_config &c = m->cfg;
+    const wgml_attn_params ap{c.seq_len, m->kv_dim, m->kv_mul, c.n_q_heads, m->head_size, 0};
+    for (uint32_t pos = 0;;) {
+        const uint32_t limit = plan_bucket(pos, c.seq_len, nullptr);
+        WGML_TRY(reserve_attention_workspace(m->ctx, ap, limit));
+        if (limit >= c.seq_len) break;
+        pos = limit;
+    }
+    return WGML_OK;
+}
+
+// Records one step (+ greedy sampling and bookkeeping) into a HIP graph, for the bucket of
+// positions that `pos` lies in.
+int build_graph(wgml_llama2 *m, uint32_t pos) {
     wgml_ctx *ctx = m->ctx;
     const wgml_llama2_config &c = m->cfg;
+    if (m->graph_fusion != m->fusion) drop_graph(m);
+    int b = 0;
+    const uint32_t plan = plan_bucket(pos, c.seq_len, &b);
+    if (m->graph_exec[b]) return WGML_OK;
     // Everything that allocates or sets function attributes happens before capture:
     // the attention workspace for the largest plan, and one eager step.
-    const wgml_attn_params ap{c.seq_len, m->kv_dim, m->kv_mul, c.n_q_heads, m->head_size, 0};
-    WGML_TRY(reserve_attention_workspace(ctx, ap, c.seq_len));
+    WGML_TRY(reserve_all_plans(m));
     // The eager step runs at position 0 and would overwrite that column of every KV
     // cache (the caller may have filled it): keep a copy and put it back.
     const size_t col = (size_t)m->kv_dim * 4;
@@ -271,7 +291,7 @@ int build_graph(wgml_llama2 *m) {
     }
     const DynState init{0, 0, 0, 0};
     hipError_t ew = hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream);
-    int rcw = ew == hipSuccess ? enqueue_step(m, true, 0, 0) : WGML_E_HIP;
+    int rcw = ew == hipSuccess ? enqueue_step(m, true, 0, 0, plan) : WGML_E_HIP;
     if (rcw == WGML_OK)
         rcw = launch_argmax_next(ctx, m->logits, c.vocab_size, m->dyn, m->d_prompt, m->d_tokens);
     for (uint32_t l = 0; l < c.n_layers; ++l) {
@@ -288,11 +308,11 @@ int build_graph(wgml_llama2 *m) {
 
     WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     const uint64_t launches0 = ctx->launches;
-    int rc = enqueue_step(m, true, 0, 0);
+    int rc = enqueue_step(m, true, 0, 0, plan);
     if (rc == WGML_OK)
         rc = launch_argmax_next(ctx, m->logits, c.vocab_size, m->dyn, m->d_prompt, m->d_tokens);
-    m->graph_launches = ctx->launches - launches0;
-    hipError_t e = hipStreamEndCapture(ctx->stream, &m->graph);
+    m->graph_launches[b] = ctx->launches - launches0;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &m->graph[b]);
     if (rc != WGML_OK) {
         drop_graph(m);
         return rc;
@@ -301,7 +321,7 @@ int build_graph(wgml_llama2 *m) {
         drop_graph(m);
         return set_error(WGML_E_HIP, "wgml_llama2: graph capture failed: %s", hipGetErrorString(e));
     }
-    e = hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0);
+    e = hipGraphInstantiate(&m->graph_exec[b], m->graph[b], nullptr, nullptr, 0);
     if (e != hipSuccess) {
         drop_graph(m);
         return set_error(WGML_E_HIP, "wgml_llama2: graph instantiate failed: %s",
@@ -319,11 +339,15 @@ int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint3
     WGML_TRY(check_ready(m));
     const bool use_graph = !graphs_disabled();
     if (use_graph) {
-        WGML_TRY(build_graph(m));
+        // every bucket this run passes through, before the first launch
+        for (uint32_t pos = start_pos; n_steps > 0;) {
+            WGML_TRY(build_graph(m, pos));
+            const uint32_t limit = plan_bucket(pos, m->cfg.seq_len, nullptr);
+            if (limit >= start_pos + n_steps || limit >= m->cfg.seq_len) break;
+            pos = limit;
+        }
     } else {
-        const wgml_attn_params ap{m->cfg.seq_len, m->kv_dim, m->kv_mul, m->cfg.n_q_heads,
-                                  m->head_size, 0};
-        WGML_TRY(reserve_attention_workspace(ctx, ap, m->cfg.seq_len));
+        WGML_TRY(reserve_all_plans(m));
     }
     if (n_prompt)
         WGML_CHECK_HIP(hipMemcpyAsync(m->d_prompt, prompt, (size_t)n_prompt * 4,
@@ -332,13 +356,15 @@ int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint3
     WGML_CHECK_HIP(hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream));
     WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));  // `init` is a stack object
     for (uint32_t i = 0; i < n_steps; ++i) {
+        int b = 0;
+        const uint32_t plan = plan_bucket(start_pos + i, m->cfg.seq_len, &b);
         if (use_graph) {
-            WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec, ctx->stream));
-            m->launches_last = m->graph_launches;
+            WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec[b], ctx->stream));
+            m->launches_last = m->graph_launches[b];
         } else {
             // the same launches, enqueued one by one (no host synchronisation either)
             const uint64_t launches0 = ctx->launches;
-            WGML_TRY(enqueue_step(m, true, 0, 0));
+            WGML_TRY(enqueue_step(m, true, 0, 0, plan));
             WGML_TRY(launch_argmax_next(ctx, m->logits, m->cfg.vocab_size, m->dyn, m->d_prompt,
                                         m->d_tokens));
             m->launches_last = ctx->launches - launches0;

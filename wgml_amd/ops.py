@@ -47,7 +47,8 @@ class GpuInstance:
 
     # keys of set_tuning (enum WGML_TUNE_* of the C header, same order)
     (TUNE_GEMV_ROWS_PER_WAVE, TUNE_GEMV_WAVES_PER_WG, TUNE_GEMV_WG_PER_CU, TUNE_GEMV_DEPTH,
-     TUNE_GEMV_F32_ACTIVATIONS, TUNE_GEMM_K_SPLIT, TUNE_PREFILL_ATTENTION_PER_TOKEN) = range(7)
+     TUNE_GEMV_F32_ACTIVATIONS, TUNE_GEMM_K_SPLIT, TUNE_PREFILL_ATTENTION_PER_TOKEN,
+     TUNE_ATTN_WIDE_POSITIONS, TUNE_ATTN_SPLITS) = range(9)
 
     def set_tuning(self, key: int, value: int) -> None:
         """Launch-shape override of this context (0 = heuristic); for sweeps and tests."""
