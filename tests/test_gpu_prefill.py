@@ -307,6 +307,12 @@ def test_prefill_rejects_bad_arguments(gpu):
         m.prefill([1, 2, MICRO.vocab_size])
     with pytest.raises(W.WgmlError):
         m.prefill([1] * 10, start_pos=MICRO.seq_len - 9)
+    # a model whose matrices have no batched product (dense f32 here) is stepped through the
+    # prompt token by token instead: same logits as the single steps
     f = Llama2(gpu, MICRO).load(synth_llama(MICRO, seed=21, scheme="f32"))
-    with pytest.raises(W.WgmlError):
-        f.prefill([1, 2, 3])
+    f.prefill([1, 2, 3])
+    got = f.logits().copy()
+    g = Llama2(gpu, MICRO).load(synth_llama(MICRO, seed=21, scheme="f32"))
+    for pos, t in enumerate([1, 2, 3]):
+        want = g.forward_logits(pos, t)
+    assert np.array_equal(got, want)

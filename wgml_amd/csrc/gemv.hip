@@ -873,10 +873,13 @@ struct PlainPolicy {
     // memory round trip to every wave's tail.
     float *out;
     float pre_bias, pre_out;
+    uint32_t pos;
+    __device__ const uint32_t *pos_ptr() const { return p.dyn_pos; }
+    __device__ void set_pos(uint32_t fetched) { pos = fetched; }
     template <int R>
     __device__ void prefetch(uint32_t g0, uint32_t GW, uint32_t my_groups, uint32_t lane) {
         out = p.out;
-        if (p.dyn_pos) out += (size_t)(*p.dyn_pos) * p.out_pos_stride;
+        if (p.dyn_pos) out += (size_t)pos * p.out_pos_stride;
         pre_bias = pre_out = 0.f;
         const uint32_t row = (g0 + (lane / R) * GW) * R + lane % R;
         if (lane < my_groups * R && row < p.nrows) {
@@ -931,11 +934,15 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     const uint32_t my_groups = (wave < nw && first < ngroups) ? (ngroups - first + GW - 1) / GW : 0;
     const uint32_t n_it = my_groups * S * nsteps;
 
-    pol.template prefetch<R>(first, GW, my_groups, lane);
-
     // The requests for x go out first, the first D weight requests after them: a
     // wave's loads return in order, so x, a cache hit, is not held up behind the
     // weights and is staged while they are in flight.
+    // The position (when it lives in device memory) is requested by a vector load ahead of
+    // x: it returns in order with x, so it is there once x has been staged, and no scalar
+    // round trip for it stands between the kernel's start and its first weight request.
+    const uint32_t *pos_src = pol.pos_ptr();
+    uint32_t pos_fetched = 0;
+    if (pos_src) pos_fetched = pos_src[opaque(0u)];
     constexpr int XP = 3;  // float4 of x per thread requested up front
     const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
     const float4 *nw4 = reinterpret_cast<const float4 *>(p.norm_w);
@@ -946,12 +953,24 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     // nv: the RMSNorm weights, or gamma of a folded LayerNorm; bv: its beta.  They are
     // requested here, ahead of the weights, so that waiting for them later does not
     // mean waiting for a weight tile.
+    // Only the first `ns` waves stage x (as few as cover it with their XP float4 per lane,
+    // in fours so that every SIMD takes part): the waves of a 1024-thread workgroup start
+    // up to a microsecond apart, and the staging would otherwise end a whole prologue after
+    // the last of them has arrived.  The other waves request their weights and wait at the
+    // barrier.  (The folded LayerNorm has barriers of its own, so there every wave stages.)
+    uint32_t ns = ((n4 + 64 * XP - 1) / (64 * XP) + 3) & ~3u;
+    if (ns > nwaves || p.ln_g) ns = nwaves;
+    const bool stager = wave < ns;
+    // a wave with neither rows nor a share of x is done: the barrier below counts only the
+    // waves that are still running, and it would be the last to reach it
+    if (n_it == 0 && !stager) return;
+    const uint32_t sthreads = ns * 64;
     float4 xv[XP], nv[XP], bv[XP];
     const float4 *gsrc = p.ln_g ? reinterpret_cast<const float4 *>(p.ln_g) : nw4;
     const float4 *bsrc = reinterpret_cast<const float4 *>(p.ln_b);
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
-        const uint32_t g4 = tid + i * blockDim.x;
+        const uint32_t g4 = stager ? tid + i * sthreads : n4;
         xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         nv[i] = make_float4(1.f, 1.f, 1.f, 1.f);
         bv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -1064,20 +1083,21 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
         // active together in every one of these branches
 #pragma unroll
         for (int i = 0; i < XP; ++i) {
-            const uint32_t g4 = tid + i * blockDim.x;
+            const uint32_t g4 = stager ? tid + i * sthreads : n4;
             if (g4 < n4) stage_one(g4, xv[i], nv[i]);
         }
-        for (uint32_t g4 = tid + XP * blockDim.x; g4 < n4; g4 += blockDim.x)
+        for (uint32_t g4 = stager ? tid + XP * sthreads : n4; g4 < n4; g4 += sthreads)
             stage_one(g4, x4[g4], p.norm_w ? nw4[g4] : make_float4(1.f, 1.f, 1.f, 1.f));
-        if (p.norm_w) {
+        if (p.norm_w && stager) {
             ss = wave_sum(ss);
             if (lane == 0) red[wave] = ss;
         }
         __syncthreads();
         if (p.norm_w) {
             // one LDS read per lane and a 16-lane DPP sum instead of a chain of
-            // dependent reads (a workgroup has at most 16 waves)
-            const float part = lane < nwaves ? red[lane] : 0.f;
+            // dependent reads (a workgroup has at most 16 waves; only the staging ones
+            // have written a partial sum)
+            const float part = lane < ns ? red[lane] : 0.f;
             const float total = readlane_f32(row16_sum(part), 0);
             out_scale = 1.0f / sqrtf(total / (float)p.ncols + p.norm_eps);
         }
@@ -1113,12 +1133,21 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     for (int d = 0; d < D; ++d) {
         const bool ok = (uint32_t)d < n_it;
         const uint32_t tile = ok ? ls * 64 + lane : lane;
-        pol.template load<WF, R>(w[d], ok ? lg : (n_it ? first : 0u), ok ? lsub : 0u, tile < ntiles ? tile : 0u, true);
+        // no tile left: the wave's own first one again, or, for a wave without rows, the
+        // first one of its workgroup (a hit in the CU's cache either way)
+        const uint32_t spare = n_it ? first : (wg * nw < ngroups ? wg * nw : 0u);
+        pol.template load<WF, R>(w[d], ok ? lg : spare, ok ? lsub : 0u, tile < ntiles ? tile : 0u, true);
         if (ok) advance_load_cursor();
     }
 
     const float out_scale = stage_x();
     if (n_it == 0) return;
+    // The epilogue's operands (bias, RoPE table entry, the value to accumulate into) are
+    // requested here, behind the first weight tiles: their addresses may depend on the
+    // position, which is a second memory round trip away from the kernel arguments, and
+    // nothing before this point waits for it.
+    pol.set_pos((uint32_t)__builtin_amdgcn_readfirstlane((int)pos_fetched));
+    pol.template prefetch<R>(first, GW, my_groups, lane);
 
     // XREG: a lane without a tile (rows shorter than 64 tiles) keeps an all-zero tile of
     // x, so that the row loop needs no condition on the lane
@@ -1203,7 +1232,7 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
 // 1024-thread workgroups share a CU).
 template <class F, int R, int D, int MAXT, int MINW = MAXT / 256>
 __global__ __launch_bounds__(MAXT, MINW) void gemv_quant_i8_kernel(const GemvParams p) {
-    PlainPolicy pol{p, nullptr, 0.f, 0.f};
+    PlainPolicy pol{p, nullptr, 0.f, 0.f, 0};
     const uint32_t ngroups = (p.nrows + R - 1) / R;
     if (p.ncols <= 64 * F::TILE)
         gemv_i8_body<F, R, D, true>(p, pol, blockIdx.x, gridDim.x, p.active_waves, ngroups);
@@ -1240,7 +1269,6 @@ struct GemvJob {
 
 struct FusedParams {
     GemvJob jobs[3];
-    int njobs;
     const float *x;
     uint32_t ncols;
     const float *norm_w;
@@ -1250,6 +1278,10 @@ struct FusedParams {
     uint32_t head_size;
     float rope_base;
     const float2 *rope_cs;  // optional: (cos, sin) of the current position per pair of a head
+    // The first field a workgroup needs sits in the last cache line of the arguments, so that
+    // the first batch of scalar loads touches every line (a line first touched by a later
+    // batch is another round trip to memory).
+    int njobs;
 };
 
 // A group is a pair of rows whose tiles a wave loads together and multiplies with one
@@ -1260,7 +1292,8 @@ struct JobPolicy {
     static constexpr int S = 1;
     const GemvJob &j;
     const GemvParams &pa, &pb;  // plane views of the two matrices
-    uint32_t pos, head_size;
+    DynPos dpos;
+    uint32_t head_size;
     float rope_base;
     const float2 *rope_cs;
     template <class WF, int R>
@@ -1284,6 +1317,9 @@ struct JobPolicy {
     // fetches what the epilogue of the first segment needs at kernel start.
     float pre_bias, pre_out;
     float2 pre_cs;
+    uint32_t pos;
+    __device__ const uint32_t *pos_ptr() const { return dpos.ptr; }
+    __device__ void set_pos(uint32_t fetched) { pos = dpos.ptr ? fetched : dpos.val; }
     __device__ float2 rope_entry(uint32_t row) const {
         if (rope_cs) return rope_cs[((row & ~1u) % head_size) >> 1];
         const float head_dim = (float)((row & ~1u) % head_size);
@@ -1339,7 +1375,7 @@ __device__ __forceinline__ void fused_job_body(const FusedParams &P, const GemvJ
     GemvParams pa = xp, pb = xp;
     pa.p0 = j.a0; pa.p1 = j.a1; pa.p2 = j.a2; pa.p3 = j.a3;
     pb.p0 = j.b0; pb.p1 = j.b1; pb.p2 = j.b2; pb.p3 = j.b3;
-    JobPolicy pol{j, pa, pb, dyn_pos(P.pos), P.head_size, P.rope_base, P.rope_cs, 0.f, 0.f, make_float2(1.f, 0.f)};
+    JobPolicy pol{j, pa, pb, P.pos, P.head_size, P.rope_base, P.rope_cs, 0.f, 0.f, make_float2(1.f, 0.f), 0};
     const uint32_t ngroups = j.mode == JOB_SILU ? j.nrows : (j.nrows + 1) / 2;
     if (P.ncols <= 64 * F::TILE)
         gemv_i8_body<F, 2, D, true>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves,
@@ -1354,10 +1390,20 @@ __device__ __forceinline__ void fused_job_body(const FusedParams &P, const GemvJ
 // of them have (smaller code, registers of that format only).
 template <int D, int MAXT, int MINW, int FMT>
 __global__ __launch_bounds__(MAXT, MINW) void gemv_fused_kernel(const FusedParams P) {
-    int ji = 0;
-    if (P.njobs > 1 && blockIdx.x >= P.jobs[1].wg_begin) ji = 1;
-    if (P.njobs > 2 && blockIdx.x >= P.jobs[2].wg_begin) ji = 2;
-    const GemvJob j = P.jobs[ji];  // a copy: fields stay in registers, not re-read in the loop
+    // All three job records are fetched at once and the workgroup's own is picked field by
+    // field afterwards: indexing the kernel arguments with the job number would put a second
+    // scalar-memory round trip (a microsecond when the arguments come from HBM) in front of
+    // the first weight request.
+    const bool is1 = P.njobs > 1 && blockIdx.x >= P.jobs[1].wg_begin;
+    const bool is2 = P.njobs > 2 && blockIdx.x >= P.jobs[2].wg_begin;
+    const GemvJob &j0 = P.jobs[0], &j1 = P.jobs[1], &j2 = P.jobs[2];
+#define WGML_PICK(f) (is2 ? j2.f : (is1 ? j1.f : j0.f))
+    const GemvJob j{WGML_PICK(a0), WGML_PICK(a1), WGML_PICK(a2), WGML_PICK(a3),
+                    WGML_PICK(b0), WGML_PICK(b1), WGML_PICK(b2), WGML_PICK(b3),
+                    WGML_PICK(out), WGML_PICK(bias), WGML_PICK(nrows), WGML_PICK(type),
+                    WGML_PICK(mode), WGML_PICK(accumulate), WGML_PICK(out_pos_stride),
+                    WGML_PICK(wg_begin), WGML_PICK(wg_count), WGML_PICK(active_waves)};
+#undef WGML_PICK
     if (FMT == WGML_Q4_K) {
         fused_job_body<IFmtQ4K, D>(P, j);
     } else if (FMT == WGML_Q6_K) {
@@ -1546,6 +1592,7 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
     const bool q8 = F::TILE == 32;
     if (!R) R = 1;
     if (!waves) waves = (q8 && p.ncols <= 1024) ? 8 : 16;  // short rows: less staging per row
+    if (waves == 12) waves = 16;  // 12-wave workgroups exist for the fused launches only
     if (!depth) depth = 1;
     if (p.ln_g && (p.ncols >> 2) > 3u * (uint32_t)waves * 64u)  // XP float4 per thread
         return set_error(WGML_E_UNSUPPORTED, "gemv_quant: %u columns are too many for the folded "
@@ -1835,6 +1882,13 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
 }
 
 int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
+    const int depth = ctx->tuning[WGML_TUNE_GEMV_DEPTH], waves = ctx->tuning[WGML_TUNE_GEMV_WAVES_PER_WG];
+    if (waves == 12) {
+        if (depth >= 2) return launch_gemv_fused_variant<2, 768, 1>(ctx, f);
+        return launch_gemv_fused_variant<1, 768, 1>(ctx, f);
+    }
+    if (depth >= 3) return launch_gemv_fused_variant<3, 1024, 1>(ctx, f);
+    if (depth == 2) return launch_gemv_fused_variant<2, 1024, 1>(ctx, f);
     return launch_gemv_fused_variant<1, 1024, 1>(ctx, f);
 }
 

@@ -107,7 +107,7 @@ int wgml_ctx_set_tuning(wgml_ctx *ctx, int key, int value) {
     bool ok = value >= 0;
     switch (key) {
     case WGML_TUNE_GEMV_ROWS_PER_WAVE: ok = value >= 0 && value <= 2; break;
-    case WGML_TUNE_GEMV_WAVES_PER_WG: ok = value == 0 || value == 4 || value == 8 || value == 16; break;
+    case WGML_TUNE_GEMV_WAVES_PER_WG: ok = value == 0 || value == 4 || value == 8 || value == 12 || value == 16; break;
     case WGML_TUNE_GEMV_DEPTH: ok = value >= 0 && value <= 4; break;
     case WGML_TUNE_GEMV_F32_ACTIVATIONS:
     case WGML_TUNE_PREFILL_ATTENTION_PER_TOKEN: ok = value == 0 || value == 1; break;
