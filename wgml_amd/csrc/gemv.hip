@@ -876,15 +876,20 @@ struct PlainPolicy {
     uint32_t pos;
     __device__ const uint32_t *pos_ptr() const { return p.dyn_pos; }
     __device__ void set_pos(uint32_t fetched) { pos = fetched; }
+    // `late` false: at kernel start, whatever does not need the position; true: behind the
+    // first weight tiles, once the position is there, the rest.
     template <int R>
-    __device__ void prefetch(uint32_t g0, uint32_t GW, uint32_t my_groups, uint32_t lane) {
-        out = p.out;
-        if (p.dyn_pos) out += (size_t)pos * p.out_pos_stride;
-        pre_bias = pre_out = 0.f;
+    __device__ void prefetch(bool late, uint32_t g0, uint32_t GW, uint32_t my_groups, uint32_t lane) {
         const uint32_t row = (g0 + (lane / R) * GW) * R + lane % R;
-        if (lane < my_groups * R && row < p.nrows) {
-            if (p.bias) pre_bias = p.bias[row];
-            if (p.accumulate) pre_out = out[row];
+        const bool mine = lane < my_groups * R && row < p.nrows;
+        if (!late) {
+            out = p.out;
+            pre_bias = pre_out = 0.f;
+            if (mine && p.bias) pre_bias = p.bias[row];
+            if (mine && p.accumulate && !p.dyn_pos) pre_out = out[row];
+        } else if (p.dyn_pos) {
+            out += (size_t)pos * p.out_pos_stride;
+            if (mine && p.accumulate) pre_out = out[row];
         }
     }
     template <int R>
@@ -933,6 +938,10 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     const uint32_t first = wg * nw + wave, GW = nwg * nw;
     const uint32_t my_groups = (wave < nw && first < ngroups) ? (ngroups - first + GW - 1) / GW : 0;
     const uint32_t n_it = my_groups * S * nsteps;
+
+    // the epilogue's operands that do not depend on the position (bias, RoPE table entry,
+    // the value to accumulate into) are requested before anything else
+    pol.template prefetch<R>(false, first, GW, my_groups, lane);
 
     // The requests for x go out first, the first D weight requests after them: a
     // wave's loads return in order, so x, a cache hit, is not held up behind the
@@ -1142,12 +1151,11 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
 
     const float out_scale = stage_x();
     if (n_it == 0) return;
-    // The epilogue's operands (bias, RoPE table entry, the value to accumulate into) are
-    // requested here, behind the first weight tiles: their addresses may depend on the
-    // position, which is a second memory round trip away from the kernel arguments, and
-    // nothing before this point waits for it.
+    // The epilogue's operands whose addresses depend on the position are requested here,
+    // behind the first weight tiles: the position is a second memory round trip away from
+    // the kernel arguments, and nothing before this point waits for it.
     pol.set_pos((uint32_t)__builtin_amdgcn_readfirstlane((int)pos_fetched));
-    pol.template prefetch<R>(first, GW, my_groups, lane);
+    pol.template prefetch<R>(true, first, GW, my_groups, lane);
 
     // XREG: a lane without a tile (rows shorter than 64 tiles) keeps an all-zero tile of
     // x, so that the row loop needs no condition on the lane
@@ -1329,16 +1337,28 @@ struct JobPolicy {
         return make_float2(cs, sn);
     }
     template <int R>
-    __device__ void prefetch(uint32_t g0, uint32_t GW, uint32_t my_groups, uint32_t lane) {
-        pre_bias = pre_out = 0.f;
-        pre_cs = make_float2(1.f, 0.f);
+    __device__ void prefetch(bool late, uint32_t g0, uint32_t GW, uint32_t my_groups, uint32_t lane) {
+        if (!late) {
+            pre_bias = pre_out = 0.f;
+            pre_cs = make_float2(1.f, 0.f);
+        }
         if (j.mode == JOB_SILU) return;
         const uint32_t row = 2 * (g0 + (lane >> 1) * GW) + (lane & 1);
-        if (lane < 2 * my_groups && row < j.nrows) {
-            const float *out = j.out + (size_t)pos * j.out_pos_stride;
+        if (!(lane < 2 * my_groups && row < j.nrows)) return;
+        // what depends on the position waits for the late call: the output column of a
+        // position-strided destination, and RoPE angles when there is no table of them
+        const bool out_needs_pos = dpos.ptr && j.out_pos_stride;
+        const bool cs_needs_pos = dpos.ptr && !rope_cs;
+        if (!late) {
             if (j.bias) pre_bias = j.bias[row];
-            if (j.accumulate) pre_out = out[row];
-            if (j.mode == JOB_ROPE) pre_cs = rope_entry(row);
+            if (j.accumulate && !out_needs_pos) pre_out = (j.out + (size_t)dpos.val * j.out_pos_stride)[row];
+            if (j.mode == JOB_ROPE && !cs_needs_pos) {
+                pos = dpos.val;
+                pre_cs = rope_entry(row);
+            }
+        } else {
+            if (j.accumulate && out_needs_pos) pre_out = (j.out + (size_t)pos * j.out_pos_stride)[row];
+            if (j.mode == JOB_ROPE && cs_needs_pos) pre_cs = rope_entry(row);
         }
     }
     template <int R>
@@ -1549,10 +1569,12 @@ int launch_variant_i8(wgml_ctx *ctx, const GemvParams &p0, size_t lds) {
     WGML_TRY(blocks_per_cu(ctx, (const void *)gemv_quant_i8_kernel<F, R, D, MAXT, MINW>, MAXT, lds,
                            &per_cu));
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
-    // every workgroup with all its waves at work (min_c): a workgroup with idle waves
-    // stages x for nothing, and idle waves re-read row-group 0
-    const WgPlan plan = plan_groups((p0.nrows + R - 1) / R, cu * (uint32_t)per_cu, MAXT / 64, 64 / R,
-                                    MAXT / 64);
+    // One workgroup per CU with all its waves at work rather than two half-empty ones
+    // (each would stage x), as long as that still gives every CU a workgroup (min_c).
+    const uint32_t ngroups = (p0.nrows + R - 1) / R;
+    uint32_t min_c = (ngroups + cu - 1) / cu;
+    if (min_c > MAXT / 64) min_c = MAXT / 64;
+    const WgPlan plan = plan_groups(ngroups, cu * (uint32_t)per_cu, MAXT / 64, 64 / R, min_c);
     GemvParams p = p0;
     p.active_waves = plan.active_waves;
     gemv_quant_i8_kernel<F, R, D, MAXT, MINW><<<dim3(plan.wgs), dim3(MAXT), lds, ctx->stream>>>(p);
@@ -1758,7 +1780,7 @@ bool gemv_fused_supported(const wgml_qmat *m) {
 }
 
 template <int D, int MAXT, int MINW>
-static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
+static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f, uint32_t *plan_only = nullptr) {
     constexpr uint32_t nwaves = MAXT / 64;
     if (f.njobs < 1 || f.njobs > 3)
         return set_error(WGML_E_INVALID, "gemv_fused: %d jobs", f.njobs);
@@ -1874,7 +1896,11 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
         if (plan.active_waves > max_nw) max_nw = plan.active_waves;
         begin += plan.wgs;
     }
-    (void)max_nw;
+    if (plan_only) {  // the caller only asks how many row pairs the launch has
+        *plan_only = 0;
+        for (int i = 0; i < f.njobs; ++i) *plan_only += ngroups[i];
+        return WGML_OK;
+    }
     kern<<<dim3(begin), dim3(MAXT), lds, ctx->stream>>>(P);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
@@ -1883,12 +1909,16 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f) {
 
 int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f) {
     const int depth = ctx->tuning[WGML_TUNE_GEMV_DEPTH], waves = ctx->tuning[WGML_TUNE_GEMV_WAVES_PER_WG];
-    if (waves == 12) {
-        if (depth >= 2) return launch_gemv_fused_variant<2, 768, 1>(ctx, f);
-        return launch_gemv_fused_variant<1, 768, 1>(ctx, f);
-    }
-    if (depth >= 3) return launch_gemv_fused_variant<3, 1024, 1>(ctx, f);
-    if (depth == 2) return launch_gemv_fused_variant<2, 1024, 1>(ctx, f);
+    (void)depth;  // deeper register rings spill in the fused kernels
+    if (waves == 12) return launch_gemv_fused_variant<1, 768, 1>(ctx, f);
+    if (waves == 16) return launch_gemv_fused_variant<1, 1024, 1>(ctx, f);
+    // 12-wave workgroups for launches with a little less than one row pair per wave of a
+    // machine full of 16-wave workgroups (Q/K/V of 4096/1024/1024 rows: 8.6 us against 9.6;
+    // small launches are better off with the 16-wave kernel: GPT-2's Q/K/V 5.1 us against 7.1)
+    uint32_t pairs = 0;
+    WGML_TRY((launch_gemv_fused_variant<1, 1024, 1>(ctx, f, &pairs)));
+    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
+    if (pairs > cu * 8 && pairs <= cu * 16) return launch_gemv_fused_variant<1, 768, 1>(ctx, f);
     return launch_gemv_fused_variant<1, 1024, 1>(ctx, f);
 }
 
