@@ -1606,16 +1606,18 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
                          kMaxLds);
     // Defaults from a sweep over the Llama-2-7B shapes on MI355X: one row per
     // wave and 16-wave workgroups (x is staged once per 16 rows in flight), and
-    // no register ring: with 16 waves per CU one tile in flight per wave already
-    // exceeds what HBM needs to stay busy, and every deeper pipeline measured
-    // slower, also with exact waits (11008x4096 Q4_K: 8.4 us at depth 1, 9.4 at 2).
+    // no register ring for Q4_K and Q6_K: a deeper pipeline measured slower at every
+    // shape, also with exact waits (11008x4096 Q4_K: 7.7 us at depth 1, 8.1 at 2, 8.8
+    // at 3; Q6_K spills from depth 2 on).
     int R = ctx->tuning[WGML_TUNE_GEMV_ROWS_PER_WAVE], waves = ctx->tuning[WGML_TUNE_GEMV_WAVES_PER_WG],
         depth = ctx->tuning[WGML_TUNE_GEMV_DEPTH];
     const bool q8 = F::TILE == 32;
     if (!R) R = 1;
     if (!waves) waves = (q8 && p.ncols <= 1024) ? 8 : 16;  // short rows: less staging per row
     if (waves == 12) waves = 16;  // 12-wave workgroups exist for the fused launches only
-    if (!depth) depth = 1;
+    // Q8_0 rows of five and more steps (over 8192 columns): four tiles in flight per wave
+    // (4096x11008: 11.0 us against 13.4); everywhere else one tile is as fast or faster
+    if (!depth) depth = (q8 && ntiles > 256 && SWEEP) ? 4 : 1;
     if (p.ln_g && (p.ncols >> 2) > 3u * (uint32_t)waves * 64u)  // XP float4 per thread
         return set_error(WGML_E_UNSUPPORTED, "gemv_quant: %u columns are too many for the folded "
                                              "LayerNorm", p.ncols);
