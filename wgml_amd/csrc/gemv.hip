@@ -1854,7 +1854,9 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f, uint32_t
     int fmt = P.jobs[0].type, slot = 0;
     for (int i = 1; i < f.njobs; ++i)
         if (P.jobs[i].type != fmt) fmt = 0;
-    void (*kern)(const FusedParams) = gemv_fused_kernel<D, MAXT, MINW, 0>;
+    // the mixed-format kernel is held to 96 registers (5 waves per SIMD): it fits without
+    // spilling, and the waves of a workgroup start sooner the fewer registers they take
+    void (*kern)(const FusedParams) = gemv_fused_kernel<D, MAXT, (MAXT == 1024 ? 5 : MINW), 0>;
     switch (fmt) {
     case WGML_Q4_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q4_K>; slot = 1; break;
     case WGML_Q6_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q6_K>; slot = 2; break;
