@@ -440,7 +440,12 @@ def main():
     tok_s = args.steps / dt
     assert np.array_equal(np.concatenate([wtoks, toks])[:args.warmup + n_sync], toks_sync), \
         "recorded and synchronous loops disagree"
-    launches_per_token = model.launches_per_token()
+    launches_per_token = model.launches_per_token()  # of the last timed step
+    # the recorded step differs between ranges of positions (attention without partial results
+    # below position 256, with a merge launch from there on): say which range the figure is for
+    launches_note = (f"{launches_per_token} at position {p0 + args.warmup + args.steps - 1} (the last "
+                     f"timed step); the step is recorded per range of positions (limits 256, 512, "
+                     f"1024, ...): attention below position 256 is one launch per layer, two from there on")
     wbytes = weights.weight_bytes_per_token()
     kv_bytes_mid = 2 * cfg.n_layers * cfg.kv_dim * 4 * (p0 + args.warmup + args.steps // 2)
     roof_tok_s = HBM_PEAK_GBS * 1e9 / wbytes
@@ -572,6 +577,7 @@ def main():
                    "roofline_tok_s_at_8TBs": round(roof_tok_s, 1),
                    "frac_of_weight_roofline": round(tok_s / roof_tok_s, 4),
                    "launches_per_token": launches_per_token,
+                   "launches_per_token_note": launches_note,
                    "tok_s_with_per_token_host_sync": round(tok_s_sync, 2),
                    "fp32_activations": fp32_act,
                    "last_token": int(toks[-1])},

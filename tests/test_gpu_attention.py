@@ -61,6 +61,22 @@ def test_attention_long_context_gqa(gpu, with_att):
         np.testing.assert_allclose(att[:, :8301], watt[:, :8301], rtol=0, atol=1e-6)
 
 
+@pytest.mark.parametrize("wide,splits", [(1024, 0), (0, 2), (0, 5), (0, 16), (0, 17), (0, 64)])
+@pytest.mark.parametrize("pos", [3, 140, 700])
+def test_attention_plans_agree(gpu, wide, splits, pos):
+    # every way of sharing a head's positions out over workgroups (one workgroup per head; 2..64
+    # workgroups with a merge of 16 or 64 partials at a time, most of them without a position
+    # at a short context) gives the oracle's result
+    gpu.set_tuning(gpu.TUNE_ATTN_WIDE_POSITIONS, wide)
+    gpu.set_tuning(gpu.TUNE_ATTN_SPLITS, splits)
+    try:
+        xb, wxb, _, _ = run(gpu, 1024, 2, 8, 128, pos, False, seed=3)
+    finally:
+        gpu.set_tuning(gpu.TUNE_ATTN_WIDE_POSITIONS, 0)
+        gpu.set_tuning(gpu.TUNE_ATTN_SPLITS, 0)
+    np.testing.assert_allclose(xb, wxb, rtol=0, atol=2e-5)
+
+
 def test_attention_invariants(gpu):
     seq_len, n_heads, hs, kv_mul = 64, 8, 64, 2
     kv_dim = n_heads // kv_mul * hs
