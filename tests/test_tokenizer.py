@@ -246,3 +246,21 @@ def test_invalid_utf8_does_not_crash(llama, gpt2):
         ids = ltok._ids("wgml_llama_tokenizer_encode", ltok._h, bad, len(bad), 0, 0)
         assert ids  # U+FFFD is no token of the vocabulary: its bytes EF BF BD + 3, per malformed byte
         assert all(t in (0xEF + 3, 0xBF + 3, 0xBD + 3) for t in ids)
+
+
+def test_llama2_chat_prompt():
+    from wgml_amd.tokenizer import llama2_chat_prompt
+
+    one = llama2_chat_prompt([{"role": "user", "content": " Hello  "}])
+    assert one == "<s>[INST] Hello [/INST]"
+    full = llama2_chat_prompt([{"role": "system", "content": "Be brief.\n"},
+                               {"role": "user", "content": "Hi"},
+                               {"role": "assistant", "content": "Hello."},
+                               {"role": "user", "content": "Bye"}])
+    assert full == ("<s>[INST] <<SYS>>\nBe brief.\n<</SYS>>\n\nHi [/INST] Hello. </s>"
+                    "<s>[INST] Bye [/INST]")
+    with pytest.raises(ValueError):
+        llama2_chat_prompt([{"role": "assistant", "content": "x"}])
+    with pytest.raises(ValueError):
+        llama2_chat_prompt([{"role": "user", "content": "a"}, {"role": "user", "content": "b"}])
+    assert llama2_chat_prompt([]) == ""

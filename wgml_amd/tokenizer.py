@@ -98,6 +98,32 @@ class LlamaTokenizer(_Tokenizer):
                           int(token)).decode("utf-8", "replace")
 
 
+def llama2_chat_prompt(messages: Sequence[dict], bos_token: str = "<s>", eos_token: str = "</s>") -> str:
+    """The Llama-2 chat prompt for a list of {"role", "content"} messages, as the reference's
+    default template for this model produces it (`LlamaTokenizer::CHAT_TEMPLATE`,
+    models/llama2/tokenizer.rs:19 with llama-2-chat.jinja): an optional leading system message
+    is wrapped in <<SYS>> markers and prepended to the first user message; user turns become
+    `bos [INST] content [/INST]`, assistant turns ` content eos`; contents are stripped of
+    surrounding whitespace; roles must alternate user / assistant.  (Only the text the template's
+    branches emit is produced: the line breaks and indentation between its blocks, which depend
+    on the template engine's whitespace settings, are not.)"""
+    msgs = list(messages)
+    system = ""
+    if msgs and msgs[0]["role"] == "system":
+        system = "<<SYS>>\n" + msgs[0]["content"].strip() + "\n<</SYS>>\n\n"
+        msgs = msgs[1:]
+    out = []
+    for i, m in enumerate(msgs):
+        if (m["role"] == "user") != (i % 2 == 0):
+            raise ValueError("Conversation roles must alternate user/assistant/user/assistant/...")
+        content = (system + m["content"] if i == 0 else m["content"]).strip()
+        if m["role"] == "user":
+            out.append(bos_token + "[INST] " + content + " [/INST]")
+        elif m["role"] == "assistant":
+            out.append(" " + content + " " + eos_token)
+    return "".join(out)
+
+
 class Gpt2Tokenizer(_Tokenizer):
     def __init__(self, tokens: Sequence[str], merges: Sequence[str], bos: int, eos: int):
         blob, offsets = _pack(tokens)
