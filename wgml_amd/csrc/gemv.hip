@@ -534,6 +534,8 @@ __global__ __launch_bounds__(MAXT) void gemv_quant_kernel(const GemvParams p) {
 // sub-block dot product is fp32.
 // =========================================================================
 
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
 }
@@ -1069,14 +1071,23 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
             sum += dpp_f32<0x4E>(sum);
             if (LPB == 8) sum += dpp_f32<0x141>(sum);
             sum *= amax * (1.0f / 32512.f);
-            const int l0 = ((X0 + 128) & 255) - 128, l1 = ((X1 + 128) & 255) - 128,
-                      l2 = ((X2 + 128) & 255) - 128, l3 = ((X3 + 128) & 255) - 128;
-            const int h0 = (X0 - l0) >> 8, h1 = (X1 - l1) >> 8, h2 = (X2 - l2) >> 8,
-                      h3 = (X3 - l3) >> 8;
-            const uint32_t hi = (uint32_t)(h0 & 255) | ((uint32_t)(h1 & 255) << 8) |
-                                ((uint32_t)(h2 & 255) << 16) | ((uint32_t)(h3 & 255) << 24);
-            const uint32_t lo = (uint32_t)(l0 & 255) | ((uint32_t)(l1 & 255) << 8) |
-                                ((uint32_t)(l2 & 255) << 16) | ((uint32_t)(l3 & 255) << 24);
+            // X = 256 hi + lo with lo the sign-extended low byte: lo is byte 0 of X as it stands
+            // and hi = (X + 128) >> 8 is byte 1 of X + 128 (|X| <= 32512, so 16 bits hold both).
+            // Two values per register as 16-bit halves, one packed add, and two byte
+            // permutes gather the four lo bytes and the four hi bytes.
+            const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)X1, (uint32_t)X0, 0x05040100u);
+            const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)X3, (uint32_t)X2, 0x05040100u);
+            const u16x2 bias128 = {128, 128};
+            u16x2 y01, y23;
+            __builtin_memcpy(&y01, &p01, 4);
+            __builtin_memcpy(&y23, &p23, 4);
+            y01 += bias128;
+            y23 += bias128;
+            uint32_t q01, q23;
+            __builtin_memcpy(&q01, &y01, 4);
+            __builtin_memcpy(&q23, &y23, 4);
+            const uint32_t lo = __builtin_amdgcn_perm(p23, p01, 0x06040200u);
+            const uint32_t hi = __builtin_amdgcn_perm(q23, q01, 0x07050301u);
             uint32_t tile, local, xb;
             F::locate(g4 * 4, tile, local, xb);
             const uint32_t dl = local >> 2, chunk = dl >> 2, sub = dl & 3;
