@@ -77,6 +77,33 @@ def test_attention_plans_agree(gpu, wide, splits, pos):
     np.testing.assert_allclose(xb, wxb, rtol=0, atol=2e-5)
 
 
+def test_bench_attention_runs_and_checks_its_arguments(gpu):
+    import ctypes as C
+
+    from wgml_amd._lib import AttnParams, View, call
+
+    seq_len, kv_mul, n_heads, hs, pos = 512, 2, 8, 64, 300
+    kv_dim = n_heads // kv_mul * hs
+    q = W.GpuVector.init(gpu, rnd(n_heads * hs, 1))
+    ks = [W.GpuVector.init(gpu, rnd(seq_len * kv_dim, 2 + i)) for i in range(2)]
+    vs = [W.GpuVector.init(gpu, rnd(seq_len * kv_dim, 5 + i)) for i in range(2)]
+    xb = W.GpuVector.uninit(gpu, n_heads * hs)
+    kv = (View * 2)(*[k.view() for k in ks])
+    vv = (View * 2)(*[v.view() for v in vs])
+    p = AttnParams(seq_len, kv_dim, kv_mul, n_heads, hs, pos)
+    ms = C.c_float(-1.0)
+    # 5 launches: the last one reads cache set 0, and leaves its result in xb
+    call("wgml_bench_attention", gpu.handle, C.byref(p), 512, q.view(), kv, vv, 2, xb.view(), 5, C.byref(ms))
+    assert ms.value > 0
+    want, _ = orc.attention(seq_len, kv_dim, kv_mul, n_heads, hs, pos, q.read(), ks[0].read(), vs[0].read())
+    np.testing.assert_allclose(xb.read(), want, rtol=0, atol=2e-5)
+    with pytest.raises(W.WgmlError):  # planned for fewer positions than the position itself
+        call("wgml_bench_attention", gpu.handle, C.byref(p), 256, q.view(), kv, vv, 2, xb.view(), 5, C.byref(ms))
+    with pytest.raises(W.WgmlError):  # caches shorter than seq_len rows
+        bad = AttnParams(2 * seq_len, kv_dim, kv_mul, n_heads, hs, pos)
+        call("wgml_bench_attention", gpu.handle, C.byref(bad), 1024, q.view(), kv, vv, 2, xb.view(), 5, C.byref(ms))
+
+
 def test_attention_invariants(gpu):
     seq_len, n_heads, hs, kv_mul = 64, 8, 64, 2
     kv_dim = n_heads // kv_mul * hs
