@@ -252,7 +252,7 @@ int launch_dequantize(wgml_ctx *ctx, float *out, const wgml_qmat *m);
 // ---- batched products for prompt processing (prefill.hip) ---------------------
 constexpr uint32_t kPrefillMaxTokens = 128;
 uint32_t prefill_tpad(uint32_t T);  // tokens rounded up to 16, 32, 64 or 128
-uint32_t prefill_kpad(uint32_t K);  // columns rounded up to a multiple of 64
+uint32_t prefill_kpad(uint32_t K);  // columns rounded up to a multiple of 128
 int ensure_prefill_scratch(wgml_ctx *ctx, size_t xh_bytes);
 // xh[tpad][kpad] (f16) <- x[T][K] (f32, rows x_stride apart): RMS-normalised with
 // norm_w first when that is non-null; replaced by up[t][k] * silu(x[t][k]) when `up`

@@ -40,6 +40,8 @@
 // of the 32 for token j); the A operand follows the same assignment of k to lanes.
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "device_utils.h"
 
@@ -49,6 +51,7 @@ namespace {
 
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // plain vector: arrays of it stay in registers
 
@@ -89,36 +92,22 @@ __device__ __forceinline__ half4 to_half4(float a, float b, float c, float d) {
 
 constexpr float kSplitScale = 2048.f;  // the low parts are stored times 2^11 (f16 range)
 
-__device__ __forceinline__ void pack_f16(const float (&w)[16], half8 (&a)[2]) {
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) a[s2][i] = (_Float16)w[8 * s2 + i];
-    }
-}
-__device__ __forceinline__ void pack_split(const float (&w)[16], half8 (&hi)[2], half8 (&lo)[2]) {
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const _Float16 h = (_Float16)w[8 * s2 + i];
-            hi[s2][i] = h;
-            lo[s2][i] = (_Float16)((w[8 * s2 + i] - (float)h) * kSplitScale);
-        }
-    }
-}
-
 // ---- weight fragments -----------------------------------------------------------
 // Lane (g, j) of a wave holds, for chunk c of row j of the tile, the 16 elements
 //     k = 64 c + 32 s2 + 8 g + 4 e + i        (s2, e in 0..1, i in 0..3)
-// load() fetches their bytes, expand() computes them as the reference's dequantize does
-// (quantization.rs:29-42, 204-244, 322-389), in fp32: w[4 (2 s2 + e) + i].  They reach the
-// matrix cores either rounded to f16 (pack_f16) or as a pair of f16 numbers whose sum is the
-// fp32 value to about 2^-22 (pack_split: hi = f16(w), lo = f16((w - hi) * 2048)).
+// load() fetches their bytes, pre() decodes what the 16 share (scales), elem<I>() computes
+// element I = 4 (2 s2 + e) + i as the reference's dequantize does (quantization.rs:29-42,
+// 204-244, 322-389), in fp32 (a fused multiply-add where the reference multiplies and subtracts:
+// one rounding less).  They reach the matrix cores either rounded to f16 or as a pair of f16
+// numbers whose sum is the fp32 value to about 2^-21 (hi = f16(w), lo = f16((w - hi) * 2048)).
+// The element-wise interface lets the kernel spread the expansion between its MFMAs.
 struct GemmQ4K {
     struct Raw {
         uint4 hdr;  // d, dmin, 12 bytes of packed scales
         uint2 qs;   // bytes 8 g .. 8 g + 7 of the chunk's 32: low nibbles s2 = 0, high s2 = 1
+    };
+    struct Pre {
+        float dd[2], mm[2];  // per s2: d * scale, dmin * min
     };
     __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, uint32_t row, uint32_t chunk,
                                 uint32_t g) {
@@ -126,7 +115,7 @@ struct GemmQ4K {
         r.hdr = *reinterpret_cast<const uint4 *>(blk);
         r.qs = *reinterpret_cast<const uint2 *>(blk + 16 + (chunk & 3) * 32 + 8 * g);
     }
-    __device__ static void expand(const Raw &r, uint32_t, uint32_t chunk, uint32_t, float (&w)[16]) {
+    __device__ static void pre(Pre &p, const Raw &r, uint32_t, uint32_t chunk, uint32_t) {
         const uint4 hdr = r.hdr;
         const uint32_t j = chunk & 3;
         const float d = f16_bits_to_f32((uint16_t)(hdr.x & 0xffffu));
@@ -147,18 +136,16 @@ struct GemmQ4K {
             s2 = ((hdr.w >> (sh + 8)) & 15u) | (((hdr.y >> (sh + 14)) & 3u) << 4);
             m2 = ((hdr.w >> (sh + 12)) & 15u) | (((hdr.z >> (sh + 14)) & 3u) << 4);
         }
-        const float d1 = d * (float)s1, mm1 = dmin * (float)m1;
-        const float d2 = d * (float)s2, mm2 = dmin * (float)m2;
-        auto four = [&](float *o, uint32_t q, float dd, float mm) {
-            o[0] = dd * (float)(q & 15u) - mm;
-            o[1] = dd * (float)((q >> 8) & 15u) - mm;
-            o[2] = dd * (float)((q >> 16) & 15u) - mm;
-            o[3] = dd * (float)((q >> 24) & 15u) - mm;
-        };
-        four(w, r.qs.x, d1, mm1);
-        four(w + 4, r.qs.y, d1, mm1);
-        four(w + 8, r.qs.x >> 4, d2, mm2);
-        four(w + 12, r.qs.y >> 4, d2, mm2);
+        p.dd[0] = d * (float)s1;
+        p.mm[0] = dmin * (float)m1;
+        p.dd[1] = d * (float)s2;
+        p.mm[1] = dmin * (float)m2;
+    }
+    template <int I>
+    __device__ static float elem(const Pre &p, const Raw &r, uint32_t) {
+        constexpr int s2 = I / 8, e = (I / 4) & 1, b = I & 3;
+        const uint32_t word = (e ? r.qs.y : r.qs.x) >> (4 * s2 + 8 * b);
+        return fmaf(p.dd[s2], (float)(word & 15u), -p.mm[s2]);
     }
 };
 
@@ -168,6 +155,10 @@ struct GemmQ6K {
         uint2 qh;     // 8 bytes of high bit pairs
         uint32_t scw;  // the four scales of this 64-element chunk
         uint32_t d;
+    };
+    struct Pre {
+        float ds[2];       // per s2: d * scale
+        uint32_t hi_nib;   // odd chunks take the high nibbles
     };
     __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, uint32_t row, uint32_t chunk,
                                 uint32_t g) {
@@ -180,28 +171,23 @@ struct GemmQ6K {
         r.scw = *reinterpret_cast<const uint32_t *>(m.p2 + blk * 16 + 8 * i + 4 * (c & 1));
         r.d = *reinterpret_cast<const uint16_t *>(m.p3 + blk * 2);
     }
-    __device__ static void expand(const Raw &r, uint32_t, uint32_t chunk, uint32_t g, float (&w)[16]) {
-        // element e = 64 (c & 1) + 32 s2 + 8 g + b of the 128-element half: quarter
-        // e / 32 = 2 (c & 1) + s2 picks the nibble (high for quarters 2, 3), the bit pair of
-        // qh[8 g + b] (shift 2 * quarter) and the scale (8 g + b) / 16 + 2 * quarter
-        const uint32_t hi_nib = chunk & 1;
+    // element e = 64 (c & 1) + 32 s2 + 8 g + b of the 128-element half: quarter
+    // e / 32 = 2 (c & 1) + s2 picks the nibble (high for quarters 2, 3), the bit pair of
+    // qh[8 g + b] (shift 2 * quarter) and the scale (8 g + b) / 16 + 2 * quarter
+    __device__ static void pre(Pre &p, const Raw &r, uint32_t, uint32_t chunk, uint32_t g) {
         const float d = f16_bits_to_f32((uint16_t)r.d);
+        p.hi_nib = chunk & 1;
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-            const float ds = d * (float)(int8_t)((r.scw >> (8 * ((g >> 1) + 2 * s2))) & 0xffu);
-            const uint32_t hsh = 2 * (2 * hi_nib + s2);
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                uint32_t l = e ? r.ql[s2].y : r.ql[s2].x;
-                if (hi_nib) l >>= 4;
-                const uint32_t h = (e ? r.qh.y : r.qh.x) >> hsh;
-#pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    const int q = (int)(((l >> (8 * b)) & 15u) | (((h >> (8 * b)) & 3u) << 4)) - 32;
-                    w[4 * (2 * s2 + e) + b] = ds * (float)q;
-                }
-            }
-        }
+        for (int s2 = 0; s2 < 2; ++s2)
+            p.ds[s2] = d * (float)(int8_t)((r.scw >> (8 * ((g >> 1) + 2 * s2))) & 0xffu);
+    }
+    template <int I>
+    __device__ static float elem(const Pre &p, const Raw &r, uint32_t) {
+        constexpr int s2 = I / 8, e = (I / 4) & 1, b = I & 3;
+        const uint32_t l = (e ? r.ql[s2].y : r.ql[s2].x) >> (4 * p.hi_nib + 8 * b);
+        const uint32_t h = (e ? r.qh.y : r.qh.x) >> (2 * (2 * p.hi_nib + s2) + 8 * b);
+        const int q = (int)((l & 15u) | ((h & 3u) << 4)) - 32;
+        return p.ds[s2] * (float)q;
     }
 };
 
@@ -210,8 +196,11 @@ struct GemmQ8_0 {
         uint2 q[2];  // per s2 (= 32-element block of the chunk): 8 quants
         uint32_t d[2];
     };
-    // rows are a multiple of 32 elements long: the second half of the last chunk may not
-    // exist; it is then read from the first half and expanded to zeros
+    struct Pre {
+        float d[2];
+    };
+    // rows are a multiple of 32 elements long: a 32-element block of the (padded) K range may
+    // not exist; the last one is then read in its place and expanded to zeros
     __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, uint32_t row, uint32_t chunk,
                                 uint32_t g) {
         const uint32_t b0 = chunk * 2, nb = ncols / 32;
@@ -222,28 +211,103 @@ struct GemmQ8_0 {
             r.d[s2] = *reinterpret_cast<const uint16_t *>(m.p1 + ((size_t)row * nb + b) * 2);
         }
     }
-    __device__ static void expand(const Raw &r, uint32_t ncols, uint32_t chunk, uint32_t, float (&w)[16]) {
+    __device__ static void pre(Pre &p, const Raw &r, uint32_t ncols, uint32_t chunk, uint32_t) {
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-            const bool exists = chunk * 2 + s2 < ncols / 32;
-            const float d = exists ? f16_bits_to_f32((uint16_t)r.d[s2]) : 0.f;
-            const uint32_t x = exists ? r.q[s2].x : 0u, y = exists ? r.q[s2].y : 0u;
-            float *o = w + 8 * s2;
-            o[0] = sb0(x) * d;
-            o[1] = sb1(x) * d;
-            o[2] = sb2(x) * d;
-            o[3] = sb3(x) * d;
-            o[4] = sb0(y) * d;
-            o[5] = sb1(y) * d;
-            o[6] = sb2(y) * d;
-            o[7] = sb3(y) * d;
-        }
+        for (int s2 = 0; s2 < 2; ++s2)
+            p.d[s2] = chunk * 2 + s2 < ncols / 32 ? f16_bits_to_f32((uint16_t)r.d[s2]) : 0.f;
+    }
+    template <int I>
+    __device__ static float elem(const Pre &p, const Raw &r, uint32_t) {
+        constexpr int s2 = I / 8, e = (I / 4) & 1, b = I & 3;
+        const uint32_t word = (e ? r.q[s2].y : r.q[s2].x) >> (8 * b);
+        return (float)(int8_t)(word & 0xffu) * p.d[s2];
     }
 };
+
+// A wave's weights for one chunk as MFMA A operands: hi[s2] (and, split precision, lo[s2]).
+template <bool SPLIT>
+struct AFrag {
+    half2v hi[2][4];
+    half2v lo[SPLIT ? 2 : 1][4];
+};
+
+// Elements 2 P and 2 P + 1 of the 16: expanded, rounded (or split) and packed.  The high part is
+// rounded toward zero in the split form (one instruction for the pair): the low part holds what
+// is left, (w - hi) * 2^11, which is exact in fp32 before its own rounding to f16.
+template <class F, bool SPLIT, int P>
+__device__ __forceinline__ void frag_pair(AFrag<SPLIT> &f, const typename F::Pre &pre, const typename F::Raw &r,
+                                          uint32_t g) {
+    const float w0 = F::template elem<2 * P>(pre, r, g), w1 = F::template elem<2 * P + 1>(pre, r, g);
+    constexpr int s2 = P / 4, i = P % 4;
+    if constexpr (SPLIT) {
+        const auto hz = __builtin_amdgcn_cvt_pkrtz(w0, w1);
+        half2v h;
+        __builtin_memcpy(&h, &hz, 4);
+        f.hi[s2][i] = h;
+        half2v l;
+        l[0] = (_Float16)((w0 - (float)h[0]) * kSplitScale);
+        l[1] = (_Float16)((w1 - (float)h[1]) * kSplitScale);
+        f.lo[s2][i] = l;
+    } else {
+        half2v h;
+        h[0] = (_Float16)w0;
+        h[1] = (_Float16)w1;
+        f.hi[s2][i] = h;
+    }
+}
+
+template <class F, bool SPLIT, int P = 0>
+__device__ __forceinline__ void frag_pairs_from(AFrag<SPLIT> &f, const typename F::Pre &pre,
+                                                const typename F::Raw &r, uint32_t g) {
+    if constexpr (P < 8) {
+        frag_pair<F, SPLIT, P>(f, pre, r, g);
+        frag_pairs_from<F, SPLIT, P + 1>(f, pre, r, g);
+    }
+}
+
+// Piece K of the nine a chunk's expansion is cut into: the shared part, then the eight pairs.
+template <class F, bool SPLIT, int K>
+__device__ __forceinline__ void frag_piece(AFrag<SPLIT> &f, typename F::Pre &pre, const typename F::Raw &r,
+                                           uint32_t ncols, uint32_t chunk, uint32_t g) {
+    if constexpr (K == 0) {
+        F::pre(pre, r, ncols, chunk, g);
+    } else {
+        frag_pair<F, SPLIT, K - 1>(f, pre, r, g);
+    }
+}
+
+// The pieces that belong to step STEP of NSTEP: piece K goes to step K * NSTEP / 9.
+template <class F, bool SPLIT, int STEP, int NSTEP, int K = 0>
+__device__ __forceinline__ void frag_pieces_of_step(AFrag<SPLIT> &f, typename F::Pre &pre,
+                                                    const typename F::Raw &r, uint32_t ncols, uint32_t chunk,
+                                                    uint32_t g) {
+    if constexpr (K < 9) {
+        if constexpr (K * NSTEP / 9 == STEP) frag_piece<F, SPLIT, K>(f, pre, r, ncols, chunk, g);
+        frag_pieces_of_step<F, SPLIT, STEP, NSTEP, K + 1>(f, pre, r, ncols, chunk, g);
+    }
+}
+
+__device__ __forceinline__ half8 as_half8(const half2v (&h)[4]) {
+    half8 v;
+    __builtin_memcpy(&v, h, 16);
+    return v;
+}
+
+template <int I, int N, class Fn>
+__device__ __forceinline__ void static_for(Fn &&fn) {
+    if constexpr (I < N) {
+        fn(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(fn);
+    }
+}
 
 // SPLIT: both operands are pairs of f16 numbers (high part, low part times 2^11); the product is
 // W_hi X_hi + 2^-11 (W_hi X_lo + W_lo X_hi), three MFMAs per sub-block instead of one, which
 // leaves an error of about 2^-22 per term instead of 2^-11.
+//
+// The loop is software-pipelined: while the matrix cores multiply the weights of iteration it,
+// the vector ALU expands those of iteration it + 1 (fetched during iteration it - 1) -- the two
+// waves of a SIMD run in step between barriers, so the overlap has to come from inside a wave.
 template <class F, int NT, bool SPLIT>
 __global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a) {
     extern __shared__ u32x4 xs[];  // [2 buffers][2 chunks][high: NT * 128 words (, low: the same)]
@@ -262,10 +326,11 @@ __global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a)
     const GemmMat &m = a.m[mi];
     const uint32_t row0 = (blockIdx.x - m.tile0) * 64 + 16 * rb;
     const uint32_t row = min(row0 + j, m.nrows - 1);  // this lane's row of the A operand
-    const uint32_t nchunks = a.kpad / KC;
-    const uint32_t per = (nchunks + a.ks - 1) / a.ks;
-    const uint32_t c0 = min(blockIdx.y * per, nchunks), c1 = min(nchunks, c0 + per);
-    const uint32_t n_it = (c1 - c0 + 1) / 2;
+    // K is walked in pairs of chunks (kpad is a multiple of two chunks)
+    const uint32_t npairs = a.kpad / (2 * KC);
+    const uint32_t per = (npairs + a.ks - 1) / a.ks;
+    const uint32_t p0 = min(blockIdx.y * per, npairs), p1 = min(npairs, p0 + per);
+    const uint32_t n_it = p1 - p0;
 
     floatx4 acc[NT], accl[SPLIT ? NT : 1];
 #pragma unroll
@@ -273,21 +338,29 @@ __global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a)
 #pragma unroll
     for (int n = 0; n < (SPLIT ? NT : 1); ++n) accl[n] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // Staged words of this thread: word tid + 512 q of the pair of chunks, q < SW.  All
-    // loads are unconditional (chunks past the end re-read the last one and are not used).
-    // In memory the low parts form a second array behind the high parts (a.xl).
-    auto gword = [&](uint32_t first_chunk, uint32_t q) {
+    // Staged words of this thread: word tid + 512 q of the pair of chunks, q < SW; in memory the
+    // low parts form a second array behind the high parts (a.xl).  All loads are unconditional:
+    // past the end the last pair is fetched again and not used.
+    const u32x4 *src[SW];
+#pragma unroll
+    for (int q = 0; q < SW; ++q) {
         const uint32_t w = min(tid + NTHREADS * q, 2 * CWX - 1);
-        const uint32_t c = min(first_chunk + w / CWX, nchunks - 1), ww = w % CWX;
-        if (SPLIT && ww >= CW) return a.xl[(size_t)c * CW + ww - CW];
-        return a.xh[(size_t)c * CW + ww];
-    };
+        const uint32_t ch = w / CWX, ww = w % CWX;
+        src[q] = (SPLIT && ww >= CW) ? a.xl + (ch * CW + ww - CW) : a.xh + (ch * CW + ww);
+    }
+    auto pair_at = [&](uint32_t it) { return min(p0 + it, npairs - 1); };  // uniform
     u32x4 st[SW];
-    typename F::Raw cur, nxt;
+    AFrag<SPLIT> A;
+    typename F::Raw rn;  // the bytes of iteration it + 1
     if (n_it > 0) {
 #pragma unroll
-        for (int q = 0; q < SW; ++q) st[q] = gword(c0, q);
-        F::load(cur, m, a.ncols, row, min(c0 + kh, nchunks - 1), g);
+        for (int q = 0; q < SW; ++q) st[q] = src[q][(size_t)p0 * 2 * CW];
+        typename F::Raw r0;
+        F::load(r0, m, a.ncols, row, 2 * p0 + kh, g);
+        F::load(rn, m, a.ncols, row, 2 * pair_at(1) + kh, g);
+        typename F::Pre pre0;
+        F::pre(pre0, r0, a.ncols, 2 * p0 + kh, g);
+        frag_pairs_from<F, SPLIT>(A, pre0, r0, g);
     }
     for (uint32_t it = 0; it < n_it; ++it) {
         u32x4 *buf = xs + (it & 1) * 2 * CWX;
@@ -296,44 +369,48 @@ __global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a)
             if (2 * CWX % NTHREADS == 0 || tid + NTHREADS * q < 2 * CWX) buf[tid + NTHREADS * q] = st[q];
         }
         __syncthreads();
+        const uint32_t pn = pair_at(it + 1);
 #pragma unroll
-        for (int q = 0; q < SW; ++q) st[q] = gword(c0 + 2 * (it + 1), q);
-        F::load(nxt, m, a.ncols, row, min(c0 + 2 * (it + 1) + kh, nchunks - 1), g);
-        const uint32_t c = c0 + 2 * it + kh;
-        if (c < c1) {  // uniform over the wave
-            const u32x4 *bsrc = buf + kh * CWX + lane;
-            // the LDS words of the first half are requested before the weights are expanded,
-            // those of the second half while the first half is multiplied
-            u32x4 bw[NT];
+        for (int q = 0; q < SW; ++q) st[q] = src[q][(size_t)pn * 2 * CW];
+        typename F::Raw rnn;
+        F::load(rnn, m, a.ncols, row, 2 * pair_at(it + 2) + kh, g);
+        // The 2 NT steps of an iteration (one token block of one half chunk each): the LDS words of
+        // step + 2 are requested, the step's MFMAs issued, and a piece of the expansion of the next
+        // iteration's weights done, in this order (nothing is scheduled across a step's end).
+        AFrag<SPLIT> An;
+        typename F::Pre pre;
+        const uint32_t cn = 2 * pn + kh;
+        const u32x4 *bsrc = buf + kh * CWX + lane;
+        constexpr int NSTEP = 2 * NT, AHEAD = 2;
+        u32x4 bh[AHEAD + 1], bl[AHEAD + 1];
 #pragma unroll
-            for (int n = 0; n < NT; ++n) bw[n] = bsrc[(n * 2) * 64];
-            float w[16];
-            F::expand(cur, a.ncols, c, g, w);
-            half8 ah[2], al[2];
-            if (SPLIT) {
-                pack_split(w, ah, al);
-            } else {
-                pack_f16(w, ah);
-            }
-#pragma unroll
-            for (int s2 = 0; s2 < 2; ++s2) {
-#pragma unroll
-                for (int n = 0; n < NT; ++n) {
-                    half8 b8;
-                    __builtin_memcpy(&b8, &bw[n], 16);
-                    acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah[s2], b8, acc[n], 0, 0, 0);
-                    if (SPLIT) {
-                        accl[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al[s2], b8, accl[n], 0, 0, 0);
-                        const u32x4 lw = bsrc[CW + (n * 2 + s2) * 64];
-                        half8 l8;
-                        __builtin_memcpy(&l8, &lw, 16);
-                        accl[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah[s2], l8, accl[n], 0, 0, 0);
-                    }
-                    if (s2 == 0) bw[n] = bsrc[(n * 2 + 1) * 64];
-                }
-            }
+        for (int d = 0; d < AHEAD && d < NSTEP; ++d) {
+            bh[d] = bsrc[((d % NT) * 2 + d / NT) * 64];
+            if (SPLIT) bl[d] = bsrc[CW + ((d % NT) * 2 + d / NT) * 64];
         }
-        cur = nxt;
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<0, NSTEP>([&](auto step_c) {
+            constexpr int step = decltype(step_c)::value;
+            constexpr int s2 = step / NT, n = step % NT, cur = step % (AHEAD + 1);
+            if constexpr (step + AHEAD < NSTEP) {
+                constexpr int sn = step + AHEAD, slot = sn % (AHEAD + 1);
+                bh[slot] = bsrc[((sn % NT) * 2 + sn / NT) * 64];
+                if (SPLIT) bl[slot] = bsrc[CW + ((sn % NT) * 2 + sn / NT) * 64];
+            }
+            half8 b8;
+            __builtin_memcpy(&b8, &bh[cur], 16);
+            acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(A.hi[s2]), b8, acc[n], 0, 0, 0);
+            if constexpr (SPLIT) {
+                accl[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(A.lo[s2]), b8, accl[n], 0, 0, 0);
+                half8 l8;
+                __builtin_memcpy(&l8, &bl[cur], 16);
+                accl[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(A.hi[s2]), l8, accl[n], 0, 0, 0);
+            }
+            frag_pieces_of_step<F, SPLIT, step, NSTEP>(An, pre, rn, a.ncols, cn, g);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        A = An;
+        rn = rnn;
     }
     if (SPLIT) {
 #pragma unroll
@@ -879,7 +956,7 @@ __global__ __launch_bounds__(256) void attn_block_kernel(const AttnRowsArgs a, u
 uint32_t gemm_k_split(const wgml_ctx *ctx, uint32_t tiles, uint32_t kpad, bool split) {
     const uint32_t nchunks = kpad / KC;
     const int forced = ctx->tuning[WGML_TUNE_GEMM_K_SPLIT];  // 0: by matrix shape
-    if (forced) return min((uint32_t)forced, max(nchunks, 1u));
+    if (forced) return min((uint32_t)forced, max(nchunks / 2, 1u));  // K is walked in pairs of chunks
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
     if (!split) {
         uint32_t ks = 1;
@@ -941,7 +1018,7 @@ int launch_gemm_fmt(wgml_ctx *ctx, GemmArgs &a, uint32_t tiles) {
 namespace wgml {
 
 uint32_t prefill_tpad(uint32_t T) { return T <= 16 ? 16 : T <= 32 ? 32 : T <= 64 ? 64 : 128; }
-uint32_t prefill_kpad(uint32_t K) { return (K + KC - 1) / KC * KC; }
+uint32_t prefill_kpad(uint32_t K) { return (K + 2 * KC - 1) / (2 * KC) * (2 * KC); }
 
 int ensure_prefill_scratch(wgml_ctx *ctx, size_t xh_bytes) {
     if (!ctx->prefill_xscale)
