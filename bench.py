@@ -318,6 +318,9 @@ def main():
                          "(for profiler runs)")
     ap.add_argument("--gemm-precision", type=int, default=1, choices=[0, 1],
                     help="with --prefill-only: 1 = split-f16 operands (default), 0 = plain f16")
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="launch-shape override, e.g. GEMM_K_SPLIT=4 (a TUNE_* key of GpuInstance); "
+                         "may be given several times (for sweeps)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every kernel uses a single device; "
@@ -384,6 +387,9 @@ def main():
         return
     model = Llama2(gpu, cfg).load(weights)
     prompt = W.prompt_tokens(4, n_prompt, cfg.vocab_size)
+    for kv in args.tune:
+        key, value = kv.split("=")
+        gpu.set_tuning(getattr(gpu, "TUNE_" + key.upper()), int(value))
     if args.prefill_only:
         gpu.set_gemm_precision(args.gemm_precision)
         model.prefill(prompt)

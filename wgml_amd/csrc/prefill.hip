@@ -11,9 +11,13 @@
 // activations are scaled per token by a power of two so that they stay in f16 range, products
 // accumulate in fp32 on v_mfma_f32_16x16x32_f16.  Two precisions:
 //   split f16 (default)  each operand is a pair of f16 numbers, hi = f16(v) and
-//                        lo = f16((v - hi) * 2^11); the product is
-//                        W_hi X_hi + 2^-11 (W_hi X_lo + W_lo X_hi): three MFMAs per term group,
-//                        results to fp32 rounding (about 1e-6 of a row's magnitude);
+//                        lo = f16(v - hi); the product is W_hi X_hi + W_hi X_lo + W_lo X_hi, three
+//                        MFMAs per term group into one fp32 accumulator, results to fp32 rounding
+//                        (about 1e-6 of a row's magnitude).  The low parts are small: weights are
+//                        expanded times 2^8 and activations scaled to 512 < max |x| <= 1024 so that
+//                        they stay clear of the bottom of the f16 range (the matrix cores take
+//                        subnormal f16 inputs as they are, so what falls below loses precision
+//                        gradually, not all at once);
 //   plain f16            both operands rounded to f16 once, one MFMA: about 3e-4 of a row's RMS.
 //
 // Tiling.  A workgroup (8 waves) owns 64 rows of one matrix -- four blocks of 16 -- and
@@ -24,13 +28,25 @@
 // exactly once, by one wave, for all NT blocks of 16 tokens (NT accumulators of 16x16 per
 // wave).  Two LDS buffers: the next pair of chunks is on its way from memory while the
 // current one is multiplied, one barrier per iteration.  At the end waves 4-7 hand
-// their sums to waves 0-3 through LDS.
+// their sums to waves 0-3 through LDS.  (K is padded to a whole number of pairs of chunks.)
+//
+// On this machine a SIMD does not overlap the vector instructions of one wave with the MFMAs
+// of another to any useful degree (measured: two MFMA-then-VALU waves per SIMD take the sum of
+// both parts), and the two waves of a SIMD run in step between barriers.  So the overlap is
+// made inside each wave: while it issues the MFMAs of iteration it, it expands the weights of
+// iteration it + 1 (fetched during iteration it - 1), a few vector instructions after every
+// MFMA, and it requests its LDS words two steps ahead.  The expansion is written for few
+// instructions: bytes masked four at a time and converted with the byte-to-float
+// instructions, one multiply-add per element, one packed conversion per pair for the high
+// parts, one mixed-precision multiply-add per element for the low parts, lane offsets of 32
+// bits on uniform bases for every load.
 //
 // One launch can cover up to three matrices that multiply the same activations (Q, K
-// and V; gate and up): their row tiles are laid side by side in grid.x.  A matrix too
-// short to give every compute unit a tile has its K range split between grid.y
-// workgroups; they leave partial sums that gemm_reduce_kernel adds in a fixed order (or,
-// for a plain `x += W h`, the prep_x_kernel that reads x next).
+// and V; gate and up): their row tiles are numbered side by side.  A matrix too short to
+// give every compute unit a tile has its K range split between ks workgroups; they leave
+// partial sums that gemm_reduce_kernel adds in a fixed order (or, for a plain `x += W h`,
+// the prep_x_kernel that reads x next).  Workgroup w takes part w % ks of tile w / ks: the
+// eight XCDs are handed workgroups in turn, so each sees 1 / ks of the activations only.
 //
 // Activations are stored in the order the B operand wants them (written by
 // prep_x_kernel): for chunk c, token block n, half s2 of the chunk, lane (g, j) finds
@@ -72,6 +88,7 @@ struct GemmArgs {
     uint32_t nmat;
     const u32x4 *xh;                   // packed f16 activations (see above)
     const u32x4 *xl;                   // their low parts in the same order (split precision only)
+    uint32_t xl_offset;                // bytes from xh to xl
     const float *xscale;               // [tpad] factor to multiply a token's results with
     uint32_t ncols, kpad, T, tpad;
     int accumulate;                    // out += result
@@ -90,16 +107,35 @@ __device__ __forceinline__ half4 to_half4(float a, float b, float c, float d) {
     return h;
 }
 
-constexpr float kSplitScale = 2048.f;  // the low parts are stored times 2^11 (f16 range)
+// Weights are expanded times 2^8 (an exact scaling, undone with the activations' factor at the
+// end): a low part f16(w - hi) of a typical weight (0.01 .. 0.1) is then a normal f16 number.
+// Weights of magnitude 256 and more would overflow f16; no model has them.
+constexpr float kWeightScale = 256.f;
+
+// The value as the compiler must take it: what follows is not merged with what computed it.
+__device__ __forceinline__ uint32_t opaque(uint32_t v) {
+    asm("" : "+v"(v));
+    return v;
+}
+
+// A load from uniform base + 32-bit lane offset.  The empty asm keeps the offset a 32-bit VGPR
+// at the point of use, so that the load takes the base from scalar registers and the offset as
+// it is: no 64-bit address arithmetic per lane and iteration.
+template <class T>
+__device__ __forceinline__ T load_at(const uint8_t *uniform_base, uint32_t lane_offset) {
+    asm volatile("" : "+v"(lane_offset));
+    return *reinterpret_cast<const T *>(uniform_base + lane_offset);
+}
 
 // ---- weight fragments -----------------------------------------------------------
 // Lane (g, j) of a wave holds, for chunk c of row j of the tile, the 16 elements
 //     k = 64 c + 32 s2 + 8 g + 4 e + i        (s2, e in 0..1, i in 0..3)
-// load() fetches their bytes, pre() decodes what the 16 share (scales), elem<I>() computes
+// lane_init() computes the lane's byte offsets into the matrix planes once (matrices are below
+// 4 GiB), load() fetches the bytes, pre() decodes what the 16 share (scales), elem<I>() computes
 // element I = 4 (2 s2 + e) + i as the reference's dequantize does (quantization.rs:29-42,
 // 204-244, 322-389), in fp32 (a fused multiply-add where the reference multiplies and subtracts:
 // one rounding less).  They reach the matrix cores either rounded to f16 or as a pair of f16
-// numbers whose sum is the fp32 value to about 2^-21 (hi = f16(w), lo = f16((w - hi) * 2048)).
+// numbers whose sum is the fp32 value to about 2^-21 (hi = f16(w), lo = f16(w - hi)), all times 2^8.
 // The element-wise interface lets the kernel spread the expansion between its MFMAs.
 struct GemmQ4K {
     struct Raw {
@@ -109,17 +145,23 @@ struct GemmQ4K {
     struct Pre {
         float dd[2], mm[2];  // per s2: d * scale, dmin * min
     };
-    __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, uint32_t row, uint32_t chunk,
-                                uint32_t g) {
-        const uint8_t *blk = m.p0 + ((size_t)row * (ncols / 256) + (chunk >> 2)) * 144;
-        r.hdr = *reinterpret_cast<const uint4 *>(blk);
-        r.qs = *reinterpret_cast<const uint2 *>(blk + 16 + (chunk & 3) * 32 + 8 * g);
+    struct Lane {
+        uint32_t hdr, qs;
+    };
+    __device__ static void lane_init(Lane &l, uint32_t ncols, uint32_t row, uint32_t g) {
+        l.hdr = row * (ncols / 256) * 144;
+        l.qs = l.hdr + 16 + 8 * g;
+    }
+    __device__ static void load(Raw &r, const GemmMat &m, uint32_t, const Lane &l, uint32_t chunk) {
+        const uint8_t *blk = m.p0 + (size_t)(chunk >> 2) * 144;
+        r.hdr = load_at<uint4>(blk, l.hdr);
+        r.qs = load_at<uint2>(blk + (chunk & 3) * 32, l.qs);
     }
     __device__ static void pre(Pre &p, const Raw &r, uint32_t, uint32_t chunk, uint32_t) {
         const uint4 hdr = r.hdr;
         const uint32_t j = chunk & 3;
-        const float d = f16_bits_to_f32((uint16_t)(hdr.x & 0xffffu));
-        const float dmin = f16_bits_to_f32((uint16_t)(hdr.x >> 16));
+        const float d = f16_bits_to_f32((uint16_t)(hdr.x & 0xffffu)) * kWeightScale;
+        const float dmin = f16_bits_to_f32((uint16_t)(hdr.x >> 16)) * kWeightScale;
         // get_scale_min_k4 for sub-blocks 2j and 2j + 1, on the three words of packed scales
         // (no byte array: the index is not a compile-time constant)
         uint32_t s1, m1, s2, m2;
@@ -144,8 +186,9 @@ struct GemmQ4K {
     template <int I>
     __device__ static float elem(const Pre &p, const Raw &r, uint32_t) {
         constexpr int s2 = I / 8, e = (I / 4) & 1, b = I & 3;
-        const uint32_t word = (e ? r.qs.y : r.qs.x) >> (4 * s2 + 8 * b);
-        return fmaf(p.dd[s2], (float)(word & 15u), -p.mm[s2]);
+        // the four nibbles of a word are masked at once; each is then one byte-to-float conversion
+        const uint32_t four = opaque(((e ? r.qs.y : r.qs.x) >> (4 * s2)) & 0x0f0f0f0fu);
+        return fmaf(p.dd[s2], (float)((four >> (8 * b)) & 0xffu), -p.mm[s2]);
     }
 };
 
@@ -157,37 +200,50 @@ struct GemmQ6K {
         uint32_t d;
     };
     struct Pre {
-        float ds[2];       // per s2: d * scale
-        uint32_t hi_nib;   // odd chunks take the high nibbles
+        float ds[2], off[2];  // per s2: d * scale, -32 d * scale
+        uint32_t hi_nib;      // odd chunks take the high nibbles
     };
-    __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, uint32_t row, uint32_t chunk,
-                                uint32_t g) {
-        const size_t blk = (size_t)row * (ncols / 256) + (chunk >> 2);
+    struct Lane {
+        uint32_t ql, qh, sc, d;
+    };
+    __device__ static void lane_init(Lane &l, uint32_t ncols, uint32_t row, uint32_t g) {
+        const uint32_t blk = row * (ncols / 256);
+        l.ql = blk * 128 + 8 * g;
+        l.qh = blk * 64 + 8 * g;
+        l.sc = blk * 16;
+        l.d = blk * 2;
+    }
+    __device__ static void load(Raw &r, const GemmMat &m, uint32_t, const Lane &l, uint32_t chunk) {
+        const size_t blk = chunk >> 2;
         const uint32_t c = chunk & 3, i = c >> 1;
-        const uint8_t *ql = m.p0 + blk * 128 + 64 * i + 8 * g;
-        r.ql[0] = *reinterpret_cast<const uint2 *>(ql);
-        r.ql[1] = *reinterpret_cast<const uint2 *>(ql + 32);
-        r.qh = *reinterpret_cast<const uint2 *>(m.p1 + blk * 64 + 32 * i + 8 * g);
-        r.scw = *reinterpret_cast<const uint32_t *>(m.p2 + blk * 16 + 8 * i + 4 * (c & 1));
-        r.d = *reinterpret_cast<const uint16_t *>(m.p3 + blk * 2);
+        const uint8_t *ql = m.p0 + blk * 128 + 64 * i;
+        r.ql[0] = load_at<uint2>(ql, l.ql);
+        r.ql[1] = load_at<uint2>(ql + 32, l.ql);
+        r.qh = load_at<uint2>(m.p1 + blk * 64 + 32 * i, l.qh);
+        r.scw = load_at<uint32_t>(m.p2 + blk * 16 + 8 * i + 4 * (c & 1), l.sc);
+        r.d = load_at<uint16_t>(m.p3 + blk * 2, l.d);
     }
     // element e = 64 (c & 1) + 32 s2 + 8 g + b of the 128-element half: quarter
     // e / 32 = 2 (c & 1) + s2 picks the nibble (high for quarters 2, 3), the bit pair of
     // qh[8 g + b] (shift 2 * quarter) and the scale (8 g + b) / 16 + 2 * quarter
     __device__ static void pre(Pre &p, const Raw &r, uint32_t, uint32_t chunk, uint32_t g) {
-        const float d = f16_bits_to_f32((uint16_t)r.d);
+        const float d = f16_bits_to_f32((uint16_t)r.d) * kWeightScale;
         p.hi_nib = chunk & 1;
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
+        for (int s2 = 0; s2 < 2; ++s2) {
             p.ds[s2] = d * (float)(int8_t)((r.scw >> (8 * ((g >> 1) + 2 * s2))) & 0xffu);
+            p.off[s2] = -32.f * p.ds[s2];
+        }
     }
     template <int I>
     __device__ static float elem(const Pre &p, const Raw &r, uint32_t) {
         constexpr int s2 = I / 8, e = (I / 4) & 1, b = I & 3;
-        const uint32_t l = (e ? r.ql[s2].y : r.ql[s2].x) >> (4 * p.hi_nib + 8 * b);
-        const uint32_t h = (e ? r.qh.y : r.qh.x) >> (2 * (2 * p.hi_nib + s2) + 8 * b);
-        const int q = (int)((l & 15u) | ((h & 3u) << 4)) - 32;
-        return p.ds[s2] * (float)q;
+        // the four 6-bit values of a word pair are put together at once (bytes 0 .. 63), each is
+        // then one byte-to-float conversion; (q - 32) ds as one multiply-add with -32 ds
+        const uint32_t l = ((e ? r.ql[s2].y : r.ql[s2].x) >> (4 * p.hi_nib)) & 0x0f0f0f0fu;
+        const uint32_t h = ((e ? r.qh.y : r.qh.x) >> (2 * (2 * p.hi_nib + s2))) & 0x03030303u;
+        const uint32_t four = opaque(l | (h << 4));
+        return fmaf(p.ds[s2], (float)((four >> (8 * b)) & 0xffu), p.off[s2]);
     }
 };
 
@@ -197,30 +253,40 @@ struct GemmQ8_0 {
         uint32_t d[2];
     };
     struct Pre {
-        float d[2];
+        float d[2], off[2];  // per s2: d, -128 d
     };
     // rows are a multiple of 32 elements long: a 32-element block of the (padded) K range may
     // not exist; the last one is then read in its place and expanded to zeros
-    __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, uint32_t row, uint32_t chunk,
-                                uint32_t g) {
+    struct Lane {
+        uint32_t q, d;
+    };
+    __device__ static void lane_init(Lane &l, uint32_t ncols, uint32_t row, uint32_t g) {
+        l.q = row * ncols + 8 * g;
+        l.d = row * (ncols / 32) * 2;
+    }
+    __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, const Lane &l, uint32_t chunk) {
         const uint32_t b0 = chunk * 2, nb = ncols / 32;
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
             const uint32_t b = min(b0 + s2, nb - 1);
-            r.q[s2] = *reinterpret_cast<const uint2 *>(m.p0 + (size_t)row * ncols + b * 32 + 8 * g);
-            r.d[s2] = *reinterpret_cast<const uint16_t *>(m.p1 + ((size_t)row * nb + b) * 2);
+            r.q[s2] = load_at<uint2>(m.p0 + (size_t)b * 32, l.q);
+            r.d[s2] = load_at<uint16_t>(m.p1 + (size_t)b * 2, l.d);
         }
     }
     __device__ static void pre(Pre &p, const Raw &r, uint32_t ncols, uint32_t chunk, uint32_t) {
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-            p.d[s2] = chunk * 2 + s2 < ncols / 32 ? f16_bits_to_f32((uint16_t)r.d[s2]) : 0.f;
+        for (int s2 = 0; s2 < 2; ++s2) {
+            p.d[s2] = chunk * 2 + s2 < ncols / 32 ? f16_bits_to_f32((uint16_t)r.d[s2]) * kWeightScale : 0.f;
+            p.off[s2] = -128.f * p.d[s2];
+        }
     }
     template <int I>
     __device__ static float elem(const Pre &p, const Raw &r, uint32_t) {
         constexpr int s2 = I / 8, e = (I / 4) & 1, b = I & 3;
-        const uint32_t word = (e ? r.q[s2].y : r.q[s2].x) >> (8 * b);
-        return (float)(int8_t)(word & 0xffu) * p.d[s2];
+        // signed bytes with the top bit flipped are q + 128 as unsigned bytes: one byte-to-float
+        // conversion each, the 128 taken off by the multiply-add (exact: |q d| needs 8 + 11 bits)
+        const uint32_t four = opaque((e ? r.q[s2].y : r.q[s2].x) ^ 0x80808080u);
+        return fmaf(p.d[s2], (float)((four >> (8 * b)) & 0xffu), p.off[s2]);
     }
 };
 
@@ -233,7 +299,7 @@ struct AFrag {
 
 // Elements 2 P and 2 P + 1 of the 16: expanded, rounded (or split) and packed.  The high part is
 // rounded toward zero in the split form (one instruction for the pair): the low part holds what
-// is left, (w - hi) * 2^11, which is exact in fp32 before its own rounding to f16.
+// is left, w - hi, which is exact in fp32 before its own rounding to f16.
 template <class F, bool SPLIT, int P>
 __device__ __forceinline__ void frag_pair(AFrag<SPLIT> &f, const typename F::Pre &pre, const typename F::Raw &r,
                                           uint32_t g) {
@@ -244,9 +310,14 @@ __device__ __forceinline__ void frag_pair(AFrag<SPLIT> &f, const typename F::Pre
         half2v h;
         __builtin_memcpy(&h, &hz, 4);
         f.hi[s2][i] = h;
+        // l = f16(w - h) per half: one mixed-precision multiply-add each takes the f16 half of h as
+        // it is, subtracts it from the fp32 value and rounds the difference to f16
+        uint32_t hb, lb;
+        __builtin_memcpy(&hb, &h, 4);
+        asm("v_fma_mixlo_f16 %0, %1, -1.0, %2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(lb) : "v"(hb), "v"(w0));
+        asm("v_fma_mixhi_f16 %0, %1, -1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(lb) : "v"(hb), "v"(w1));
         half2v l;
-        l[0] = (_Float16)((w0 - (float)h[0]) * kSplitScale);
-        l[1] = (_Float16)((w1 - (float)h[1]) * kSplitScale);
+        __builtin_memcpy(&l, &lb, 4);
         f.lo[s2][i] = l;
     } else {
         half2v h;
@@ -276,14 +347,15 @@ __device__ __forceinline__ void frag_piece(AFrag<SPLIT> &f, typename F::Pre &pre
     }
 }
 
-// The pieces that belong to step STEP of NSTEP: piece K goes to step K * NSTEP / 9.
-template <class F, bool SPLIT, int STEP, int NSTEP, int K = 0>
+// The pieces of row block B (of RB) that belong to step STEP of NSTEP: the RB x 9 pieces of a wave
+// are spread evenly, piece K of block B goes to step (B * 9 + K) * NSTEP / (9 RB).
+template <class F, bool SPLIT, int STEP, int NSTEP, int RB, int B, int K = 0>
 __device__ __forceinline__ void frag_pieces_of_step(AFrag<SPLIT> &f, typename F::Pre &pre,
                                                     const typename F::Raw &r, uint32_t ncols, uint32_t chunk,
                                                     uint32_t g) {
     if constexpr (K < 9) {
-        if constexpr (K * NSTEP / 9 == STEP) frag_piece<F, SPLIT, K>(f, pre, r, ncols, chunk, g);
-        frag_pieces_of_step<F, SPLIT, STEP, NSTEP, K + 1>(f, pre, r, ncols, chunk, g);
+        if constexpr ((B * 9 + K) * NSTEP / (9 * RB) == STEP) frag_piece<F, SPLIT, K>(f, pre, r, ncols, chunk, g);
+        frag_pieces_of_step<F, SPLIT, STEP, NSTEP, RB, B, K + 1>(f, pre, r, ncols, chunk, g);
     }
 }
 
@@ -301,68 +373,92 @@ __device__ __forceinline__ void static_for(Fn &&fn) {
     }
 }
 
-// SPLIT: both operands are pairs of f16 numbers (high part, low part times 2^11); the product is
-// W_hi X_hi + 2^-11 (W_hi X_lo + W_lo X_hi), three MFMAs per sub-block instead of one, which
-// leaves an error of about 2^-22 per term instead of 2^-11.
+// SPLIT: both operands are pairs of f16 numbers (high part, low part); the product is
+// W_hi X_hi + W_hi X_lo + W_lo X_hi, three MFMAs per sub-block instead of one, which leaves an
+// error of about 2^-22 per term instead of 2^-11.
 //
 // The loop is software-pipelined: while the matrix cores multiply the weights of iteration it,
 // the vector ALU expands those of iteration it + 1 (fetched during iteration it - 1) -- the two
 // waves of a SIMD run in step between barriers, so the overlap has to come from inside a wave.
-template <class F, int NT, bool SPLIT>
+// RB: blocks of 16 rows per wave (a tile is 64 RB rows); every block multiplies the same LDS words.
+template <class F, int NT, bool SPLIT, int RB>
 __global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a) {
     extern __shared__ u32x4 xs[];  // [2 buffers][2 chunks][high: NT * 128 words (, low: the same)]
     constexpr uint32_t CW = NT * 128;               // words of one chunk of one part
     constexpr uint32_t CWX = SPLIT ? 2 * CW : CW;   // words of one chunk in LDS
     constexpr uint32_t NTHREADS = KWAVES * 64;
     constexpr int SW = (2 * CWX + NTHREADS - 1) / NTHREADS;  // staged words per thread
+    constexpr uint32_t TILE = 64 * RB;              // rows of a workgroup
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t j = lane & 15, g = lane >> 4;
     const uint32_t rb = wave & 3, kh = wave >> 2;
+    // Workgroup w works on part w % ks of the K range of tile w / ks.  Workgroups are handed to
+    // the eight XCDs in turn, each with an L2 cache of its own: with the part index varying
+    // fastest an XCD sees only every (8 / ks)-th part of the activations, which every tile reads
+    // again, instead of all of them.
+    const uint32_t ky = blockIdx.x % a.ks, tile = blockIdx.x / a.ks;
     // which matrix this tile belongs to (uniform over the workgroup)
     uint32_t mi = 0;
-    if (a.nmat > 1 && blockIdx.x >= a.m[1].tile0) mi = 1;
-    if (a.nmat > 2 && blockIdx.x >= a.m[2].tile0) mi = 2;
+    if (a.nmat > 1 && tile >= a.m[1].tile0) mi = 1;
+    if (a.nmat > 2 && tile >= a.m[2].tile0) mi = 2;
     const GemmMat &m = a.m[mi];
-    const uint32_t row0 = (blockIdx.x - m.tile0) * 64 + 16 * rb;
-    const uint32_t row = min(row0 + j, m.nrows - 1);  // this lane's row of the A operand
+    // a wave's RB blocks of 16 rows: blocks rb, rb + 4, .. of the tile
+    const uint32_t row0 = (tile - m.tile0) * TILE + 16 * rb;
+    typename F::Lane wl[RB];  // where this lane's rows of the A operands lie
+#pragma unroll
+    for (int b = 0; b < RB; ++b) F::lane_init(wl[b], a.ncols, min(row0 + 64 * b + j, m.nrows - 1), g);
     // K is walked in pairs of chunks (kpad is a multiple of two chunks)
     const uint32_t npairs = a.kpad / (2 * KC);
     const uint32_t per = (npairs + a.ks - 1) / a.ks;
-    const uint32_t p0 = min(blockIdx.y * per, npairs), p1 = min(npairs, p0 + per);
+    const uint32_t p0 = min(ky * per, npairs), p1 = min(npairs, p0 + per);
     const uint32_t n_it = p1 - p0;
 
-    floatx4 acc[NT], accl[SPLIT ? NT : 1];
+    floatx4 acc[RB][NT];
 #pragma unroll
-    for (int n = 0; n < NT; ++n) acc[n] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int b = 0; b < RB; ++b) {
 #pragma unroll
-    for (int n = 0; n < (SPLIT ? NT : 1); ++n) accl[n] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int n = 0; n < NT; ++n) acc[b][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
 
     // Staged words of this thread: word tid + 512 q of the pair of chunks, q < SW; in memory the
-    // low parts form a second array behind the high parts (a.xl).  All loads are unconditional:
-    // past the end the last pair is fetched again and not used.
-    const u32x4 *src[SW];
+    // low parts form a second array behind the high parts (a.xl, within 2 GiB of a.xh: the
+    // launcher checks), so one uniform base per iteration and a 32-bit offset per word address
+    // them all.  All loads are unconditional: past the end the last pair is fetched again and
+    // not used.
+    uint32_t soff[SW];  // byte offsets from the pair's first high word
 #pragma unroll
     for (int q = 0; q < SW; ++q) {
         const uint32_t w = min(tid + NTHREADS * q, 2 * CWX - 1);
         const uint32_t ch = w / CWX, ww = w % CWX;
-        src[q] = (SPLIT && ww >= CW) ? a.xl + (ch * CW + ww - CW) : a.xh + (ch * CW + ww);
+        soff[q] = (SPLIT && ww >= CW) ? a.xl_offset + (ch * CW + ww - CW) * 16 : (ch * CW + ww) * 16;
     }
     auto pair_at = [&](uint32_t it) { return min(p0 + it, npairs - 1); };  // uniform
-    u32x4 st[SW];
-    AFrag<SPLIT> A;
-    typename F::Raw rn;  // the bytes of iteration it + 1
-    if (n_it > 0) {
+    auto stage_load = [&](u32x4 (&st)[SW], uint32_t pair) {
+        const char *base = reinterpret_cast<const char *>(a.xh) + (size_t)pair * (2 * CW * 16);
 #pragma unroll
-        for (int q = 0; q < SW; ++q) st[q] = src[q][(size_t)p0 * 2 * CW];
-        typename F::Raw r0;
-        F::load(r0, m, a.ncols, row, 2 * p0 + kh, g);
-        F::load(rn, m, a.ncols, row, 2 * pair_at(1) + kh, g);
-        typename F::Pre pre0;
-        F::pre(pre0, r0, a.ncols, 2 * p0 + kh, g);
-        frag_pairs_from<F, SPLIT>(A, pre0, r0, g);
+        for (int q = 0; q < SW; ++q) st[q] = load_at<u32x4>(reinterpret_cast<const uint8_t *>(base), soff[q]);
+    };
+    u32x4 st[SW];
+    // Two sets of operands and of fetched bytes, used in turn: iteration it multiplies with
+    // A[it & 1] while it expands R[it & 1] (the bytes of iteration it + 1) into A[~it & 1] and
+    // fetches the bytes of iteration it + 2 into R[~it & 1].
+    AFrag<SPLIT> A0[RB], A1[RB];
+    typename F::Raw R0[RB], R1[RB];
+    if (n_it > 0) {
+        stage_load(st, p0);
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            typename F::Raw r0;
+            F::load(r0, m, a.ncols, wl[b], 2 * p0 + kh);
+            F::load(R0[b], m, a.ncols, wl[b], 2 * pair_at(1) + kh);
+            typename F::Pre pre0;
+            F::pre(pre0, r0, a.ncols, 2 * p0 + kh, g);
+            frag_pairs_from<F, SPLIT>(A0[b], pre0, r0, g);
+        }
     }
-    for (uint32_t it = 0; it < n_it; ++it) {
+    auto iteration = [&](uint32_t it, const AFrag<SPLIT>(&A)[RB], AFrag<SPLIT>(&An)[RB],
+                         const typename F::Raw(&rn)[RB], typename F::Raw(&rnn)[RB]) {
         u32x4 *buf = xs + (it & 1) * 2 * CWX;
 #pragma unroll
         for (int q = 0; q < SW; ++q) {
@@ -370,15 +466,14 @@ __global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a)
         }
         __syncthreads();
         const uint32_t pn = pair_at(it + 1);
+        stage_load(st, pn);
 #pragma unroll
-        for (int q = 0; q < SW; ++q) st[q] = src[q][(size_t)pn * 2 * CW];
-        typename F::Raw rnn;
-        F::load(rnn, m, a.ncols, row, 2 * pair_at(it + 2) + kh, g);
+        for (int b = 0; b < RB; ++b) F::load(rnn[b], m, a.ncols, wl[b], 2 * pair_at(it + 2) + kh);
         // The 2 NT steps of an iteration (one token block of one half chunk each): the LDS words of
-        // step + 2 are requested, the step's MFMAs issued, and a piece of the expansion of the next
-        // iteration's weights done, in this order (nothing is scheduled across a step's end).
-        AFrag<SPLIT> An;
-        typename F::Pre pre;
+        // step + 2 are requested, the step's MFMAs issued (every row block of the wave uses the same
+        // words), and a piece of the expansion of the next iteration's weights done, in this order
+        // (nothing is scheduled across a step's end).
+        typename F::Pre pre[RB];
         const uint32_t cn = 2 * pn + kh;
         const u32x4 *bsrc = buf + kh * CWX + lane;
         constexpr int NSTEP = 2 * NT, AHEAD = 2;
@@ -397,79 +492,90 @@ __global__ __launch_bounds__(KWAVES * 64) void gemm_lds_kernel(const GemmArgs a)
                 bh[slot] = bsrc[((sn % NT) * 2 + sn / NT) * 64];
                 if (SPLIT) bl[slot] = bsrc[CW + ((sn % NT) * 2 + sn / NT) * 64];
             }
-            half8 b8;
+            half8 b8, l8;
             __builtin_memcpy(&b8, &bh[cur], 16);
-            acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(A.hi[s2]), b8, acc[n], 0, 0, 0);
-            if constexpr (SPLIT) {
-                accl[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(A.lo[s2]), b8, accl[n], 0, 0, 0);
-                half8 l8;
-                __builtin_memcpy(&l8, &bl[cur], 16);
-                accl[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(A.hi[s2]), l8, accl[n], 0, 0, 0);
-            }
-            frag_pieces_of_step<F, SPLIT, step, NSTEP>(An, pre, rn, a.ncols, cn, g);
+            if constexpr (SPLIT) __builtin_memcpy(&l8, &bl[cur], 16);
+            static_for<0, RB>([&](auto b_c) {
+                constexpr int b = decltype(b_c)::value;
+                acc[b][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(A[b].hi[s2]), b8, acc[b][n], 0, 0, 0);
+                if constexpr (SPLIT) {
+                    acc[b][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(A[b].lo[s2]), b8, acc[b][n], 0, 0, 0);
+                    acc[b][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(A[b].hi[s2]), l8, acc[b][n], 0, 0, 0);
+                }
+            });
+            // pieces of this step: the RB blocks' nine pieces each, one block after the other
+            static_for<0, RB>([&](auto b_c) {
+                constexpr int b = decltype(b_c)::value;
+                frag_pieces_of_step<F, SPLIT, step, NSTEP, RB, b>(An[b], pre[b], rn[b], a.ncols, cn, g);
+            });
             __builtin_amdgcn_sched_barrier(0);
         });
-        A = An;
-        rn = rnn;
-    }
-    if (SPLIT) {
-#pragma unroll
-        for (int n = 0; n < NT; ++n) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[n][i] = fmaf(accl[n][i], 1.0f / kSplitScale, acc[n][i]);
-        }
+    };
+    for (uint32_t it = 0; it < n_it; it += 2) {
+        iteration(it, A0, A1, R0, R1);
+        if (it + 1 < n_it) iteration(it + 1, A1, A0, R1, R0);
     }
     // waves 4-7 hand their sums to waves 0-3 through LDS
     __syncthreads();
-    float4 *red = reinterpret_cast<float4 *>(xs);  // [4 row blocks][NT][64]
+    float4 *red = reinterpret_cast<float4 *>(xs);  // [RB][4 row blocks][NT][64]
     if (kh == 1) {
 #pragma unroll
-        for (int n = 0; n < NT; ++n)
-            red[(rb * NT + n) * 64 + lane] = make_float4(acc[n][0], acc[n][1], acc[n][2], acc[n][3]);
+        for (int b = 0; b < RB; ++b) {
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+                red[((b * 4 + rb) * NT + n) * 64 + lane] =
+                    make_float4(acc[b][n][0], acc[b][n][1], acc[b][n][2], acc[b][n][3]);
+        }
     }
     __syncthreads();
     if (kh == 1) return;
-    const uint32_t r4 = row0 + 4 * g;  // acc[n] = rows r4 .. r4 + 3 of token 16 n + j
 #pragma unroll
-    for (int n = 0; n < NT; ++n) {
-        const float4 p = red[(rb * NT + n) * 64 + lane];
-        float4 v = make_float4(acc[n][0] + p.x, acc[n][1] + p.y, acc[n][2] + p.z, acc[n][3] + p.w);
-        const uint32_t tok = n * 16 + j;
-        if (tok >= a.T || r4 >= m.nrows) continue;
-        float *o;
-        bool add = false;
-        if (a.ks > 1) {
-            // plain partial sum
-            o = a.part + ((size_t)blockIdx.y * a.T + tok) * a.total_rows + m.roff + r4;
-        } else {
-            const float xs_t = a.xscale ? a.xscale[tok] : 1.f;
-            v = make_float4(v.x * xs_t, v.y * xs_t, v.z * xs_t, v.w * xs_t);
-            if (m.bias) {
-                if (r4 + 3 < m.nrows) {
-                    v.x += m.bias[r4];
-                    v.y += m.bias[r4 + 1];
-                    v.z += m.bias[r4 + 2];
-                    v.w += m.bias[r4 + 3];
-                } else {
-                    v.x += m.bias[r4];
-                    if (r4 + 1 < m.nrows) v.y += m.bias[r4 + 1];
-                    if (r4 + 2 < m.nrows) v.z += m.bias[r4 + 2];
+    for (int b = 0; b < RB; ++b) {
+        const uint32_t r4 = row0 + 64 * b + 4 * g;  // acc[b][n] = rows r4 .. r4 + 3 of token 16 n + j
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+            const float4 p = red[((b * 4 + rb) * NT + n) * 64 + lane];
+            // the sums carry the factor the weights were expanded with: an exact scaling back
+            constexpr float u = 1.0f / kWeightScale;
+            float4 v = make_float4((acc[b][n][0] + p.x) * u, (acc[b][n][1] + p.y) * u, (acc[b][n][2] + p.z) * u,
+                                   (acc[b][n][3] + p.w) * u);
+            const uint32_t tok = n * 16 + j;
+            if (tok >= a.T || r4 >= m.nrows) continue;
+            float *o;
+            bool add = false;
+            if (a.ks > 1) {
+                // plain partial sum
+                o = a.part + ((size_t)ky * a.T + tok) * a.total_rows + m.roff + r4;
+            } else {
+                const float xs_t = a.xscale ? a.xscale[tok] : 1.f;
+                v = make_float4(v.x * xs_t, v.y * xs_t, v.z * xs_t, v.w * xs_t);
+                if (m.bias) {
+                    if (r4 + 3 < m.nrows) {
+                        v.x += m.bias[r4];
+                        v.y += m.bias[r4 + 1];
+                        v.z += m.bias[r4 + 2];
+                        v.w += m.bias[r4 + 3];
+                    } else {
+                        v.x += m.bias[r4];
+                        if (r4 + 1 < m.nrows) v.y += m.bias[r4 + 1];
+                        if (r4 + 2 < m.nrows) v.z += m.bias[r4 + 2];
+                    }
                 }
+                o = m.out + (size_t)tok * m.out_stride + r4;
+                add = a.accumulate != 0;
             }
-            o = m.out + (size_t)tok * m.out_stride + r4;
-            add = a.accumulate != 0;
-        }
-        if (r4 + 3 < m.nrows && (reinterpret_cast<uintptr_t>(o) & 15u) == 0) {
-            if (add) {
-                const float4 q = *reinterpret_cast<const float4 *>(o);
-                v = make_float4(q.x + v.x, q.y + v.y, q.z + v.z, q.w + v.w);
+            if (r4 + 3 < m.nrows && (reinterpret_cast<uintptr_t>(o) & 15u) == 0) {
+                if (add) {
+                    const float4 q = *reinterpret_cast<const float4 *>(o);
+                    v = make_float4(q.x + v.x, q.y + v.y, q.z + v.z, q.w + v.w);
+                }
+                *reinterpret_cast<float4 *>(o) = v;
+            } else {
+                o[0] = add ? o[0] + v.x : v.x;
+                if (r4 + 1 < m.nrows) o[1] = add ? o[1] + v.y : v.y;
+                if (r4 + 2 < m.nrows) o[2] = add ? o[2] + v.z : v.z;
+                if (r4 + 3 < m.nrows) o[3] = add ? o[3] + v.w : v.w;
             }
-            *reinterpret_cast<float4 *>(o) = v;
-        } else {
-            o[0] = add ? o[0] + v.x : v.x;
-            if (r4 + 1 < m.nrows) o[1] = add ? o[1] + v.y : v.y;
-            if (r4 + 2 < m.nrows) o[2] = add ? o[2] + v.z : v.z;
-            if (r4 + 3 < m.nrows) o[3] = add ? o[3] + v.w : v.w;
         }
     }
 }
@@ -494,8 +600,8 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmArgs a) {
 
 // One workgroup per token: X[t] (fp32, optionally RMS-normalised with weights w as
 // the reference does: (x * rsqrt(mean(x^2) + eps)) * w, ops/rms_norm.rs:55-63) -> f16
-// in the packed order described at the top, divided by a power of two if needed so that
-// |x| <= 1024; the factor to undo it goes to xscale[t].  Tokens from T on and columns
+// in the packed order described at the top, times the power of two that brings the row's
+// largest |x| into (512, 1024]; the factor to undo it goes to xscale[t].  Tokens from T on and columns
 // from K on are zero.  With `up` non-null the input is the gated activation
 // up[k] * silu(x[k]) (ops/silu.wgsl:13-27) instead of x itself (no normalisation then).
 constexpr int PREP_THREADS = 1024;
@@ -647,14 +753,18 @@ __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict_
         down *= 0.5f;
         undo *= 2.f;
     }
-    // high parts f16(v); low parts f16((v - high) * 2^11) when the split-precision product is on
+    for (int it = 0; it < 100 && amax > 0.f && amax * down <= 512.f; ++it) {
+        down *= 2.f;
+        undo *= 0.5f;
+    }
+    // high parts f16(v); low parts f16(v - high) when the split-precision product is on
     auto store = [&](uint32_t k8, const float(&f)[8]) {
         _Float16 h[8], lo[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const float v = f[e] * down;
             h[e] = (_Float16)v;
-            lo[e] = (_Float16)((v - (float)h[e]) * kSplitScale);
+            lo[e] = (_Float16)(v - (float)h[e]);
         }
         uint4 w;
         __builtin_memcpy(&w, h, 16);
@@ -975,30 +1085,31 @@ uint32_t gemm_k_split(const wgml_ctx *ctx, uint32_t tiles, uint32_t kpad, bool s
     return best;
 }
 
-template <class F, int NT, bool SPLIT>
+template <class F, int NT, bool SPLIT, int RB>
 int launch_gemm_kernel(wgml_ctx *ctx, const GemmArgs &a, dim3 grid) {
-    const size_t lds = (size_t)NT * 8192 * (SPLIT ? 2 : 1);  // 2 buffers x 2 chunks x NT x 2 KiB (x 2 parts)
-    wgml_kernel_info &ki = ctx->kernel_info[(const void *)gemm_lds_kernel<F, NT, SPLIT>];
+    // 2 buffers x 2 chunks x NT x 2 KiB (x 2 parts); the sums handed over at the end need RB x NT x 4 KiB
+    const size_t lds = max((size_t)NT * 8192 * (SPLIT ? 2 : 1), (size_t)RB * NT * 4096);
+    wgml_kernel_info &ki = ctx->kernel_info[(const void *)gemm_lds_kernel<F, NT, SPLIT, RB>];
     if (lds > 64 * 1024 && !ki.opted_in) {
         // gfx950 has 160 KB of LDS per CU; above 64 KB a kernel must opt in once
-        WGML_CHECK_HIP(hipFuncSetAttribute((const void *)gemm_lds_kernel<F, NT, SPLIT>,
+        WGML_CHECK_HIP(hipFuncSetAttribute((const void *)gemm_lds_kernel<F, NT, SPLIT, RB>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         ki.opted_in = true;
     }
-    gemm_lds_kernel<F, NT, SPLIT><<<grid, dim3(KWAVES * 64), lds, ctx->stream>>>(a);
+    gemm_lds_kernel<F, NT, SPLIT, RB><<<grid, dim3(KWAVES * 64), lds, ctx->stream>>>(a);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
 }
 
-template <class F, bool SPLIT>
+template <class F, bool SPLIT, int RB>
 int launch_gemm_prec(wgml_ctx *ctx, GemmArgs &a, uint32_t tiles) {
-    const dim3 grid(tiles, a.ks);
+    const dim3 grid(tiles * a.ks);
     switch (a.tpad / 16) {  // token blocks: 1, 2, 4 or 8
-    case 8: WGML_TRY((launch_gemm_kernel<F, 8, SPLIT>(ctx, a, grid))); break;
-    case 4: WGML_TRY((launch_gemm_kernel<F, 4, SPLIT>(ctx, a, grid))); break;
-    case 2: WGML_TRY((launch_gemm_kernel<F, 2, SPLIT>(ctx, a, grid))); break;
-    default: WGML_TRY((launch_gemm_kernel<F, 1, SPLIT>(ctx, a, grid))); break;
+    case 8: WGML_TRY((launch_gemm_kernel<F, 8, SPLIT, RB>(ctx, a, grid))); break;
+    case 4: WGML_TRY((launch_gemm_kernel<F, 4, SPLIT, RB>(ctx, a, grid))); break;
+    case 2: WGML_TRY((launch_gemm_kernel<F, 2, SPLIT, RB>(ctx, a, grid))); break;
+    default: WGML_TRY((launch_gemm_kernel<F, 1, SPLIT, RB>(ctx, a, grid))); break;
     }
     if (a.ks > 1 && !a.defer) {
         gemm_reduce_kernel<<<dim3((a.total_rows + 255) / 256, a.T), dim3(256), 0, ctx->stream>>>(a);
@@ -1010,7 +1121,9 @@ int launch_gemm_prec(wgml_ctx *ctx, GemmArgs &a, uint32_t tiles) {
 
 template <class F>
 int launch_gemm_fmt(wgml_ctx *ctx, GemmArgs &a, uint32_t tiles) {
-    return a.xl ? launch_gemm_prec<F, true>(ctx, a, tiles) : launch_gemm_prec<F, false>(ctx, a, tiles);
+    // one block of 16 rows per wave: two (tiles of 128 rows, half the LDS reads per MFMA) ran each
+    // iteration 20 % faster per row but filled the compute units worse, no gain over a prompt pass
+    return a.xl ? launch_gemm_prec<F, true, 1>(ctx, a, tiles) : launch_gemm_prec<F, false, 1>(ctx, a, tiles);
 }
 
 }  // namespace
@@ -1122,6 +1235,13 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
     a.nmat = (uint32_t)n;
     a.xh = reinterpret_cast<const u32x4 *>(xh);
     a.xl = ctx->gemm_precise ? reinterpret_cast<const u32x4 *>(ctx->prefill_xl) : nullptr;
+    if (a.xl) {
+        // the kernel addresses the low parts relative to the high parts with 32 bits
+        const ptrdiff_t d = reinterpret_cast<const char *>(a.xl) - reinterpret_cast<const char *>(a.xh);
+        if (d <= 0 || d >= (ptrdiff_t(1) << 31))
+            return set_error(WGML_E_INVALID, "gemm_quant: the activations are not the context's packed buffer");
+        a.xl_offset = (uint32_t)d;
+    }
     a.xscale = xscale;
     a.ncols = first->ncols;
     a.kpad = prefill_kpad(first->ncols);
