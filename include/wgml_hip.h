@@ -155,8 +155,10 @@ WGML_API int wgml_gemv_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, w
  * cores pairs of f16 numbers per operand (high part + low part), three MFMAs per
  * product term group, fp32 sums: results agree with n_tokens calls of
  * wgml_gemv_quant to fp32 rounding (about 1e-6 of a row's magnitude).  Level 0 rounds
- * weights and vectors to f16 once: 1.6x faster, about 3e-4 of a row's magnitude
- * (up to 1.4e-3 for single elements).  m must be WGML_Q8_0, WGML_Q4_K or WGML_Q6_K. */
+ * weights and vectors to f16 once: 1.4x faster, about 3e-4 of a row's magnitude
+ * (up to 1.4e-3 for single elements).  m must be WGML_Q8_0, WGML_Q4_K or WGML_Q6_K.
+ * Vectors of any magnitude are taken (scaled per vector by a power of two); the
+ * dequantized weights must be below 256 in magnitude (they pass through f16 times 2^8). */
 WGML_API int wgml_ctx_set_gemm_precision(wgml_ctx *ctx, int level);
 WGML_API int wgml_gemm_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, wgml_view x,
                              uint32_t n_tokens);

