@@ -162,3 +162,10 @@ def test_argmax_first_maximum(gpu):  # models/sampler.rs:54-56
     v[[123, 45000, 69999]] = 7.0  # ties: the first index wins
     assert s.sample_argmax(vec(gpu, v)) == 123
     assert s.sample_argmax(vec(gpu, np.full(3000, -np.inf, dtype=np.float32))) == 0
+    # sub-views that do not start on a 16-byte boundary, every length down to one element
+    v = rnd(9000, 5)
+    whole = vec(gpu, v)
+    for start, count in ((1, 8999), (2, 8000), (3, 4097), (1, 3), (3, 2), (2, 1), (5, 70)):
+        assert s.sample_argmax(whole.rows(start, count)) == orc.argmax(v[start:start + count])
+    v[1] = v[4000] = v[8999] = 99.0  # a tie between the unaligned head, the middle and the tail
+    assert s.sample_argmax(vec(gpu, v).rows(1, 8999)) == 0
