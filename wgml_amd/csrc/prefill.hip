@@ -1218,6 +1218,10 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
         const wgml_qmat *q = targets[i].m;
         if (q->type != first->type || q->ncols != first->ncols)
             return set_error(WGML_E_INVALID, "gemm_quant: matrices of one launch differ in format or width");
+        // the kernel addresses a matrix plane with 32-bit lane offsets (at most 1 byte per element)
+        if ((uint64_t)q->nrows * q->ncols >= (uint64_t(1) << 32) - 4096)
+            return set_error(WGML_E_UNSUPPORTED, "gemm_quant: a matrix of %u x %u elements (below 2^32 only)",
+                             q->nrows, q->ncols);
         GemmMat &g = a.m[i];
         g.p0 = q->p0;
         g.p1 = q->p1;
