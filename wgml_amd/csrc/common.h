@@ -285,12 +285,24 @@ struct GemmTarget {
     float *out;
     uint32_t out_stride;
     const float *bias;
+    bool rope = false;  // rotate the rows of this product (see GemmRope)
+};
+// Rotary position encoding of the targets marked `rope`, applied by the kernel that adds up the
+// partial sums of a K-split product (the rows of a pair meet there anyway): token t sits at
+// position pos0 + t.  `applied` tells the caller whether it happened (not when K was not split
+// or a target has an odd number of rows: launch_rope_rows then).
+struct GemmRope {
+    int variant;  // WGML_ROPE_ORIGINAL or WGML_ROPE_NEOX
+    uint32_t head_size, pos0;
+    float base_freq;
+    bool applied;
 };
 int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, const void *xh,
                             const float *xscale, uint32_t T, int accumulate,
-                            bool defer_reduce = false);
+                            bool defer_reduce = false, GemmRope *rope = nullptr);
 int launch_embed_rows(wgml_ctx *ctx, float *x, const float *table, const uint32_t *d_tokens,
                       uint32_t dim, uint32_t T);
+// q (q_len wide) and k (kv_dim wide) of T tokens rotated in place; either may be null
 int launch_rope_rows(wgml_ctx *ctx, int variant, uint32_t head_size, uint32_t kv_dim, uint32_t pos0,
                      float base_freq, float *q, uint32_t q_len, uint32_t q_stride, float *k,
                      uint32_t k_stride, uint32_t T);

@@ -403,27 +403,35 @@ int enqueue_prefill_run(wgml_llama2 *m, const uint32_t *tokens, uint32_t T, uint
         WGML_TRY(launch_prefill_prep(ctx, m->pf_x, dim, nullptr, w.attn_norm, c.rms_norm_eps, xh, xs,
                                      dim, T));
         // Q, K and V in as few launches as their formats allow (one launch takes matrices
-        // of one format); K and V go straight to their cache rows
+        // of one format); K and V go straight to their cache rows.  Q and K are rotated by the
+        // kernel that adds up the partial sums of their launch where there is one, by a launch
+        // of their own otherwise.
+        bool roped[3] = {false, false, true};
         {
-            const GemmTarget tq{w.attn_q, m->pf_q, dim, w.bq}, tk{w.attn_k, kc, kv_dim, w.bk},
+            GemmTarget tq{w.attn_q, m->pf_q, dim, w.bq}, tk{w.attn_k, kc, kv_dim, w.bk},
                 tv{w.attn_v, vc, kv_dim, w.bv};
+            tq.rope = tk.rope = true;
             GemmTarget group[3] = {tq, tk, tv};
             bool done[3] = {false, false, false};
             for (int i = 0; i < 3; ++i) {
                 if (done[i]) continue;
                 GemmTarget launch[3];
-                int n = 0;
+                int n = 0, members[3];
                 for (int k = i; k < 3; ++k) {
                     if (!done[k] && group[k].m->type == group[i].m->type) {
+                        members[n] = k;
                         launch[n++] = group[k];
                         done[k] = true;
                     }
                 }
-                WGML_TRY(launch_gemm_quant_multi(ctx, launch, n, xh, xs, T, 0));
+                GemmRope rope{variant, m->head_size, pos0, c.rope_base_freq, false};
+                WGML_TRY(launch_gemm_quant_multi(ctx, launch, n, xh, xs, T, 0, false, &rope));
+                for (int k = 0; k < n; ++k) roped[members[k]] = roped[members[k]] || rope.applied;
             }
         }
-        WGML_TRY(launch_rope_rows(ctx, variant, m->head_size, kv_dim, pos0, c.rope_base_freq,
-                                  m->pf_q, dim, dim, kc, kv_dim, T));
+        if (!roped[0] || !roped[1])
+            WGML_TRY(launch_rope_rows(ctx, variant, m->head_size, kv_dim, pos0, c.rope_base_freq,
+                                      roped[0] ? nullptr : m->pf_q, dim, dim, roped[1] ? nullptr : kc, kv_dim, T));
         WGML_TRY(launch_attention_rows(ctx, ap, pos0, T, m->pf_q, dim, w.key_cache, w.value_cache,
                                        m->pf_xb, dim));
         WGML_TRY(launch_prefill_prep(ctx, m->pf_xb, dim, nullptr, nullptr, 0.f, xh, xs, dim, T));

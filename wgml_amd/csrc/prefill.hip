@@ -81,6 +81,7 @@ struct GemmMat {
     uint32_t nrows, out_stride;
     uint32_t tile0;                    // first 64-row tile of this matrix in grid.x
     uint32_t roff;                     // rows of the matrices before this one in the launch
+    uint32_t rope;                     // the reduction rotates this matrix' rows (GemmArgs::rope_*)
 };
 
 struct GemmArgs {
@@ -96,6 +97,10 @@ struct GemmArgs {
     uint32_t ks;                       // ways K is split between workgroups (grid.y)
     uint32_t total_rows;               // rows of all matrices of the launch
     int defer;                         // ks > 1: leave the partial sums to the next kernel
+    // rotary encoding applied by gemm_reduce_rope_kernel to the matrices marked `rope`
+    uint32_t rope_head_size, rope_pos0;
+    float rope_base;
+    int rope_neox;
 };
 
 __device__ __forceinline__ half4 to_half4(float a, float b, float c, float d) {
@@ -598,6 +603,52 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmArgs a) {
     *o = a.accumulate ? *o + v : v;
 }
 
+// The same for pairs of rows, with the rotary position encoding of the matrices marked for it
+// (ops/rope.wgsl:35-78, the arithmetic of rope_rows_kernel below): thread (i, t) adds up the two
+// rows of pair i of token t -- rows 2 i and 2 i + 1, or i' and i' + head_size / 2 within a head
+// in the Neox variant -- and rotates them by the angle of position pos0 + t.  Every matrix of
+// the launch has an even number of rows; nothing is accumulated onto the output.
+__global__ __launch_bounds__(256) void gemm_reduce_rope_kernel(const GemmArgs a) {
+    const uint32_t pg = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;  // pair among all matrices
+    if (2 * pg >= a.total_rows) return;
+    uint32_t mi = 0;
+    if (a.nmat > 1 && 2 * pg >= a.m[1].roff) mi = 1;
+    if (a.nmat > 2 && 2 * pg >= a.m[2].roff) mi = 2;
+    const GemmMat &m = a.m[mi];
+    const uint32_t i = pg - m.roff / 2, hs = a.rope_head_size;
+    uint32_t ra = 2 * i, rb = 2 * i + 1;
+    if (m.rope && a.rope_neox) {
+        ra = i + (2 * i / hs) * (hs / 2);
+        rb = ra + hs / 2;
+    }
+    const float *pa = a.part + (size_t)t * a.total_rows + m.roff + ra;
+    const float *pb = a.part + (size_t)t * a.total_rows + m.roff + rb;
+    float x = pa[0], y = pb[0];
+    for (uint32_t k = 1; k < a.ks; ++k) {
+        x += pa[(size_t)k * a.T * a.total_rows];
+        y += pb[(size_t)k * a.T * a.total_rows];
+    }
+    const float xs_t = a.xscale ? a.xscale[t] : 1.f;
+    x *= xs_t;
+    y *= xs_t;
+    if (m.bias) {
+        x += m.bias[ra];
+        y += m.bias[rb];
+    }
+    float *o = m.out + (size_t)t * m.out_stride;
+    if (m.rope) {
+        const float head_dim = (float)((i * 2) % hs);
+        const float theta = powf(a.rope_base, -head_dim / (float)hs);
+        float sn, cs;
+        sincosf((float)(a.rope_pos0 + t) * theta, &sn, &cs);
+        o[ra] = cs * x - sn * y;
+        o[rb] = sn * x + cs * y;
+    } else {
+        o[ra] = x;
+        o[rb] = y;
+    }
+}
+
 // One workgroup per token: X[t] (fp32, optionally RMS-normalised with weights w as
 // the reference does: (x * rsqrt(mean(x^2) + eps)) * w, ops/rms_norm.rs:55-63) -> f16
 // in the packed order described at the top, times the power of two that brings the row's
@@ -820,12 +871,12 @@ __global__ void rope_rows_kernel(float *__restrict__ q, uint32_t q_stride, float
         a = i + head_id * head_size / 2;
         b = a + head_size / 2;
     }
-    {
+    if (q) {
         const float x = qt[a], y = qt[b];
         qt[a] = cs * x - sn * y;
         qt[b] = sn * x + cs * y;
     }
-    if (i * 2 < kv_dim) {
+    if (k && i * 2 < kv_dim) {
         const float x = kt[a], y = kt[b];
         kt[a] = cs * x - sn * y;
         kt[b] = sn * x + cs * y;
@@ -1112,7 +1163,10 @@ int launch_gemm_prec(wgml_ctx *ctx, GemmArgs &a, uint32_t tiles) {
     default: WGML_TRY((launch_gemm_kernel<F, 1, SPLIT, RB>(ctx, a, grid))); break;
     }
     if (a.ks > 1 && !a.defer) {
-        gemm_reduce_kernel<<<dim3((a.total_rows + 255) / 256, a.T), dim3(256), 0, ctx->stream>>>(a);
+        if (a.rope_head_size)
+            gemm_reduce_rope_kernel<<<dim3((a.total_rows / 2 + 255) / 256, a.T), dim3(256), 0, ctx->stream>>>(a);
+        else
+            gemm_reduce_kernel<<<dim3((a.total_rows + 255) / 256, a.T), dim3(256), 0, ctx->stream>>>(a);
         WGML_CHECK_LAUNCH();
         ctx->launches++;
     }
@@ -1207,7 +1261,8 @@ int ensure_gemm_partials(wgml_ctx *ctx, size_t bytes) {
 }
 
 int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, const void *xh,
-                            const float *xscale, uint32_t T, int accumulate, bool defer_reduce) {
+                            const float *xscale, uint32_t T, int accumulate, bool defer_reduce,
+                            GemmRope *rope) {
     if (T == 0 || T > kPrefillMaxTokens)
         return set_error(WGML_E_INVALID, "gemm_quant: %u tokens (1..%u)", T, kPrefillMaxTokens);
     if (n < 1 || n > 3) return set_error(WGML_E_INVALID, "gemm_quant: %d matrices (1..3)", n);
@@ -1230,6 +1285,7 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
         g.out = targets[i].out;
         g.bias = targets[i].bias;
         g.nrows = q->nrows;
+        g.rope = targets[i].rope ? 1u : 0u;
         g.out_stride = targets[i].out_stride;
         g.tile0 = tiles;
         g.roff = a.total_rows;
@@ -1269,6 +1325,21 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
         if (a.defer) {
             ctx->gemm_pending_ks = a.ks;
             ctx->gemm_pending_pair = pair ? 1 : 0;
+        }
+    }
+    if (rope) {
+        // the kernel that adds the partial sums rotates the marked targets, if there is one and
+        // rows come in pairs
+        bool pairs = a.ks > 1 && !a.defer && !accumulate && rope->head_size >= 2 && rope->head_size % 2 == 0;
+        for (int i = 0; i < n; ++i)
+            pairs = pairs && targets[i].m->nrows % 2 == 0 &&
+                    (!targets[i].rope || targets[i].m->nrows % rope->head_size == 0);
+        rope->applied = pairs;
+        if (pairs) {
+            a.rope_head_size = rope->head_size;
+            a.rope_pos0 = rope->pos0;
+            a.rope_base = rope->base_freq;
+            a.rope_neox = rope->variant == WGML_ROPE_NEOX;
         }
     }
     switch (first->type) {
