@@ -655,6 +655,47 @@ __global__ __launch_bounds__(256) void gemm_reduce_rope_kernel(const GemmArgs a)
 // largest |x| into (512, 1024]; the factor to undo it goes to xscale[t].  Tokens from T on and columns
 // from K on are zero.  With `up` non-null the input is the gated activation
 // up[k] * silu(x[k]) (ops/silu.wgsl:13-27) instead of x itself (no normalisation then).
+// acc[n][0..7] += part[y .. y + B - 1][off[n] .. off[n] + 7], part by part in the order of y; the
+// loads of all B parts are requested before the first sum (a chain of memory round trips
+// otherwise).  ystride: floats from one part to the next.
+template <int B, int N>
+__device__ __forceinline__ void add_part_batch(float (&acc)[N][8], const float *__restrict__ part, size_t ystride,
+                                               const size_t (&off)[N], uint32_t y) {
+    float4 q[B][N][2];
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+#pragma unroll
+        for (int n = 0; n < N; ++n) {
+            const float4 *p = reinterpret_cast<const float4 *>(part + (size_t)(y + b) * ystride + off[n]);
+            q[b][n][0] = p[0];
+            q[b][n][1] = p[1];
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+#pragma unroll
+        for (int n = 0; n < N; ++n) {
+            acc[n][0] += q[b][n][0].x;
+            acc[n][1] += q[b][n][0].y;
+            acc[n][2] += q[b][n][0].z;
+            acc[n][3] += q[b][n][0].w;
+            acc[n][4] += q[b][n][1].x;
+            acc[n][5] += q[b][n][1].y;
+            acc[n][6] += q[b][n][1].z;
+            acc[n][7] += q[b][n][1].w;
+        }
+    }
+}
+// all ks parts, four, two or one at a time
+template <int N>
+__device__ __forceinline__ void add_parts(float (&acc)[N][8], const float *__restrict__ part, size_t ystride,
+                                          const size_t (&off)[N], uint32_t ks) {
+    uint32_t y = 0;
+    for (; y + 4 <= ks; y += 4) add_part_batch<4, N>(acc, part, ystride, off, y);
+    for (; y + 2 <= ks; y += 2) add_part_batch<2, N>(acc, part, ystride, off, y);
+    for (; y < ks; ++y) add_part_batch<1, N>(acc, part, ystride, off, y);
+}
+
 constexpr int PREP_THREADS = 1024;
 constexpr int PREP_GROUPS = 2;  // groups of 8 columns a thread keeps in registers
 __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict__ x, uint32_t x_stride,
@@ -718,40 +759,25 @@ __global__ __launch_bounds__(PREP_THREADS) void prep_x_kernel(float *__restrict_
             for (int e = 0; e < 8; ++e) v[i][e] = 0.f;
             if (k0 < K && part_ks && part_pair) {
                 const size_t wide = 2 * (size_t)K;
-                float g8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, u8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                for (uint32_t y = 0; y < part_ks; ++y) {
-                    const float4 *pg = reinterpret_cast<const float4 *>(part + ((size_t)y * T + t) * wide + k0);
-                    const float4 *pu = reinterpret_cast<const float4 *>(part + ((size_t)y * T + t) * wide + K + k0);
-                    const float4 g0 = pg[0], g1 = pg[1], u0 = pu[0], u1 = pu[1];
-                    const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
-                    const float uv[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        g8[e] += gv[e];
-                        u8[e] += uv[e];
-                    }
-                }
+                float gu[2][8] = {};  // sums of the gate parts and of the up parts
+                const size_t off[2] = {(size_t)t * wide + k0, (size_t)t * wide + K + k0};
+                add_parts<2>(gu, part, (size_t)T * wide, off, part_ks);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    const float xv = g8[e] * old_scale;
-                    v[i][e] = (u8[e] * old_scale) * (xv / (1.0f + expf(-xv)));
+                    const float xv = gu[0][e] * old_scale;
+                    v[i][e] = (gu[1][e] * old_scale) * (xv / (1.0f + expf(-xv)));
                 }
             } else if (k0 < K) {
                 float4 *xp = reinterpret_cast<float4 *>(xr + k0);
                 float4 a0 = xp[0], a1 = xp[1];
                 if (part_ks) {
-                    const float4 *pp = reinterpret_cast<const float4 *>(part + (size_t)t * K + k0);
-                    float4 s0 = pp[0], s1 = pp[1];
-                    for (uint32_t y = 1; y < part_ks; ++y) {
-                        const float4 *py = reinterpret_cast<const float4 *>(part + ((size_t)y * T + t) * K + k0);
-                        const float4 q0 = py[0], q1 = py[1];
-                        s0 = make_float4(s0.x + q0.x, s0.y + q0.y, s0.z + q0.z, s0.w + q0.w);
-                        s1 = make_float4(s1.x + q1.x, s1.y + q1.y, s1.z + q1.z, s1.w + q1.w);
-                    }
-                    a0 = make_float4(a0.x + s0.x * old_scale, a0.y + s0.y * old_scale,
-                                     a0.z + s0.z * old_scale, a0.w + s0.w * old_scale);
-                    a1 = make_float4(a1.x + s1.x * old_scale, a1.y + s1.y * old_scale,
-                                     a1.z + s1.z * old_scale, a1.w + s1.w * old_scale);
+                    float sp[1][8] = {};
+                    const size_t off[1] = {(size_t)t * K + k0};
+                    add_parts<1>(sp, part, (size_t)T * K, off, part_ks);
+                    a0 = make_float4(a0.x + sp[0][0] * old_scale, a0.y + sp[0][1] * old_scale,
+                                     a0.z + sp[0][2] * old_scale, a0.w + sp[0][3] * old_scale);
+                    a1 = make_float4(a1.x + sp[0][4] * old_scale, a1.y + sp[0][5] * old_scale,
+                                     a1.z + sp[0][6] * old_scale, a1.w + sp[0][7] * old_scale);
                     xp[0] = a0;
                     xp[1] = a1;
                 }
