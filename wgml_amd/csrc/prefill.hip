@@ -260,8 +260,6 @@ struct GemmQ8_0 {
     struct Pre {
         float d[2], off[2];  // per s2: d, -128 d
     };
-    // rows are a multiple of 32 elements long: a 32-element block of the (padded) K range may
-    // not exist; the last one is then read in its place and expanded to zeros
     struct Lane {
         uint32_t q, d;
     };
@@ -269,6 +267,8 @@ struct GemmQ8_0 {
         l.q = row * ncols + 8 * g;
         l.d = row * (ncols / 32) * 2;
     }
+    // rows are a multiple of 32 elements long: a 32-element block of the (padded) K range may
+    // not exist; the last one is then read in its place and expanded to zeros
     __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, const Lane &l, uint32_t chunk) {
         const uint32_t b0 = chunk * 2, nb = ncols / 32;
 #pragma unroll
