@@ -124,6 +124,42 @@ def time_gate_up(W, gpu, cfg, weights):
     return best, nbytes
 
 
+READ_CHAIN_ROWS = (4096, 11008, 22016, 46400)  # 9.4 / 25.4 / 50.7 / 106.9 MB per launch
+
+
+def read_chain(gpu, use_graph=True):
+    """The machine's own ceiling for a chain of launches: a kernel that only reads, with the
+    Q4_K GEMV's access pattern (wgml_bench_read_chain), at four sizes.  A least-squares line
+    through time per launch against bytes gives what a launch boundary costs (intercept) and
+    what loads sustain (1 / slope)."""
+    from wgml_amd._lib import call
+
+    pts = []
+    ms = C.c_float()
+    for nrows in READ_CHAIN_ROWS:
+        nbytes = nrows * 2304
+        iters = max(64, min(600, (3 << 30) // nbytes))
+        best = None
+        for _ in range(3):
+            call("wgml_bench_read_chain", gpu.handle, nrows, iters, 1 if use_graph else 0, C.byref(ms))
+            us = ms.value * 1e3 / iters
+            best = us if best is None else min(best, us)
+        pts.append((nbytes, best))
+    n = len(pts)
+    sx = sum(b for b, _ in pts)
+    sy = sum(t for _, t in pts)
+    sxx = sum(b * b for b, _ in pts)
+    sxy = sum(b * t for b, t in pts)
+    slope = (n * sxy - sx * sy) / (n * sxx - sx * sx)  # us per byte
+    icpt = (sy - slope * sx) / n
+    return {"points": [{"bytes": b, "us_per_launch": round(t, 3), "GB/s": round(b / t * 1e-3, 1)}
+                       for b, t in pts],
+            "GB/s": round(1e-3 / slope, 1), "launch_overhead_us": round(icpt, 3),
+            "how": "bare read kernel with the Q4_K GEMV's access pattern, one launch after the other "
+                   + ("in a recorded graph" if use_graph else "launch by launch")
+                   + ", rotating over a 1.5 GB pool; line through us per launch against bytes"}
+
+
 def gemv_sweep(W, gpu, nrows, ncols, cpu_threads, min_total_bytes=640 << 20, formats=None):
     """One matrix shape for Q8_0 / Q4_K / Q6_K: GB/s and fraction of HBM peak on the GPU (the
     default integer-dot kernels and the fp32-activation kernels), and the CPU oracle's
@@ -201,6 +237,56 @@ def cpu_baseline(weights, prompt, n_steps, threads_all):
                             "sample": "the same steps, rows of every matrix-vector product shared "
                                       "out over the host cores (OpenMP); identical results"}
     return out, logits
+
+
+def parity_at_timed_positions(W, gpu, model, weights, prompt, generated, first, p0, warmup, steps, cores):
+    """The GPU step against the CPU oracle at positions the timed region covers.  The oracle
+    (all host cores; same sums for any thread count) is fed the prompt and then the tokens the
+    GPU chose, so both sides see the same context; its logits at up to four timed positions
+    (the first two, one a little later, and the last one within a budget of 40 decode
+    positions) are compared with the GPU's step at those positions, for the default
+    integer-dot step and for the step with fp32 activations in every GEMV."""
+    import numpy as np
+
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle as orc
+
+    seq = np.concatenate([np.asarray(prompt, dtype=np.int64), [first], np.asarray(generated, dtype=np.int64)])
+    # seq[pos] = the token fed at position pos
+    t_first = p0 + warmup
+    t_last = min(t_first + steps - 1, p0 + 39)
+    cand = sorted({t_first, min(t_first + 1, t_last), min(t_first + 7, t_last), t_last})
+    cand = [c for c in cand if c >= t_first]
+    orc.set_threads(cores)
+    t0 = time.perf_counter()
+    ref = orc.Llama2(weights, predequantize=True)
+    want = {}
+    for pos in range(cand[-1] + 1):
+        lg = ref.forward(int(seq[pos]), pos)
+        if pos in cand:
+            want[pos] = lg.astype(np.float64).copy()
+    orc.set_threads(1)
+    dt = time.perf_counter() - t0
+
+    def worst_error():
+        worst = 0.0
+        for pos in cand:
+            got = model.forward_logits(pos, int(seq[pos])).astype(np.float64)
+            worst = max(worst, float(np.abs(got - want[pos]).max() / np.abs(want[pos]).max()))
+        return worst
+
+    e_default = worst_error()
+    gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 1)
+    e_f32 = worst_error()
+    gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 0)
+    log(f"  GPU step vs oracle logits at positions {cand} (oracle through {cand[-1] + 1} positions on "
+        f"{cores} cores: {dt:.0f}s): {e_default:.2e} of max|logit| (integer-dot step), {e_f32:.2e} "
+        f"(fp32 activations); budget 1e-3")
+    return {"max_logit_err_over_max_logit": float(f"{e_default:.3e}"),
+            "fp32_activations_max_logit_err_over_max_logit": float(f"{e_f32:.3e}"),
+            "positions": cand, "timed_positions": [t_first, t_first + steps - 1], "budget": 1e-3,
+            "against": "CPU oracle fed the prompt and the tokens the GPU generated (same weights), "
+                       "logits at positions inside the timed region"}
 
 
 def host_cores():
@@ -288,6 +374,53 @@ def bench_8b_gqa(args, W, gpu):
             "roofline": None, "cpu_baseline": None}
 
 
+def attention_leg(W, gpu):
+    """Decode attention on its own at the Llama-3-8B head layout (32 query / 8 KV heads of 128),
+    position 8192: GB/s of the K and V rows read, launches rotating over eight cache sets
+    (553 MB, nothing stays cached), position read from device memory as in a recorded step."""
+    import numpy as np
+    from wgml_amd._lib import AttnParams, View, call
+
+    seq_len, n_heads, kv_mul, hs, pos = 8448, 32, 4, 128, 8192
+    kv_dim = n_heads // kv_mul * hs
+    n_sets = 8
+    q = W.GpuVector.init(gpu, W.rng_normal(71, n_heads * hs))
+    sets = [(W.GpuVector.init(gpu, W.rng_normal(72 + 2 * i, seq_len * kv_dim)),
+             W.GpuVector.init(gpu, W.rng_normal(73 + 2 * i, seq_len * kv_dim))) for i in range(n_sets)]
+    xb = W.GpuVector.uninit(gpu, n_heads * hs)
+    kv = (View * n_sets)(*[k.view() for k, _ in sets])
+    vv = (View * n_sets)(*[v.view() for _, v in sets])
+    p = AttnParams(seq_len, kv_dim, kv_mul, n_heads, hs, pos)
+    ms, iters, best = C.c_float(), 64, None
+    for _ in range(3):
+        call("wgml_bench_attention", gpu.handle, C.byref(p), seq_len, q.view(), kv, vv, n_sets, xb.view(),
+             iters, C.byref(ms))
+        us = ms.value * 1e3 / iters
+        best = us if best is None else min(best, us)
+    nbytes = 2 * kv_dim * 4 * (pos + 1)
+    return {"workload": "decode attention, 32 query / 8 KV heads of 128, position 8192 (attention + "
+                        "merge of the partial results), f32 caches",
+            "us_per_layer": round(best, 3), "kv_bytes": nbytes, "GB/s": round(nbytes / best * 1e-3, 1),
+            "frac_hbm_peak": round(nbytes / best * 1e-3 / HBM_PEAK_GBS, 4)}
+
+
+def gpt2_leg(W, gpu, steps=288):
+    from wgml_amd.models import GPT2_124M, Gpt2, synth_gpt2
+
+    p = GPT2_124M
+    m = Gpt2(gpu, p).load(synth_gpt2(p, seed=3))
+    prompt = W.prompt_tokens(3, 32, p.n_vocab)
+    n = min(32 + steps, p.n_seq)
+    m.generate_greedy(prompt, min(64, n))  # records the step
+    gpu.synchronize()
+    t0 = time.perf_counter()
+    m.generate_greedy(prompt, n)
+    gpu.synchronize()
+    dt = time.perf_counter() - t0
+    return {"workload": f"gpt2-124m q8_0 bs1 greedy: 32-token prompt, positions 0..{n - 1}",
+            "tok_s": round(n / dt, 1), "launches_per_token": m.launches_per_token()}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -316,6 +449,11 @@ def main():
     ap.add_argument("--prefill-only", action="store_true",
                     help="only the batched prompt pass over the prompt, 1 untimed + 3 timed calls "
                          "(for profiler runs)")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="only the machine's own read ceiling: a bare read kernel with the Q4_K "
+                         "GEMV's access pattern at 9.4 / 25.4 / 50.7 / 106.9 MB per launch, in a "
+                         "recorded graph and launch by launch (for profiler runs: set "
+                         "WGML_DISABLE_GRAPHS=1)")
     ap.add_argument("--gemm-precision", type=int, default=1, choices=[0, 1],
                     help="with --prefill-only: 1 = split-f16 operands (default), 0 = plain f16")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
@@ -335,6 +473,10 @@ def main():
     name, n_cu = gpu.info()
     cores = host_cores()
     log(f"device: {name}, {n_cu} CUs; host cores for the CPU legs: {cores}")
+    if args.ceiling:
+        print(json.dumps({"read_chain_in_graph": read_chain(gpu, True),
+                          "read_chain_launch_by_launch": read_chain(gpu, False)}), flush=True)
+        return
     if args.model in ("gpt2", "8b-gqa"):
         if args.steps is None:
             args.steps = 256
@@ -527,13 +669,23 @@ def main():
             tj = json.load(open(tpath))
             traffic = tj.get("gemv_fused_gate_up_bytes_per_launch")
             traffic_src = tj.get("source")
+            # the counters were read for the kernel as it was then: say so when it has changed
+            ksrc = os.path.join(ROOT, "wgml_amd", "csrc", "gemv.hip")
+            if os.path.exists(ksrc) and os.path.getmtime(ksrc) > os.path.getmtime(tpath) + 1:
+                log("WARNING: wgml_amd/csrc/gemv.hip is newer than profiles/traffic.json: "
+                    "roofline.traffic was measured for an earlier build of the kernel")
+                traffic_src = (traffic_src or "") + " (measured before the kernel source last changed)"
         gate = [W.GpuQuantMatrix(gpu, W.Q4_K, cfg.hidden_dim, cfg.dim, l["ffn_gate"].data)
                 for l in weights.layers[:24]]
         us1 = time_gemv(W, gpu, gate, cfg.hidden_dim, cfg.dim, iters=4 * len(gate))
         b1 = gemv_bytes(gate[0].gguf_bytes(), cfg.hidden_dim, cfg.dim)
         del gate
+        chain = read_chain(gpu, True)
+        log(f"machine read ceiling (bare read chain in a graph): {chain['GB/s']:.0f} GB/s sustained, "
+            f"{chain['launch_overhead_us']:.2f} us per launch boundary")
         roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                    "achievable": chain,
                     "traffic_source": traffic_src,
                     "kernel": "gemv_fused_kernel, gate+up launch: 2 x Q4_K 11008x4096, RMSNorm "
                               "folded into staging, SiLU epilogue",
@@ -562,15 +714,18 @@ def main():
     if not args.no_cpu_baseline:
         n = args.cpu_steps or (2 if args.model == "7b" else 16)
         n = min(n, n_prompt)
-        cpu, ref_logits = cpu_baseline(weights, prompt, n, cores)
-        # the GPU step on the same positions against the oracle's logits
-        worst = 0.0
-        for pos in range(n):
-            got = model.forward_logits(pos, int(prompt[pos])).astype(np.float64)
-            worst = max(worst, float(np.abs(got - ref_logits[pos]).max() / np.abs(ref_logits[pos]).max()))
-        parity = {"max_logit_err_over_max_logit": float(f"{worst:.3e}"), "positions": n, "budget": 1e-3,
-                  "against": "CPU oracle, same weights and tokens (the steps of cpu_baseline)"}
-        log(f"  GPU step vs oracle logits on positions 0..{n - 1}: {worst:.2e} of max|logit| (budget 1e-3)")
+        cpu, _ = cpu_baseline(weights, prompt, n, cores)
+        parity = parity_at_timed_positions(W, gpu, model, weights, prompt, np.concatenate([wtoks, toks]),
+                                           first, p0, args.warmup, args.steps, cores)
+
+    other = None
+    if args.model == "7b" and not args.no_sweep:
+        # cheap legs of the two other large workloads, so that the one line carries them
+        other = {"attention_8b_gqa_pos8192": attention_leg(W, gpu), "gpt2_124m_q8_0": gpt2_leg(W, gpu)}
+        log(f"other workloads: attention at the 8B-GQA layout, position 8192: "
+            f"{other['attention_8b_gqa_pos8192']['us_per_layer']:.2f} us per layer, "
+            f"{other['attention_8b_gqa_pos8192']['GB/s']:.0f} GB/s; GPT-2 124M: "
+            f"{other['gpt2_124m_q8_0']['tok_s']:.0f} tok/s")
 
     line = {
         "metric": "decode tok/s bs1 Llama-2-7B-shape Q4_K" if args.model == "7b"
@@ -593,7 +748,7 @@ def main():
                    "fp32_activations": fp32_act,
                    "last_token": int(toks[-1])},
         "roofline": roofline, "cpu_baseline": cpu, "parity": parity, "prefill": prefill,
-        "gemv_sweep": sweep,
+        "gemv_sweep": sweep, "other_workloads": other,
     }
     print(json.dumps(line), flush=True)
 

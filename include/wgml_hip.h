@@ -77,20 +77,29 @@ typedef struct {
 WGML_API int wgml_ctx_create(int device, wgml_ctx **out);
 WGML_API int wgml_ctx_destroy(wgml_ctx *ctx);
 WGML_API int wgml_ctx_synchronize(wgml_ctx *ctx);
+/* The HIP stream (a hipStream_t) on which every call of this context enqueues its work, in
+ * call order: the counterpart of the wgpu queue / compute pass the reference's dispatch calls
+ * record into (e.g. ops/gemv_quant.rs:243-250).  For callers that order HIP work of their own
+ * against the library's, or capture its launches into a HIP graph. */
+WGML_API int wgml_ctx_stream(wgml_ctx *ctx, void **stream);
 /* Launch-shape overrides of one context, for kernel sweeps and for tests that must reach every
  * kernel variant; value 0 restores the heuristic.  The reference has compile-time constants in
  * this role (USE_OPTIMIZED, ops/gemv_quant.rs:15; USE_MATMUL_ATTN, models/llama2/transformer.rs:444).
- * Results stay within the documented tolerances for every setting. */
+ * Results stay within the documented tolerances for every setting.  Values outside a key's range
+ * are refused.  A model re-records its decode step the next time it runs after a change (launch
+ * sequences recorded under other settings are dropped). */
 enum {
     WGML_TUNE_GEMV_ROWS_PER_WAVE = 0,        /* 1 or 2 rows of a quantized GEMV per wave and step */
-    WGML_TUNE_GEMV_WAVES_PER_WG,             /* 4, 8 or 16 */
-    WGML_TUNE_GEMV_WG_PER_CU,                /* cap on resident workgroups per compute unit */
+    WGML_TUNE_GEMV_WAVES_PER_WG,             /* 4, 8 or 16; 12 for the multi-matrix launches only
+                                                (single-matrix launches then use 16) */
+    WGML_TUNE_GEMV_WG_PER_CU,                /* cap on resident workgroups per compute unit, 1..8 */
     WGML_TUNE_GEMV_DEPTH,                    /* weight tiles in flight per wave, 1..4 */
     WGML_TUNE_GEMV_F32_ACTIVATIONS,          /* 1: fp32 activations instead of 16-bit block fixed point */
     WGML_TUNE_GEMM_K_SPLIT,                  /* 1..8 workgroups share the K range of a batched product */
     WGML_TUNE_PREFILL_ATTENTION_PER_TOKEN,   /* 1: one workgroup per (head, token) in the prompt pass */
-    WGML_TUNE_ATTN_WIDE_POSITIONS,           /* decode attention planned for up to this many positions runs
-                                                as one workgroup per head group, without partial results */
+    WGML_TUNE_ATTN_WIDE_POSITIONS,           /* decode attention planned for up to this many positions
+                                                (at most 2^20) runs as one workgroup per head group,
+                                                without partial results */
     WGML_TUNE_ATTN_SPLITS,                   /* workgroups that share the positions of a head group, 2..64 */
     WGML_TUNE_COUNT
 };
@@ -134,6 +143,11 @@ WGML_API int wgml_quant_matrix_shape(const wgml_qmat *m, int *type, uint32_t *nr
                                      uint32_t *ncols); /* GpuQuantMatrix::shape */
 /* Size of the tensor in GGUF bytes (the algorithmic weight traffic of one GEMV). */
 WGML_API uint64_t wgml_quant_matrix_gguf_bytes(const wgml_qmat *m);
+/* An upper bound on the magnitude of the matrix's dequantized weights, computed on the device
+ * when the matrix is created (Q8_0 / Q4_K / Q6_K; 0 for other formats; infinity when a block
+ * scale is NaN or infinite).  The reference has no counterpart: it is what decides whether the
+ * batched product (wgml_gemm_quant) takes the matrix. */
+WGML_API int wgml_quant_matrix_weight_bound(const wgml_qmat *m, float *bound);
 
 /* Host helpers (no device needed): bytes of `nelems` elements in a format
  * (0 if unsupported / not a whole number of blocks). */
@@ -158,7 +172,11 @@ WGML_API int wgml_gemv_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, w
  * weights and vectors to f16 once: 1.4x faster, about 3e-4 of a row's magnitude
  * (up to 1.4e-3 for single elements).  m must be WGML_Q8_0, WGML_Q4_K or WGML_Q6_K.
  * Vectors of any magnitude are taken (scaled per vector by a power of two); the
- * dequantized weights must be below 256 in magnitude (they pass through f16 times 2^8). */
+ * dequantized weights must not exceed 255.875 in magnitude (they pass through f16 times 2^8,
+ * and 65504 is the largest finite f16): a bound on the largest weight is computed when the
+ * matrix is created, and a matrix whose bound is larger is refused with WGML_E_UNSUPPORTED
+ * (wgml_gemv_quant takes any value;
+ * wgml_llama2_prefill steps through the prompt token by token for such a model). */
 WGML_API int wgml_ctx_set_gemm_precision(wgml_ctx *ctx, int level);
 WGML_API int wgml_gemm_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, wgml_view x,
                              uint32_t n_tokens);
@@ -212,6 +230,17 @@ typedef struct {
 WGML_API int wgml_attention(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
                             wgml_view key_cache, wgml_view value_cache, wgml_view att,
                             wgml_view xb);
+/* The pair BatchedMultiqueryAttention::dispatch_multi + GemvQuant::dispatch that every decoder
+ * layer runs (models/llama2/transformer.rs:366-383, models/gpt2/transformer.rs:355-395):
+ * out = m * attention(q, caches), or out += ... when accumulate != 0 (the add_assign that
+ * follows in the reference).  m is n x (n_heads * head_size).  Where m is Q8_0 / Q4_K / Q6_K
+ * the attention launch leaves per-workgroup partial results and the product merges them while
+ * it stages its input: there is no merge launch and `xb` is not written; otherwise the two
+ * launches run as they would on their own.  xb: n_heads * head_size floats of scratch whose
+ * contents after the call are unspecified. */
+WGML_API int wgml_attention_gemv_quant(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
+                                       wgml_view key_cache, wgml_view value_cache, wgml_view xb,
+                                       const wgml_qmat *m, wgml_view out, int accumulate);
 /* No counterpart in the reference.  wgml_attention without the `att` output, for callers
  * that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc): the partial results of the position-split launches live
@@ -221,14 +250,19 @@ WGML_API int wgml_attention(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view 
  * floats; 1.06 MB for 32 heads of 128 at 8192 positions) exceed the array is refused with
  * WGML_E_UNSUPPORTED.  Results equal
  * wgml_attention's.  Every call on a GPU uses that GPU's one array: calls that overlap on
- * one GPU (two contexts, two streams) race. */
+ * one GPU (two contexts, two streams) race.  The array's address is looked up when the context
+ * is created; the call itself only launches kernels, so it may be recorded under stream capture
+ * (wgml_ctx_stream) and replayed. */
 WGML_API int wgml_attention_noalloc(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
                                     wgml_view key_cache, wgml_view value_cache, wgml_view xb);
 
 /* Silu::dispatch (ops/silu.rs:18-34): h1 = h2 * h1 / (1 + exp(-h1)). */
 WGML_API int wgml_silu(wgml_ctx *ctx, wgml_view h1, wgml_view h2);
 
-/* UnaryOp (ops/unary.rs:16-38), same order. */
+/* UnaryOp (ops/unary.rs:16-38), same order.  Each follows the shader (ops/unary.wgsl); where the
+ * reference's CPU twin differs from its shader the shader wins, this being the device op:
+ * WGML_UNARY_SGN is WGSL `sign` (ops/unary.wgsl:27): 0 at +0 and -0 (and for NaN), whereas
+ * UnaryOp::eval's f32::signum (ops/unary.rs:90) gives +1 / -1 at the two zeros. */
 enum {
     WGML_UNARY_ABS = 0, WGML_UNARY_SGN, WGML_UNARY_NEG, WGML_UNARY_STEP, WGML_UNARY_ELU,
     WGML_UNARY_GELU, WGML_UNARY_GELU_QUICK, WGML_UNARY_SILU, WGML_UNARY_TANH, WGML_UNARY_RELU,
@@ -401,6 +435,17 @@ WGML_API int wgml_gpt2_launches_per_token(const wgml_gpt2 *m);
  * part of the measurement. */
 WGML_API int wgml_bench_gemv_quant(wgml_ctx *ctx, const wgml_qmat *const *mats, uint32_t n_mats,
                                    wgml_view out, wgml_view v, uint32_t iters, int use_graph,
+                                   float *total_ms);
+
+/* The machine's own ceiling for such a chain of launches (no counterpart in the reference):
+ * `iters` launches of a kernel that only reads, with the access pattern of the Q4_K GEMV
+ * (rows of 4096 columns = 2304 bytes, a wave per row, one 64-element tile per lane in
+ * flight, one workgroup of 16 waves per compute unit), each launch over its own `nrows` rows
+ * of a 1.5 GB pool that the call allocates and frees.  nrows 4096 / 11008 / 22016 / 46400 read
+ * 9.4 / 25.4 / 50.7 / 106.9 MB per launch.  Returns the elapsed milliseconds between two GPU
+ * timestamps; use_graph != 0 records the launches into a HIP graph first.  Time per launch as a
+ * function of the bytes gives what a launch boundary costs and what loads sustain. */
+WGML_API int wgml_bench_read_chain(wgml_ctx *ctx, uint32_t nrows, uint32_t iters, int use_graph,
                                    float *total_ms);
 
 /* The same loop for the fused launches of the decoder: launch i covers the

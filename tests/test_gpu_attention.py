@@ -6,6 +6,7 @@ long-context cases of the benchmark configurations."""
 import numpy as np
 import pytest
 
+import npref
 import oracle as orc
 import wgml_amd as W
 
@@ -75,6 +76,105 @@ def test_attention_plans_agree(gpu, wide, splits, pos):
         gpu.set_tuning(gpu.TUNE_ATTN_WIDE_POSITIONS, 0)
         gpu.set_tuning(gpu.TUNE_ATTN_SPLITS, 0)
     np.testing.assert_allclose(xb, wxb, rtol=0, atol=2e-5)
+
+
+def run_with_projection(gpu, qtype, seq_len, kv_mul, n_heads, hs, pos, nrows, accumulate, seed=0):
+    """attention + output projection as one call, against the oracle's attention followed by the
+    exact product of the dequantized matrix with it (f64)."""
+    kv_dim = n_heads // kv_mul * hs
+    dim = n_heads * hs
+    q = rnd(dim, seed + 1)
+    kc, vc = rnd(seq_len * kv_dim, seed + 2), rnd(seq_len * kv_dim, seed + 3)
+    vals = rnd(nrows * dim, seed + 4, 0.02)
+    if qtype == W.F32:
+        raw, w = vals.view(np.uint8), vals
+    elif qtype in (W.Q8_0, W.Q4_K, W.Q6_K):
+        raw = W.quantize(qtype, vals)
+        w = orc.dequantize(qtype, raw, nrows * dim)
+    else:  # no quantizer for these: random blocks with finite scales
+        raw = npref.random_blocks(qtype, nrows * dim // npref.BLOCK_ELEMS[qtype], seed=seed + 4)
+        w = orc.dequantize(qtype, raw, nrows * dim)
+    m = W.GpuQuantMatrix(gpu, qtype, nrows, dim, raw)
+    p = W.BatchedMultiqueryAttentionParams(seq_len, kv_dim, kv_mul, n_heads, hs, pos)
+    gq, gk, gv = (W.GpuVector.init(gpu, a) for a in (q, kc, vc))
+    xb = W.GpuVector.init(gpu, np.full(dim, np.nan, dtype=np.float32))
+    out0 = rnd(nrows, seed + 5)
+    out = W.GpuVector.init(gpu, out0)
+    W.BatchedMultiqueryAttention.from_device(gpu).dispatch_with_projection(p, gq, gk, gv, xb, m, out,
+                                                                            accumulate)
+    want_xb, _ = orc.attention(seq_len, kv_dim, kv_mul, n_heads, hs, pos, q, kc, vc)
+    want = w.reshape(nrows, dim).astype(np.float64) @ want_xb.astype(np.float64)
+    if accumulate:
+        want = want + out0
+    return out.read(), want
+
+
+@pytest.mark.parametrize("qtype", [W.Q4_K, W.Q6_K, W.Q8_0])
+@pytest.mark.parametrize("pos", [0, 3, 31, 140, 255, 256, 700, 1023])
+def test_attention_with_projection(gpu, qtype, pos):
+    # the product merges attention's per-workgroup partial results while it stages its input
+    # (2 to 16 partial results per head, depending on the position; at the first positions
+    # most of them are neutral); GEMV tolerance as in tests/test_gpu_gemv.py
+    got, want = run_with_projection(gpu, qtype, 1024, 1, 8, 128, pos, 192, False, seed=pos)
+    assert np.abs(got - want).max() <= 5e-4 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("kv_mul,n_heads,hs", [(4, 32, 128), (2, 8, 64), (1, 12, 64), (1, 6, 48), (8, 16, 128),
+                                               (1, 2, 256)])
+@pytest.mark.parametrize("pos", [5, 383])
+def test_attention_with_projection_head_layouts(gpu, kv_mul, n_heads, hs, pos):
+    # grouped queries, head sizes that fill a lane group only partly (48) and that need the
+    # four-wave kernel (256), accumulation into the output
+    dim = n_heads * hs
+    qtype = W.Q8_0 if dim % 256 else W.Q4_K
+    got, want = run_with_projection(gpu, qtype, 512, kv_mul, n_heads, hs, pos, 96, True, seed=kv_mul)
+    assert np.abs(got - want).max() <= 5e-4 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("wide,splits", [(1024, 0), (0, 2), (0, 8), (0, 9), (0, 16), (0, 17), (0, 64)])
+def test_attention_with_projection_plans(gpu, wide, splits):
+    # forced plans: one workgroup per head (nothing to merge), 2..16 partial results merged by the
+    # product (eight at a time), 17 and 64 through the merge launch
+    gpu.set_tuning(gpu.TUNE_ATTN_WIDE_POSITIONS, wide)
+    gpu.set_tuning(gpu.TUNE_ATTN_SPLITS, splits)
+    try:
+        for pos in (3, 140, 700):
+            got, want = run_with_projection(gpu, W.Q4_K, 1024, 2, 8, 128, pos, 128, True, seed=3)
+            assert np.abs(got - want).max() <= 5e-4 * np.abs(want).max(), pos
+    finally:
+        gpu.set_tuning(gpu.TUNE_ATTN_WIDE_POSITIONS, 0)
+        gpu.set_tuning(gpu.TUNE_ATTN_SPLITS, 0)
+
+
+@pytest.mark.parametrize("qtype", [W.F32, W.Q5_K, W.Q4_0])
+def test_attention_with_projection_other_formats(gpu, qtype):
+    # formats without a merging product: the two launches run as they would on their own
+    got, want = run_with_projection(gpu, qtype, 256, 1, 4, 64, 77, 64, True, seed=11)
+    assert np.abs(got - want).max() <= 5e-4 * np.abs(want).max()
+
+
+def test_attention_with_projection_fp32_activations(gpu):
+    gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 1)
+    try:
+        got, want = run_with_projection(gpu, W.Q4_K, 512, 1, 8, 128, 300, 64, False, seed=2)
+    finally:
+        gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 0)
+    assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+
+
+def test_attention_with_projection_argument_checks(gpu):
+    a = W.BatchedMultiqueryAttention.from_device(gpu)
+    raw = W.quantize(W.Q8_0, rnd(32 * 128, 1, 0.02))
+    m = W.GpuQuantMatrix(gpu, W.Q8_0, 32, 128, raw)
+    v = W.GpuVector.uninit(gpu, 4096)
+    p = W.BatchedMultiqueryAttentionParams(16, 128, 1, 2, 64, 3)
+    with pytest.raises(W.WgmlError):  # out does not have the matrix's rows
+        a.dispatch_with_projection(p, v.rows(0, 128), v.rows(0, 2048), v.rows(0, 2048), v.rows(0, 128), m,
+                                   v.rows(0, 31))
+    bad = W.BatchedMultiqueryAttentionParams(16, 64, 1, 1, 64, 3)
+    with pytest.raises(W.WgmlError):  # attention output shorter than the matrix's columns
+        a.dispatch_with_projection(bad, v.rows(0, 64), v.rows(0, 1024), v.rows(0, 1024), v.rows(0, 64), m,
+                                   v.rows(0, 32))
 
 
 def test_bench_attention_runs_and_checks_its_arguments(gpu):

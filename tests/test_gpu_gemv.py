@@ -238,6 +238,48 @@ def test_fused_gate_up_silu_launch(gpu, nrows, ncols):
 OTHER = [W.Q4_0, W.Q4_1, W.Q5_0, W.Q5_1, W.Q5_K, W.Q8_K]
 
 
+@pytest.mark.parametrize("qtype", QT + OTHER)
+@pytest.mark.parametrize("nrows", [1, 3, 9, 15])
+@pytest.mark.parametrize("ncols", [256, 1024, 8192])
+def test_gemv_fewer_rows_than_waves(gpu, qtype, nrows, ncols):
+    # Workgroups of 8 or 16 waves, fewer rows than that: the waves without a row either stage a
+    # share of x and wait at the barrier, or (no share either: 256 columns need one staging wave
+    # in four, 8192 all of them) end before it.  The barrier counts only waves that are still
+    # running (a terminated wave is not waited for on this hardware), which this case relies on.
+    be = npref.BLOCK_ELEMS[qtype]
+    raw = npref.random_blocks(qtype, nrows * ncols // be, seed=500 + qtype + nrows)
+    x = W.rng_normal(600 + ncols, ncols)
+    _, ref = orc.gemv_quant(qtype, raw, nrows, ncols, x)
+    ok, e = close(gemv(gpu, qtype, raw, nrows, ncols, x), ref)
+    assert ok, e
+
+
+@pytest.mark.parametrize("qtype", QT)
+@pytest.mark.parametrize("nrows", [1, 2, 7])
+def test_fused_launch_with_fewer_row_pairs_than_waves(gpu, qtype, nrows):
+    # the multi-matrix launch with so few (gate, up) pairs that most waves of its one
+    # workgroup have none
+    import ctypes as C
+
+    from wgml_amd._lib import call
+
+    ncols = 512
+    gate_raw, up_raw = weights(qtype, nrows, ncols, 15), weights(qtype, nrows, ncols, 16)
+    x = W.rng_normal(17, ncols)
+    gate = W.GpuQuantMatrix(gpu, qtype, nrows, ncols, gate_raw)
+    up = W.GpuQuantMatrix(gpu, qtype, nrows, ncols, up_raw)
+    out = W.GpuVector.init(gpu, np.full(nrows, np.nan, dtype=np.float32))
+    xv = W.GpuVector.init(gpu, x)
+    a, b = (C.c_void_p * 1)(gate.handle), (C.c_void_p * 1)(up.handle)
+    modes, ms = (C.c_int * 1)(2), C.c_float()
+    call("wgml_bench_gemv_fused", gpu.handle, a, b, modes, 1, 1, out.view(), nrows, xv.view(), None, 1,
+         C.byref(ms))
+    _, g = orc.gemv_quant(qtype, gate_raw, nrows, ncols, x)
+    _, u = orc.gemv_quant(qtype, up_raw, nrows, ncols, x)
+    ok, e = close(out.read(), u * (g / (1.0 + np.exp(-g))))
+    assert ok, e
+
+
 @pytest.mark.parametrize("qtype", OTHER)
 @pytest.mark.parametrize("nrows,ncols", [(4, 256), (1, 512), (37, 768), (33, 4096), (260, 11008),
                                          (4096, 4096), (7, 14336)])

@@ -94,6 +94,33 @@ def test_llama_recorded_loop_matches_oracle(gpu, model_type):
         assert np.array_equal(m.generate_greedy(prompt, MICRO.seq_len), want), fusion
 
 
+def test_tuning_change_rerecords_the_step(gpu):
+    # a launch-shape override set after a model has recorded its step must take effect: the
+    # captures are dropped and made again.  Seventeen workgroups per head are more than the output
+    # projection merges itself, so each layer gains a merge launch; tokens stay the same.
+    w = synth_llama(MICRO, seed=21, scheme="q8_0")
+    spice(w, MICRO, 5, biases=False)
+    m = Llama2(gpu, MICRO).load(w)
+    prompt = [3, 300, 17]
+    base = m.generate_greedy(prompt, 20)
+    n0 = m.launches_per_token()
+    gpu.set_tuning(gpu.TUNE_ATTN_WIDE_POSITIONS, 1)  # no single-workgroup plan at this length
+    gpu.set_tuning(gpu.TUNE_ATTN_SPLITS, 17)
+    try:
+        again = m.generate_greedy(prompt, 20)
+        assert m.launches_per_token() == n0 + MICRO.n_layers
+    finally:
+        gpu.set_tuning(gpu.TUNE_ATTN_WIDE_POSITIONS, 0)
+        gpu.set_tuning(gpu.TUNE_ATTN_SPLITS, 0)
+    assert np.array_equal(base, again)
+    assert np.array_equal(m.generate_greedy(prompt, 20), base)
+    assert m.launches_per_token() == n0
+    for key, bad in ((gpu.TUNE_GEMV_WG_PER_CU, 9), (gpu.TUNE_ATTN_WIDE_POSITIONS, (1 << 20) + 1),
+                     (gpu.TUNE_GEMV_WAVES_PER_WG, 5), (gpu.TUNE_ATTN_SPLITS, 65)):
+        with pytest.raises(W.WgmlError):
+            gpu.set_tuning(key, bad)
+
+
 def test_llama_decode_from_uploaded_kv(gpu):
     # pre-filled cache then decode, as the long-context configuration does
     w = synth_llama(MICRO, seed=23, scheme="q6_k")

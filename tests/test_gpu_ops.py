@@ -133,6 +133,16 @@ def test_unary_ops(gpu, op):  # ops/unary.rs:273-348, epsilon 1e-5
     np.testing.assert_allclose(g.read(), _unary_ref(op, x, args), rtol=1e-5, atol=1e-5)
 
 
+def test_unary_sgn_at_zero_follows_the_shader(gpu):
+    # WGSL sign (ops/unary.wgsl:27) is 0 at both zeros; the reference's CPU twin (f32::signum,
+    # ops/unary.rs:90) would give +1 / -1 there.  The device op follows the shader; its test in
+    # the reference (ops/unary.rs:273-348) draws random values and never meets a zero.
+    x = np.array([0.0, -0.0, 1e-30, -1e-30, 3.5, -2.0, np.inf, -np.inf], dtype=np.float32)
+    g = vec(gpu, x)
+    W.UnaryInplace(gpu, W.UnaryOp.Sgn).dispatch(g, None)
+    assert g.read().tolist() == [0.0, 0.0, 1.0, -1.0, 1.0, -1.0, 1.0, -1.0]
+
+
 def test_unary_needs_args(gpu):  # ops/unary.rs:173-176
     with pytest.raises(W.WgmlError, match="needs arguments"):
         W.UnaryInplace(gpu, W.UnaryOp.Scale).dispatch(W.GpuVector.uninit(gpu, 4), None)

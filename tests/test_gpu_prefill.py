@@ -19,6 +19,7 @@ import pytest
 
 import oracle as orc
 import wgml_amd as W
+from wgml_amd._lib import E_UNSUPPORTED
 
 pytestmark = pytest.mark.gpu
 QT = [W.Q8_0, W.Q4_K, W.Q6_K]
@@ -128,13 +129,54 @@ def test_gemm_large_activations_stay_finite(gpu, k_split, qtype):
 def test_gemm_operand_magnitudes(gpu, qtype, x_scale, w_std):
     # The low parts of the split operands are small numbers: activations are scaled per token into
     # (512, 1024] (up as well as down) and weights expanded times 2^8 so that they stay f16
-    # numbers.  Small and large activations, small and large weights (|w| < 256 is the limit),
+    # numbers.  Small and large activations, small and large weights (|w| <= 255.875 is the limit),
     # one outlier in a row: the bounds hold unchanged (observed 2e-7 rms, 2e-6 worst, split f16).
     nrows, ncols, T = 96, 2048, 40
     raw = W.quantize(qtype, W.rng_normal(31, nrows * ncols, 0, w_std))
     x = (W.rng_normal(32, T * ncols) * np.float32(x_scale)).reshape(T, ncols)
     x[3, 17] = 40 * x_scale
     check(gemm(gpu, qtype, raw, nrows, ncols, x), reference(qtype, raw, nrows, ncols, x))
+
+
+@pytest.mark.parametrize("qtype", QT)
+def test_gemm_weight_magnitude_limit(gpu, qtype):
+    # Weights pass through f16 times 2^8, so a matrix is taken only while a bound on its largest
+    # dequantized weight stays within 65504 / 256 = 255.875 (computed when the matrix is created: exact for Q8_0,
+    # the ends of each sub-block's quant range for Q4_K, |d| |scale| 32 for Q6_K).  Just inside the limit the product
+    # is as accurate as anywhere else; at or beyond it the call is refused and the per-token
+    # product, which takes any value, still answers.
+    nrows, ncols, T = 64, 1024, 20
+    u = W.rng_normal(41, nrows * ncols)
+    u = np.clip(u / 3.0, -1.0, 1.0).astype(np.float32)
+    x = W.rng_normal(42, T * ncols).reshape(T, ncols)
+    inside = {W.Q8_0: 250.0, W.Q6_K: 240.0, W.Q4_K: 150.0}[qtype]
+    raw = W.quantize(qtype, u * np.float32(inside))
+    m = W.GpuQuantMatrix(gpu, qtype, nrows, ncols, raw)
+    w = orc.dequantize(qtype, raw, nrows * ncols)
+    assert float(np.abs(w).max()) <= m.weight_bound() <= 255.875
+    check(gemm(gpu, qtype, raw, nrows, ncols, x), reference(qtype, raw, nrows, ncols, x))
+    for amp in (256.0, 300.0, 7e4):
+        vals = u * np.float32(amp)
+        vals[5] = amp  # the largest weight itself reaches the amplitude
+        raw = W.quantize(qtype, vals)
+        m = W.GpuQuantMatrix(gpu, qtype, nrows, ncols, raw)
+        w = orc.dequantize(qtype, raw, nrows * ncols)
+        if not np.isfinite(w).all():
+            continue  # beyond what the format's f16 scale holds
+        assert m.weight_bound() >= float(np.abs(w).max()) >= 255.0
+        if m.weight_bound() <= 255.875:
+            # the f16 scale rounded the largest weight to within the limit: taken
+            check(gemm(gpu, qtype, raw, nrows, ncols, x), reference(qtype, raw, nrows, ncols, x))
+            continue
+        xv = W.GpuVector.init(gpu, x.reshape(-1))
+        out = W.GpuVector.init(gpu, np.zeros(T * nrows, dtype=np.float32))
+        with pytest.raises(W.WgmlError) as e:
+            W.GemmQuant.from_device(gpu).dispatch(out, m, xv, T)
+        assert e.value.code == E_UNSUPPORTED
+        o1 = W.GpuVector.init(gpu, np.zeros(nrows, dtype=np.float32))
+        W.GemvQuant.from_device(gpu).dispatch(o1, m, W.GpuVector.init(gpu, x[0]))
+        ref = reference(qtype, raw, nrows, ncols, x[:1])[0]
+        assert np.abs(o1.read() - ref).max() <= 5e-4 * np.abs(ref).max()
 
 
 @pytest.mark.parametrize("qtype", QT)
@@ -330,3 +372,22 @@ def test_prefill_rejects_bad_arguments(gpu):
     for pos, t in enumerate([1, 2, 3]):
         want = g.forward_logits(pos, t)
     assert np.array_equal(got, want)
+
+
+def test_prefill_steps_through_a_model_with_large_weights(gpu):
+    # one matrix whose weights do not fit the batched product: the prompt then goes through the
+    # per-token steps, and the state equals the oracle's as for any other model
+    w = synth_llama(MICRO, seed=21, scheme="q8_0")
+    spice(w, MICRO, 5, biases=False)
+    hm = w.layers[1]["ffn_down"]
+    vals = orc.dequantize(hm.qtype, hm.data, hm.nrows * hm.ncols).copy()
+    vals[7] = 300.0
+    w.layers[1]["ffn_down"] = type(hm)(hm.qtype, hm.nrows, hm.ncols, W.quantize(hm.qtype, vals))
+    ref = orc.Llama2(w)
+    toks = W.prompt_tokens(3, 9, MICRO.vocab_size)
+    for pos, t in enumerate(toks):
+        want = ref.forward(int(t), pos)
+    m = Llama2(gpu, MICRO).load(w)
+    m.prefill(toks)
+    assert np.isfinite(m.logits()).all()
+    assert_state_matches(m, ref, MICRO, 9, want, tol=1e-3)

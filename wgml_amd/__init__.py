@@ -13,3 +13,4 @@ from .models import prompt_tokens  # noqa: F401
 from .gguf import (Gguf, GgufTensor, gpt2_params_from_gguf, gpt2_weights_from_gguf,  # noqa: F401
                    llama2_config_from_gguf, llama2_weights_from_gguf)
 from .tokenizer import Gpt2Tokenizer, LlamaTokenizer, llama2_chat_prompt  # noqa: F401
+from .chat_template import ChatTemplate, Prompt, TemplateError, LLAMA2_CHAT_TEMPLATE  # noqa: F401

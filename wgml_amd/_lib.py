@@ -92,6 +92,7 @@ PROTOTYPES = {
     "wgml_ctx_create": (_i, [_i, _PP]),
     "wgml_ctx_destroy": (_i, [_P]),
     "wgml_ctx_synchronize": (_i, [_P]),
+    "wgml_ctx_stream": (_i, [_P, _PP]),
     "wgml_ctx_info": (_i, [_P, C.c_char_p, C.c_size_t, C.POINTER(_i)]),
     "wgml_timer_start": (_i, [_P]),
     "wgml_timer_stop": (_i, [_P, _fp]),
@@ -106,6 +107,7 @@ PROTOTYPES = {
     "wgml_quant_matrix_destroy": (_i, [_P]),
     "wgml_quant_matrix_shape": (_i, [_P, C.POINTER(_i), _u32p, _u32p]),
     "wgml_quant_matrix_gguf_bytes": (_u64, [_P]),
+    "wgml_quant_matrix_weight_bound": (_i, [_P, _fp]),
     "wgml_quant_bytes": (_u64, [_i, _u64]),
     "wgml_quant_block_elems": (_u32, [_i]),
     "wgml_gemv_quant": (_i, [_P, View, _P, View]),
@@ -120,6 +122,7 @@ PROTOTYPES = {
     "wgml_softmax": (_i, [_P, View, _u32, _u32, _u32]),
     "wgml_attention": (_i, [_P, C.POINTER(AttnParams), View, View, View, View, View]),
     "wgml_attention_noalloc": (_i, [_P, C.POINTER(AttnParams), View, View, View, View]),
+    "wgml_attention_gemv_quant": (_i, [_P, C.POINTER(AttnParams), View, View, View, View, _P, View, _i]),
     "wgml_silu": (_i, [_P, View, View]),
     "wgml_unary_inplace": (_i, [_P, _i, View, _fp]),
     "wgml_op_assign": (_i, [_P, _i, View, View]),
@@ -151,6 +154,7 @@ PROTOTYPES = {
     "wgml_gpt2_set_fusion": (_i, [_P, _i]),
     "wgml_gpt2_launches_per_token": (_i, [_P]),
     "wgml_bench_gemv_quant": (_i, [_P, _PP, _u32, View, View, _u32, _i, _fp]),
+    "wgml_bench_read_chain": (_i, [_P, _u32, _u32, _i, _fp]),
     "wgml_bench_gemv_fused": (_i, [_P, _PP, _PP, C.POINTER(C.c_int), _u32, _u32, View, _u32, View,
                                    C.POINTER(View), _u32, _fp]),
     "wgml_bench_attention": (_i, [_P, C.POINTER(AttnParams), _u32, View, C.POINTER(View), C.POINTER(View),

@@ -35,11 +35,15 @@ struct AttnArgs {
     const float *q, *kc, *vc;
     float *att;  // optional: raw scores here, normalised by the merge kernel
     float *xb;
-    float *ws;  // partials: [head][wg_y][2 + HSP]
+    // partial results of the workgroups that share a head's positions: the weighted sums of V
+    // as ws[head][wg_y][HSP] (rows of HSP floats, 16-byte aligned), and (max, sum) as
+    // ws_ml[head][wg_y][2]
+    float *ws, *ws_ml;
     uint32_t seq_len, kv_dim, kv_mul, n_heads, head_size;
     DynPos pos;
     uint32_t chunk;  // positions per wave
     uint32_t spec_rows;  // rows of the caches that exist (may be read before pos is known)
+    uint32_t spec_sets;  // register sets whose quads are requested before pos is known (>= 1)
     uint32_t n_wg_y;
     int direct;  // 1: grid.y == 1 and the workgroup writes xb itself
 };
@@ -147,12 +151,12 @@ __global__ __launch_bounds__(WAVES * 64) void attn_split_kernel(const AttnArgs a
         if (a.direct) {
             if (d < hs) a.xb[(size_t)(h0 + m) * hs + d] = o / L;
         } else {
-            float *p = a.ws + ((size_t)(h0 + m) * a.n_wg_y + blockIdx.y) * (2 + HSP);
+            const size_t slot = (size_t)(h0 + m) * a.n_wg_y + blockIdx.y;
             if (d == 0) {
-                p[0] = M;
-                p[1] = L;
+                a.ws_ml[slot * 2] = M;
+                a.ws_ml[slot * 2 + 1] = L;
             }
-            p[2 + d] = o;
+            a.ws[slot * HSP + d] = o;
         }
     }
 }
@@ -176,8 +180,9 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnArgs a, uint3
     __shared__ float sm_ML[2];
     const uint32_t h = blockIdx.x;
     const uint32_t pos = dyn_pos(a.pos);
-    const uint32_t stride = 2 + hsp;
+    const uint32_t stride = hsp;
     const float *base = a.ws + (size_t)h * a.n_wg_y * stride;
+    const float *ml = a.ws_ml + (size_t)h * a.n_wg_y * 2;
     // workgroups whose positions start beyond pos hold no partial
     // (chunk == 0: partials of the fast kernel)
     const uint32_t n_used = a.chunk ? min(a.n_wg_y, pos / (a.chunk * WAVES) + 1)
@@ -186,8 +191,8 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnArgs a, uint3
     float M, L;
     if (n_used <= MERGE_MAX_Y) {
         if (tid < 64) {  // wave 0: one partial per lane
-            const float my = lane < n_used ? base[(size_t)lane * stride] : -INFINITY;
-            const float ly = lane < n_used ? base[(size_t)lane * stride + 1] : 0.f;
+            const float my = lane < n_used ? ml[lane * 2] : -INFINITY;
+            const float ly = lane < n_used ? ml[lane * 2 + 1] : 0.f;
             const float mm = wave_max(my);
             const float wgt = my == -INFINITY ? 0.f : __expf(my - mm);
             const float ll = wave_sum(ly * wgt);
@@ -206,7 +211,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnArgs a, uint3
                 float v[8];
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
-                    v[k] = y0 + k < n_used ? base[(size_t)(y0 + k) * stride + 2 + d] : 0.f;
+                    v[k] = y0 + k < n_used ? base[(size_t)(y0 + k) * stride + d] : 0.f;
 #pragma unroll
                 for (int k = 0; k < 8; ++k) o = fmaf(v[k], y0 + k < n_used ? sm_w[y0 + k] : 0.f, o);
             }
@@ -214,19 +219,19 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnArgs a, uint3
         }
     } else {
         M = -INFINITY;
-        for (uint32_t y = 0; y < n_used; ++y) M = fmaxf(M, base[(size_t)y * stride]);
+        for (uint32_t y = 0; y < n_used; ++y) M = fmaxf(M, ml[y * 2]);
         L = 0.f;
         for (uint32_t y = 0; y < n_used; ++y) {
-            const float my = base[(size_t)y * stride];
+            const float my = ml[y * 2];
             const float wgt = my == -INFINITY ? 0.f : __expf(my - M);
-            L = fmaf(base[(size_t)y * stride + 1], wgt, L);
+            L = fmaf(ml[y * 2 + 1], wgt, L);
         }
         for (uint32_t d = tid; d < a.head_size; d += blockDim.x) {
             float o = 0.f;
             for (uint32_t y = 0; y < n_used; ++y) {
-                const float my = base[(size_t)y * stride];
+                const float my = ml[y * 2];
                 const float wgt = my == -INFINITY ? 0.f : __expf(my - M);
-                o = fmaf(base[(size_t)y * stride + 2 + d], wgt, o);
+                o = fmaf(base[(size_t)y * stride + d], wgt, o);
             }
             a.xb[(size_t)h * a.head_size + d] = o / L;
         }
@@ -246,15 +251,16 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const AttnArgs a, uint3
 template <int B>
 __global__ __launch_bounds__(256) void attn_merge_fast_kernel(const AttnArgs a, uint32_t hsp) {
     const uint32_t h = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
-    const uint32_t stride = 2 + hsp, ny = a.n_wg_y;  // ny <= MERGE_MAX_Y = 64
+    const uint32_t stride = hsp, ny = a.n_wg_y;  // ny <= MERGE_MAX_Y = 64
     const float *base = a.ws + (size_t)h * ny * stride;
-    const float my = lane < ny ? base[(size_t)lane * stride] : -INFINITY;
-    const float ly = lane < ny ? base[(size_t)lane * stride + 1] : 0.f;
+    const float *ml = a.ws_ml + (size_t)h * ny * 2;
+    const float my = lane < ny ? ml[lane * 2] : -INFINITY;
+    const float ly = lane < ny ? ml[lane * 2 + 1] : 0.f;
     float v[B];
     const bool has_d = tid < a.head_size;  // head sizes up to 256: one dimension per thread
 #pragma unroll
     for (int k = 0; k < B; ++k)
-        v[k] = (has_d && (uint32_t)k < ny) ? base[(size_t)k * stride + 2 + tid] : 0.f;
+        v[k] = (has_d && (uint32_t)k < ny) ? base[(size_t)k * stride + tid] : 0.f;
     const float M = wave_max(my);
     const float wgt = my == -INFINITY ? 0.f : __expf(my - M);
     const float L = wave_sum(ly * wgt);
@@ -267,7 +273,7 @@ __global__ __launch_bounds__(256) void attn_merge_fast_kernel(const AttnArgs a, 
     for (uint32_t y0 = B; y0 < ny; y0 += B) {
 #pragma unroll
         for (int k = 0; k < B; ++k)
-            v[k] = (has_d && y0 + k < ny) ? base[(size_t)(y0 + k) * stride + 2 + tid] : 0.f;
+            v[k] = (has_d && y0 + k < ny) ? base[(size_t)(y0 + k) * stride + tid] : 0.f;
 #pragma unroll
         for (int k = 0; k < B; ++k) {
             const float wk = __shfl(wgt, (int)(y0 + k), 64);
@@ -324,7 +330,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
 
     // This wave's quads are gid, gid + total, ...  NS register sets of two quads
     // each take turns: while one is consumed the others' loads are in flight.  The
-    // very first quad is requested before the position is known (`spec_rows` rows
+    // quads of the first set are requested before the position is known (`spec_rows` rows
     // of the caches may be read; rows beyond the position are masked out below),
     // the others once it is, and only those that hold a position <= pos.
     float4 kS[NS][2][NV4], vS[NS][2][NV4];
@@ -353,8 +359,18 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
             }
         }
     };
-    const bool spec = gid * 4 < a.spec_rows;
-    if (spec) request(kS[0], vS[0], 0, a.spec_rows - 1, 0, gid + 1);
+    // Quads that lie inside the caches whatever the position are requested right away: those
+    // of the first set, and at short planned lengths (spec_sets = NS; the launch is then bound
+    // by the chain of memory round trips, not by what it reads) those of every set.
+    const uint32_t spec_quads = a.spec_rows / 4;  // whole quads below spec_rows
+    int n_spec[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const uint32_t q0 = (uint32_t)(2 * s) * total + gid;
+        n_spec[s] = ((uint32_t)s < a.spec_sets && q0 < spec_quads) ? (q0 + total < spec_quads ? 2 : 1) : 0;
+        if (n_spec[s])
+            request(kS[s], vS[s], 2 * s, a.spec_rows - 1, 0, n_spec[s] == 2 ? spec_quads : q0 + 1);
+    }
 
     float4 q[KM][NV4], acc[KM][NV4];
     float mx[KM], l[KM];
@@ -377,7 +393,7 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
         // no position for this workgroup: a neutral partial (max -inf, sum 0), so that the
         // merge need not know the position to tell which partials count
         if (threadIdx.x < KM) {
-            float *p = a.ws + ((size_t)(h0 + threadIdx.x) * a.n_wg_y + blockIdx.y) * (2 + HSP);
+            float *p = a.ws_ml + ((size_t)(h0 + threadIdx.x) * a.n_wg_y + blockIdx.y) * 2;
             p[0] = -INFINITY;
             p[1] = 0.f;
         }
@@ -407,9 +423,8 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
             }
         }
     };
-    request(kS[0], vS[0], 0, pos, spec ? 1 : 0, nq);
 #pragma unroll
-    for (int s = 1; s < NS; ++s) request(kS[s], vS[s], 2 * s, pos, 0, nq);
+    for (int s = 0; s < NS; ++s) request(kS[s], vS[s], 2 * s, pos, n_spec[s], nq);
     for (uint32_t i0 = 0; i0 * total + gid < nq; i0 += 2 * NS) {
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
@@ -470,12 +485,12 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
         if (a.n_wg_y == 1) {
             if (d < hs) a.xb[(size_t)(h0 + m) * hs + d] = o / L;
         } else {
-            float *p = a.ws + ((size_t)(h0 + m) * a.n_wg_y + blockIdx.y) * (2 + HSP);
+            const size_t slot = (size_t)(h0 + m) * a.n_wg_y + blockIdx.y;
             if (d == 0) {
-                p[0] = M;
-                p[1] = L;
+                a.ws_ml[slot * 2] = M;
+                a.ws_ml[slot * 2 + 1] = L;
             }
-            p[2 + d] = o;
+            a.ws[slot * HSP + d] = o;
         }
     }
 }
@@ -484,28 +499,29 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
 // results (max, sum, weighted V per workgroup and head) live in this fixed array instead of a
 // workspace from hipMalloc.  Every GPU the library runs on holds its own copy for the life of
 // the process.  In host code the array's name is only a handle for hipGetSymbolAddress: the
-// device address it returns, kept per device, is what kernels and copies are given.
+// device address it returns, kept in every context of that device, is what kernels and copies
+// are given.
 constexpr size_t kNoAllocScratchBytes = 2u << 20;
 static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
-constexpr int kMaxDevices = 64;
-static void *g_scratch_ptr[kMaxDevices];
 
-// The device address of `scratch` on the context's device (looked up once per device, with
-// that device current).
-int noalloc_scratch(wgml_ctx *ctx, float **ptr) {
-    if (ctx->device < 0 || ctx->device >= kMaxDevices)
-        return set_error(WGML_E_UNSUPPORTED, "wgml_attention_noalloc: device %d beyond %d",
-                         ctx->device, kMaxDevices);
-    if (!g_scratch_ptr[ctx->device]) {
-        WGML_CHECK_HIP(hipSetDevice(ctx->device));
-        void *p = nullptr;
-        WGML_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
-        if (!p) return set_error(WGML_E_HIP, "wgml_attention_noalloc: null scratch address");
-        g_scratch_ptr[ctx->device] = p;
-    }
-    *ptr = reinterpret_cast<float *>(g_scratch_ptr[ctx->device]);
+}  // namespace
+
+namespace wgml {
+
+// Looks up the device address of `scratch` on the context's device and keeps it in the
+// context.  Called by wgml_ctx_create with that device current, so that the entry point itself
+// neither switches devices nor touches the symbol table (it may run under stream capture).
+int resolve_noalloc_scratch(wgml_ctx *ctx) {
+    void *p = nullptr;
+    WGML_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return set_error(WGML_E_HIP, "wgml_ctx_create: null address for the fixed scratch array");
+    ctx->noalloc_scratch = reinterpret_cast<float *>(p);
     return WGML_OK;
 }
+
+}  // namespace wgml
+
+namespace {
 
 int ensure_ws(wgml_ctx *ctx, size_t bytes) {
     if (bytes <= ctx->attn_ws_bytes) return WGML_OK;
@@ -590,14 +606,19 @@ static bool fast_ok(const wgml_attn_params &p, bool aligned, bool wants_scores) 
 }
 
 constexpr uint32_t kWidePositions = 256;  // up to here one workgroup per head group
+// the most partial results per head that a consumer merges while it stages its input
+// (launch_gemv_quant with GemvEpilogue::partials)
+constexpr uint32_t kMaxFoldedPartials = 16;
 
 static int make_fast_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions,
-                          AttnPlan &pl) {
+                          AttnPlan &pl, bool folded = false) {
     const uint32_t hs = p.head_size;
     pl.nv = (int)((hs + 63) / 64);  // float4 per lane: 16 lanes x 4 floats x nv
     const int wide_tune = ctx->tuning[WGML_TUNE_ATTN_WIDE_POSITIONS];
     const uint32_t wide_limit = wide_tune > 0 ? (uint32_t)wide_tune : kWidePositions;
-    pl.wide = (plan_positions <= wide_limit && pl.nv <= 2) ? 1 : 0;
+    // (a caller that merges the partial results in its own next launch gets the split grid at
+    // every length: the merge launch is what made one workgroup per head the better plan)
+    pl.wide = (plan_positions <= wide_limit && pl.nv <= 2 && !(folded && wide_tune <= 0)) ? 1 : 0;
     pl.km = 1;
     if (p.kv_mul == 2 || p.kv_mul == 4) pl.km = (int)p.kv_mul;
     if (p.kv_mul == 8) pl.km = 4;
@@ -617,7 +638,16 @@ static int make_fast_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pla
     // quads per wave; measured on 32 x 128 and 12 x 64 heads, shorter shares only add
     // partial results for the merge to read)
     uint32_t n_wg_y = (2 * cu + pl.groups - 1) / pl.groups;
-    const uint32_t max_y = (plan_positions + 16 * WAVES - 1) / (16 * WAVES);
+    uint32_t max_y = (plan_positions + 16 * WAVES - 1) / (16 * WAVES);
+    // short contexts of a folded plan: up to one workgroup per CU
+    if (folded && plan_positions <= kWidePositions) {
+        max_y = (cu + pl.groups - 1) / pl.groups;
+        // four quads per wave: both register sets, all of them requested before the position
+        // is known; and few partial results, which every workgroup of the consumer merges
+        const uint32_t enough = (plan_positions + 16 * WAVES - 1) / (16 * WAVES);
+        if (max_y > enough) max_y = enough;
+        if (max_y > kMaxFoldedPartials) max_y = kMaxFoldedPartials;
+    }
     if (n_wg_y > max_y) n_wg_y = max_y;
     if (n_wg_y > (uint32_t)MERGE_MAX_Y) n_wg_y = MERGE_MAX_Y;  // what the merge takes in one go
     if (ctx->tuning[WGML_TUNE_ATTN_SPLITS] > 0) n_wg_y = (uint32_t)ctx->tuning[WGML_TUNE_ATTN_SPLITS];
@@ -656,9 +686,11 @@ int reserve_attention_workspace(wgml_ctx *ctx, const wgml_attn_params &p, uint32
     WGML_TRY(make_plan(ctx, p, plan_positions, pl));
     size_t bytes = (size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4;
     if (fast_ok(p, true, false)) {
-        WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl));
-        const size_t fast = (size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4;
-        if (fast > bytes) bytes = fast;
+        for (int folded = 0; folded < 2; ++folded) {
+            WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl, folded != 0));
+            const size_t fast = (size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4;
+            if (fast > bytes) bytes = fast;
+        }
     }
     return ensure_ws(ctx, bytes);
 }
@@ -669,8 +701,13 @@ int reserve_attention_workspace(wgml_ctx *ctx, const wgml_attn_params &p, uint32
 int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
                              uint32_t plan_positions, uint32_t cache_rows, const float *q,
                              const float *kc, const float *vc, float *att, float *xb,
-                             float *ext_ws, size_t ext_ws_bytes) {
+                             float *ext_ws, size_t ext_ws_bytes, AttnPartials *keep) {
     AttnPlan pl;
+    if (keep) *keep = AttnPartials{};
+    // a caller that merges the partial results itself gets the plan with partial results also
+    // where one workgroup per head would do, as long as there are few enough of them
+    const bool want_partials = keep != nullptr && att == nullptr;
+    if (!want_partials) keep = nullptr;
     auto workspace = [&](size_t bytes, float **ws) -> int {
         if (ext_ws) {
             if (bytes > ext_ws_bytes)
@@ -686,7 +723,12 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
     };
     const bool aligned = (((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) & 15u) == 0;
     if (fast_ok(p, aligned, att != nullptr)) {
-        WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl));
+        WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl, want_partials));
+        if (want_partials && (pl.wide || pl.n_wg_y > kMaxFoldedPartials)) {
+            // more partial results than a consumer merges: the plan with a merge launch
+            keep = nullptr;
+            WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl, false));
+        }
         AttnArgs a{};
         a.q = q;
         a.kc = kc;
@@ -700,10 +742,21 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
         a.pos = pos;
         a.n_wg_y = pl.n_wg_y;
         a.spec_rows = cache_rows;
+        a.spec_sets = plan_positions <= kWidePositions ? 8u : 1u;
         const dim3 grid(pl.groups, pl.n_wg_y);
         if (pl.wide) return launch_fast<16>(ctx, a, pl.nv, pl.km, grid);
         WGML_TRY(workspace((size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4, &a.ws));
+        a.ws_ml = a.ws + (size_t)p.n_heads * pl.n_wg_y * pl.hsp;
         WGML_TRY(launch_fast<WAVES>(ctx, a, pl.nv, pl.km, grid));
+        if (keep) {
+            // the caller's next launch merges the partial results while it stages its input
+            keep->o = a.ws;
+            keep->ml = a.ws_ml;
+            keep->n = pl.n_wg_y;
+            keep->hsp = pl.hsp;
+            keep->head_size = p.head_size;
+            return WGML_OK;
+        }
         if (pl.n_wg_y > 16)
             attn_merge_fast_kernel<64><<<dim3(p.n_heads), dim3(256), 0, ctx->stream>>>(a, pl.hsp);
         else
@@ -734,7 +787,10 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
     a.direct = (n_wg_y == 1 && att == nullptr) ? 1 : 0;
     a.ws = nullptr;
     const uint32_t hsp = pl.hsp;
-    if (!a.direct) WGML_TRY(workspace((size_t)p.n_heads * n_wg_y * (2 + hsp) * 4, &a.ws));
+    if (!a.direct) {
+        WGML_TRY(workspace((size_t)p.n_heads * n_wg_y * (2 + hsp) * 4, &a.ws));
+        a.ws_ml = a.ws + (size_t)p.n_heads * n_wg_y * hsp;
+    }
     const dim3 grid(groups, n_wg_y);
     switch (nv) {
     case 1: WGML_TRY(launch_nv<1>(ctx, a, km, grid)); break;
@@ -754,7 +810,7 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
 int launch_attention(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos, uint32_t cache_rows,
                      const float *q, const float *kc, const float *vc, float *att, float *xb) {
     return launch_attention_planned(ctx, p, pos, pos.ptr ? p.seq_len : pos.val + 1, cache_rows, q,
-                                    kc, vc, att, xb, nullptr, 0);
+                                    kc, vc, att, xb, nullptr, 0, nullptr);
 }
 
 }  // namespace wgml
@@ -763,7 +819,7 @@ extern "C" {
 
 static int attention_entry(const char *name, wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
                            wgml_view key_cache, wgml_view value_cache, wgml_view att, wgml_view xb,
-                           float *ext_ws, size_t ext_ws_bytes) {
+                           float *ext_ws, size_t ext_ws_bytes, AttnPartials *keep = nullptr) {
     WGML_REQUIRE(ctx && p, "%s: null argument", name);
     WGML_TRY(check_view(q, "attention: q"));
     WGML_TRY(check_view(key_cache, "attention: key_cache"));
@@ -794,12 +850,31 @@ static int attention_entry(const char *name, wgml_ctx *ctx, const wgml_attn_para
     return launch_attention_planned(ctx, *p, pos, p->pos + 1,
                                     (uint32_t)(rows < p->seq_len ? rows : p->seq_len), view_ptr(q),
                                     view_ptr(key_cache), view_ptr(value_cache), att_ptr,
-                                    view_ptr(xb), ext_ws, ext_ws_bytes);
+                                    view_ptr(xb), ext_ws, ext_ws_bytes, keep);
 }
 
 int wgml_attention(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q, wgml_view key_cache,
                    wgml_view value_cache, wgml_view att, wgml_view xb) {
     return attention_entry("wgml_attention", ctx, p, q, key_cache, value_cache, att, xb, nullptr, 0);
+}
+
+int wgml_attention_gemv_quant(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
+                              wgml_view key_cache, wgml_view value_cache, wgml_view xb,
+                              const wgml_qmat *m, wgml_view out, int accumulate) {
+    WGML_REQUIRE(ctx && p && m, "wgml_attention_gemv_quant: null argument");
+    WGML_TRY(check_view(out, "wgml_attention_gemv_quant: out"));
+    WGML_REQUIRE((uint64_t)m->ncols == (uint64_t)p->n_heads * p->head_size && out.len == m->nrows,
+                 "wgml_attention_gemv_quant: the matrix is %ux%u, attention gives %llu values and "
+                 "out holds %u", m->nrows, m->ncols, (unsigned long long)p->n_heads * p->head_size,
+                 out.len);
+    const wgml_view no_att{nullptr, 0, 0};
+    AttnPartials parts;
+    WGML_TRY(attention_entry("wgml_attention_gemv_quant", ctx, p, q, key_cache, value_cache, no_att,
+                             xb, nullptr, 0, gemv_partials_supported(ctx, m) ? &parts : nullptr));
+    GemvEpilogue e;
+    e.accumulate = accumulate ? 1 : 0;
+    e.partials = parts;
+    return launch_gemv_quant(ctx, view_ptr(out), m, view_ptr(xb), e);
 }
 
 // The same launches as wgml_attention with no `att` output, partial results in the library's
@@ -808,8 +883,8 @@ int wgml_attention(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q, wgml_v
 int wgml_attention_noalloc(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
                            wgml_view key_cache, wgml_view value_cache, wgml_view xb) {
     WGML_REQUIRE(ctx != nullptr, "wgml_attention_noalloc: null context");
-    float *ws = nullptr;
-    WGML_TRY(noalloc_scratch(ctx, &ws));
+    float *ws = ctx->noalloc_scratch;  // resolved when the context was created
+    WGML_REQUIRE(ws != nullptr, "wgml_attention_noalloc: the context holds no scratch address");
     const wgml_view no_att{nullptr, 0, 0};
     return attention_entry("wgml_attention_noalloc", ctx, p, q, key_cache, value_cache, no_att, xb,
                            ws, kNoAllocScratchBytes);

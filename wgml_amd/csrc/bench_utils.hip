@@ -6,7 +6,98 @@
 
 using namespace wgml;
 
+namespace {
+
+// A kernel that only reads: rows of 2304 bytes (4096 columns of Q4_K: sixteen 144-byte
+// super-blocks), one wave per row and step, each lane requesting the three 16-byte words of
+// its 64-element tile (header + two words of nibbles) with one tile in flight, rows dealt out
+// to the waves of the machine the way the GEMV kernels deal them out.  Nothing is computed and
+// nothing is stored: what it takes is what the memory system takes to deliver the bytes to
+// the compute units with this access pattern.
+__global__ __launch_bounds__(1024) void read_chain_kernel(const uint8_t *__restrict__ base,
+                                                          uint32_t nrows, uint32_t *sink) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const uint32_t gw = blockIdx.x * nw + wave, GW = gridDim.x * nw;
+    constexpr size_t kRowBytes = 16 * 144;
+    uint4 buf[3];
+    auto load = [&](uint32_t row) {
+        const uint8_t *blk = base + (size_t)row * kRowBytes + (lane >> 2) * 144;
+        buf[0] = *reinterpret_cast<const uint4 *>(blk);
+        buf[1] = *reinterpret_cast<const uint4 *>(blk + 16 + (lane & 3) * 32);
+        buf[2] = *reinterpret_cast<const uint4 *>(blk + 32 + (lane & 3) * 32);
+    };
+    uint32_t next = gw, acc = 0;
+    if (next < nrows) load(next);
+    next += GW;
+    for (uint32_t r = gw; r < nrows; r += GW) {
+        acc ^= buf[0].x ^ buf[1].y ^ buf[2].z ^ buf[1].w ^ buf[2].x;
+        if (next < nrows) load(next);
+        next += GW;
+    }
+    if (acc == 0x12345678u) sink[0] = acc;  // keeps the loads alive; the pool holds no such word
+}
+
+}  // namespace
+
 extern "C" {
+
+int wgml_bench_read_chain(wgml_ctx *ctx, uint32_t nrows, uint32_t iters, int use_graph,
+                          float *total_ms) {
+    WGML_REQUIRE(ctx && total_ms && nrows > 0 && iters > 0, "wgml_bench_read_chain: bad argument");
+    constexpr size_t kRowBytes = 16 * 144;
+    const size_t bytes = (size_t)nrows * kRowBytes;
+    const size_t pool_bytes = (size_t)1536 << 20;  // six times the 256 MB memory-side cache
+    WGML_REQUIRE(bytes * 2 <= pool_bytes, "wgml_bench_read_chain: %u rows exceed half the pool", nrows);
+    const uint32_t ncopies = (uint32_t)(pool_bytes / bytes);
+    uint8_t *pool = nullptr;
+    hipError_t e = hipMalloc((void **)&pool, pool_bytes + 4096);
+    if (e != hipSuccess)
+        return set_error(WGML_E_OOM, "wgml_bench_read_chain: hipMalloc: %s", hipGetErrorString(e));
+    uint32_t *sink = ctx->d_scalar + 16;
+    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
+    auto launch = [&](uint32_t i) {
+        read_chain_kernel<<<dim3(cu), dim3(1024), 0, ctx->stream>>>(
+            pool + (size_t)(i % ncopies) * bytes, nrows, sink);
+    };
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    e = hipMemsetAsync(pool, 1, pool_bytes, ctx->stream);
+    if (e == hipSuccess) {
+        launch(0);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    const bool graphed = use_graph && !graphs_disabled();
+    if (e == hipSuccess && graphed) {
+        e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+        if (e == hipSuccess) {
+            for (uint32_t i = 0; i < iters; ++i) launch(i);
+            e = hipStreamEndCapture(ctx->stream, &graph);
+        }
+        if (e == hipSuccess) e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+        if (e == hipSuccess) e = hipGraphLaunch(exec, ctx->stream);  // warm replay, untimed
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    }
+    if (e == hipSuccess) e = hipEventRecord(ctx->ev_start, ctx->stream);
+    if (e == hipSuccess) {
+        if (graphed) {
+            e = hipGraphLaunch(exec, ctx->stream);
+        } else {
+            for (uint32_t i = 0; i < iters; ++i) launch(i);
+            e = hipGetLastError();
+        }
+    }
+    if (e == hipSuccess) e = hipEventRecord(ctx->ev_stop, ctx->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(ctx->ev_stop);
+    if (e == hipSuccess) e = hipEventElapsedTime(total_ms, ctx->ev_start, ctx->ev_stop);
+    (void)hipStreamSynchronize(ctx->stream);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    (void)hipFree(pool);
+    ctx->launches += iters;
+    if (e != hipSuccess) return set_error(WGML_E_HIP, "wgml_bench_read_chain: %s", hipGetErrorString(e));
+    return WGML_OK;
+}
 
 int wgml_bench_gemv_quant(wgml_ctx *ctx, const wgml_qmat *const *mats, uint32_t n_mats,
                           wgml_view out, wgml_view v, uint32_t iters, int use_graph,

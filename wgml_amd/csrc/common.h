@@ -64,6 +64,9 @@ struct wgml_ctx {
     float *attn_ws = nullptr;
     size_t attn_ws_bytes = 0;
     std::vector<void *> retired;  // outgrown workspaces, freed with the context
+    // device address of the library's fixed scratch array on this context's device
+    // (wgml_attention_noalloc), looked up when the context is created
+    float *noalloc_scratch = nullptr;
     // f16 copy of the activations of a batched matrix product (+ one scale per token),
     // grown on demand
     void *prefill_xh = nullptr;
@@ -81,6 +84,7 @@ struct wgml_ctx {
     uint64_t launches = 0;  // kernels enqueued so far (diagnostics)
     // launch-shape overrides for sweeps and tests (wgml_ctx_set_tuning), 0 = heuristic
     int tuning[WGML_TUNE_COUNT] = {0};
+    uint64_t tuning_generation = 0;  // counts changes of `tuning` (recorded launches go stale)
     std::unordered_map<const void *, wgml_kernel_info> kernel_info;
     // Buffers, matrices and models keep their context alive: the device objects
     // are torn down when the last reference goes, whatever order handles are
@@ -111,7 +115,15 @@ struct wgml_qmat {
     uint8_t *base = nullptr;  // device allocation
     uint64_t alloc_bytes = 0;
     uint8_t *p0 = nullptr, *p1 = nullptr, *p2 = nullptr, *p3 = nullptr;  // planes
+    // upper bound on |w| over the dequantized matrix (Q8_0 / Q4_K / Q6_K; inf for NaN / inf
+    // scales): the batched products need it below kGemmMaxWeight
+    float max_abs = 0.f;
 };
+
+// The batched products (prefill.hip) expand weights into f16 times 2^8: a dequantized weight
+// beyond 65504 / 2^8 (the largest finite f16) would round to infinity there, so a matrix whose
+// bound exceeds this goes through the per-token kernels, which take any f32 value.
+constexpr float kGemmMaxWeight = 65504.f / 256.f;  // 255.875
 
 namespace wgml {
 
@@ -124,6 +136,7 @@ inline float *view_ptr(const wgml_view &v) {
 // being replayed as HIP graphs (same kernels, same order; useful under profilers
 // that cannot trace graph launches).
 bool graphs_disabled();
+int resolve_noalloc_scratch(wgml_ctx *ctx);  // attention.hip, where the array lives
 void ctx_retain(wgml_ctx *ctx);
 void ctx_release(wgml_ctx *ctx);
 
@@ -146,6 +159,16 @@ __device__ __forceinline__ uint32_t dyn_pos(const DynPos &p) {
 }
 
 // ---- internal launchers (async on ctx->stream, raw device pointers) --------
+// Unmerged output of a decode-attention launch: for every head, n partial results of the
+// flash-decoding scheme: weighted sums of V rows o[head][y][hsp] (hsp floats per row, the
+// first head_size used) and (running maximum, sum of weights) ml[head][y][2].  A partial with
+// maximum -inf is neutral and its o row is undefined.  The merged output is
+//   xb[head][d] = sum_y o[y][d] e^(m_y - M) / sum_y l_y e^(m_y - M),   M = max_y m_y.
+struct AttnPartials {
+    const float *o = nullptr, *ml = nullptr;
+    uint32_t n = 0, hsp = 0, head_size = 0;
+};
+
 struct GemvEpilogue {
     // out[r] = acc (+ bias[r]) (+ out[r] if accumulate)
     const float *bias = nullptr;
@@ -163,6 +186,10 @@ struct GemvEpilogue {
     // activation applied to acc + bias before it is stored: 0 none, 1 GELU (tanh form,
     // ops/unary.rs:106-110)
     int act = 0;
+    // partials.n > 0: the input vector is the merged attention output of these partial results
+    // (the `v` argument is ignored); integer-dot kernels of Q8_0 / Q4_K / Q6_K only, up to 16
+    // partial results per head
+    AttnPartials partials;
 };
 
 // One launch for up to three quantized matrices that consume the same vector
@@ -195,6 +222,8 @@ struct FusedGemv {
     const float *rope_cs = nullptr;
 };
 bool gemv_fused_supported(const wgml_qmat *m);
+// launch_gemv_quant takes GemvEpilogue::partials for this matrix (with the context's settings)
+bool gemv_partials_supported(const wgml_ctx *ctx, const wgml_qmat *m);
 int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f);
 
 int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float *v,
@@ -230,10 +259,15 @@ inline uint32_t plan_bucket(uint32_t pos, uint32_t seq_len, int *index) {
     return limit < seq_len ? limit : seq_len;
 }
 int reserve_attention_workspace(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions);
+// `keep` (optional): the launch may leave the attention output unmerged, as per-workgroup
+// partial results that the caller's next launch merges while it stages its input
+// (GemvEpilogue::partials); keep->n > 0 then, and xb has NOT been written.  keep->n == 0: xb
+// holds the result as usual.
 int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos pos,
                              uint32_t plan_positions, uint32_t cache_rows, const float *q,
                              const float *kc, const float *vc, float *att, float *xb,
-                             float *ext_ws = nullptr, size_t ext_ws_bytes = 0);
+                             float *ext_ws = nullptr, size_t ext_ws_bytes = 0,
+                             AttnPartials *keep = nullptr);
 int launch_silu(wgml_ctx *ctx, float *h1, const float *h2, uint32_t n);
 int launch_unary(wgml_ctx *ctx, int op, float *x, uint32_t n, const float *args4);
 int launch_op_assign(wgml_ctx *ctx, int op, float *a, const float *b, uint32_t n);

@@ -49,7 +49,81 @@ struct GemvParams {
     // integer-dot kernels: the first `active_waves` waves of every workgroup walk
     // the row-groups with stride gridDim.x * active_waves
     uint32_t active_waves;
+    // part_n > 0: x is the merged output of a decode-attention launch that left part_n partial
+    // results per head (AttnPartials in common.h); x itself is then not read
+    const float *part_o, *part_ml;
+    uint32_t part_n, part_hsp, part_hs;
 };
+
+// Merging attention partial results (see AttnPartials) for float4 number g4 of the merged
+// output: the partial results of its head are taken in eight at a time, the way an online
+// softmax takes in new scores.  PartialChunk holds one round of loads, so that a caller can
+// request it early and merge it later.
+struct PartialChunk {
+    float2 s[8];  // (maximum, sum of weights)
+    float4 v[8];  // weighted sums of V
+};
+__device__ __forceinline__ void load_partials(PartialChunk &c, const GemvParams &p, uint32_t g4,
+                                              uint32_t y0) {
+    const uint32_t e = g4 * 4, h = e / p.part_hs, d = e - h * p.part_hs, P = p.part_n;
+    const float *o = p.part_o + (size_t)h * P * p.part_hsp + d;
+    const float2 *ml = reinterpret_cast<const float2 *>(p.part_ml) + (size_t)h * P;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        c.s[k] = make_float2(-INFINITY, 0.f);
+        c.v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (y0 + k < P) {
+            c.s[k] = ml[y0 + k];
+            c.v[k] = *reinterpret_cast<const float4 *>(o + (size_t)(y0 + k) * p.part_hsp);
+        }
+    }
+}
+struct PartialState {
+    float M = -INFINITY, L = 0.f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+};
+__device__ __forceinline__ void merge_partials(PartialState &st, const PartialChunk &c) {
+    float Mc = st.M;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) Mc = fmaxf(Mc, c.s[k].x);
+    // the running state is rescaled to the new maximum (M = -inf only while nothing has been
+    // taken in, and then L and acc are zero)
+    const float r = st.M == -INFINITY ? 0.f : __expf(st.M - Mc);
+    st.L *= r;
+    st.acc.x *= r;
+    st.acc.y *= r;
+    st.acc.z *= r;
+    st.acc.w *= r;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        // a neutral partial (maximum -inf) has undefined values: they must not be touched
+        const bool live = c.s[k].x != -INFINITY;
+        const float wk = live ? __expf(c.s[k].x - Mc) : 0.f;
+        st.L = fmaf(c.s[k].y, wk, st.L);
+        st.acc.x = fmaf(live ? c.v[k].x : 0.f, wk, st.acc.x);
+        st.acc.y = fmaf(live ? c.v[k].y : 0.f, wk, st.acc.y);
+        st.acc.z = fmaf(live ? c.v[k].z : 0.f, wk, st.acc.z);
+        st.acc.w = fmaf(live ? c.v[k].w : 0.f, wk, st.acc.w);
+    }
+    st.M = Mc;
+}
+// `first`: the partial results 0..7, already requested; the others are fetched here.
+__device__ __forceinline__ float4 merged_partials(const GemvParams &p, uint32_t g4,
+                                                  const PartialChunk &first) {
+    PartialState st;
+    merge_partials(st, first);
+    for (uint32_t y0 = 8; y0 < p.part_n; y0 += 8) {
+        PartialChunk c;
+        load_partials(c, p, g4, y0);
+        merge_partials(st, c);
+    }
+    return make_float4(st.acc.x / st.L, st.acc.y / st.L, st.acc.z / st.L, st.acc.w / st.L);
+}
+__device__ __forceinline__ float4 merged_partials(const GemvParams &p, uint32_t g4) {
+    PartialChunk c;
+    load_partials(c, p, g4, 0);
+    return merged_partials(p, g4, c);
+}
 
 // Hides a value from the optimizer (no instruction is emitted).  Used on masked
 // 32-bit words so that the four bytes are converted with v_cvt_f32_ubyte0..3 of
@@ -916,7 +990,8 @@ struct PlainPolicy {
 // LDS: uint4 xq[step][plane(2)][chunk(PCH)][lane(64)], then float meta[tile][MF].
 // XREG: rows fit one step (ncols <= 64 tiles), so a lane's tile of x is the same
 // for every row and is read from LDS once instead of once per row.
-template <class F, int R, int D, bool XREG, class Policy>
+// XPART: x is not read from p.x but merged from attention partial results (merged_partials).
+template <class F, int R, int D, bool XREG, class Policy, bool XPART = false>
 __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, uint32_t wg,
                                              uint32_t nwg, uint32_t nw, uint32_t ngroups) {
     using WF = typename F::W;
@@ -969,8 +1044,9 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     // up to a microsecond apart, and the staging would otherwise end a whole prologue after
     // the last of them has arrived.  The other waves request their weights and wait at the
     // barrier.  (The folded LayerNorm has barriers of its own, so there every wave stages.)
+    // (Merging partial results is several loads per float4: every wave takes a share.)
     uint32_t ns = ((n4 + 64 * XP - 1) / (64 * XP) + 3) & ~3u;
-    if (ns > nwaves || p.ln_g) ns = nwaves;
+    if (ns > nwaves || p.ln_g || XPART) ns = nwaves;
     const bool stager = wave < ns;
     // a wave with neither rows nor a share of x is done: the barrier below counts only the
     // waves that are still running, and it would be the last to reach it
@@ -986,10 +1062,17 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
         nv[i] = make_float4(1.f, 1.f, 1.f, 1.f);
         bv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (g4 < n4) {
-            xv[i] = x4[g4];
+            if constexpr (!XPART) xv[i] = x4[g4];
             if (gsrc) nv[i] = gsrc[g4];
             if (p.ln_g && bsrc) bv[i] = bsrc[g4];
         }
+    }
+    // XPART: the first eight partial results of each thread's first float4 are requested here,
+    // ahead of the weights, and merged in stage_x once they are there (merging them here would
+    // put a memory round trip in front of the first weight request)
+    PartialChunk early;
+    if constexpr (XPART) {
+        if (tid < n4) load_partials(early, p, tid, 0);
     }
 
     // Stage x as 16-bit block fixed point (two int8 planes) + per-block scale and sum.
@@ -1002,6 +1085,12 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
         float out_scale = 1.f;
         uint32_t *xq32 = reinterpret_cast<uint32_t *>(xq);
         float ss = 0.f;
+        if constexpr (XPART) {  // every wave stages (sthreads == blockDim.x)
+            if (tid < n4) xv[0] = merged_partials(p, tid, early);
+#pragma unroll
+            for (int i = 1; i < XP; ++i)
+                if (tid + i * sthreads < n4) xv[i] = merged_partials(p, tid + i * sthreads);
+        }
         if (p.ln_g) {
             // LayerNorm folded in (host guarantees that the XP float4 per thread cover
             // x): mean, then variance about the mean (two exact passes over registers,
@@ -1107,7 +1196,8 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
             if (g4 < n4) stage_one(g4, xv[i], nv[i]);
         }
         for (uint32_t g4 = stager ? tid + XP * sthreads : n4; g4 < n4; g4 += sthreads)
-            stage_one(g4, x4[g4], p.norm_w ? nw4[g4] : make_float4(1.f, 1.f, 1.f, 1.f));
+            stage_one(g4, XPART ? merged_partials(p, g4) : x4[g4],
+                      p.norm_w ? nw4[g4] : make_float4(1.f, 1.f, 1.f, 1.f));
         if (p.norm_w && stager) {
             ss = wave_sum(ss);
             if (lane == 0) red[wave] = ss;
@@ -1249,14 +1339,16 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
 // MINW: waves per SIMD the register allocation must leave room for (MAXT / 256 = one
 // workgroup per CU; twice that caps the kernel at 64 vector registers, so that two
 // 1024-thread workgroups share a CU).
-template <class F, int R, int D, int MAXT, int MINW = MAXT / 256>
+template <class F, int R, int D, int MAXT, int MINW = MAXT / 256, bool XPART = false>
 __global__ __launch_bounds__(MAXT, MINW) void gemv_quant_i8_kernel(const GemvParams p) {
     PlainPolicy pol{p, nullptr, 0.f, 0.f, 0};
     const uint32_t ngroups = (p.nrows + R - 1) / R;
     if (p.ncols <= 64 * F::TILE)
-        gemv_i8_body<F, R, D, true>(p, pol, blockIdx.x, gridDim.x, p.active_waves, ngroups);
+        gemv_i8_body<F, R, D, true, PlainPolicy, XPART>(p, pol, blockIdx.x, gridDim.x, p.active_waves,
+                                                        ngroups);
     else
-        gemv_i8_body<F, R, D, false>(p, pol, blockIdx.x, gridDim.x, p.active_waves, ngroups);
+        gemv_i8_body<F, R, D, false, PlainPolicy, XPART>(p, pol, blockIdx.x, gridDim.x, p.active_waves,
+                                                         ngroups);
 }
 
 // ------------------------------------------------------------------------
@@ -1574,11 +1666,11 @@ WgPlan plan_groups(uint32_t ngroups, uint32_t max_wgs, uint32_t max_waves, uint3
     return {c, nw, wgs};
 }
 
-template <class F, int R, int D, int MAXT, int MINW = MAXT / 256>
+template <class F, int R, int D, int MAXT, int MINW = MAXT / 256, bool XPART = false>
 int launch_variant_i8(wgml_ctx *ctx, const GemvParams &p0, size_t lds) {
     int per_cu = 1;
-    WGML_TRY(blocks_per_cu(ctx, (const void *)gemv_quant_i8_kernel<F, R, D, MAXT, MINW>, MAXT, lds,
-                           &per_cu));
+    WGML_TRY(blocks_per_cu(ctx, (const void *)gemv_quant_i8_kernel<F, R, D, MAXT, MINW, XPART>, MAXT,
+                           lds, &per_cu));
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
     // One workgroup per CU with all its waves at work rather than two half-empty ones
     // (each would stage x), as long as that still gives every CU a workgroup (min_c).
@@ -1588,7 +1680,7 @@ int launch_variant_i8(wgml_ctx *ctx, const GemvParams &p0, size_t lds) {
     const WgPlan plan = plan_groups(ngroups, cu * (uint32_t)per_cu, MAXT / 64, 64 / R, min_c);
     GemvParams p = p0;
     p.active_waves = plan.active_waves;
-    gemv_quant_i8_kernel<F, R, D, MAXT, MINW><<<dim3(plan.wgs), dim3(MAXT), lds, ctx->stream>>>(p);
+    gemv_quant_i8_kernel<F, R, D, MAXT, MINW, XPART><<<dim3(plan.wgs), dim3(MAXT), lds, ctx->stream>>>(p);
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
@@ -1632,6 +1724,12 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
     if (p.ln_g && (p.ncols >> 2) > 3u * (uint32_t)waves * 64u)  // XP float4 per thread
         return set_error(WGML_E_UNSUPPORTED, "gemv_quant: %u columns are too many for the folded "
                                              "LayerNorm", p.ncols);
+    if (p.part_n) {
+        // the input is merged from attention partial results: one configuration (16-wave
+        // workgroups with room for the partial results in registers)
+        if constexpr (SWEEP) return launch_variant_i8<F, 1, 1, 1024, 4, true>(ctx, p, lds);
+        return set_error(WGML_E_UNSUPPORTED, "gemv_quant: no merging kernel for this format");
+    }
     if constexpr (SWEEP) {
         if (R == 2) {
             if (depth >= 2) return launch_rd_i8<F, 2, 2>(ctx, p, lds, waves);
@@ -1712,10 +1810,12 @@ int launch_gemv_f32(wgml_ctx *ctx, float *out, const float *a, uint32_t nrows, u
     return WGML_OK;
 }
 
+bool gemv_partials_supported(const wgml_ctx *ctx, const wgml_qmat *m) {
+    return gemv_fused_supported(m) && !ctx->tuning[WGML_TUNE_GEMV_F32_ACTIVATIONS];
+}
+
 int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float *v,
                       const GemvEpilogue &ep) {
-    if ((uintptr_t)v % 16 != 0)
-        return set_error(WGML_E_INVALID, "gemv_quant: the input vector must be 16-byte aligned");
     GemvParams p{};
     p.p0 = m->p0;
     p.p1 = m->p1;
@@ -1735,6 +1835,22 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
     p.ln_b = ep.ln_beta;
     p.act = ep.act;
     const bool main_fmt = m->type == WGML_Q4_K || m->type == WGML_Q6_K || m->type == WGML_Q8_0;
+    if (ep.partials.n) {
+        const AttnPartials &a = ep.partials;
+        if (!gemv_partials_supported(ctx, m) || a.n > 16 || !a.o || !a.ml || a.head_size == 0 ||
+            a.head_size % 4 != 0 || a.hsp < a.head_size || a.hsp % 4 != 0 ||
+            m->ncols % a.head_size != 0 || ep.ln_gamma)
+            return set_error(WGML_E_INVALID, "gemv_quant: these attention partial results cannot "
+                                             "be merged by this product");
+        p.part_o = a.o;
+        p.part_ml = a.ml;
+        p.part_n = a.n;
+        p.part_hsp = a.hsp;
+        p.part_hs = a.head_size;
+        p.x = nullptr;
+    } else if ((uintptr_t)v % 16 != 0) {
+        return set_error(WGML_E_INVALID, "gemv_quant: the input vector must be 16-byte aligned");
+    }
     if ((p.ln_g || p.act) &&
         (m->type == WGML_F32 || (main_fmt && ctx->tuning[WGML_TUNE_GEMV_F32_ACTIVATIONS])))
         return set_error(WGML_E_UNSUPPORTED,

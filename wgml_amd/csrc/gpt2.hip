@@ -38,6 +38,7 @@ struct wgml_gpt2 {
     uint64_t graph_launches[kMaxPlanBuckets] = {};  // launches of the recorded step
     int fusion = 1;  // 0: one launch per op group as before; 1: folded launches
     int graph_fusion = -1;
+    uint64_t graph_tuning = 0;  // the context's tuning generation the captures were made under
     uint64_t launches_last = 0;   // launches of the last step that ran
 };
 
@@ -281,13 +282,19 @@ int enqueue_step(wgml_gpt2 *m, bool dynamic, uint32_t token, uint32_t pos,
             WGML_CHECK_HIP(hipMemcpyAsync(w.value_cache + (size_t)pos * n, m->curr_2304 + 2 * n,
                                           (size_t)n * 4, hipMemcpyDeviceToDevice, ctx->stream));
         }
+        // with the fused launches, attention may leave per-workgroup partial results that the
+        // projection merges while it stages its input (no merge launch)
+        AttnPartials parts;
         WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, ap.seq_len, m->curr_2304,
-                                          w.key_cache, w.value_cache, nullptr, m->curr_768));
+                                          w.key_cache, w.value_cache, nullptr, m->curr_768, nullptr, 0,
+                                          fold && gemv_partials_supported(ctx, w.proj_w) ? &parts
+                                                                                         : nullptr));
         // layer_input += proj_w * attn + proj_b   (:372-395)
         {
             GemvEpilogue e;
             e.bias = w.proj_b;
             e.accumulate = 1;
+            e.partials = parts;
             WGML_TRY(launch_gemv_quant(ctx, m->layer_input, w.proj_w, m->curr_768, e));
         }
         if (fold) {
@@ -354,7 +361,8 @@ int build_graph(wgml_gpt2 *m, uint32_t pos) {
     wgml_ctx *ctx = m->ctx;
     const wgml_gpt2_params &p = m->p;
     const uint32_t n = p.n_embd;
-    if (m->graph_fusion != m->fusion) drop_graph(m);
+    // captures made at another fusion level or under other launch-shape overrides are stale
+    if (m->graph_fusion != m->fusion || m->graph_tuning != ctx->tuning_generation) drop_graph(m);
     int b = 0;
     const uint32_t plan = plan_bucket(pos, p.n_seq, &b);
     if (m->graph_exec[b]) return WGML_OK;
@@ -407,6 +415,7 @@ int build_graph(wgml_gpt2 *m, uint32_t pos) {
         return rc;
     }
     m->graph_fusion = m->fusion;
+    m->graph_tuning = ctx->tuning_generation;
     return WGML_OK;
 }
 

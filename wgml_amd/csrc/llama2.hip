@@ -47,6 +47,7 @@ struct wgml_llama2 {
     hipGraphExec_t graph_exec[kMaxPlanBuckets] = {};
     uint64_t graph_launches[kMaxPlanBuckets] = {};  // launches of the recorded step
     int graph_fusion = -1;
+    uint64_t graph_tuning = 0;  // the context's tuning generation the captures were made under
     // state of the batched prompt pass, allocated at its first use: one row per token
     // of a run (up to kPrefillMaxTokens)
     float *pf_x = nullptr, *pf_xb = nullptr, *pf_q = nullptr, *pf_hb = nullptr, *pf_hb2 = nullptr;
@@ -153,11 +154,19 @@ int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos,
             if (!rope_fused)
                 WGML_TRY(launch_rope(ctx, variant, m->head_size, kv_dim, dpos, c.rope_base_freq,
                                      m->q, dim, w.key_cache, kv_dim));
+            // attention leaves its output as per-workgroup partial results where it can, and
+            // the output projection merges them while it stages its input: no merge launch,
+            // and no reason to hold short contexts to one workgroup per head
+            AttnPartials parts;
             WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, ap.seq_len, m->q, w.key_cache,
-                                              w.value_cache, nullptr, m->xb));
+                                              w.value_cache, nullptr, m->xb, nullptr, 0,
+                                              gemv_partials_supported(ctx, w.attn_output) ? &parts
+                                                                                          : nullptr));
             GemvEpilogue eacc;
             eacc.accumulate = 1;
-            WGML_TRY(launch_gemv_quant(ctx, m->x, w.attn_output, m->xb, eacc));
+            GemvEpilogue ewo = eacc;
+            ewo.partials = parts;
+            WGML_TRY(launch_gemv_quant(ctx, m->x, w.attn_output, m->xb, ewo));
             FusedGemv g;
             g.njobs = 1;
             g.x = m->x;
@@ -271,7 +280,8 @@ int reserve_all_plans(wgml_llama2 *m) {
 int build_graph(wgml_llama2 *m, uint32_t pos) {
     wgml_ctx *ctx = m->ctx;
     const wgml_llama2_config &c = m->cfg;
-    if (m->graph_fusion != m->fusion) drop_graph(m);
+    // captures made at another fusion level or under other launch-shape overrides are stale
+    if (m->graph_fusion != m->fusion || m->graph_tuning != ctx->tuning_generation) drop_graph(m);
     int b = 0;
     const uint32_t plan = plan_bucket(pos, c.seq_len, &b);
     if (m->graph_exec[b]) return WGML_OK;
@@ -328,6 +338,7 @@ int build_graph(wgml_llama2 *m, uint32_t pos) {
                          hipGetErrorString(e));
     }
     m->graph_fusion = m->fusion;
+    m->graph_tuning = ctx->tuning_generation;
     return WGML_OK;
 }
 
@@ -376,8 +387,10 @@ int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint3
     return WGML_OK;
 }
 
+// The batched products take these formats, and weights that fit their f16 operands.
 bool gemm_supported(const wgml_qmat *q) {
-    return q->type == WGML_Q8_0 || q->type == WGML_Q4_K || q->type == WGML_Q6_K;
+    return (q->type == WGML_Q8_0 || q->type == WGML_Q4_K || q->type == WGML_Q6_K) &&
+           q->max_abs <= kGemmMaxWeight;
 }
 
 // One run of T <= kPrefillMaxTokens prompt tokens at positions pos0 .. pos0 + T - 1: the
@@ -655,8 +668,8 @@ int wgml_llama2_prefill(wgml_llama2 *m, const uint32_t *tokens, uint32_t n_token
                                    w.ffn_down})
             if (!gemm_supported(q)) batched = false;
     if (!batched) {
-        // The batched products exist for Q8_0, Q4_K and Q6_K.  A model with a matrix in another
-        // format takes the prompt the way the reference does: one step per token
+        // The batched products exist for Q8_0, Q4_K and Q6_K with weights of at most 255.875
+        // in magnitude.  A model with any other matrix takes the prompt the way the reference does: one step per token
         // (chat_llama2.rs:155-228), which leaves the same state.
         const uint64_t launches0 = ctx->launches;
         for (uint32_t i = 0; i < n_tokens; ++i) WGML_TRY(enqueue_step(m, false, tokens[i], start_pos + i));

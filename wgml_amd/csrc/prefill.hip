@@ -114,7 +114,8 @@ __device__ __forceinline__ half4 to_half4(float a, float b, float c, float d) {
 
 // Weights are expanded times 2^8 (an exact scaling, undone with the activations' factor at the
 // end): a low part f16(w - hi) of a typical weight (0.01 .. 0.1) is then a normal f16 number.
-// Weights of magnitude 256 and more would overflow f16; no model has them.
+// Weights beyond 65504 / 2^8 = 255.875 would overflow f16: launch_gemm_quant_multi refuses a
+// matrix whose bound (wgml_qmat::max_abs) exceeds that.
 constexpr float kWeightScale = 256.f;
 
 // The value as the compiler must take it: what follows is not merged with what computed it.
@@ -1299,6 +1300,11 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
         const wgml_qmat *q = targets[i].m;
         if (q->type != first->type || q->ncols != first->ncols)
             return set_error(WGML_E_INVALID, "gemm_quant: matrices of one launch differ in format or width");
+        if (!(q->max_abs <= kGemmMaxWeight))
+            return set_error(WGML_E_UNSUPPORTED,
+                             "gemm_quant: a weight of magnitude up to %g does not fit the f16 operands of "
+                             "the batched product (up to %g only); use the per-token product",
+                             (double)q->max_abs, (double)kGemmMaxWeight);
         // the kernel addresses a matrix plane with 32-bit lane offsets (at most 1 byte per element)
         if ((uint64_t)q->nrows * q->ncols >= (uint64_t(1) << 32) - 4096)
             return set_error(WGML_E_UNSUPPORTED, "gemm_quant: a matrix of %u x %u elements (below 2^32 only)",

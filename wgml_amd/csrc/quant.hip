@@ -49,6 +49,53 @@ __global__ void repack_q6_k(const uint16_t *__restrict__ raw, uint16_t *__restri
     else d[b] = v;
 }
 
+// ---- largest weight magnitude (computed once per matrix at load) --------------
+// An upper bound on |w| over the dequantized matrix: Q8_0 |d| max|q| (exact); Q4_K
+// max(|dmin m|, |d sc 15 - dmin m|) per sub-block (the two ends of the quant range); Q6_K
+// |d| |scale| 32 per sub-block.  The batched
+// products expand weights into f16 times 2^8 and need it within 255.875.  NaN / inf scales give
+// inf.  Non-negative floats order like their bit patterns, so the maximum is an atomicMax on
+// the bits.
+__device__ __forceinline__ float nan_to_inf(float v) { return v == v ? v : INFINITY; }
+
+__global__ void max_abs_kernel(int type, const uint8_t *__restrict__ p0,
+                               const uint8_t *__restrict__ p1, const uint8_t *__restrict__ p2,
+                               const uint8_t *__restrict__ p3, uint64_t nblocks,
+                               uint32_t *__restrict__ out_bits) {
+    float best = 0.f;
+    for (uint64_t b = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; b < nblocks;
+         b += (uint64_t)gridDim.x * blockDim.x) {
+        float v = 0.f;
+        if (type == WGML_Q8_0) {
+            const int8_t *q = reinterpret_cast<const int8_t *>(p0) + b * 32;
+            int m = 0;
+            for (int k = 0; k < 32; ++k) m = max(m, abs((int)q[k]));
+            v = fabsf(f16_bits_to_f32(reinterpret_cast<const uint16_t *>(p1)[b])) * (float)m;
+        } else if (type == WGML_Q4_K) {
+            const uint8_t *blk = p0 + b * Q4_K_BYTES;
+            const float d = f16_bits_to_f32(*(const uint16_t *)(blk + 0));
+            const float dmin = f16_bits_to_f32(*(const uint16_t *)(blk + 2));
+            for (uint32_t j = 0; j < 8; ++j) {
+                uint8_t sc, m;
+                get_scale_min_k4(j, blk + 4, sc, m);
+                // w = d sc q - dmin m is linear in q = 0..15: the extremes are its ends.  A term
+                // with a zero factor counts as zero even when the other factor is inf.
+                const float a = sc ? d * (float)sc * 15.f : 0.f, c = m ? dmin * (float)m : 0.f;
+                v = fmaxf(v, fmaxf(nan_to_inf(fabsf(c)), nan_to_inf(fabsf(a - c))));
+            }
+        } else {  // WGML_Q6_K
+            const float d = fabsf(f16_bits_to_f32(reinterpret_cast<const uint16_t *>(p3)[b]));
+            const int8_t *sc = reinterpret_cast<const int8_t *>(p2) + b * 16;
+            int m = 0;
+            for (int k = 0; k < 16; ++k) m = max(m, abs((int)sc[k]));
+            v = m ? d * (float)m * 32.f : 0.f;
+        }
+        best = fmaxf(best, nan_to_inf(v));
+    }
+    best = wave_max(best);
+    if ((threadIdx.x & 63) == 0) atomicMax(out_bits, __float_as_uint(best));
+}
+
 // ---- dequantization kernels ---------------------------------------------------
 
 // quantization.rs:38-41
@@ -368,6 +415,22 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
         (void)hipFree(raw);
         if (e != hipSuccess) return fail(e, "re-layout");
     }
+    if (type == WGML_Q8_0 || type == WGML_Q4_K || type == WGML_Q6_K) {
+        // the formats the batched products take: bound their largest weight once
+        uint32_t *bits = ctx->d_scalar + 8;
+        e = hipMemsetAsync(bits, 0, 4, ctx->stream);
+        if (e == hipSuccess) {
+            const uint64_t want = (nblocks + 255) / 256;
+            max_abs_kernel<<<dim3((unsigned)(want < 2048 ? want : 2048)), dim3(256), 0, ctx->stream>>>(
+                type, m->p0, m->p1, m->p2, m->p3, nblocks, bits);
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess)
+            e = hipMemcpyAsync(ctx->h_scalar + 8, bits, 4, hipMemcpyDeviceToHost, ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) return fail(e, "weight bound");
+        memcpy(&m->max_abs, ctx->h_scalar + 8, 4);
+    }
     *out = m;
     return WGML_OK;
 }
@@ -390,6 +453,12 @@ int wgml_quant_matrix_shape(const wgml_qmat *m, int *type, uint32_t *nrows, uint
 }
 
 uint64_t wgml_quant_matrix_gguf_bytes(const wgml_qmat *m) { return m ? m->gguf_bytes : 0; }
+
+int wgml_quant_matrix_weight_bound(const wgml_qmat *m, float *bound) {
+    WGML_REQUIRE(m && bound, "wgml_quant_matrix_weight_bound: null argument");
+    *bound = m->max_abs;
+    return WGML_OK;
+}
 
 int wgml_dequantize(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m) {
     WGML_REQUIRE(ctx && m, "wgml_dequantize: null argument");

@@ -88,6 +88,11 @@ int wgml_ctx_create(int device, wgml_ctx **out) {
         wgml_ctx_destroy(ctx);
         return set_error(WGML_E_HIP, "wgml_ctx_create: %s", hipGetErrorString(err));
     }
+    const int rc = resolve_noalloc_scratch(ctx);  // the device is current (hipSetDevice above)
+    if (rc != WGML_OK) {
+        wgml_ctx_destroy(ctx);
+        return rc;
+    }
     *out = ctx;
     return WGML_OK;
 }
@@ -108,6 +113,8 @@ int wgml_ctx_set_tuning(wgml_ctx *ctx, int key, int value) {
     switch (key) {
     case WGML_TUNE_GEMV_ROWS_PER_WAVE: ok = value >= 0 && value <= 2; break;
     case WGML_TUNE_GEMV_WAVES_PER_WG: ok = value == 0 || value == 4 || value == 8 || value == 12 || value == 16; break;
+    case WGML_TUNE_GEMV_WG_PER_CU: ok = value >= 0 && value <= 8; break;
+    case WGML_TUNE_ATTN_WIDE_POSITIONS: ok = value >= 0 && value <= (1 << 20); break;
     case WGML_TUNE_GEMV_DEPTH: ok = value >= 0 && value <= 4; break;
     case WGML_TUNE_GEMV_F32_ACTIVATIONS:
     case WGML_TUNE_PREFILL_ATTENTION_PER_TOKEN: ok = value == 0 || value == 1; break;
@@ -116,6 +123,8 @@ int wgml_ctx_set_tuning(wgml_ctx *ctx, int key, int value) {
     default: break;
     }
     WGML_REQUIRE(ok, "wgml_ctx_set_tuning: value %d is not valid for key %d", value, key);
+    // models drop the launch sequences they recorded under other settings (build_graph)
+    if (ctx->tuning[key] != value) ++ctx->tuning_generation;
     ctx->tuning[key] = value;
     return WGML_OK;
 }
@@ -123,6 +132,12 @@ int wgml_ctx_set_tuning(wgml_ctx *ctx, int key, int value) {
 int wgml_ctx_synchronize(wgml_ctx *ctx) {
     WGML_REQUIRE(ctx != nullptr, "wgml_ctx_synchronize: null context");
     WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    return WGML_OK;
+}
+
+int wgml_ctx_stream(wgml_ctx *ctx, void **stream) {
+    WGML_REQUIRE(ctx && stream, "wgml_ctx_stream: null argument");
+    *stream = ctx->stream;
     return WGML_OK;
 }
 

@@ -45,6 +45,13 @@ class GpuInstance:
     def synchronize(self) -> None:
         call("wgml_ctx_synchronize", self._h)
 
+    def stream(self) -> int:
+        """The context's HIP stream (a hipStream_t as an integer), on which every call of this
+        context enqueues its work in call order."""
+        st = C.c_void_p()
+        call("wgml_ctx_stream", self._h, C.byref(st))
+        return st.value or 0
+
     # keys of set_tuning (enum WGML_TUNE_* of the C header, same order)
     (TUNE_GEMV_ROWS_PER_WAVE, TUNE_GEMV_WAVES_PER_WG, TUNE_GEMV_WG_PER_CU, TUNE_GEMV_DEPTH,
      TUNE_GEMV_F32_ACTIVATIONS, TUNE_GEMM_K_SPLIT, TUNE_PREFILL_ATTENTION_PER_TOKEN,
@@ -201,6 +208,12 @@ class GpuQuantMatrix:
     def gguf_bytes(self) -> int:
         return _lib.lib.wgml_quant_matrix_gguf_bytes(self._h)
 
+    def weight_bound(self) -> float:
+        """Upper bound on |w| of the dequantized matrix (Q8_0 / Q4_K / Q6_K), else 0."""
+        b = C.c_float()
+        call("wgml_quant_matrix_weight_bound", self._h, C.byref(b))
+        return b.value
+
     def __del__(self):
         try:
             if self._h:
@@ -332,6 +345,18 @@ class BatchedMultiqueryAttention(_Op):
 
     def dispatch_multi(self, params, q, key_cache, value_cache, xb) -> None:
         self.dispatch(params, q, key_cache, value_cache, None, xb)
+
+    def dispatch_with_projection(self, params: BatchedMultiqueryAttentionParams, q: GpuVector,
+                                 key_cache: GpuVector, value_cache: GpuVector, xb: GpuVector,
+                                 m: "GpuQuantMatrix", out: GpuVector, accumulate: bool = False) -> None:
+        """`dispatch_multi` followed by `GemvQuant::dispatch(out, m, xb)` (and the `add_assign`
+        into `out` when `accumulate`), the pair of models/llama2/transformer.rs:366-383, as one
+        call: the product merges attention's partial results itself where the format allows.
+        `xb` is scratch."""
+        p = AttnParams(params.seq_len, params.kv_dim, params.kv_mul, params.n_heads,
+                       params.head_size, params.pos)
+        call("wgml_attention_gemv_quant", self.gpu.handle, C.byref(p), q.view(), key_cache.view(),
+             value_cache.view(), xb.view(), m.handle, out.view(), 1 if accumulate else 0)
 
     def dispatch_noalloc(self, params: BatchedMultiqueryAttentionParams, q: GpuVector,
                          key_cache: GpuVector, value_cache: GpuVector, xb: GpuVector) -> None:

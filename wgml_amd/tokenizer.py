@@ -106,7 +106,8 @@ def llama2_chat_prompt(messages: Sequence[dict], bos_token: str = "<s>", eos_tok
     `bos [INST] content [/INST]`, assistant turns ` content eos`; contents are stripped of
     surrounding whitespace; roles must alternate user / assistant.  (Only the text the template's
     branches emit is produced: the line breaks and indentation between its blocks, which depend
-    on the template engine's whitespace settings, are not.)"""
+    on the template engine's whitespace settings, are not.  `wgml_amd.ChatTemplate` renders that
+    template, or any other, whitespace included.)"""
     msgs = list(messages)
     system = ""
     if msgs and msgs[0]["role"] == "system":
