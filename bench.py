@@ -473,6 +473,9 @@ def main():
     name, n_cu = gpu.info()
     cores = host_cores()
     log(f"device: {name}, {n_cu} CUs; host cores for the CPU legs: {cores}")
+    for kv in args.tune:
+        key, value = kv.split("=")
+        gpu.set_tuning(getattr(gpu, "TUNE_" + key.upper()), int(value))
     if args.ceiling:
         print(json.dumps({"read_chain_in_graph": read_chain(gpu, True),
                           "read_chain_launch_by_launch": read_chain(gpu, False)}), flush=True)
@@ -529,9 +532,6 @@ def main():
         return
     model = Llama2(gpu, cfg).load(weights)
     prompt = W.prompt_tokens(4, n_prompt, cfg.vocab_size)
-    for kv in args.tune:
-        key, value = kv.split("=")
-        gpu.set_tuning(getattr(gpu, "TUNE_" + key.upper()), int(value))
     if args.prefill_only:
         gpu.set_gemm_precision(args.gemm_precision)
         model.prefill(prompt)
@@ -606,11 +606,9 @@ def main():
         f"{launches_per_token} launches/token; with a host read-back per token: "
         f"{tok_s_sync:.1f} tok/s")
 
-    # the same decode with fp32 activations in every GEMV (no 16-bit rounding of x): the
-    # fused launches exist for the integer-dot kernels only, so this is the level with one
-    # launch per matrix (norms still folded into the staging of x)
+    # the same decode with fp32 activations in every GEMV (no 16-bit rounding of x; the
+    # arithmetic of the reference's shaders), same fused launches
     gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 1)
-    model.set_fusion(2)
     n32 = min(args.steps, 64)
     model.decode_greedy(first, p0, 2)
     gpu.synchronize()
@@ -620,9 +618,8 @@ def main():
     dt32 = time.perf_counter() - t0
     fp32_act = {"tok_s": round(n32 / dt32, 2), "steps": n32, "launches_per_token": model.launches_per_token(),
                 "same_tokens_as_default": bool(np.array_equal(toks32, np.concatenate([wtoks, toks])[:n32])),
-                "note": "one launch per matrix (fusion level 2), fp32 activations staged in LDS"}
+                "note": "fp32 activations staged in LDS, the same fused launches as the default step"}
     gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 0)
-    model.set_fusion(3)
     log(f"decode with fp32 activations: {n32 / dt32:.1f} tok/s ({fp32_act['launches_per_token']} launches/token), "
         f"same tokens: {fp32_act['same_tokens_as_default']}")
 

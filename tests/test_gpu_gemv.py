@@ -306,3 +306,63 @@ def test_gemv_remaining_formats_all_ones_vector_sums_rows(gpu, qtype):
     x = np.ones(ncols, np.float32)
     got = gemv(gpu, qtype, raw, nrows, ncols, x)
     np.testing.assert_allclose(got, w.sum(axis=1), rtol=2e-5, atol=2e-5 * np.abs(w).sum(axis=1).max())
+
+
+def _fused(gpu, mats, partner, modes, nrows, x, norm_w=None):
+    """One fused launch through the benchmark entry point; returns the concatenated outputs."""
+    import ctypes as C
+
+    from wgml_amd._lib import call
+
+    nj = len(mats)
+    out = W.GpuVector.init(gpu, np.full(nj * nrows, np.nan, dtype=np.float32))
+    xv = W.GpuVector.init(gpu, x)
+    a = (C.c_void_p * nj)(*[m.handle for m in mats])
+    b = (C.c_void_p * nj)(*[(p.handle if p is not None else None) for p in partner]) if any(partner) else None
+    ms = C.c_float()
+    nwv = None
+    if norm_w is not None:
+        nwv = W.GpuVector.init(gpu, norm_w)
+        view = nwv.view()
+    call("wgml_bench_gemv_fused", gpu.handle, a, b, (C.c_int * nj)(*modes), nj, 1, out.view(), nrows,
+         xv.view(), C.byref(view) if norm_w is not None else None, 1, C.byref(ms))
+    return out.read().reshape(nj, nrows)
+
+
+def _rope0(v):
+    return v  # rotation at position 0 is the identity
+
+
+@pytest.mark.parametrize("qtype", QT + OTHER)
+@pytest.mark.parametrize("ncols", [512, 4096, 8192])
+def test_fused_launches_in_every_format(gpu, mode, qtype, ncols):
+    # Q/K/V-like (two rotated matrices + a plain one; position 0, so the rotation is the identity)
+    # and gate/up-like launches with all matrices in one format, for the nine quantized formats
+    # on the integer-dot path and the three main ones with fp32 activations
+    if mode == "f32_act" and qtype in OTHER:
+        pytest.skip("fp32 activations exist for Q8_0 / Q4_K / Q6_K")
+    nrows = 96
+    be = npref.BLOCK_ELEMS[qtype]
+    raws = [npref.random_blocks(qtype, nrows * ncols // be, seed=700 + qtype + i) for i in range(3)]
+    mats = [W.GpuQuantMatrix(gpu, qtype, nrows, ncols, r) for r in raws]
+    x = W.rng_normal(800 + ncols, ncols)
+    nw = (1.0 + 0.1 * W.rng_normal(801, ncols)).astype(np.float32)
+    xn = orc.rms_norm(x, nw, 1e-5)
+    refs = [orc.gemv_quant(qtype, r, nrows, ncols, xn)[1] for r in raws]
+    got = _fused(gpu, mats, [None] * 3, [1, 1, 0], nrows, x, nw)
+    for i in range(3):
+        ok, e = close(got[i], refs[i])
+        assert ok, (i, e)
+    got = _fused(gpu, mats[:1], mats[1:2], [2], nrows, x, nw)
+    g, u = refs[0], refs[1]
+    ok, e = close(got[0], u * (g / (1.0 + np.exp(-g))))
+    assert ok, e
+
+
+def test_fused_launch_refuses_a_mix_with_the_other_formats(gpu):
+    nrows, ncols = 32, 512
+    a = W.GpuQuantMatrix(gpu, W.Q4_K, nrows, ncols, weights(W.Q4_K, nrows, ncols, 1))
+    b = W.GpuQuantMatrix(gpu, W.Q5_K, nrows, ncols,
+                         npref.random_blocks(W.Q5_K, nrows * ncols // 256, seed=2))
+    with pytest.raises(W.WgmlError):
+        _fused(gpu, [a, b], [None, None], [0, 0], nrows, W.rng_normal(3, ncols))

@@ -121,6 +121,31 @@ def test_tuning_change_rerecords_the_step(gpu):
             gpu.set_tuning(key, bad)
 
 
+@pytest.mark.parametrize("scheme", ["q8_0", "q4_k", "q6_k", "q4_k_m"])
+@pytest.mark.parametrize("model_type", [LlamaModelType.Llama, LlamaModelType.Qwen2])
+def test_llama_micro_fp32_activations_fused(gpu, scheme, model_type):
+    # the step with fp32 activations in every GEMV (the arithmetic of the reference's shaders)
+    # takes the same fused launches as the integer-dot step: 5 launches per layer
+    gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 1)
+    try:
+        w = synth_llama(MICRO, seed=21, scheme=scheme)
+        spice(w, MICRO, 5, biases=model_type == LlamaModelType.Qwen2)
+        ref = orc.Llama2(w, rope_variant=model_type)
+        m = Llama2(gpu, MICRO, model_type).load(w)
+        for pos, t in enumerate([3, 300, 17, 17, 250, 9, 1]):
+            want = ref.forward(t, pos)
+            got = m.forward_logits(pos, t)
+            scale = float(np.abs(want).max())
+            assert np.abs(got - want).max() <= 2e-4 * scale, pos
+        extra = MICRO.n_layers if model_type == LlamaModelType.Qwen2 else 0  # Neox RoPE launch
+        assert m.launches_per_token() == 1 + 5 * MICRO.n_layers + 1 + extra
+        prompt = W.prompt_tokens(5, 4, MICRO.vocab_size)
+        want_t, _ = orc.Llama2(w, rope_variant=model_type).generate_greedy(prompt, 24)
+        assert np.array_equal(Llama2(gpu, MICRO, model_type).load(w).generate_greedy(prompt, 24), want_t)
+    finally:
+        gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 0)
+
+
 def test_llama_decode_from_uploaded_kv(gpu):
     # pre-filled cache then decode, as the long-context configuration does
     w = synth_llama(MICRO, seed=23, scheme="q6_k")
@@ -353,8 +378,10 @@ def test_gpt2_matrix_replaced_after_a_recorded_run(gpu):
 @pytest.mark.parametrize("qtype", [W.Q4_0, W.Q4_1, W.Q5_0, W.Q5_1, W.Q5_K, W.Q8_K])
 def test_llama_micro_in_the_remaining_block_formats(gpu, qtype):
     # a model whose matrices are all in one of the formats beside Q8_0 / Q4_K / Q6_K: they
-    # stay quantized on the device (one launch per matrix, no fused launches), the prompt pass
-    # falls back to one step per token; logits, KV rows and greedy tokens against the oracle
+    # stay quantized on the device and take the same fused Q/K/V and gate/up launches (a launch
+    # holds matrices of one format), the prompt pass falls back to one step per token; logits,
+    # KV rows and greedy tokens against the oracle, and the fused step against the step with
+    # one launch per matrix
     import npref
 
     w = synth_llama(MICRO, seed=61, scheme="f32")
@@ -372,9 +399,16 @@ def test_llama_micro_in_the_remaining_block_formats(gpu, qtype):
     for pos, t in enumerate(toks):
         ok, e = logits_close(m.forward_logits(pos, t), ref.forward(t, pos))
         assert ok, (pos, e)
+    assert m.launches_per_token() == 1 + 5 * MICRO.n_layers + 1  # embed, 5 per layer, output
     want_k = ref.key_cache(1)[:len(toks)].copy()
     np.testing.assert_allclose(m.kv_download(1, 0, 0, len(toks)), want_k, rtol=0,
                                atol=1e-3 * np.abs(want_k).max())
+    unfused = Llama2(gpu, MICRO).load(w)
+    unfused.set_fusion(2)
+    for pos, t in enumerate(toks):
+        lg = unfused.forward_logits(pos, t)
+    assert unfused.launches_per_token() > m.launches_per_token()
+    assert np.abs(lg - m.forward_logits(len(toks) - 1, toks[-1])).max() <= 1e-4 * np.abs(lg).max()
     m2 = Llama2(gpu, MICRO).load(w)
     m2.prefill(toks)  # no batched product for these formats: steps through the prompt
     ok, e = logits_close(m2.logits(), ref.forward(toks[-1], len(toks) - 1))

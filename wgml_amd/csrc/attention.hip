@@ -360,8 +360,9 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
         }
     };
     // Quads that lie inside the caches whatever the position are requested right away: those
-    // of the first set, and at short planned lengths (spec_sets = NS; the launch is then bound
-    // by the chain of memory round trips, not by what it reads) those of every set.
+    // of the first `spec_sets` register sets (one: a recorded step is planned for a range of
+    // positions whose lower end lies beyond what the first sets of all waves cover, so nothing
+    // is read in vain).
     const uint32_t spec_quads = a.spec_rows / 4;  // whole quads below spec_rows
     int n_spec[NS];
 #pragma unroll
@@ -609,6 +610,8 @@ constexpr uint32_t kWidePositions = 256;  // up to here one workgroup per head g
 // the most partial results per head that a consumer merges while it stages its input
 // (launch_gemv_quant with GemvEpilogue::partials)
 constexpr uint32_t kMaxFoldedPartials = 16;
+// ... and the most bytes of partial results that the consumer's workgroups together may read
+constexpr uint64_t kMaxFoldedBytes = 4u << 20;
 
 static int make_fast_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions,
                           AttnPlan &pl, bool folded = false) {
@@ -703,6 +706,8 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
                              const float *kc, const float *vc, float *att, float *xb,
                              float *ext_ws, size_t ext_ws_bytes, AttnPartials *keep) {
     AttnPlan pl;
+    const uint32_t consumer_wgs = keep && keep->consumer_wgs ? keep->consumer_wgs
+                                                             : (ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u);
     if (keep) *keep = AttnPartials{};
     // a caller that merges the partial results itself gets the plan with partial results also
     // where one workgroup per head would do, as long as there are few enough of them
@@ -724,8 +729,12 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
     const bool aligned = (((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) & 15u) == 0;
     if (fast_ok(p, aligned, att != nullptr)) {
         WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl, want_partials));
-        if (want_partials && (pl.wide || pl.n_wg_y > kMaxFoldedPartials)) {
-            // more partial results than a consumer merges: the plan with a merge launch
+        // Every workgroup of the consumer reads all partial results: what they pull through
+        // the L2s together must stay small beside the consumer's own weights, or the merge
+        // launch is the cheaper way (a 4096-wide vector with 8 partial results per head is
+        // 33 MB over 256 workgroups and costs the consumer 4 us; GPT-2's 768-wide one 1 MB).
+        const uint64_t pulled = (uint64_t)pl.n_wg_y * p.n_heads * pl.hsp * 4 * consumer_wgs;
+        if (want_partials && (pl.wide || pl.n_wg_y > kMaxFoldedPartials || pulled > kMaxFoldedBytes)) {
             keep = nullptr;
             WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl, false));
         }
@@ -742,7 +751,9 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
         a.pos = pos;
         a.n_wg_y = pl.n_wg_y;
         a.spec_rows = cache_rows;
-        a.spec_sets = plan_positions <= kWidePositions ? 8u : 1u;
+        // (all sets at short planned lengths was measured: the launch reads up to twice the
+        // rows it needs and gets slower, 5.1 against 4.7 us with four workgroups per head)
+        a.spec_sets = 1u;
         const dim3 grid(pl.groups, pl.n_wg_y);
         if (pl.wide) return launch_fast<16>(ctx, a, pl.nv, pl.km, grid);
         WGML_TRY(workspace((size_t)p.n_heads * pl.n_wg_y * (2 + pl.hsp) * 4, &a.ws));
@@ -869,6 +880,7 @@ int wgml_attention_gemv_quant(wgml_ctx *ctx, const wgml_attn_params *p, wgml_vie
                  out.len);
     const wgml_view no_att{nullptr, 0, 0};
     AttnPartials parts;
+    parts.consumer_wgs = gemv_consumer_wgs(ctx, m->nrows);
     WGML_TRY(attention_entry("wgml_attention_gemv_quant", ctx, p, q, key_cache, value_cache, no_att,
                              xb, nullptr, 0, gemv_partials_supported(ctx, m) ? &parts : nullptr));
     GemvEpilogue e;

@@ -167,7 +167,17 @@ __device__ __forceinline__ uint32_t dyn_pos(const DynPos &p) {
 struct AttnPartials {
     const float *o = nullptr, *ml = nullptr;
     uint32_t n = 0, hsp = 0, head_size = 0;
+    // in, for launch_attention_planned: workgroups of the launch that will merge the partial
+    // results (each reads all of them); 0 = one per compute unit
+    uint32_t consumer_wgs = 0;
 };
+
+// Workgroups launch_gemv_quant uses for a matrix of `nrows` rows, roughly: what a caller tells
+// launch_attention_planned about the consumer of its partial results.
+inline uint32_t gemv_consumer_wgs(const wgml_ctx *ctx, uint32_t nrows) {
+    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u, wgs = (nrows + 15) / 16;
+    return wgs < cu ? (wgs ? wgs : 1u) : cu;
+}
 
 struct GemvEpilogue {
     // out[r] = acc (+ bias[r]) (+ out[r] if accumulate)
@@ -222,6 +232,9 @@ struct FusedGemv {
     const float *rope_cs = nullptr;
 };
 bool gemv_fused_supported(const wgml_qmat *m);
+// the matrices can share one launch_gemv_fused (with the context's settings): one format, or a
+// mix of Q4_K / Q6_K / Q8_0
+bool gemv_fused_set_supported(const wgml_ctx *ctx, const wgml_qmat *const *mats, int n);
 // launch_gemv_quant takes GemvEpilogue::partials for this matrix (with the context's settings)
 bool gemv_partials_supported(const wgml_ctx *ctx, const wgml_qmat *m);
 int launch_gemv_fused(wgml_ctx *ctx, const FusedGemv &f);

@@ -52,7 +52,7 @@ struct GemvParams {
     // part_n > 0: x is the merged output of a decode-attention launch that left part_n partial
     // results per head (AttnPartials in common.h); x itself is then not read
     const float *part_o, *part_ml;
-    uint32_t part_n, part_hsp, part_hs;
+    uint32_t part_n, part_hsp, part_hs, part_hs_inv;  // part_hs_inv = ceil(2^32 / part_hs)
 };
 
 // Merging attention partial results (see AttnPartials) for float4 number g4 of the merged
@@ -65,27 +65,31 @@ struct PartialChunk {
 };
 __device__ __forceinline__ void load_partials(PartialChunk &c, const GemvParams &p, uint32_t g4,
                                               uint32_t y0) {
-    const uint32_t e = g4 * 4, h = e / p.part_hs, d = e - h * p.part_hs, P = p.part_n;
+    // h = e / head_size by multiplication with ceil(2^32 / head_size): exact for the e < 2^20
+    // and head sizes up to 256 that occur here
+    const uint32_t e = g4 * 4, h = __umulhi(e, p.part_hs_inv), d = e - h * p.part_hs, P = p.part_n;
     const float *o = p.part_o + (size_t)h * P * p.part_hsp + d;
     const float2 *ml = reinterpret_cast<const float2 *>(p.part_ml) + (size_t)h * P;
+    // The loads are unconditional (a partial result beyond the last one re-reads the last one
+    // and is masked out when it is merged): with a load under a condition the compiler cannot
+    // count the loads in flight, and the wait for these would also wait for the weight tiles
+    // requested after them.
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-        c.s[k] = make_float2(-INFINITY, 0.f);
-        c.v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (y0 + k < P) {
-            c.s[k] = ml[y0 + k];
-            c.v[k] = *reinterpret_cast<const float4 *>(o + (size_t)(y0 + k) * p.part_hsp);
-        }
+        const uint32_t y = min(y0 + (uint32_t)k, P - 1);
+        c.s[k] = ml[y];
+        c.v[k] = *reinterpret_cast<const float4 *>(o + (size_t)y * p.part_hsp);
     }
 }
 struct PartialState {
     float M = -INFINITY, L = 0.f;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 };
-__device__ __forceinline__ void merge_partials(PartialState &st, const PartialChunk &c) {
+// `n`: how many of the chunk's eight partial results exist.
+__device__ __forceinline__ void merge_partials(PartialState &st, const PartialChunk &c, uint32_t n) {
     float Mc = st.M;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) Mc = fmaxf(Mc, c.s[k].x);
+    for (int k = 0; k < 8; ++k) Mc = fmaxf(Mc, (uint32_t)k < n ? c.s[k].x : -INFINITY);
     // the running state is rescaled to the new maximum (M = -inf only while nothing has been
     // taken in, and then L and acc are zero)
     const float r = st.M == -INFINITY ? 0.f : __expf(st.M - Mc);
@@ -97,7 +101,7 @@ __device__ __forceinline__ void merge_partials(PartialState &st, const PartialCh
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         // a neutral partial (maximum -inf) has undefined values: they must not be touched
-        const bool live = c.s[k].x != -INFINITY;
+        const bool live = (uint32_t)k < n && c.s[k].x != -INFINITY;
         const float wk = live ? __expf(c.s[k].x - Mc) : 0.f;
         st.L = fmaf(c.s[k].y, wk, st.L);
         st.acc.x = fmaf(live ? c.v[k].x : 0.f, wk, st.acc.x);
@@ -111,11 +115,11 @@ __device__ __forceinline__ void merge_partials(PartialState &st, const PartialCh
 __device__ __forceinline__ float4 merged_partials(const GemvParams &p, uint32_t g4,
                                                   const PartialChunk &first) {
     PartialState st;
-    merge_partials(st, first);
+    merge_partials(st, first, p.part_n);
     for (uint32_t y0 = 8; y0 < p.part_n; y0 += 8) {
         PartialChunk c;
         load_partials(c, p, g4, y0);
-        merge_partials(st, c);
+        merge_partials(st, c, p.part_n - y0);
     }
     return make_float4(st.acc.x / st.L, st.acc.y / st.L, st.acc.z / st.L, st.acc.w / st.L);
 }
@@ -470,126 +474,6 @@ __device__ __forceinline__ void load_group(typename F::Row (&w)[R], const GemvPa
     }
 }
 
-template <int R>
-__device__ __forceinline__ void reduce_and_store(const GemvParams &p, uint32_t g,
-                                                 const float (&acc)[R], uint32_t lane) {
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const float total = wave_sum(acc[r]);
-        const uint32_t row = g * R + r;
-        if (lane == 0 && row < p.nrows) {
-            float *out = p.out;
-            if (p.dyn_pos) out += (size_t)(*p.dyn_pos) * p.out_pos_stride;
-            float v = total;
-            if (p.bias) v += p.bias[row];
-            if (p.accumulate) v += out[row];
-            out[row] = v;
-        }
-    }
-}
-
-// Persistent kernel: the grid is sized to the machine, every wave walks over
-// row-groups (R consecutive rows) with stride = total waves.  The (group, step)
-// pairs of a wave form one sequence that is software-pipelined D deep: D
-// register sets hold weights in flight (a ring, unrolled so that no register
-// copies are needed), so D-1 loads stay outstanding while one set is consumed.
-template <class F, int R, int D, int MAXT>
-__global__ __launch_bounds__(MAXT) void gemv_quant_kernel(const GemvParams p) {
-    extern __shared__ float4 smem[];
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t nwaves = blockDim.x >> 6;
-    const uint32_t ntiles = p.ncols / F::TILE;
-    const uint32_t nsteps = (ntiles + 63) >> 6;
-    const uint32_t ntiles_pad = nsteps << 6;
-    float *sums = reinterpret_cast<float *>(smem + (size_t)ntiles_pad * F::CHUNKS);
-
-    const uint32_t gw = blockIdx.x * nwaves + wave, GW = gridDim.x * nwaves;
-    const uint32_t ngroups = (p.nrows + R - 1) / R;
-    // this wave's sequence: groups gw, gw+GW, ... ; nsteps steps each
-    const uint32_t my_groups = gw < ngroups ? (ngroups - gw + GW - 1) / GW : 0;
-    const uint32_t n_it = my_groups * nsteps;
-
-    // Requests for the first D (group, step) pairs go out before x is staged:
-    // they do not depend on it.
-    typename F::Row w[D][R];
-    uint32_t lg = gw, ls = 0;  // (group, step) of the next load
-#pragma unroll
-    for (int d = 0; d < D; ++d) {
-        if ((uint32_t)d < n_it) {
-            const uint32_t tile = ls * 64 + lane;
-            if (tile < ntiles) load_group<F, R>(w[d], p, lg, tile);
-            if (++ls == nsteps) {
-                ls = 0;
-                lg += GW;
-            }
-        }
-    }
-
-    // Stage x (lane-transposed) and the per-tile sums of x.
-    __shared__ float red[16];
-    float rms = 1.f;
-    if (p.norm_w) rms = block_rms_scale(p, red);
-    const float4 *x4 = reinterpret_cast<const float4 *>(p.x);
-    const float4 *nw4 = reinterpret_cast<const float4 *>(p.norm_w);
-    const uint32_t n4 = p.ncols >> 2;
-    for (uint32_t g4 = tid; g4 < n4; g4 += blockDim.x) {
-        uint32_t tile, chunk;
-        F::map(g4, tile, chunk);
-        float4 v = x4[g4];
-        if (p.norm_w) v = apply_norm(v, rms, nw4[g4]);
-        smem[lds_slot<F>(tile, chunk)] = v;
-    }
-    __syncthreads();
-    {
-        constexpr int CPS = F::CHUNKS / F::NSUM;  // chunks per sum
-        for (uint32_t t = tid; t < ntiles * F::NSUM; t += blockDim.x) {
-            const uint32_t tile = t % ntiles, si = t / ntiles;
-            float a = 0.f;
-#pragma unroll
-            for (int c = 0; c < CPS; ++c) {
-                const float4 v = smem[lds_slot<F>(tile, si * CPS + c)];
-                a += (v.x + v.y) + (v.z + v.w);
-            }
-            sums[tile * F::NSUM + si] = a;
-        }
-        __syncthreads();
-    }
-    if (n_it == 0) return;
-
-    uint32_t g = gw, step = 0;  // (group, step) being computed
-    float acc[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = 0.f;
-    for (uint32_t base = 0; base < n_it; base += D) {
-#pragma unroll
-        for (int d = 0; d < D; ++d) {
-            const uint32_t it = base + d;
-            if (it < n_it) {
-                const uint32_t tile = step * 64 + lane;
-                if (tile < ntiles)
-                    F::template accumulate<R>(w[d], smem + (size_t)step * F::CHUNKS * 64 + lane,
-                                              sums + (size_t)tile * F::NSUM, tile, acc);
-                if (++step == nsteps) {
-                    reduce_and_store<R>(p, g, acc, lane);
-#pragma unroll
-                    for (int r = 0; r < R; ++r) acc[r] = 0.f;
-                    step = 0;
-                    g += GW;
-                }
-                // refill this register set with the pair D positions ahead
-                if (it + D < n_it) {
-                    const uint32_t tile_n = ls * 64 + lane;
-                    if (tile_n < ntiles) load_group<F, R>(w[d], p, lg, tile_n);
-                    if (++ls == nsteps) {
-                        ls = 0;
-                        lg += GW;
-                    }
-                }
-            }
-        }
-    }
-}
-
 // =========================================================================
 // Integer-dot path (default).  The fp32 path above spends ~3 VALU operations
 // per weight element (convert, multiply-add, unpack), which makes the 4-bit
@@ -622,6 +506,7 @@ __device__ __forceinline__ float dpp_max(float v) {
 // --- formats: TILE elements per lane, XB elements per activation block ------
 struct IFmtQ4K {
     using W = FmtQ4K;
+    static constexpr bool F32X = false;
     static constexpr int TILE = 64, XB = 32, NXB = 2, NSUM = 2;
     // element index e of x -> tile, element within tile, block within tile
     __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
@@ -687,6 +572,7 @@ struct IFmtQ4K {
 
 struct IFmtQ6K {
     using W = FmtQ6K;
+    static constexpr bool F32X = false;
     static constexpr int TILE = 64, XB = 16, NXB = 4, NSUM = 4;
     __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
         const uint32_t blk = e >> 8, i = (e >> 7) & 1, quarter = (e >> 5) & 3, s = (e >> 4) & 1;
@@ -750,6 +636,7 @@ struct IFmtQ6K {
 
 struct IFmtQ8_0 {
     using W = FmtQ8_0;
+    static constexpr bool F32X = false;
     static constexpr int TILE = 32, XB = 32, NXB = 1, NSUM = 0;
     __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
         tile = e >> 5;
@@ -796,6 +683,7 @@ __device__ __forceinline__ uint32_t spread_bit4(uint32_t b) {
 template <int BYTES, bool HAS_M, bool HAS_QH>
 struct IFmtLegacy {
     using W = FmtLegacy<BYTES, HAS_M, HAS_QH>;
+    static constexpr bool F32X = false;
     static constexpr int TILE = 32, XB = 32, NXB = 1, NSUM = 1;
     __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
         tile = e >> 5;
@@ -850,6 +738,7 @@ using IFmtQ5_1 = IFmtLegacy<24, true, true>;
 
 struct IFmtQ8K {
     using W = FmtQ8K;
+    static constexpr bool F32X = false;
     static constexpr int TILE = 32, XB = 32, NXB = 1, NSUM = 0;
     __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
         tile = e >> 5;
@@ -879,6 +768,7 @@ struct IFmtQ8K {
 
 struct IFmtQ5K {
     using W = FmtQ5K;
+    static constexpr bool F32X = false;
     static constexpr int TILE = 64, XB = 32, NXB = 2, NSUM = 2;
     __device__ static void locate(uint32_t e, uint32_t &tile, uint32_t &local, uint32_t &xb) {
         IFmtQ4K::locate(e, tile, local, xb);
@@ -930,6 +820,20 @@ struct IFmtQ5K {
             acc[r] += v;
         }
     }
+};
+
+// The fp32-activation twin of a format: x is staged in LDS as it is (RMSNorm / LayerNorm applied),
+// float4 xs[step][chunk][lane] followed by the NSUM sums of x per tile, and the weights are
+// expanded with one conversion and one multiply-add per element (FmtQ4K / FmtQ6K / FmtQ8_0
+// ::accumulate).  The arithmetic the reference's shaders use (ops/gemv_quant.rs:243-348 multiply
+// f32 vectors); about 3 VALU operations per weight against 1 on the integer-dot path.
+template <class WFmt>
+struct FFmt {
+    using W = WFmt;
+    static constexpr bool F32X = true;
+    static constexpr int TILE = WFmt::TILE, CHUNKS = WFmt::CHUNKS, NSUM = WFmt::NSUM;
+    static constexpr int XB = WFmt::TILE / WFmt::NSUM, NXB = 0;  // elements per sum of x
+    struct X {};
 };
 
 // Row source / sink of a plain single-matrix GEMV: group g = rows g*R .. g*R+R-1.
@@ -998,7 +902,8 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     constexpr int S = Policy::S;
     constexpr int PCH = F::TILE / 16;         // 16-byte chunks per plane per tile
     constexpr int MF = F::NXB + F::NSUM;      // floats of meta per tile
-    constexpr int LPB = F::XB / 4;            // lanes (float4) per activation block
+    constexpr int LPB = F::XB / 4;            // lanes (float4) per activation block (fp32: per sum)
+    static_assert(!(F::F32X && XREG), "fp32 activations are read from LDS tile by tile");
     extern __shared__ float4 smem4[];
     uint4 *xq = reinterpret_cast<uint4 *>(smem4);
     // the wave index is read through readfirstlane: the compiler then knows that it,
@@ -1011,6 +916,8 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     const uint32_t nsteps = (ntiles + 63) >> 6;
     const uint32_t ntiles_pad = nsteps << 6;
     float *meta = reinterpret_cast<float *>(xq + (size_t)ntiles_pad * 2 * PCH);
+    // fp32 activations: the tile sums follow the ntiles_pad * CHUNKS float4 of x
+    float *fsums = reinterpret_cast<float *>(smem4 + (size_t)ntiles_pad * (F::TILE / 4));
 
     const uint32_t first = wg * nw + wave, GW = nwg * nw;
     const uint32_t my_groups = (wave < nw && first < ngroups) ? (ngroups - first + GW - 1) / GW : 0;
@@ -1072,7 +979,10 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     // put a memory round trip in front of the first weight request)
     PartialChunk early;
     if constexpr (XPART) {
-        if (tid < n4) load_partials(early, p, tid, 0);
+        load_partials(early, p, min(tid, n4 - 1), 0);  // unconditional, see there
+        // the compiler must not move the weight requests below ahead of these (a wave's loads
+        // return in the order they were issued)
+        asm volatile("" ::: "memory");
     }
 
     // Stage x as 16-bit block fixed point (two int8 planes) + per-block scale and sum.
@@ -1135,6 +1045,30 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
             }
         }
         auto stage_one = [&](uint32_t g4, float4 v, const float4 nw) {
+            if constexpr (F::F32X) {
+                if (p.norm_w) {
+                    ss = fmaf(v.x, v.x, ss);
+                    ss = fmaf(v.y, v.y, ss);
+                    ss = fmaf(v.z, v.z, ss);
+                    ss = fmaf(v.w, v.w, ss);
+                    v.x *= nw.x;
+                    v.y *= nw.y;
+                    v.z *= nw.z;
+                    v.w *= nw.w;
+                }
+                uint32_t tile, chunk;
+                WF::map(g4, tile, chunk);
+                smem4[lds_slot<WF>(tile, chunk)] = v;
+                if constexpr (F::NSUM > 0) {
+                    // the sum of x over the LPB consecutive float4 that one sum covers
+                    float sum = (v.x + v.y) + (v.z + v.w);
+                    sum += dpp_f32<0xB1>(sum);
+                    sum += dpp_f32<0x4E>(sum);
+                    if (LPB == 8) sum += dpp_f32<0x141>(sum);
+                    constexpr int CPS = F::CHUNKS / F::NSUM;  // chunks per sum
+                    if ((g4 & (LPB - 1)) == 0) fsums[tile * F::NSUM + chunk / CPS] = sum;
+                }
+            } else {
             if (p.norm_w) {
                 ss = fmaf(v.x, v.x, ss);
                 ss = fmaf(v.y, v.y, ss);
@@ -1187,6 +1121,7 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
                 meta[tile * MF + xb] = amax * (1.0f / 32512.f);
                 if (F::NSUM > 0) meta[tile * MF + F::NXB + xb] = sum;
             }
+            }  // integer-dot staging
         };
         // ncols is a multiple of the tile size, so the LPB lanes of a block are
         // active together in every one of these branches
@@ -1261,7 +1196,9 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     // XREG: a lane without a tile (rows shorter than 64 tiles) keeps an all-zero tile of
     // x, so that the row loop needs no condition on the lane
     typename F::X xr{};
-    if (XREG && lane < ntiles) F::load_x(xr, xq + lane, meta + (size_t)lane * MF);
+    if constexpr (XREG) {
+        if (lane < ntiles) F::load_x(xr, xq + lane, meta + (size_t)lane * MF);
+    }
     uint32_t step = 0;  // step within the row being computed
     float acc[R];
 #pragma unroll
@@ -1272,7 +1209,11 @@ __device__ __forceinline__ void gemv_i8_body(const GemvParams &p, Policy &pol, u
     // reduction when the row is complete (no memory operation, LDS aside)
     auto compute = [&](typename WF::Row(&wd)[R]) {
         const uint32_t tile = step * 64 + lane;
-        if (XREG) {
+        if constexpr (F::F32X) {
+            if (tile < ntiles)
+                WF::template accumulate<R>(wd, smem4 + (size_t)step * F::CHUNKS * 64 + lane,
+                                           fsums + (size_t)tile * F::NSUM, tile, acc);
+        } else if constexpr (XREG) {
             F::template accumulate<R>(wd, xr, lane, acc);
         } else if (tile < ntiles) {
             typename F::X xt;
@@ -1343,12 +1284,15 @@ template <class F, int R, int D, int MAXT, int MINW = MAXT / 256, bool XPART = f
 __global__ __launch_bounds__(MAXT, MINW) void gemv_quant_i8_kernel(const GemvParams p) {
     PlainPolicy pol{p, nullptr, 0.f, 0.f, 0};
     const uint32_t ngroups = (p.nrows + R - 1) / R;
-    if (p.ncols <= 64 * F::TILE)
-        gemv_i8_body<F, R, D, true, PlainPolicy, XPART>(p, pol, blockIdx.x, gridDim.x, p.active_waves,
-                                                        ngroups);
-    else
-        gemv_i8_body<F, R, D, false, PlainPolicy, XPART>(p, pol, blockIdx.x, gridDim.x, p.active_waves,
-                                                         ngroups);
+    if constexpr (!F::F32X) {
+        if (p.ncols <= 64 * F::TILE) {
+            gemv_i8_body<F, R, D, true, PlainPolicy, XPART>(p, pol, blockIdx.x, gridDim.x,
+                                                            p.active_waves, ngroups);
+            return;
+        }
+    }
+    gemv_i8_body<F, R, D, false, PlainPolicy, XPART>(p, pol, blockIdx.x, gridDim.x, p.active_waves,
+                                                     ngroups);
 }
 
 // ------------------------------------------------------------------------
@@ -1500,18 +1444,36 @@ __device__ __forceinline__ void fused_job_body(const FusedParams &P, const GemvJ
     pb.p0 = j.b0; pb.p1 = j.b1; pb.p2 = j.b2; pb.p3 = j.b3;
     JobPolicy pol{j, pa, pb, P.pos, P.head_size, P.rope_base, P.rope_cs, 0.f, 0.f, make_float2(1.f, 0.f), 0};
     const uint32_t ngroups = j.mode == JOB_SILU ? j.nrows : (j.nrows + 1) / 2;
-    if (P.ncols <= 64 * F::TILE)
-        gemv_i8_body<F, 2, D, true>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves,
-                                    ngroups);
-    else
-        gemv_i8_body<F, 2, D, false>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves,
-                                     ngroups);
+    if constexpr (!F::F32X) {
+        if (P.ncols <= 64 * F::TILE) {
+            gemv_i8_body<F, 2, D, true>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves,
+                                        ngroups);
+            return;
+        }
+    }
+    gemv_i8_body<F, 2, D, false>(xp, pol, blockIdx.x - j.wg_begin, j.wg_count, j.active_waves, ngroups);
 }
 
+// The format struct of a GGUF type: integer-dot (F32 false) or fp32-activation.
+template <int TYPE, bool F32> struct FusedFmt;
+template <> struct FusedFmt<WGML_Q4_K, false> { using T = IFmtQ4K; };
+template <> struct FusedFmt<WGML_Q6_K, false> { using T = IFmtQ6K; };
+template <> struct FusedFmt<WGML_Q8_0, false> { using T = IFmtQ8_0; };
+template <> struct FusedFmt<WGML_Q4_K, true> { using T = FFmt<FmtQ4K>; };
+template <> struct FusedFmt<WGML_Q6_K, true> { using T = FFmt<FmtQ6K>; };
+template <> struct FusedFmt<WGML_Q8_0, true> { using T = FFmt<FmtQ8_0>; };
+template <> struct FusedFmt<WGML_Q5_K, false> { using T = IFmtQ5K; };
+template <> struct FusedFmt<WGML_Q8_K, false> { using T = IFmtQ8K; };
+template <> struct FusedFmt<WGML_Q4_0, false> { using T = IFmtQ4_0; };
+template <> struct FusedFmt<WGML_Q4_1, false> { using T = IFmtQ4_1; };
+template <> struct FusedFmt<WGML_Q5_0, false> { using T = IFmtQ5_0; };
+template <> struct FusedFmt<WGML_Q5_1, false> { using T = IFmtQ5_1; };
+
 // MINW: waves per SIMD the register budget must allow.  FMT: 0 = the matrices of
-// a launch may differ in format (decided per workgroup), else the one format all
-// of them have (smaller code, registers of that format only).
-template <int D, int MAXT, int MINW, int FMT>
+// a launch may differ in format (Q4_K / Q6_K / Q8_0, decided per workgroup), else the one
+// format all of them have (smaller code, registers of that format only).  F32: fp32
+// activations (the three main formats only).
+template <int D, int MAXT, int MINW, int FMT, bool F32 = false>
 __global__ __launch_bounds__(MAXT, MINW) void gemv_fused_kernel(const FusedParams P) {
     // All three job records are fetched at once and the workgroup's own is picked field by
     // field afterwards: indexing the kernel arguments with the job number would put a second
@@ -1527,17 +1489,13 @@ __global__ __launch_bounds__(MAXT, MINW) void gemv_fused_kernel(const FusedParam
                     WGML_PICK(mode), WGML_PICK(accumulate), WGML_PICK(out_pos_stride),
                     WGML_PICK(wg_begin), WGML_PICK(wg_count), WGML_PICK(active_waves)};
 #undef WGML_PICK
-    if (FMT == WGML_Q4_K) {
-        fused_job_body<IFmtQ4K, D>(P, j);
-    } else if (FMT == WGML_Q6_K) {
-        fused_job_body<IFmtQ6K, D>(P, j);
-    } else if (FMT == WGML_Q8_0) {
-        fused_job_body<IFmtQ8_0, D>(P, j);
+    if constexpr (FMT != 0) {
+        fused_job_body<typename FusedFmt<FMT, F32>::T, D>(P, j);
     } else {
         switch (j.type) {
-        case WGML_Q4_K: fused_job_body<IFmtQ4K, D>(P, j); break;
-        case WGML_Q6_K: fused_job_body<IFmtQ6K, D>(P, j); break;
-        default: fused_job_body<IFmtQ8_0, D>(P, j); break;
+        case WGML_Q4_K: fused_job_body<typename FusedFmt<WGML_Q4_K, F32>::T, D>(P, j); break;
+        case WGML_Q6_K: fused_job_body<typename FusedFmt<WGML_Q6_K, F32>::T, D>(P, j); break;
+        default: fused_job_body<typename FusedFmt<WGML_Q8_0, F32>::T, D>(P, j); break;
         }
     }
 }
@@ -1617,24 +1575,6 @@ int blocks_per_cu(wgml_ctx *ctx, const void *fn, int threads, size_t lds, int *b
     *blocks = ki.blocks_per_cu;
     const int cap = ctx->tuning[WGML_TUNE_GEMV_WG_PER_CU];
     if (cap > 0 && cap < *blocks) *blocks = cap;
-    return WGML_OK;
-}
-
-template <class F, int R, int D, int MAXT>
-int launch_variant(wgml_ctx *ctx, const GemvParams &p, size_t lds) {
-    int per_cu = 1;
-    WGML_TRY(blocks_per_cu(ctx, (const void *)gemv_quant_kernel<F, R, D, MAXT>, MAXT, lds, &per_cu));
-    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
-    const uint32_t nwaves = MAXT / 64;
-    const uint32_t ngroups = (p.nrows + R - 1) / R;
-    // Balanced persistent grid: every wave gets k or k-1 groups, k minimal such
-    // that the grid fits the machine.
-    const uint32_t resident_waves = cu * (uint32_t)per_cu * nwaves;
-    const uint32_t k = (ngroups + resident_waves - 1) / resident_waves;
-    uint32_t grid = (ngroups + nwaves * k - 1) / (nwaves * k);
-    gemv_quant_kernel<F, R, D, MAXT><<<dim3(grid), dim3(MAXT), lds, ctx->stream>>>(p);
-    WGML_CHECK_LAUNCH();
-    ctx->launches++;
     return WGML_OK;
 }
 
@@ -1751,34 +1691,26 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
     }
 }
 
-// fp32-activation path: one configuration per format
-template <class F, int R, int D>
-int launch_rd(wgml_ctx *ctx, const GemvParams &p, size_t lds, int) {
-    return launch_variant<F, R, D, 512>(ctx, p, lds);
-}
-
-template <class F, int R>
-int launch_r(wgml_ctx *ctx, const GemvParams &p, size_t lds, int waves, int) {
-    return launch_rd<F, R, 2>(ctx, p, lds, waves);
-}
-
-template <class F>
-int launch_fmt(wgml_ctx *ctx, const GemvParams &p) {
-    constexpr int NS = F::NSUM;
+// fp32-activation path: the same body with x staged as floats.  16-wave workgroups, one per
+// compute unit (the expansion needs the registers), or 8-wave workgroups with two tiles in flight
+// per wave when WGML_TUNE_GEMV_WAVES_PER_WG is 8.
+template <class WF>
+int launch_fmt_f32(wgml_ctx *ctx, const GemvParams &p) {
+    using F = FFmt<WF>;
     const uint32_t ntiles = p.ncols / F::TILE;
     const uint32_t ntiles_pad = ((ntiles + 63) / 64) * 64;
-    const size_t lds = (size_t)ntiles_pad * F::CHUNKS * 16 + (size_t)ntiles_pad * NS * 4;
+    const size_t lds = (size_t)ntiles_pad * F::CHUNKS * 16 + (size_t)ntiles_pad * F::NSUM * 4;
     if (lds > kMaxLds)
         return set_error(WGML_E_UNSUPPORTED,
                          "gemv_quant: %u columns need %zu bytes of LDS (limit %zu)", p.ncols, lds,
                          kMaxLds);
-    int R = ctx->tuning[WGML_TUNE_GEMV_ROWS_PER_WAVE], waves = ctx->tuning[WGML_TUNE_GEMV_WAVES_PER_WG],
-        depth = ctx->tuning[WGML_TUNE_GEMV_DEPTH];
-    if (!R) R = 1;
-    if (!waves) waves = 8;
-    if (!depth) depth = 2;
-    (void)R;
-    return launch_r<F, 1>(ctx, p, lds, waves, depth);
+    if (p.part_n) return launch_variant_i8<F, 1, 1, 1024, 4, true>(ctx, p, lds);
+    const int waves = ctx->tuning[WGML_TUNE_GEMV_WAVES_PER_WG];
+    if (p.ln_g && (p.ncols >> 2) > 3u * (waves == 8 ? 512u : 1024u))  // XP float4 per thread
+        return set_error(WGML_E_UNSUPPORTED, "gemv_quant: %u columns are too many for the folded "
+                                             "LayerNorm", p.ncols);
+    if (waves == 8) return launch_variant_i8<F, 1, 2, 512, 2>(ctx, p, lds);
+    return launch_variant_i8<F, 1, 1, 1024, 4>(ctx, p, lds);
 }
 
 }  // namespace
@@ -1810,8 +1742,8 @@ int launch_gemv_f32(wgml_ctx *ctx, float *out, const float *a, uint32_t nrows, u
     return WGML_OK;
 }
 
-bool gemv_partials_supported(const wgml_ctx *ctx, const wgml_qmat *m) {
-    return gemv_fused_supported(m) && !ctx->tuning[WGML_TUNE_GEMV_F32_ACTIVATIONS];
+bool gemv_partials_supported(const wgml_ctx *, const wgml_qmat *m) {
+    return m && (m->type == WGML_Q4_K || m->type == WGML_Q6_K || m->type == WGML_Q8_0);
 }
 
 int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float *v,
@@ -1839,7 +1771,7 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
         const AttnPartials &a = ep.partials;
         if (!gemv_partials_supported(ctx, m) || a.n > 16 || !a.o || !a.ml || a.head_size == 0 ||
             a.head_size % 4 != 0 || a.hsp < a.head_size || a.hsp % 4 != 0 ||
-            m->ncols % a.head_size != 0 || ep.ln_gamma)
+            m->ncols % a.head_size != 0 || m->ncols >= (1u << 20) || a.head_size > 4096 || ep.ln_gamma)
             return set_error(WGML_E_INVALID, "gemv_quant: these attention partial results cannot "
                                              "be merged by this product");
         p.part_o = a.o;
@@ -1847,14 +1779,15 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
         p.part_n = a.n;
         p.part_hsp = a.hsp;
         p.part_hs = a.head_size;
+        p.part_hs_inv = (uint32_t)(((uint64_t(1) << 32) + a.head_size - 1) / a.head_size);
         p.x = nullptr;
     } else if ((uintptr_t)v % 16 != 0) {
         return set_error(WGML_E_INVALID, "gemv_quant: the input vector must be 16-byte aligned");
     }
-    if ((p.ln_g || p.act) &&
-        (m->type == WGML_F32 || (main_fmt && ctx->tuning[WGML_TUNE_GEMV_F32_ACTIVATIONS])))
+    (void)main_fmt;
+    if ((p.ln_g || p.act) && m->type == WGML_F32)
         return set_error(WGML_E_UNSUPPORTED,
-                         "gemv_quant: LayerNorm / activation folding needs the integer-dot path");
+                         "gemv_quant: LayerNorm / activation folding needs a quantized matrix");
     if (m->type == WGML_F32) {
         const size_t lds = (size_t)m->ncols * 4;
         if (lds > kMaxLds)
@@ -1885,27 +1818,55 @@ int launch_gemv_quant(wgml_ctx *ctx, float *out, const wgml_qmat *m, const float
         }
     }
     switch (m->type) {
-    case WGML_Q4_K: return launch_fmt<FmtQ4K>(ctx, p);
-    case WGML_Q6_K: return launch_fmt<FmtQ6K>(ctx, p);
-    case WGML_Q8_0: return launch_fmt<FmtQ8_0>(ctx, p);
+    case WGML_Q4_K: return launch_fmt_f32<FmtQ4K>(ctx, p);
+    case WGML_Q6_K: return launch_fmt_f32<FmtQ6K>(ctx, p);
+    case WGML_Q8_0: return launch_fmt_f32<FmtQ8_0>(ctx, p);
     default: return set_error(WGML_E_UNSUPPORTED, "gemv_quant: unsupported type %d", m->type);
     }
 }
 
-static size_t lds_bytes_i8(int type, uint32_t ncols) {
-    uint32_t tile, pch, mf;
+// LDS a workgroup of the shared body needs for x: two int8 planes + per-tile scales and sums
+// (integer dot), or the floats themselves + per-tile sums (fp32 activations).
+template <class F>
+static size_t lds_bytes_of(uint32_t ncols) {
+    const uint32_t ntiles = ncols / F::TILE;
+    const size_t ntiles_pad = ((ntiles + 63) / 64) * 64;
+    if (F::F32X) return ntiles_pad * (F::TILE / 4) * 16 + ntiles_pad * F::NSUM * 4;
+    return ntiles_pad * 2 * (F::TILE / 16) * 16 + ntiles_pad * (F::NXB + F::NSUM) * 4;
+}
+static size_t lds_bytes_fused(int type, uint32_t ncols, bool f32) {
     switch (type) {
-    case WGML_Q4_K: tile = 64; pch = 4; mf = IFmtQ4K::NXB + IFmtQ4K::NSUM; break;
-    case WGML_Q6_K: tile = 64; pch = 4; mf = IFmtQ6K::NXB + IFmtQ6K::NSUM; break;
-    default: tile = 32; pch = 2; mf = IFmtQ8_0::NXB + IFmtQ8_0::NSUM; break;
+    case WGML_Q4_K: return f32 ? lds_bytes_of<FFmt<FmtQ4K>>(ncols) : lds_bytes_of<IFmtQ4K>(ncols);
+    case WGML_Q6_K: return f32 ? lds_bytes_of<FFmt<FmtQ6K>>(ncols) : lds_bytes_of<IFmtQ6K>(ncols);
+    case WGML_Q8_0: return f32 ? lds_bytes_of<FFmt<FmtQ8_0>>(ncols) : lds_bytes_of<IFmtQ8_0>(ncols);
+    case WGML_Q5_K: return lds_bytes_of<IFmtQ5K>(ncols);
+    case WGML_Q8_K: return lds_bytes_of<IFmtQ8K>(ncols);
+    default: return lds_bytes_of<IFmtQ4_0>(ncols);  // the four 32-element block formats
     }
-    const uint32_t ntiles = ncols / tile;
-    const uint32_t ntiles_pad = ((ntiles + 63) / 64) * 64;
-    return (size_t)ntiles_pad * 2 * pch * 16 + (size_t)ntiles_pad * mf * 4;
 }
 
+static bool main_format(int type) { return type == WGML_Q4_K || type == WGML_Q6_K || type == WGML_Q8_0; }
+
 bool gemv_fused_supported(const wgml_qmat *m) {
-    return m && (m->type == WGML_Q4_K || m->type == WGML_Q6_K || m->type == WGML_Q8_0);
+    if (!m) return false;
+    switch (m->type) {
+    case WGML_Q4_K: case WGML_Q6_K: case WGML_Q8_0: case WGML_Q5_K: case WGML_Q8_K: case WGML_Q4_0:
+    case WGML_Q4_1: case WGML_Q5_0: case WGML_Q5_1: return true;
+    default: return false;
+    }
+}
+
+// One launch takes matrices of one format (any of the nine), or a mix of Q4_K / Q6_K / Q8_0; with
+// fp32 activations only those three.
+bool gemv_fused_set_supported(const wgml_ctx *ctx, const wgml_qmat *const *mats, int n) {
+    bool same = true, all_main = true;
+    for (int i = 0; i < n; ++i) {
+        if (!gemv_fused_supported(mats[i])) return false;
+        same = same && mats[i]->type == mats[0]->type;
+        all_main = all_main && main_format(mats[i]->type);
+    }
+    if (ctx->tuning[WGML_TUNE_GEMV_F32_ACTIVATIONS]) return all_main;
+    return same || all_main;
 }
 
 template <int D, int MAXT, int MINW>
@@ -1928,6 +1889,7 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f, uint32_t
     P.rope_cs = reinterpret_cast<const float2 *>(f.rope_cs);
     const uint32_t ncols = f.jobs[0].a->ncols;
     P.ncols = ncols;
+    const bool f32 = ctx->tuning[WGML_TUNE_GEMV_F32_ACTIVATIONS] != 0;
     size_t lds = 0;
     uint64_t bytes[3] = {0, 0, 0};
     uint32_t ngroups[3];
@@ -1935,6 +1897,9 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f, uint32_t
         const FusedGemvJob &s = f.jobs[i];
         if (!gemv_fused_supported(s.a) || s.a->ncols != ncols)
             return set_error(WGML_E_INVALID, "gemv_fused: job %d has an unsupported matrix", i);
+        if (f32 && !main_format(s.a->type))
+            return set_error(WGML_E_UNSUPPORTED, "gemv_fused: fp32 activations exist for Q4_K, Q6_K "
+                                                 "and Q8_0 only");
         GemvJob &j = P.jobs[i];
         j.a0 = s.a->p0; j.a1 = s.a->p1; j.a2 = s.a->p2; j.a3 = s.a->p3;
         j.out = s.out;
@@ -1944,11 +1909,17 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f, uint32_t
             const uint32_t n = s.nrows ? s.nrows : s.a->nrows - s.row0;
             if (s.mode == JOB_SILU || (uint64_t)s.row0 + n > s.a->nrows)
                 return set_error(WGML_E_INVALID, "gemv_fused: job %d: bad row slice", i);
-            const uint64_t r = s.row0, nb = r * (ncols / 256);
+            const uint64_t r = s.row0, nb = r * (ncols / 256), nb32 = r * (ncols / 32);
             switch (s.a->type) {
             case WGML_Q4_K: j.a0 += nb * 144; break;
+            case WGML_Q5_K: j.a0 += nb * 176; break;
+            case WGML_Q8_K: j.a0 += nb * 292; break;
             case WGML_Q6_K: j.a0 += nb * 128; j.a1 += nb * 64; j.a2 += nb * 16; j.a3 += nb * 2; break;
-            default: j.a0 += r * ncols; j.a1 += r * (ncols / 32) * 2; break;  // Q8_0
+            case WGML_Q8_0: j.a0 += r * ncols; j.a1 += nb32 * 2; break;
+            case WGML_Q4_0: j.a0 += nb32 * 18; break;
+            case WGML_Q4_1: j.a0 += nb32 * 20; break;
+            case WGML_Q5_0: j.a0 += nb32 * 22; break;
+            default: j.a0 += nb32 * 24; break;  // Q5_1
             }
             j.nrows = n;
         }
@@ -1968,7 +1939,7 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f, uint32_t
                 return set_error(WGML_E_INVALID, "gemv_fused: RoPE needs even row counts");
             ngroups[i] = (j.nrows + 1) / 2;
         }
-        const size_t l = lds_bytes_i8(j.type, ncols);
+        const size_t l = lds_bytes_fused(j.type, ncols, f32);
         if (l > lds) lds = l;
     }
     if (lds > kMaxLds)
@@ -1981,16 +1952,37 @@ static int launch_gemv_fused_variant(wgml_ctx *ctx, const FusedGemv &f, uint32_t
     int fmt = P.jobs[0].type, slot = 0;
     for (int i = 1; i < f.njobs; ++i)
         if (P.jobs[i].type != fmt) fmt = 0;
+    if (fmt == 0)
+        for (int i = 0; i < f.njobs; ++i)
+            if (!main_format(P.jobs[i].type))
+                return set_error(WGML_E_UNSUPPORTED, "gemv_fused: formats can be mixed among Q4_K, "
+                                                     "Q6_K and Q8_0 only");
     // the mixed-format kernel is held to 96 registers (5 waves per SIMD): it fits without
     // spilling, and the waves of a workgroup start sooner the fewer registers they take
     void (*kern)(const FusedParams) = gemv_fused_kernel<D, MAXT, (MAXT == 1024 ? 5 : MINW), 0>;
-    switch (fmt) {
-    case WGML_Q4_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q4_K>; slot = 1; break;
-    case WGML_Q6_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q6_K>; slot = 2; break;
-    case WGML_Q8_0: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q8_0>; slot = 3; break;
-    default: break;
-    }
     (void)slot;
+    if (f32) {
+        kern = gemv_fused_kernel<D, MAXT, MINW, 0, true>;
+        switch (fmt) {
+        case WGML_Q4_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q4_K, true>; break;
+        case WGML_Q6_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q6_K, true>; break;
+        case WGML_Q8_0: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q8_0, true>; break;
+        default: break;
+        }
+    } else {
+        switch (fmt) {
+        case WGML_Q4_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q4_K>; break;
+        case WGML_Q6_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q6_K>; break;
+        case WGML_Q8_0: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q8_0>; break;
+        case WGML_Q5_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q5_K>; break;
+        case WGML_Q8_K: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q8_K>; break;
+        case WGML_Q4_0: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q4_0>; break;
+        case WGML_Q4_1: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q4_1>; break;
+        case WGML_Q5_0: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q5_0>; break;
+        case WGML_Q5_1: kern = gemv_fused_kernel<D, MAXT, MINW, WGML_Q5_1>; break;
+        default: break;
+        }
+    }
     int cached_blocks = 1;
     WGML_TRY(blocks_per_cu(ctx, (const void *)kern, MAXT, lds, &cached_blocks));
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;

@@ -122,9 +122,10 @@ int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos,
 
     for (uint32_t l = 0; l < c.n_layers; ++l) {
         const LlamaLayer &w = m->layers[l];
-        if (fusion >= 3 && gemv_fused_supported(w.attn_q) && gemv_fused_supported(w.attn_k) &&
-            gemv_fused_supported(w.attn_v) && gemv_fused_supported(w.ffn_gate) &&
-            gemv_fused_supported(w.ffn_up) && w.ffn_gate->type == w.ffn_up->type) {
+        const wgml_qmat *const qkv[3] = {w.attn_q, w.attn_k, w.attn_v};
+        const wgml_qmat *const gate_up[2] = {w.ffn_gate, w.ffn_up};
+        if (fusion >= 3 && gemv_fused_set_supported(ctx, qkv, 3) &&
+            gemv_fused_set_supported(ctx, gate_up, 2) && w.ffn_gate->type == w.ffn_up->type) {
             // 5 launches per layer: [norm + Q,K,V + bias + RoPE + KV-cache write],
             // attention (+ merge), [Wo + residual], [norm + gate,up + SiLU], [down + residual]
             const bool rope_fused = variant == WGML_ROPE_ORIGINAL;
@@ -158,6 +159,7 @@ int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos,
             // the output projection merges them while it stages its input: no merge launch,
             // and no reason to hold short contexts to one workgroup per head
             AttnPartials parts;
+            parts.consumer_wgs = gemv_consumer_wgs(ctx, w.attn_output->nrows);
             WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, ap.seq_len, m->q, w.key_cache,
                                               w.value_cache, nullptr, m->xb, nullptr, 0,
                                               gemv_partials_supported(ctx, w.attn_output) ? &parts
