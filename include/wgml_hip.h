@@ -170,7 +170,8 @@ WGML_API int wgml_gemv_quant(wgml_ctx *ctx, wgml_view out, const wgml_qmat *m, w
  * product term group, fp32 sums: results agree with n_tokens calls of
  * wgml_gemv_quant to fp32 rounding (about 1e-6 of a row's magnitude).  Level 0 rounds
  * weights and vectors to f16 once: 1.4x faster, about 3e-4 of a row's magnitude
- * (up to 1.4e-3 for single elements).  m must be WGML_Q8_0, WGML_Q4_K or WGML_Q6_K.
+ * (up to 1.4e-3 for single elements).  m: any of the nine quantized block formats
+ * (Q8_0, Q4_K, Q6_K, Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, Q8_K); not F32 / F16.
  * Vectors of any magnitude are taken (scaled per vector by a power of two); the
  * dequantized weights must not exceed 255.875 in magnitude (they pass through f16 times 2^8,
  * and 65504 is the largest finite f16): a bound on the largest weight is computed when the
@@ -357,8 +358,9 @@ WGML_API int wgml_llama2_decode_greedy_sync(wgml_llama2 *m, uint32_t first_token
  * fp32 implementations do (2e-4 of their range is the bound the tests use); with
  * level 0 a product is within about 3e-4 and a whole model adds that up (3e-3 of
  * the logits' range on 2-layer models, 6e-3 on the 32-layer 7B shape).  The batched
- * products exist for WGML_Q8_0, WGML_Q4_K and WGML_Q6_K: a model with a layer matrix in
- * another format takes the prompt one step per token, as the reference does.
+ * products exist for the nine quantized block formats: a model with a layer matrix that is
+ * F32 / F16, or whose weights exceed what the products take (see wgml_gemm_quant), takes the
+ * prompt one step per token, as the reference does.
  * Enqueues and returns. */
 WGML_API int wgml_llama2_prefill(wgml_llama2 *m, const uint32_t *tokens, uint32_t n_tokens,
                                  uint32_t start_pos);

@@ -379,9 +379,8 @@ def test_gpt2_matrix_replaced_after_a_recorded_run(gpu):
 def test_llama_micro_in_the_remaining_block_formats(gpu, qtype):
     # a model whose matrices are all in one of the formats beside Q8_0 / Q4_K / Q6_K: they
     # stay quantized on the device and take the same fused Q/K/V and gate/up launches (a launch
-    # holds matrices of one format), the prompt pass falls back to one step per token; logits,
-    # KV rows and greedy tokens against the oracle, and the fused step against the step with
-    # one launch per matrix
+    # holds matrices of one format) and the batched prompt pass; logits, KV rows and greedy
+    # tokens against the oracle, and the fused step against the step with one launch per matrix
     import npref
 
     w = synth_llama(MICRO, seed=61, scheme="f32")
@@ -410,7 +409,7 @@ def test_llama_micro_in_the_remaining_block_formats(gpu, qtype):
     assert unfused.launches_per_token() > m.launches_per_token()
     assert np.abs(lg - m.forward_logits(len(toks) - 1, toks[-1])).max() <= 1e-4 * np.abs(lg).max()
     m2 = Llama2(gpu, MICRO).load(w)
-    m2.prefill(toks)  # no batched product for these formats: steps through the prompt
+    m2.prefill(toks)  # the batched prompt pass
     ok, e = logits_close(m2.logits(), ref.forward(toks[-1], len(toks) - 1))
     assert ok, e
     prompt = W.prompt_tokens(61, 4, MICRO.vocab_size)

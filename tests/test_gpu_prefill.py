@@ -17,6 +17,7 @@ Two precisions (wgml_ctx_set_gemm_precision), both tested:
 import numpy as np
 import pytest
 
+import npref
 import oracle as orc
 import wgml_amd as W
 from wgml_amd._lib import E_UNSUPPORTED
@@ -87,6 +88,53 @@ def test_gemm_q8_0_rows_not_a_multiple_of_64(gpu, k_split, ncols, T):
     raw = W.quantize(W.Q8_0, W.rng_normal(3, nrows * ncols, 0, 0.02))
     x = W.rng_normal(4, T * ncols).reshape(T, ncols)
     check(gemm(gpu, W.Q8_0, raw, nrows, ncols, x), reference(W.Q8_0, raw, nrows, ncols, x))
+
+
+OTHER = [W.Q4_0, W.Q4_1, W.Q5_0, W.Q5_1, W.Q5_K, W.Q8_K]
+
+
+def small_blocks(qtype, n_elems, seed):
+    """Blocks of a format that has no quantizer here: the closest-value encoder of the test
+    helpers over N(0, 0.02) values (weights of ordinary size, well inside the f16 operands)."""
+    vals = W.rng_normal(seed, n_elems, 0, 0.02)
+    return npref.encode_simple(qtype, vals)
+
+
+@pytest.mark.parametrize("qtype", OTHER)
+@pytest.mark.parametrize("T", [1, 17, 64, 128])
+@pytest.mark.parametrize("nrows,ncols", [(16, 256), (100, 768), (333, 2048)])
+def test_gemm_in_the_remaining_block_formats(gpu, k_split, qtype, T, nrows, ncols):
+    # the batched product for Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q5_K / Q8_K: same bounds as for the
+    # three main formats, against the exact product of the bit-exactly dequantized weights
+    raw = small_blocks(qtype, nrows * ncols, 40 + nrows)
+    x = W.rng_normal(50 + T, T * ncols).reshape(T, ncols)
+    check(gemm(gpu, qtype, raw, nrows, ncols, x), reference(qtype, raw, nrows, ncols, x))
+
+
+@pytest.mark.parametrize("qtype", [W.Q4_0, W.Q4_1, W.Q5_0, W.Q5_1])
+@pytest.mark.parametrize("ncols", [32, 96, 160, 2080])
+def test_gemm_32_element_blocks_rows_not_a_multiple_of_64(gpu, k_split, qtype, ncols):
+    nrows, T = 21, 9
+    raw = small_blocks(qtype, nrows * ncols, 3)
+    x = W.rng_normal(4, T * ncols).reshape(T, ncols)
+    check(gemm(gpu, qtype, raw, nrows, ncols, x), reference(qtype, raw, nrows, ncols, x))
+
+
+@pytest.mark.parametrize("qtype", OTHER)
+def test_gemm_remaining_formats_random_block_bits(gpu, qtype):
+    # every bit pattern of quants, fifth bits and 6-bit scales (scales kept small enough for the
+    # weights to fit the f16 operands: matrices beyond that are refused, see the limit test)
+    nrows, ncols, T = 48, 1024, 20
+    raw = npref.random_blocks(qtype, nrows * ncols // npref.BLOCK_ELEMS[qtype], seed=77)
+    m = W.GpuQuantMatrix(gpu, qtype, nrows, ncols, raw)
+    x = W.rng_normal(78, T * ncols).reshape(T, ncols)
+    w = orc.dequantize(qtype, raw, nrows * ncols)
+    assert m.weight_bound() >= float(np.abs(w).max()) * (1 - 1e-6)
+    if m.weight_bound() <= 255.875:
+        check(gemm(gpu, qtype, raw, nrows, ncols, x), reference(qtype, raw, nrows, ncols, x))
+    else:
+        with pytest.raises(W.WgmlError):
+            gemm(gpu, qtype, raw, nrows, ncols, x)
 
 
 @pytest.mark.parametrize("qtype", QT)
@@ -391,3 +439,26 @@ def test_prefill_steps_through_a_model_with_large_weights(gpu):
     m.prefill(toks)
     assert np.isfinite(m.logits()).all()
     assert_state_matches(m, ref, MICRO, 9, want, tol=1e-3)
+
+
+@pytest.mark.parametrize("qtype", OTHER)
+def test_prefill_in_the_remaining_block_formats(gpu, qtype):
+    # a model all in one of the six other formats goes through the batched prompt pass too
+    from wgml_amd.models import HostMatrix
+    w = synth_llama(MICRO, seed=61, scheme="f32")
+    for layer in w.layers:
+        for name, v in list(layer.items()):
+            if isinstance(v, HostMatrix):
+                layer[name] = HostMatrix(qtype, v.nrows, v.ncols,
+                                         npref.encode_simple(qtype, v.data.view(np.float32)))
+    w.output = HostMatrix(qtype, w.output.nrows, w.output.ncols,
+                          npref.encode_simple(qtype, w.output.data.view(np.float32)))
+    spice(w, MICRO, 9, biases=False)
+    ref = orc.Llama2(w)
+    toks = W.prompt_tokens(3, 19, MICRO.vocab_size)
+    for pos, t in enumerate(toks):
+        want = ref.forward(int(t), pos)
+    m = Llama2(gpu, MICRO).load(w)
+    m.prefill(toks)
+    assert m.launches_per_token() < 19 * 5  # batched: far fewer launches than 19 steps
+    assert_state_matches(m, ref, MICRO, 19, want)

@@ -391,8 +391,7 @@ int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint3
 
 // The batched products take these formats, and weights that fit their f16 operands.
 bool gemm_supported(const wgml_qmat *q) {
-    return (q->type == WGML_Q8_0 || q->type == WGML_Q4_K || q->type == WGML_Q6_K) &&
-           q->max_abs <= kGemmMaxWeight;
+    return gemv_fused_supported(q) && q->max_abs <= kGemmMaxWeight;  // the nine quantized formats
 }
 
 // One run of T <= kPrefillMaxTokens prompt tokens at positions pos0 .. pos0 + T - 1: the
@@ -670,8 +669,8 @@ int wgml_llama2_prefill(wgml_llama2 *m, const uint32_t *tokens, uint32_t n_token
                                    w.ffn_down})
             if (!gemm_supported(q)) batched = false;
     if (!batched) {
-        // The batched products exist for Q8_0, Q4_K and Q6_K with weights of at most 255.875
-        // in magnitude.  A model with any other matrix takes the prompt the way the reference does: one step per token
+        // The batched products exist for the quantized formats, with weights of at most
+        // 255.875 in magnitude.  A model with any other matrix takes the prompt the way the reference does: one step per token
         // (chat_llama2.rs:155-228), which leaves the same state.
         const uint64_t launches0 = ctx->launches;
         for (uint32_t i = 0; i < n_tokens; ++i) WGML_TRY(enqueue_step(m, false, tokens[i], start_pos + i));

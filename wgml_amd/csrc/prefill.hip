@@ -296,6 +296,166 @@ struct GemmQ8_0 {
     }
 };
 
+// Q5_K (176 B: d, dmin, scales[12] as Q4_K, 32 bytes of fifth bits, 128 bytes of nibbles;
+// quantization.rs:249-317).  Chunk c is the 64-element group j = c & 3 of super-block c >> 2:
+// sub-block 2 j + s2 takes the low (s2 = 0) or high nibbles of qs[32 j + l] and bit 2 j + s2 of
+// qh[l], l = 8 g + 4 e + i.
+struct GemmQ5K {
+    struct Raw {
+        uint4 hdr;
+        uint2 qs, qh;
+    };
+    struct Pre {
+        float dd[2], mm[2];
+        uint32_t j2;  // 2 j
+    };
+    struct Lane {
+        uint32_t hdr, qs, qh;
+    };
+    __device__ static void lane_init(Lane &l, uint32_t ncols, uint32_t row, uint32_t g) {
+        l.hdr = row * (ncols / 256) * 176;
+        l.qh = l.hdr + 16 + 8 * g;
+        l.qs = l.hdr + 48 + 8 * g;
+    }
+    __device__ static void load(Raw &r, const GemmMat &m, uint32_t, const Lane &l, uint32_t chunk) {
+        const uint8_t *blk = m.p0 + (size_t)(chunk >> 2) * 176;
+        r.hdr = load_at<uint4>(blk, l.hdr);
+        r.qh = load_at<uint2>(blk, l.qh);
+        r.qs = load_at<uint2>(blk + (chunk & 3) * 32, l.qs);
+    }
+    __device__ static void pre(Pre &p, const Raw &r, uint32_t ncols, uint32_t chunk, uint32_t g) {
+        GemmQ4K::Raw q4;
+        q4.hdr = r.hdr;
+        q4.qs = r.qs;
+        GemmQ4K::Pre p4;
+        GemmQ4K::pre(p4, q4, ncols, chunk, g);  // the scale / min layout is Q4_K's
+        p.dd[0] = p4.dd[0];
+        p.dd[1] = p4.dd[1];
+        p.mm[0] = p4.mm[0];
+        p.mm[1] = p4.mm[1];
+        p.j2 = 2 * (chunk & 3);
+    }
+    template <int I>
+    __device__ static float elem(const Pre &p, const Raw &r, uint32_t) {
+        constexpr int s2 = I / 8, e = (I / 4) & 1, b = I & 3;
+        const uint32_t lo = ((e ? r.qs.y : r.qs.x) >> (4 * s2)) & 0x0f0f0f0fu;
+        const uint32_t hb = (((e ? r.qh.y : r.qh.x) >> (p.j2 + s2)) & 0x01010101u) << 4;
+        const uint32_t four = opaque(lo | hb);
+        return fmaf(p.dd[s2], (float)((four >> (8 * b)) & 0xffu), -p.mm[s2]);
+    }
+};
+
+// Q8_K (292 B: f32 d, 256 int8, 16 sums that dequantization does not use; quantization.rs:170-199).
+struct GemmQ8K {
+    struct Raw {
+        uint2 q[2];
+        float d;
+    };
+    struct Pre {
+        float d, off;
+    };
+    struct Lane {
+        uint32_t d, q;
+    };
+    __device__ static void lane_init(Lane &l, uint32_t ncols, uint32_t row, uint32_t g) {
+        l.d = row * (ncols / 256) * 292;
+        l.q = l.d + 4 + 8 * g;
+    }
+    __device__ static void load(Raw &r, const GemmMat &m, uint32_t, const Lane &l, uint32_t chunk) {
+        const uint8_t *blk = m.p0 + (size_t)(chunk >> 2) * 292;
+        r.d = load_at<float>(blk, l.d);
+        r.q[0] = load_at<uint2>(blk + (chunk & 3) * 64, l.q);
+        r.q[1] = load_at<uint2>(blk + (chunk & 3) * 64 + 32, l.q);
+    }
+    __device__ static void pre(Pre &p, const Raw &r, uint32_t, uint32_t, uint32_t) {
+        p.d = r.d * kWeightScale;
+        p.off = -128.f * p.d;
+    }
+    template <int I>
+    __device__ static float elem(const Pre &p, const Raw &r, uint32_t) {
+        constexpr int s2 = I / 8, e = (I / 4) & 1, b = I & 3;
+        const uint32_t four = opaque((e ? r.q[s2].y : r.q[s2].x) ^ 0x80808080u);  // q + 128 as bytes
+        return fmaf(p.d, (float)((four >> (8 * b)) & 0xffu), p.off);
+    }
+};
+
+// The 32-element blocks Q4_0 (18 B: d, 16 B of nibbles), Q4_1 (20 B: d, m, nibbles), Q5_0 (22 B:
+// d, 32 fifth bits, nibbles), Q5_1 (24 B: d, m, fifth bits, nibbles); quantization.rs:47-162.
+// Element t of a block is the low nibble of qs[t] for t < 16 and the high nibble of qs[t - 16]
+// otherwise, with bit t of qh as its fifth bit.  Chunk c holds blocks 2 c (s2 = 0) and 2 c + 1;
+// a lane's t = 8 g + 4 e + i, so lanes g < 2 take low nibbles and g >= 2 high nibbles of the
+// same eight bytes.  Blocks are 2-byte aligned: the loads below are unaligned, which gfx950
+// serves.  A block of the padded K range that does not exist reads the last one and expands to 0.
+template <int BYTES, bool HAS_M, bool HAS_QH>
+struct GemmLegacy {
+    struct Raw {
+        uint2 q[2];
+        uint32_t qh[2];
+        uint32_t dm[2];  // d (low half) and m (high half) as stored
+    };
+    struct Pre {
+        float d[2], off[2];
+        uint32_t hi_nib, shift;  // g >= 2; bit of qh that belongs to this lane's first element
+    };
+    struct Lane {
+        uint32_t blk, q;
+    };
+    static constexpr uint32_t QS = 2 + (HAS_M ? 2 : 0) + (HAS_QH ? 4 : 0);
+    __device__ static void lane_init(Lane &l, uint32_t ncols, uint32_t row, uint32_t g) {
+        l.blk = row * (ncols / 32) * BYTES;
+        l.q = l.blk + QS + 8 * (g & 1);
+    }
+    __device__ static void load(Raw &r, const GemmMat &m, uint32_t ncols, const Lane &l, uint32_t chunk) {
+        const uint32_t b0 = chunk * 2, nb = ncols / 32;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            const uint8_t *blk = m.p0 + (size_t)min(b0 + s2, nb - 1) * BYTES;
+            // 2-byte aligned: halfwords are loaded as such and put together
+            const uint32_t d = load_at<uint16_t>(blk, l.blk);
+            uint32_t mm = 0;
+            if (HAS_M) mm = load_at<uint16_t>(blk + 2, l.blk);
+            r.dm[s2] = d | (mm << 16);
+            r.qh[s2] = 0;
+            if (HAS_QH)
+                r.qh[s2] = (uint32_t)load_at<uint16_t>(blk + (HAS_M ? 4 : 2), l.blk) |
+                           ((uint32_t)load_at<uint16_t>(blk + (HAS_M ? 6 : 4), l.blk) << 16);
+            const uint32_t q0 = (uint32_t)load_at<uint16_t>(blk, l.q) | ((uint32_t)load_at<uint16_t>(blk + 2, l.q) << 16);
+            const uint32_t q1 = (uint32_t)load_at<uint16_t>(blk + 4, l.q) | ((uint32_t)load_at<uint16_t>(blk + 6, l.q) << 16);
+            r.q[s2] = make_uint2(q0, q1);
+        }
+    }
+    __device__ static void pre(Pre &p, const Raw &r, uint32_t ncols, uint32_t chunk, uint32_t g) {
+        p.hi_nib = g >> 1;
+        p.shift = 8 * g;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            const bool exists = chunk * 2 + s2 < ncols / 32;
+            const float d = exists ? f16_bits_to_f32((uint16_t)(r.dm[s2] & 0xffffu)) * kWeightScale : 0.f;
+            p.d[s2] = d;
+            if (HAS_M)  // y = d q + m
+                p.off[s2] = exists ? f16_bits_to_f32((uint16_t)(r.dm[s2] >> 16)) * kWeightScale : 0.f;
+            else  // y = d (q - 8) or d (q - 16)
+                p.off[s2] = (HAS_QH ? -16.f : -8.f) * d;
+        }
+    }
+    template <int I>
+    __device__ static float elem(const Pre &p, const Raw &r, uint32_t) {
+        constexpr int s2 = I / 8, e = (I / 4) & 1, b = I & 3;
+        uint32_t four = ((e ? r.q[s2].y : r.q[s2].x) >> (4 * p.hi_nib)) & 0x0f0f0f0fu;
+        if (HAS_QH) {
+            // bits t .. t + 3 of qh (t = 8 g + 4 e) moved to bit 4 of bytes 0 .. 3
+            const uint32_t bits = (r.qh[s2] >> (p.shift + 4 * e)) & 15u;
+            four |= ((bits * 0x00204081u) & 0x01010101u) << 4;
+        }
+        four = opaque(four);
+        return fmaf(p.d[s2], (float)((four >> (8 * b)) & 0xffu), p.off[s2]);
+    }
+};
+using GemmQ4_0 = GemmLegacy<18, false, false>;
+using GemmQ4_1 = GemmLegacy<20, true, false>;
+using GemmQ5_0 = GemmLegacy<22, false, true>;
+using GemmQ5_1 = GemmLegacy<24, true, true>;
+
 // A wave's weights for one chunk as MFMA A operands: hi[s2] (and, split precision, lo[s2]).
 template <bool SPLIT>
 struct AFrag {
@@ -1378,9 +1538,15 @@ int launch_gemm_quant_multi(wgml_ctx *ctx, const GemmTarget *targets, int n, con
     case WGML_Q4_K: return launch_gemm_fmt<GemmQ4K>(ctx, a, tiles);
     case WGML_Q6_K: return launch_gemm_fmt<GemmQ6K>(ctx, a, tiles);
     case WGML_Q8_0: return launch_gemm_fmt<GemmQ8_0>(ctx, a, tiles);
+    case WGML_Q5_K: return launch_gemm_fmt<GemmQ5K>(ctx, a, tiles);
+    case WGML_Q8_K: return launch_gemm_fmt<GemmQ8K>(ctx, a, tiles);
+    case WGML_Q4_0: return launch_gemm_fmt<GemmQ4_0>(ctx, a, tiles);
+    case WGML_Q4_1: return launch_gemm_fmt<GemmQ4_1>(ctx, a, tiles);
+    case WGML_Q5_0: return launch_gemm_fmt<GemmQ5_0>(ctx, a, tiles);
+    case WGML_Q5_1: return launch_gemm_fmt<GemmQ5_1>(ctx, a, tiles);
     default:
-        return set_error(WGML_E_UNSUPPORTED, "gemm_quant: matrix type %d (Q8_0, Q4_K, Q6_K only)",
-                         first->type);
+        return set_error(WGML_E_UNSUPPORTED, "gemm_quant: matrix type %d has no batched product "
+                                             "(the nine quantized block formats only)", first->type);
     }
 }
 

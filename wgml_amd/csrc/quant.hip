@@ -50,9 +50,9 @@ __global__ void repack_q6_k(const uint16_t *__restrict__ raw, uint16_t *__restri
 }
 
 // ---- largest weight magnitude (computed once per matrix at load) --------------
-// An upper bound on |w| over the dequantized matrix: Q8_0 |d| max|q| (exact); Q4_K
-// max(|dmin m|, |d sc 15 - dmin m|) per sub-block (the two ends of the quant range); Q6_K
-// |d| |scale| 32 per sub-block.  The batched
+// An upper bound on |w| over the dequantized matrix: Q8_0 and Q8_K |d| max|q| (exact); Q4_K and
+// Q5_K max(|dmin m|, |d sc 15 (31) - dmin m|) per sub-block (the two ends of the quant range);
+// Q6_K |d| |scale| 32 per sub-block; the 32-element blocks the ends of their ranges likewise.  The batched
 // products expand weights into f16 times 2^8 and need it within 255.875.  NaN / inf scales give
 // inf.  Non-negative floats order like their bit patterns, so the maximum is an atomicMax on
 // the bits.
@@ -83,12 +83,42 @@ __global__ void max_abs_kernel(int type, const uint8_t *__restrict__ p0,
                 const float a = sc ? d * (float)sc * 15.f : 0.f, c = m ? dmin * (float)m : 0.f;
                 v = fmaxf(v, fmaxf(nan_to_inf(fabsf(c)), nan_to_inf(fabsf(a - c))));
             }
-        } else {  // WGML_Q6_K
+        } else if (type == WGML_Q6_K) {
             const float d = fabsf(f16_bits_to_f32(reinterpret_cast<const uint16_t *>(p3)[b]));
             const int8_t *sc = reinterpret_cast<const int8_t *>(p2) + b * 16;
             int m = 0;
             for (int k = 0; k < 16; ++k) m = max(m, abs((int)sc[k]));
             v = m ? d * (float)m * 32.f : 0.f;
+        } else if (type == WGML_Q5_K) {  // as Q4_K with quants 0..31
+            const uint8_t *blk = p0 + b * 176;
+            const float d = f16_bits_to_f32(*(const uint16_t *)(blk + 0));
+            const float dmin = f16_bits_to_f32(*(const uint16_t *)(blk + 2));
+            for (uint32_t j = 0; j < 8; ++j) {
+                uint8_t sc, m;
+                get_scale_min_k4(j, blk + 4, sc, m);
+                const float a = sc ? d * (float)sc * 31.f : 0.f, c = m ? dmin * (float)m : 0.f;
+                v = fmaxf(v, fmaxf(nan_to_inf(fabsf(c)), nan_to_inf(fabsf(a - c))));
+            }
+        } else if (type == WGML_Q8_K) {
+            const uint8_t *blk = p0 + b * 292;
+            float d;
+            __builtin_memcpy(&d, blk, 4);
+            const int8_t *q = reinterpret_cast<const int8_t *>(blk + 4);
+            int m = 0;
+            for (int k = 0; k < 256; ++k) m = max(m, abs((int)q[k]));
+            v = m ? fabsf(d) * (float)m : 0.f;
+        } else {  // the 32-element blocks: y = d (q - 8), d q + m, d (q - 16), d q + m
+            const bool has_m = type == WGML_Q4_1 || type == WGML_Q5_1;
+            const bool has_qh = type == WGML_Q5_0 || type == WGML_Q5_1;
+            const uint32_t bytes = 18 + (has_m ? 2 : 0) + (has_qh ? 4 : 0);
+            const uint8_t *blk = p0 + b * bytes;
+            uint16_t db, mb = 0;
+            __builtin_memcpy(&db, blk, 2);
+            if (has_m) __builtin_memcpy(&mb, blk + 2, 2);
+            const float d = f16_bits_to_f32(db), m = f16_bits_to_f32(mb);
+            const float top = has_qh ? 31.f : 15.f;
+            if (has_m) v = fmaxf(nan_to_inf(fabsf(m)), nan_to_inf(fabsf(d * top + m)));
+            else v = fabsf(d) * (has_qh ? 16.f : 8.f);
         }
         best = fmaxf(best, nan_to_inf(v));
     }
@@ -415,7 +445,7 @@ int wgml_quant_matrix_create(wgml_ctx *ctx, int type, uint32_t nrows, uint32_t n
         (void)hipFree(raw);
         if (e != hipSuccess) return fail(e, "re-layout");
     }
-    if (type == WGML_Q8_0 || type == WGML_Q4_K || type == WGML_Q6_K) {
+    if (block_bytes(type) && type != WGML_F16 && type != WGML_F32) {
         // the formats the batched products take: bound their largest weight once
         uint32_t *bits = ctx->d_scalar + 8;
         e = hipMemsetAsync(bits, 0, 4, ctx->stream);
