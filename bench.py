@@ -269,10 +269,16 @@ def parity_at_timed_positions(W, gpu, model, weights, prompt, generated, first, 
     dt = time.perf_counter() - t0
 
     def worst_error():
+        # the state the timed steps ran on: the prompt through the batched pass at its default
+        # precision, then one step per position (every step rewrites its own KV row)
+        gpu.set_gemm_precision(1)
+        model.prefill(prompt)
         worst = 0.0
-        for pos in cand:
-            got = model.forward_logits(pos, int(seq[pos])).astype(np.float64)
-            worst = max(worst, float(np.abs(got - want[pos]).max() / np.abs(want[pos]).max()))
+        for pos in range(p0, cand[-1] + 1):
+            got = model.forward_logits(pos, int(seq[pos]))
+            if pos in want:
+                worst = max(worst, float(np.abs(got.astype(np.float64) - want[pos]).max() /
+                                         np.abs(want[pos]).max()))
         return worst
 
     e_default = worst_error()

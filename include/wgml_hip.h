@@ -101,6 +101,12 @@ enum {
                                                 (at most 2^20) runs as one workgroup per head group,
                                                 without partial results */
     WGML_TUNE_ATTN_SPLITS,                   /* workgroups that share the positions of a head group, 2..64 */
+    WGML_TUNE_ATTN_FOLD_MERGE,               /* attention followed by a quantized GEMV on its output
+                                                (wgml_attention_gemv_quant, the decoders' layers): 1 = the
+                                                GEMV merges attention's partial results itself while it
+                                                stages its input (up to 16 per head) instead of a merge
+                                                launch.  Off by default: every workgroup of the GEMV then
+                                                reads all partial results, which costs more than the launch */
     WGML_TUNE_COUNT
 };
 WGML_API int wgml_ctx_set_tuning(wgml_ctx *ctx, int key, int value);
@@ -234,11 +240,11 @@ WGML_API int wgml_attention(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view 
 /* The pair BatchedMultiqueryAttention::dispatch_multi + GemvQuant::dispatch that every decoder
  * layer runs (models/llama2/transformer.rs:366-383, models/gpt2/transformer.rs:355-395):
  * out = m * attention(q, caches), or out += ... when accumulate != 0 (the add_assign that
- * follows in the reference).  m is n x (n_heads * head_size).  Where m is Q8_0 / Q4_K / Q6_K
- * the attention launch leaves per-workgroup partial results and the product merges them while
- * it stages its input: there is no merge launch and `xb` is not written; otherwise the two
- * launches run as they would on their own.  xb: n_heads * head_size floats of scratch whose
- * contents after the call are unspecified. */
+ * follows in the reference).  m is n x (n_heads * head_size).  The two launches run as they
+ * would on their own; with WGML_TUNE_ATTN_FOLD_MERGE set and m in Q8_0 / Q4_K / Q6_K the
+ * attention launch leaves per-workgroup partial results and the product merges them while it
+ * stages its input (no merge launch, `xb` not written).  xb: n_heads * head_size floats of
+ * scratch whose contents after the call are unspecified. */
 WGML_API int wgml_attention_gemv_quant(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view q,
                                        wgml_view key_cache, wgml_view value_cache, wgml_view xb,
                                        const wgml_qmat *m, wgml_view out, int accumulate);

@@ -78,6 +78,15 @@ def test_attention_plans_agree(gpu, wide, splits, pos):
     np.testing.assert_allclose(xb, wxb, rtol=0, atol=2e-5)
 
 
+@pytest.fixture(params=["merge_launch", "merged_by_product"])
+def fold(gpu, request):
+    """Both ways the pair runs: attention's own merge launch (the default), and the product
+    merging the partial results while it stages its input."""
+    gpu.set_tuning(gpu.TUNE_ATTN_FOLD_MERGE, 1 if request.param == "merged_by_product" else 0)
+    yield request.param
+    gpu.set_tuning(gpu.TUNE_ATTN_FOLD_MERGE, 0)
+
+
 def run_with_projection(gpu, qtype, seq_len, kv_mul, n_heads, hs, pos, nrows, accumulate, seed=0):
     """attention + output projection as one call, against the oracle's attention followed by the
     exact product of the dequantized matrix with it (f64)."""
@@ -111,10 +120,10 @@ def run_with_projection(gpu, qtype, seq_len, kv_mul, n_heads, hs, pos, nrows, ac
 
 @pytest.mark.parametrize("qtype", [W.Q4_K, W.Q6_K, W.Q8_0])
 @pytest.mark.parametrize("pos", [0, 3, 31, 140, 255, 256, 700, 1023])
-def test_attention_with_projection(gpu, qtype, pos):
-    # the product merges attention's per-workgroup partial results while it stages its input
-    # (2 to 16 partial results per head, depending on the position; at the first positions
-    # most of them are neutral); GEMV tolerance as in tests/test_gpu_gemv.py
+def test_attention_with_projection(gpu, fold, qtype, pos):
+    # with `fold` the product merges attention's per-workgroup partial results while it stages
+    # its input (2 to 16 partial results per head, depending on the position; at the first
+    # positions most of them are neutral); GEMV tolerance as in tests/test_gpu_gemv.py
     got, want = run_with_projection(gpu, qtype, 1024, 1, 8, 128, pos, 192, False, seed=pos)
     assert np.abs(got - want).max() <= 5e-4 * np.abs(want).max()
 
@@ -122,7 +131,7 @@ def test_attention_with_projection(gpu, qtype, pos):
 @pytest.mark.parametrize("kv_mul,n_heads,hs", [(4, 32, 128), (2, 8, 64), (1, 12, 64), (1, 6, 48), (8, 16, 128),
                                                (1, 2, 256)])
 @pytest.mark.parametrize("pos", [5, 383])
-def test_attention_with_projection_head_layouts(gpu, kv_mul, n_heads, hs, pos):
+def test_attention_with_projection_head_layouts(gpu, fold, kv_mul, n_heads, hs, pos):
     # grouped queries, head sizes that fill a lane group only partly (48) and that need the
     # four-wave kernel (256), accumulation into the output
     dim = n_heads * hs
@@ -132,7 +141,7 @@ def test_attention_with_projection_head_layouts(gpu, kv_mul, n_heads, hs, pos):
 
 
 @pytest.mark.parametrize("wide,splits", [(1024, 0), (0, 2), (0, 8), (0, 9), (0, 16), (0, 17), (0, 64)])
-def test_attention_with_projection_plans(gpu, wide, splits):
+def test_attention_with_projection_plans(gpu, fold, wide, splits):
     # forced plans: one workgroup per head (nothing to merge), 2..16 partial results merged by the
     # product (eight at a time), 17 and 64 through the merge launch
     gpu.set_tuning(gpu.TUNE_ATTN_WIDE_POSITIONS, wide)
@@ -147,13 +156,13 @@ def test_attention_with_projection_plans(gpu, wide, splits):
 
 
 @pytest.mark.parametrize("qtype", [W.F32, W.Q5_K, W.Q4_0])
-def test_attention_with_projection_other_formats(gpu, qtype):
+def test_attention_with_projection_other_formats(gpu, fold, qtype):
     # formats without a merging product: the two launches run as they would on their own
     got, want = run_with_projection(gpu, qtype, 256, 1, 4, 64, 77, 64, True, seed=11)
     assert np.abs(got - want).max() <= 5e-4 * np.abs(want).max()
 
 
-def test_attention_with_projection_fp32_activations(gpu):
+def test_attention_with_projection_fp32_activations(gpu, fold):
     gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 1)
     try:
         got, want = run_with_projection(gpu, W.Q4_K, 512, 1, 8, 128, 300, 64, False, seed=2)

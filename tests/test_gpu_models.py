@@ -116,9 +116,29 @@ def test_tuning_change_rerecords_the_step(gpu):
     assert np.array_equal(m.generate_greedy(prompt, 20), base)
     assert m.launches_per_token() == n0
     for key, bad in ((gpu.TUNE_GEMV_WG_PER_CU, 9), (gpu.TUNE_ATTN_WIDE_POSITIONS, (1 << 20) + 1),
-                     (gpu.TUNE_GEMV_WAVES_PER_WG, 5), (gpu.TUNE_ATTN_SPLITS, 65)):
+                     (gpu.TUNE_GEMV_WAVES_PER_WG, 5), (gpu.TUNE_ATTN_SPLITS, 65),
+                     (gpu.TUNE_ATTN_FOLD_MERGE, 2)):
         with pytest.raises(W.WgmlError):
             gpu.set_tuning(key, bad)
+
+
+def test_output_projection_merging_attention_partials(gpu):
+    # on request the layer's output projection merges attention's partial results itself: the
+    # step keeps its launch count at a short context (no merge launch either way) and its tokens
+    w = synth_llama(MICRO, seed=22, scheme="q4_k")
+    spice(w, MICRO, 6, biases=False)
+    prompt = W.prompt_tokens(6, 5, MICRO.vocab_size)
+    want_t, _ = orc.Llama2(w).generate_greedy(prompt, 24)
+    m = Llama2(gpu, MICRO).load(w)
+    assert np.array_equal(m.generate_greedy(prompt, 24), want_t)
+    n0 = m.launches_per_token()
+    gpu.set_tuning(gpu.TUNE_ATTN_FOLD_MERGE, 1)
+    try:
+        got = m.generate_greedy(prompt, 24)
+        assert m.launches_per_token() == n0
+    finally:
+        gpu.set_tuning(gpu.TUNE_ATTN_FOLD_MERGE, 0)
+    assert np.array_equal(got, want_t)
 
 
 @pytest.mark.parametrize("scheme", ["q8_0", "q4_k", "q6_k", "q4_k_m"])

@@ -610,8 +610,6 @@ constexpr uint32_t kWidePositions = 256;  // up to here one workgroup per head g
 // the most partial results per head that a consumer merges while it stages its input
 // (launch_gemv_quant with GemvEpilogue::partials)
 constexpr uint32_t kMaxFoldedPartials = 16;
-// ... and the most bytes of partial results that the consumer's workgroups together may read
-constexpr uint64_t kMaxFoldedBytes = 4u << 20;
 
 static int make_fast_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t plan_positions,
                           AttnPlan &pl, bool folded = false) {
@@ -706,12 +704,15 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
                              const float *kc, const float *vc, float *att, float *xb,
                              float *ext_ws, size_t ext_ws_bytes, AttnPartials *keep) {
     AttnPlan pl;
-    const uint32_t consumer_wgs = keep && keep->consumer_wgs ? keep->consumer_wgs
-                                                             : (ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u);
     if (keep) *keep = AttnPartials{};
-    // a caller that merges the partial results itself gets the plan with partial results also
-    // where one workgroup per head would do, as long as there are few enough of them
-    const bool want_partials = keep != nullptr && att == nullptr;
+    // A caller that merges the partial results itself gets the plan with partial results also
+    // where one workgroup per head would do, as long as there are few enough of them.  Only on
+    // request (WGML_TUNE_ATTN_FOLD_MERGE): every workgroup of the consumer then reads all
+    // partial results through the L2s, which was measured to cost more than the merge launch it
+    // saves (7B shape: the 4096-wide output projection grows from 3.9 to 8.4 us with eight
+    // partial results per head, 7.4 with four, against 3.0 us for the merge launch; GPT-2 124M
+    // over 1024 positions 3199 against 3273 tok/s).
+    const bool want_partials = keep != nullptr && att == nullptr && ctx->tuning[WGML_TUNE_ATTN_FOLD_MERGE] == 1;
     if (!want_partials) keep = nullptr;
     auto workspace = [&](size_t bytes, float **ws) -> int {
         if (ext_ws) {
@@ -729,12 +730,8 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
     const bool aligned = (((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) & 15u) == 0;
     if (fast_ok(p, aligned, att != nullptr)) {
         WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl, want_partials));
-        // Every workgroup of the consumer reads all partial results: what they pull through
-        // the L2s together must stay small beside the consumer's own weights, or the merge
-        // launch is the cheaper way (a 4096-wide vector with 8 partial results per head is
-        // 33 MB over 256 workgroups and costs the consumer 4 us; GPT-2's 768-wide one 1 MB).
-        const uint64_t pulled = (uint64_t)pl.n_wg_y * p.n_heads * pl.hsp * 4 * consumer_wgs;
-        if (want_partials && (pl.wide || pl.n_wg_y > kMaxFoldedPartials || pulled > kMaxFoldedBytes)) {
+        if (want_partials && (pl.wide || pl.n_wg_y > kMaxFoldedPartials)) {
+            // more partial results than a consumer merges: the plan with a merge launch
             keep = nullptr;
             WGML_TRY(make_fast_plan(ctx, p, plan_positions, pl, false));
         }
@@ -880,7 +877,6 @@ int wgml_attention_gemv_quant(wgml_ctx *ctx, const wgml_attn_params *p, wgml_vie
                  out.len);
     const wgml_view no_att{nullptr, 0, 0};
     AttnPartials parts;
-    parts.consumer_wgs = gemv_consumer_wgs(ctx, m->nrows);
     WGML_TRY(attention_entry("wgml_attention_gemv_quant", ctx, p, q, key_cache, value_cache, no_att,
                              xb, nullptr, 0, gemv_partials_supported(ctx, m) ? &parts : nullptr));
     GemvEpilogue e;

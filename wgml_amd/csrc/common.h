@@ -167,17 +167,7 @@ __device__ __forceinline__ uint32_t dyn_pos(const DynPos &p) {
 struct AttnPartials {
     const float *o = nullptr, *ml = nullptr;
     uint32_t n = 0, hsp = 0, head_size = 0;
-    // in, for launch_attention_planned: workgroups of the launch that will merge the partial
-    // results (each reads all of them); 0 = one per compute unit
-    uint32_t consumer_wgs = 0;
 };
-
-// Workgroups launch_gemv_quant uses for a matrix of `nrows` rows, roughly: what a caller tells
-// launch_attention_planned about the consumer of its partial results.
-inline uint32_t gemv_consumer_wgs(const wgml_ctx *ctx, uint32_t nrows) {
-    const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u, wgs = (nrows + 15) / 16;
-    return wgs < cu ? (wgs ? wgs : 1u) : cu;
-}
 
 struct GemvEpilogue {
     // out[r] = acc (+ bias[r]) (+ out[r] if accumulate)

@@ -285,7 +285,6 @@ int enqueue_step(wgml_gpt2 *m, bool dynamic, uint32_t token, uint32_t pos,
         // with the fused launches, attention may leave per-workgroup partial results that the
         // projection merges while it stages its input (no merge launch)
         AttnPartials parts;
-        parts.consumer_wgs = gemv_consumer_wgs(ctx, w.proj_w->nrows);
         WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, ap.seq_len, m->curr_2304,
                                           w.key_cache, w.value_cache, nullptr, m->curr_768, nullptr, 0,
                                           fold && gemv_partials_supported(ctx, w.proj_w) ? &parts

@@ -159,7 +159,6 @@ int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos,
             // the output projection merges them while it stages its input: no merge launch,
             // and no reason to hold short contexts to one workgroup per head
             AttnPartials parts;
-            parts.consumer_wgs = gemv_consumer_wgs(ctx, w.attn_output->nrows);
             WGML_TRY(launch_attention_planned(ctx, ap, dpos, plan, ap.seq_len, m->q, w.key_cache,
                                               w.value_cache, nullptr, m->xb, nullptr, 0,
                                               gemv_partials_supported(ctx, w.attn_output) ? &parts
