@@ -101,7 +101,7 @@ enum {
                                                 (at most 2^20) runs as one workgroup per head group,
                                                 without partial results */
     WGML_TUNE_ATTN_SPLITS,                   /* workgroups that share the positions of a head group, 2..64 */
-    WGML_TUNE_ATTN_FOLD_MERGE,               /* attention followed by a quantized GEMV on its output
+    WGML_TUNE_ATTN_MERGE,                    /* attention followed by a quantized GEMV on its output
                                                 (wgml_attention_gemv_quant, the decoders' layers): 1 = the
                                                 GEMV merges attention's partial results itself while it
                                                 stages its input (up to 16 per head) instead of a merge
@@ -241,7 +241,7 @@ WGML_API int wgml_attention(wgml_ctx *ctx, const wgml_attn_params *p, wgml_view 
  * layer runs (models/llama2/transformer.rs:366-383, models/gpt2/transformer.rs:355-395):
  * out = m * attention(q, caches), or out += ... when accumulate != 0 (the add_assign that
  * follows in the reference).  m is n x (n_heads * head_size).  The two launches run as they
- * would on their own; with WGML_TUNE_ATTN_FOLD_MERGE set and m in Q8_0 / Q4_K / Q6_K the
+ * would on their own; with WGML_TUNE_ATTN_MERGE = 1 and m in Q8_0 / Q4_K / Q6_K the
  * attention launch leaves per-workgroup partial results and the product merges them while it
  * stages its input (no merge launch, `xb` not written).  xb: n_heads * head_size floats of
  * scratch whose contents after the call are unspecified. */

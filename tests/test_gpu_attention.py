@@ -82,9 +82,9 @@ def test_attention_plans_agree(gpu, wide, splits, pos):
 def fold(gpu, request):
     """Both ways the pair runs: attention's own merge launch (the default), and the product
     merging the partial results while it stages its input."""
-    gpu.set_tuning(gpu.TUNE_ATTN_FOLD_MERGE, 1 if request.param == "merged_by_product" else 0)
+    gpu.set_tuning(gpu.TUNE_ATTN_MERGE, 1 if request.param == "merged_by_product" else 0)
     yield request.param
-    gpu.set_tuning(gpu.TUNE_ATTN_FOLD_MERGE, 0)
+    gpu.set_tuning(gpu.TUNE_ATTN_MERGE, 0)
 
 
 def run_with_projection(gpu, qtype, seq_len, kv_mul, n_heads, hs, pos, nrows, accumulate, seed=0):

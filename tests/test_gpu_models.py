@@ -117,7 +117,7 @@ def test_tuning_change_rerecords_the_step(gpu):
     assert m.launches_per_token() == n0
     for key, bad in ((gpu.TUNE_GEMV_WG_PER_CU, 9), (gpu.TUNE_ATTN_WIDE_POSITIONS, (1 << 20) + 1),
                      (gpu.TUNE_GEMV_WAVES_PER_WG, 5), (gpu.TUNE_ATTN_SPLITS, 65),
-                     (gpu.TUNE_ATTN_FOLD_MERGE, 2)):
+                     (gpu.TUNE_ATTN_MERGE, 2)):
         with pytest.raises(W.WgmlError):
             gpu.set_tuning(key, bad)
 
@@ -132,12 +132,12 @@ def test_output_projection_merging_attention_partials(gpu):
     m = Llama2(gpu, MICRO).load(w)
     assert np.array_equal(m.generate_greedy(prompt, 24), want_t)
     n0 = m.launches_per_token()
-    gpu.set_tuning(gpu.TUNE_ATTN_FOLD_MERGE, 1)
+    gpu.set_tuning(gpu.TUNE_ATTN_MERGE, 1)
     try:
         got = m.generate_greedy(prompt, 24)
         assert m.launches_per_token() == n0
     finally:
-        gpu.set_tuning(gpu.TUNE_ATTN_FOLD_MERGE, 0)
+        gpu.set_tuning(gpu.TUNE_ATTN_MERGE, 0)
     assert np.array_equal(got, want_t)
 
 

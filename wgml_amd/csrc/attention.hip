@@ -22,8 +22,14 @@
 // a recorded launch has work at any position.  Up to 128 positions one 16-wave
 // workgroup per head group does everything and writes the result (one launch, no
 // workspace); beyond that 4-wave workgroups write partials for the merge kernel.
-// (Merging in the workgroup that arrives last was tried and dropped: every
-// device-scope fence is an L2 write-back here, 20 us per launch.)
+// (Merging in the workgroup that arrives last was tried twice and dropped.  With
+// device-scope fences every fence is an L2 write-back here, 20 us per launch.  Without
+// fences -- partial results stored and loaded at device scope, a relaxed arrival counter
+// per head group, every thread waiting for its own stores before the workgroup is counted
+// in -- the results equal the merge launch's bit for bit, but the three dependent trips to
+// memory (store acknowledgement, counter, loads) cost what the launch costs: +0.6 % on 32
+// heads of 128 beyond position 256, -1.2 % on 12 heads of 64, -16 % at 8192 positions of
+// 8 KV heads, where one workgroup merges the four heads of its group in turn.)
 #include "common.h"
 #include "device_utils.h"
 
@@ -707,12 +713,12 @@ int launch_attention_planned(wgml_ctx *ctx, const wgml_attn_params &p, DynPos po
     if (keep) *keep = AttnPartials{};
     // A caller that merges the partial results itself gets the plan with partial results also
     // where one workgroup per head would do, as long as there are few enough of them.  Only on
-    // request (WGML_TUNE_ATTN_FOLD_MERGE): every workgroup of the consumer then reads all
+    // request (WGML_TUNE_ATTN_MERGE): every workgroup of the consumer then reads all
     // partial results through the L2s, which was measured to cost more than the merge launch it
     // saves (7B shape: the 4096-wide output projection grows from 3.9 to 8.4 us with eight
     // partial results per head, 7.4 with four, against 3.0 us for the merge launch; GPT-2 124M
     // over 1024 positions 3199 against 3273 tok/s).
-    const bool want_partials = keep != nullptr && att == nullptr && ctx->tuning[WGML_TUNE_ATTN_FOLD_MERGE] == 1;
+    const bool want_partials = keep != nullptr && att == nullptr && ctx->tuning[WGML_TUNE_ATTN_MERGE] == 1;
     if (!want_partials) keep = nullptr;
     auto workspace = [&](size_t bytes, float **ws) -> int {
         if (ext_ws) {

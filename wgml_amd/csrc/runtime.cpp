@@ -120,7 +120,7 @@ int wgml_ctx_set_tuning(wgml_ctx *ctx, int key, int value) {
     case WGML_TUNE_PREFILL_ATTENTION_PER_TOKEN: ok = value == 0 || value == 1; break;
     case WGML_TUNE_GEMM_K_SPLIT: ok = value >= 0 && value <= 8; break;
     case WGML_TUNE_ATTN_SPLITS: ok = value == 0 || (value >= 2 && value <= 64); break;
-    case WGML_TUNE_ATTN_FOLD_MERGE: ok = value == 0 || value == 1; break;
+    case WGML_TUNE_ATTN_MERGE: ok = value == 0 || value == 1; break;
     default: break;
     }
     WGML_REQUIRE(ok, "wgml_ctx_set_tuning: value %d is not valid for key %d", value, key);

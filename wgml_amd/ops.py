@@ -55,7 +55,7 @@ class GpuInstance:
     # keys of set_tuning (enum WGML_TUNE_* of the C header, same order)
     (TUNE_GEMV_ROWS_PER_WAVE, TUNE_GEMV_WAVES_PER_WG, TUNE_GEMV_WG_PER_CU, TUNE_GEMV_DEPTH,
      TUNE_GEMV_F32_ACTIVATIONS, TUNE_GEMM_K_SPLIT, TUNE_PREFILL_ATTENTION_PER_TOKEN,
-     TUNE_ATTN_WIDE_POSITIONS, TUNE_ATTN_SPLITS, TUNE_ATTN_FOLD_MERGE) = range(10)
+     TUNE_ATTN_WIDE_POSITIONS, TUNE_ATTN_SPLITS, TUNE_ATTN_MERGE) = range(10)
 
     def set_tuning(self, key: int, value: int) -> None:
         """Launch-shape override of this context (0 = heuristic); for sweeps and tests."""
