@@ -366,3 +366,26 @@ def test_fused_launch_refuses_a_mix_with_the_other_formats(gpu):
                          npref.random_blocks(W.Q5_K, nrows * ncols // 256, seed=2))
     with pytest.raises(W.WgmlError):
         _fused(gpu, [a, b], [None, None], [0, 0], nrows, W.rng_normal(3, ncols))
+
+
+def test_bench_read_chain_runs_and_checks_its_arguments(gpu):
+    # the bare chain of read-only launches that prices the machine (bench.py --ceiling):
+    # a time comes back for both ways of launching; sizes beyond half its pool are refused
+    import ctypes as C
+
+    from wgml_amd._lib import call
+
+    ms = C.c_float(-1.0)
+    for use_graph in (0, 1):
+        call("wgml_bench_read_chain", gpu.handle, 4096, 8, use_graph, C.byref(ms))
+        assert 0 < ms.value < 50.0
+    with pytest.raises(W.WgmlError):
+        call("wgml_bench_read_chain", gpu.handle, 400000, 8, 0, C.byref(ms))
+    with pytest.raises(W.WgmlError):
+        call("wgml_bench_read_chain", gpu.handle, 0, 8, 0, C.byref(ms))
+
+
+def test_context_stream_handle(gpu):
+    # the stream every call of the context enqueues on: a stable, non-null handle
+    assert gpu.stream() != 0
+    assert gpu.stream() == gpu.stream()

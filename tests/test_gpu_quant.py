@@ -91,6 +91,20 @@ def test_remaining_block_formats_stay_quantized(gpu, name, qtype):
         np.testing.assert_allclose(out.read(), ref[:, col], rtol=1e-6, atol=0)
 
 
+@pytest.mark.parametrize("name,qtype", [("q8_0", W.Q8_0), ("q4_k", W.Q4_K), ("q6_k", W.Q6_K)] + OTHER)
+def test_weight_bound_of_every_quantized_format(gpu, name, qtype):
+    # the bound the batched product checks (computed from the block scales when the matrix is
+    # created) is never below the largest dequantized weight, and not far above it: random bits
+    # reach the ends of a block's range
+    nrows, nblk = 24, 8
+    ncols = nblk * npref.BLOCK_ELEMS[qtype]
+    raw = npref.random_blocks(qtype, nrows * nblk, seed=300 + qtype)
+    w = orc.dequantize(qtype, raw, nrows * ncols)
+    m = W.GpuQuantMatrix(gpu, qtype, nrows, ncols, raw)
+    top = float(np.abs(w).max())
+    assert top <= m.weight_bound() <= 1.5 * top, (name, top, m.weight_bound())
+
+
 def test_f16_matrix_expanded_at_load(gpu):
     h = np.arange(4 * 64, dtype=np.uint16) * 97 % 31744  # finite halves
     want = np.array([orc.decode_f16(int(b)) for b in h], dtype=np.float32)

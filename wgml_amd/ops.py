@@ -209,7 +209,9 @@ class GpuQuantMatrix:
         return _lib.lib.wgml_quant_matrix_gguf_bytes(self._h)
 
     def weight_bound(self) -> float:
-        """Upper bound on |w| of the dequantized matrix (Q8_0 / Q4_K / Q6_K), else 0."""
+        """Upper bound on |w| of the dequantized matrix, from its block scales (the nine
+        quantized formats; 0 for f32 matrices): what the batched product checks against its
+        limit of 255.875."""
         b = C.c_float()
         call("wgml_quant_matrix_weight_bound", self._h, C.byref(b))
         return b.value
