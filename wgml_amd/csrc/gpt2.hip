@@ -35,6 +35,10 @@ struct wgml_gpt2 {
     // the recorded step, one capture per bucket of positions (plan_bucket)
     hipGraph_t graph[kMaxPlanBuckets] = {};
     hipGraphExec_t graph_exec[kMaxPlanBuckets] = {};
+    // kStepsPerGraph consecutive steps as one graph, replayed where that many steps stay inside
+    // a bucket (a replay costs the same between two graphs whatever the graph holds)
+    hipGraph_t graph_multi[kMaxPlanBuckets] = {};
+    hipGraphExec_t graph_exec_multi[kMaxPlanBuckets] = {};
     uint64_t graph_launches[kMaxPlanBuckets] = {};  // launches of the recorded step
     int fusion = 1;  // 0: one launch per op group as before; 1: folded launches
     int graph_fusion = -1;
@@ -337,6 +341,10 @@ void drop_graph(wgml_gpt2 *m) {
         if (m->graph[b]) (void)hipGraphDestroy(m->graph[b]);
         m->graph_exec[b] = nullptr;
         m->graph[b] = nullptr;
+        if (m->graph_exec_multi[b]) (void)hipGraphExecDestroy(m->graph_exec_multi[b]);
+        if (m->graph_multi[b]) (void)hipGraphDestroy(m->graph_multi[b]);
+        m->graph_exec_multi[b] = nullptr;
+        m->graph_multi[b] = nullptr;
     }
     m->graph_fusion = -1;
 }
@@ -355,9 +363,35 @@ int reserve_all_plans(wgml_gpt2 *m) {
     return WGML_OK;
 }
 
+constexpr uint32_t kStepsPerGraph = 8;
+
+// Records `steps` consecutive steps (each followed by greedy sampling and the loop's
+// bookkeeping, all on the device) into one HIP graph.
+int capture_steps(wgml_gpt2 *m, uint32_t plan, uint32_t steps, hipGraph_t *graph,
+                  hipGraphExec_t *exec, uint64_t *launches_per_step) {
+    wgml_ctx *ctx = m->ctx;
+    WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    const uint64_t launches0 = ctx->launches;
+    int rc = WGML_OK;
+    for (uint32_t k = 0; k < steps && rc == WGML_OK; ++k) {
+        rc = enqueue_step(m, true, 0, 0, plan);
+        if (rc == WGML_OK)
+            rc = launch_argmax_next(ctx, m->curr_vocab, m->p.n_vocab, m->dyn, m->d_prompt, m->d_tokens);
+    }
+    if (launches_per_step) *launches_per_step = (ctx->launches - launches0) / steps;
+    hipError_t e = hipStreamEndCapture(ctx->stream, graph);
+    if (rc != WGML_OK) return rc;
+    if (e != hipSuccess)
+        return set_error(WGML_E_HIP, "wgml_gpt2: graph capture failed: %s", hipGetErrorString(e));
+    e = hipGraphInstantiate(exec, *graph, nullptr, nullptr, 0);
+    if (e != hipSuccess)
+        return set_error(WGML_E_HIP, "wgml_gpt2: graph instantiate failed: %s", hipGetErrorString(e));
+    return WGML_OK;
+}
+
 // Records one step (+ greedy sampling and bookkeeping) into a HIP graph, for the bucket of
-// positions that `pos` lies in.
-int build_graph(wgml_gpt2 *m, uint32_t pos) {
+// positions that `pos` lies in; with `multi` also the graph of kStepsPerGraph steps.
+int build_graph(wgml_gpt2 *m, uint32_t pos, bool multi = false) {
     wgml_ctx *ctx = m->ctx;
     const wgml_gpt2_params &p = m->p;
     const uint32_t n = p.n_embd;
@@ -365,7 +399,15 @@ int build_graph(wgml_gpt2 *m, uint32_t pos) {
     if (m->graph_fusion != m->fusion || m->graph_tuning != ctx->tuning_generation) drop_graph(m);
     int b = 0;
     const uint32_t plan = plan_bucket(pos, p.n_seq, &b);
-    if (m->graph_exec[b]) return WGML_OK;
+    if (m->graph_exec[b]) {
+        if (multi && !m->graph_exec_multi[b]) {
+            const int rc = capture_steps(m, plan, kStepsPerGraph, &m->graph_multi[b],
+                                         &m->graph_exec_multi[b], nullptr);
+            if (rc != WGML_OK) drop_graph(m);
+            return rc;
+        }
+        return WGML_OK;
+    }
     WGML_TRY(reserve_all_plans(m));
     // An eager step first (function attributes, lazy loading); it runs at position 0
     // and would overwrite that column of every cache: keep a copy and put it back.
@@ -395,21 +437,9 @@ int build_graph(wgml_gpt2 *m, uint32_t pos) {
     if (ew != hipSuccess)
         return set_error(WGML_E_HIP, "wgml_gpt2: warm-up step failed: %s", hipGetErrorString(ew));
 
-    WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
-    const uint64_t launches0 = ctx->launches;
-    int rc = enqueue_step(m, true, 0, 0, plan);
-    if (rc == WGML_OK)
-        rc = launch_argmax_next(ctx, m->curr_vocab, p.n_vocab, m->dyn, m->d_prompt, m->d_tokens);
-    m->graph_launches[b] = ctx->launches - launches0;
-    hipError_t e = hipStreamEndCapture(ctx->stream, &m->graph[b]);
-    if (rc == WGML_OK && e != hipSuccess)
-        rc = set_error(WGML_E_HIP, "wgml_gpt2: graph capture failed: %s", hipGetErrorString(e));
-    if (rc == WGML_OK) {
-        e = hipGraphInstantiate(&m->graph_exec[b], m->graph[b], nullptr, nullptr, 0);
-        if (e != hipSuccess)
-            rc = set_error(WGML_E_HIP, "wgml_gpt2: graph instantiate failed: %s",
-                           hipGetErrorString(e));
-    }
+    int rc = capture_steps(m, plan, 1, &m->graph[b], &m->graph_exec[b], &m->graph_launches[b]);
+    if (rc == WGML_OK && multi)
+        rc = capture_steps(m, plan, kStepsPerGraph, &m->graph_multi[b], &m->graph_exec_multi[b], nullptr);
     if (rc != WGML_OK) {
         drop_graph(m);
         return rc;
@@ -487,8 +517,9 @@ int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_p
     if (use_graph) {
         // every bucket this run passes through, before the first launch
         for (uint32_t pos = 0; n_total > 0;) {
-            WGML_TRY(build_graph(m, pos));
             const uint32_t limit = plan_bucket(pos, m->p.n_seq, nullptr);
+            const uint32_t end = limit < n_total ? limit : n_total;
+            WGML_TRY(build_graph(m, pos, end - pos >= kStepsPerGraph));
             if (limit >= n_total || limit >= m->p.n_seq) break;
             pos = limit;
         }
@@ -504,7 +535,14 @@ int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_p
         int b = 0;
         const uint32_t plan = plan_bucket(i, m->p.n_seq, &b);
         if (use_graph) {
-            WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec[b], ctx->stream));
+            // steps left in this run that stay inside the bucket (positions below `plan`)
+            const uint32_t in_bucket = plan > i ? plan - i : 1;
+            if (m->graph_exec_multi[b] && n_total - i >= kStepsPerGraph && in_bucket >= kStepsPerGraph) {
+                WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec_multi[b], ctx->stream));
+                i += kStepsPerGraph - 1;
+            } else {
+                WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec[b], ctx->stream));
+            }
             m->launches_last = m->graph_launches[b];
         } else {
             const uint64_t l0 = ctx->launches;

@@ -46,6 +46,11 @@ struct wgml_llama2 {
     hipGraph_t graph[kMaxPlanBuckets] = {};
     hipGraphExec_t graph_exec[kMaxPlanBuckets] = {};
     uint64_t graph_launches[kMaxPlanBuckets] = {};  // launches of the recorded step
+    // kStepsPerGraph consecutive steps as one graph (the token loop replays it where that many
+    // steps stay inside a bucket): a replay costs the host a call and the GPU a few microseconds
+    // between two graphs, whatever the graph holds
+    hipGraph_t graph_multi[kMaxPlanBuckets] = {};
+    hipGraphExec_t graph_exec_multi[kMaxPlanBuckets] = {};
     int graph_fusion = -1;
     uint64_t graph_tuning = 0;  // the context's tuning generation the captures were made under
     // state of the batched prompt pass, allocated at its first use: one row per token
@@ -92,6 +97,10 @@ void drop_graph(wgml_llama2 *m) {
         if (m->graph[b]) (void)hipGraphDestroy(m->graph[b]);
         m->graph_exec[b] = nullptr;
         m->graph[b] = nullptr;
+        if (m->graph_exec_multi[b]) (void)hipGraphExecDestroy(m->graph_exec_multi[b]);
+        if (m->graph_multi[b]) (void)hipGraphDestroy(m->graph_multi[b]);
+        m->graph_exec_multi[b] = nullptr;
+        m->graph_multi[b] = nullptr;
     }
     m->graph_fusion = -1;
 }
@@ -276,16 +285,52 @@ int reserve_all_plans(wgml_llama2 *m) {
     return WGML_OK;
 }
 
+constexpr uint32_t kStepsPerGraph = 8;
+
+// Records `steps` consecutive steps (each followed by greedy sampling and the loop's
+// bookkeeping, all on the device) into one HIP graph.
+int capture_steps(wgml_llama2 *m, uint32_t plan, uint32_t steps, hipGraph_t *graph,
+                  hipGraphExec_t *exec, uint64_t *launches_per_step) {
+    wgml_ctx *ctx = m->ctx;
+    const wgml_llama2_config &c = m->cfg;
+    WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    const uint64_t launches0 = ctx->launches;
+    int rc = WGML_OK;
+    for (uint32_t k = 0; k < steps && rc == WGML_OK; ++k) {
+        rc = enqueue_step(m, true, 0, 0, plan);
+        if (rc == WGML_OK)
+            rc = launch_argmax_next(ctx, m->logits, c.vocab_size, m->dyn, m->d_prompt, m->d_tokens);
+    }
+    if (launches_per_step) *launches_per_step = (ctx->launches - launches0) / steps;
+    hipError_t e = hipStreamEndCapture(ctx->stream, graph);
+    if (rc != WGML_OK) return rc;
+    if (e != hipSuccess)
+        return set_error(WGML_E_HIP, "wgml_llama2: graph capture failed: %s", hipGetErrorString(e));
+    e = hipGraphInstantiate(exec, *graph, nullptr, nullptr, 0);
+    if (e != hipSuccess)
+        return set_error(WGML_E_HIP, "wgml_llama2: graph instantiate failed: %s",
+                         hipGetErrorString(e));
+    return WGML_OK;
+}
+
 // Records one step (+ greedy sampling and bookkeeping) into a HIP graph, for the bucket of
-// positions that `pos` lies in.
-int build_graph(wgml_llama2 *m, uint32_t pos) {
+// positions that `pos` lies in; with `multi` also the graph of kStepsPerGraph steps.
+int build_graph(wgml_llama2 *m, uint32_t pos, bool multi = false) {
     wgml_ctx *ctx = m->ctx;
     const wgml_llama2_config &c = m->cfg;
     // captures made at another fusion level or under other launch-shape overrides are stale
     if (m->graph_fusion != m->fusion || m->graph_tuning != ctx->tuning_generation) drop_graph(m);
     int b = 0;
     const uint32_t plan = plan_bucket(pos, c.seq_len, &b);
-    if (m->graph_exec[b]) return WGML_OK;
+    if (m->graph_exec[b]) {
+        if (multi && !m->graph_exec_multi[b]) {
+            const int rc = capture_steps(m, plan, kStepsPerGraph, &m->graph_multi[b],
+                                         &m->graph_exec_multi[b], nullptr);
+            if (rc != WGML_OK) drop_graph(m);
+            return rc;
+        }
+        return WGML_OK;
+    }
     // Everything that allocates or sets function attributes happens before capture:
     // the attention workspace for the largest plan, and one eager step.
     WGML_TRY(reserve_all_plans(m));
@@ -317,26 +362,12 @@ int build_graph(wgml_llama2 *m, uint32_t pos) {
     if (ew != hipSuccess)
         return set_error(WGML_E_HIP, "wgml_llama2: warm-up step failed: %s", hipGetErrorString(ew));
 
-    WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
-    const uint64_t launches0 = ctx->launches;
-    int rc = enqueue_step(m, true, 0, 0, plan);
-    if (rc == WGML_OK)
-        rc = launch_argmax_next(ctx, m->logits, c.vocab_size, m->dyn, m->d_prompt, m->d_tokens);
-    m->graph_launches[b] = ctx->launches - launches0;
-    hipError_t e = hipStreamEndCapture(ctx->stream, &m->graph[b]);
+    int rc = capture_steps(m, plan, 1, &m->graph[b], &m->graph_exec[b], &m->graph_launches[b]);
+    if (rc == WGML_OK && multi)
+        rc = capture_steps(m, plan, kStepsPerGraph, &m->graph_multi[b], &m->graph_exec_multi[b], nullptr);
     if (rc != WGML_OK) {
         drop_graph(m);
         return rc;
-    }
-    if (e != hipSuccess) {
-        drop_graph(m);
-        return set_error(WGML_E_HIP, "wgml_llama2: graph capture failed: %s", hipGetErrorString(e));
-    }
-    e = hipGraphInstantiate(&m->graph_exec[b], m->graph[b], nullptr, nullptr, 0);
-    if (e != hipSuccess) {
-        drop_graph(m);
-        return set_error(WGML_E_HIP, "wgml_llama2: graph instantiate failed: %s",
-                         hipGetErrorString(e));
     }
     m->graph_fusion = m->fusion;
     m->graph_tuning = ctx->tuning_generation;
@@ -353,8 +384,9 @@ int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint3
     if (use_graph) {
         // every bucket this run passes through, before the first launch
         for (uint32_t pos = start_pos; n_steps > 0;) {
-            WGML_TRY(build_graph(m, pos));
             const uint32_t limit = plan_bucket(pos, m->cfg.seq_len, nullptr);
+            const uint32_t end = limit < start_pos + n_steps ? limit : start_pos + n_steps;
+            WGML_TRY(build_graph(m, pos, end - pos >= kStepsPerGraph));
             if (limit >= start_pos + n_steps || limit >= m->cfg.seq_len) break;
             pos = limit;
         }
@@ -371,7 +403,15 @@ int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint3
         int b = 0;
         const uint32_t plan = plan_bucket(start_pos + i, m->cfg.seq_len, &b);
         if (use_graph) {
-            WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec[b], ctx->stream));
+            // steps left in this run that stay inside the bucket (positions below `plan`;
+            // the last bucket also takes what lies beyond, as single steps do)
+            const uint32_t in_bucket = plan > start_pos + i ? plan - (start_pos + i) : 1;
+            if (m->graph_exec_multi[b] && n_steps - i >= kStepsPerGraph && in_bucket >= kStepsPerGraph) {
+                WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec_multi[b], ctx->stream));
+                i += kStepsPerGraph - 1;
+            } else {
+                WGML_CHECK_HIP(hipGraphLaunch(m->graph_exec[b], ctx->stream));
+            }
             m->launches_last = m->graph_launches[b];
         } else {
             // the same launches, enqueued one by one (no host synchronisation either)
