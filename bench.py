@@ -314,7 +314,8 @@ def bench_gpt2(args, W, gpu):
     m = Gpt2(gpu, p).load(w)
     prompt = W.prompt_tokens(3, 32, p.n_vocab)
     n = min(32 + args.steps, p.n_seq)
-    m.generate_greedy(prompt, min(64, n))  # records the step
+    m.generate_greedy(prompt, min(64, n))  # warm-up
+    m.record_steps(n)  # the recorded steps of every range of positions the timed run passes
     gpu.synchronize()
     t0 = time.perf_counter()
     toks = m.generate_greedy(prompt, n)
@@ -357,7 +358,8 @@ def bench_8b_gqa(args, W, gpu):
             kv = W.rng_normal(1000 + 2 * layer + which, n_pre * cfg.kv_dim).reshape(n_pre, cfg.kv_dim)
             m.kv_upload(layer, which, 0, kv)
     gpu.synchronize()
-    m.decode_greedy(7, n_pre, 4)  # records the step
+    m.record_steps(n_pre, n)
+    m.decode_greedy(7, n_pre, 4)  # warm-up
     gpu.synchronize()
     t0 = time.perf_counter()
     toks = m.decode_greedy(7, n_pre, n)
@@ -417,7 +419,8 @@ def gpt2_leg(W, gpu, steps=288):
     m = Gpt2(gpu, p).load(synth_gpt2(p, seed=3))
     prompt = W.prompt_tokens(3, 32, p.n_vocab)
     n = min(32 + steps, p.n_seq)
-    m.generate_greedy(prompt, min(64, n))  # records the step
+    m.generate_greedy(prompt, min(64, n))  # warm-up
+    m.record_steps(n)  # the recorded steps of every range of positions the timed run passes
     gpu.synchronize()
     t0 = time.perf_counter()
     m.generate_greedy(prompt, n)
@@ -559,6 +562,11 @@ def main():
     first = int(np.argmax(model.logits()))
     p0 = n_prompt  # position of the first decode step
 
+    # the steps are recorded (captured as graphs, one per range of positions) before anything
+    # is timed: a run that crosses position 256 would otherwise record the next range inside
+    # the timed region
+    model.record_steps(p0, args.warmup + args.steps)
+
     if args.decode_only:
         wtoks = model.decode_greedy(first, p0, args.warmup)
         gpu.synchronize()
@@ -616,6 +624,7 @@ def main():
     # arithmetic of the reference's shaders), same fused launches
     gpu.set_tuning(gpu.TUNE_GEMV_F32_ACTIVATIONS, 1)
     n32 = min(args.steps, 64)
+    model.record_steps(p0, n32)  # (a changed override drops the recorded steps)
     model.decode_greedy(first, p0, 2)
     gpu.synchronize()
     t0 = time.perf_counter()

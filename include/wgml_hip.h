@@ -345,6 +345,13 @@ WGML_API int wgml_llama2_generate_greedy(wgml_llama2 *m, const uint32_t *prompt,
  * for positions < start_pos; first consumed token is `first_token`. */
 WGML_API int wgml_llama2_decode_greedy(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos,
                                        uint32_t n_steps, uint32_t *out_tokens);
+/* Records, ahead of time, the steps that the token loops replay for positions
+ * start_pos .. start_pos + n_steps - 1 (one capture per range of positions, limits 256, 512,
+ * 1024, ...: what the first run through such a range would otherwise do before its first
+ * launch, a few milliseconds per range).  No counterpart in the reference, which has nothing
+ * to record; KV caches and logits are left as they were.  Without graphs
+ * (WGML_DISABLE_GRAPHS) it only reserves the attention workspace. */
+WGML_API int wgml_llama2_record_steps(wgml_llama2 *m, uint32_t start_pos, uint32_t n_steps);
 /* The same loop with a blocking read-back of the sampled token after every
  * step, as the reference's chat loop does (chat_llama2.rs:205-220). */
 WGML_API int wgml_llama2_decode_greedy_sync(wgml_llama2 *m, uint32_t first_token,
@@ -425,6 +432,8 @@ WGML_API int wgml_gpt2_read_logits(wgml_gpt2 *m, float *host_out);
 /* ChatGpt2::forward's loop with greedy sampling (wgml-chat/src/chat_gpt2.rs:43-151). */
 WGML_API int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_prompt,
                                        uint32_t n_total, uint32_t *out_tokens);
+/* As wgml_llama2_record_steps, for positions 0 .. n_total - 1. */
+WGML_API int wgml_gpt2_record_steps(wgml_gpt2 *m, uint32_t n_total);
 /* 0: layernorm, GELU and the q/k/v copies are launches of their own and the token
  * loop reads every token back (mirrors Gpt2::dispatch and chat_gpt2.rs one to
  * one); 1 (default): LayerNorm folded into the GEMV that consumes it, bias /

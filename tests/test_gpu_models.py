@@ -122,6 +122,26 @@ def test_tuning_change_rerecords_the_step(gpu):
             gpu.set_tuning(key, bad)
 
 
+def test_recording_steps_ahead_of_time(gpu):
+    # record_steps captures what the token loop replays (single steps and runs of eight) for a
+    # range of positions without touching caches or logits; the loop that follows gives the
+    # oracle's tokens, also for step counts that are no multiple of eight
+    w = synth_llama(MICRO, seed=23, scheme="q8_0")
+    spice(w, MICRO, 7, biases=False)
+    prompt = W.prompt_tokens(8, 3, MICRO.vocab_size)
+    want_t, _ = orc.Llama2(w).generate_greedy(prompt, 29)
+    m = Llama2(gpu, MICRO).load(w)
+    m.record_steps(0, MICRO.seq_len)
+    for n in (29, 8, 7, 17):
+        assert np.array_equal(m.generate_greedy(prompt, n), want_t[:n]), n
+    # a decode that continues from a cache the caller filled: recording must leave it alone
+    kv0 = m.kv_download(0, 0, 0, 8).copy()
+    m.record_steps(8, 16)
+    assert np.array_equal(m.kv_download(0, 0, 0, 8), kv0)
+    with pytest.raises(W.WgmlError):
+        m.record_steps(MICRO.seq_len - 1, 2)
+
+
 def test_output_projection_merging_attention_partials(gpu):
     # on request the layer's output projection merges attention's partial results itself: the
     # step keeps its launch count at a short context (no merge launch either way) and its tokens
@@ -364,8 +384,13 @@ def test_gpt2_micro_greedy_with_norm_affine(gpu):
     prompt = W.prompt_tokens(9, 6, p.n_vocab)
     want, _ = orc.Gpt2(w).generate_greedy(prompt, p.n_seq)
     m = Gpt2(gpu, p).load(w)
-    assert np.array_equal(m.generate_greedy(prompt, p.n_seq), want)
+    m.record_steps(p.n_seq)  # ahead of the first run; step counts that are no multiple of eight
+    for n in (p.n_seq, 13, 8, 3):
+        assert np.array_equal(m.generate_greedy(prompt, n), want[:n]), n
+    with pytest.raises(W.WgmlError):
+        m.record_steps(p.n_seq + 1)
     m.set_fusion(0)
+    m.record_steps(p.n_seq)  # nothing to record for the loop with one launch per op
     assert np.array_equal(m.generate_greedy(prompt, p.n_seq), want)
 
 

@@ -138,6 +138,8 @@ PROTOTYPES = {
     "wgml_llama2_prefill": (_i, [_P, _P, _u32, _u32]),
     "wgml_llama2_prefill_decode_greedy": (_i, [_P, _P, _u32, _u32, _P]),
     "wgml_llama2_decode_greedy": (_i, [_P, _u32, _u32, _u32, _P]),
+    "wgml_llama2_record_steps": (_i, [_P, _u32, _u32]),
+    "wgml_gpt2_record_steps": (_i, [_P, _u32]),
     "wgml_llama2_decode_greedy_sync": (_i, [_P, _u32, _u32, _u32, _P]),
     "wgml_llama2_kv_upload": (_i, [_P, _u32, _i, _u32, _u32, _P]),
     "wgml_llama2_kv_download": (_i, [_P, _u32, _i, _u32, _u32, _P]),

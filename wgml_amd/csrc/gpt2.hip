@@ -386,12 +386,42 @@ int capture_steps(wgml_gpt2 *m, uint32_t plan, uint32_t steps, hipGraph_t *graph
     e = hipGraphInstantiate(exec, *graph, nullptr, nullptr, 0);
     if (e != hipSuccess)
         return set_error(WGML_E_HIP, "wgml_gpt2: graph instantiate failed: %s", hipGetErrorString(e));
+    if (steps > 1) {
+        // A graph's first replay costs milliseconds (uploading the graph ahead of time does
+        // not remove it): do it here, from position 0, with the cache rows it writes saved
+        // and put back.
+        const size_t bytes = (size_t)steps * m->p.n_embd * 4;
+        void *saved = nullptr;
+        WGML_CHECK_HIP(hipMalloc(&saved, bytes * 2 * m->p.n_layer));
+        for (uint32_t l = 0; l < m->p.n_layer; ++l) {
+            (void)hipMemcpyAsync((char *)saved + bytes * (2 * l), m->layers[l].key_cache, bytes,
+                                 hipMemcpyDeviceToDevice, ctx->stream);
+            (void)hipMemcpyAsync((char *)saved + bytes * (2 * l + 1), m->layers[l].value_cache, bytes,
+                                 hipMemcpyDeviceToDevice, ctx->stream);
+        }
+        const DynState init{0, 0, 0, 0};
+        e = hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipGraphLaunch(*exec, ctx->stream);
+        for (uint32_t l = 0; l < m->p.n_layer; ++l) {
+            (void)hipMemcpyAsync(m->layers[l].key_cache, (char *)saved + bytes * (2 * l), bytes,
+                                 hipMemcpyDeviceToDevice, ctx->stream);
+            (void)hipMemcpyAsync(m->layers[l].value_cache, (char *)saved + bytes * (2 * l + 1), bytes,
+                                 hipMemcpyDeviceToDevice, ctx->stream);
+        }
+        const hipError_t es = hipStreamSynchronize(ctx->stream);  // `init` is a stack object
+        (void)hipFree(saved);
+        if (e == hipSuccess) e = es;
+        if (e != hipSuccess)
+            return set_error(WGML_E_HIP, "wgml_gpt2: first replay failed: %s", hipGetErrorString(e));
+    }
     return WGML_OK;
 }
 
 // Records one step (+ greedy sampling and bookkeeping) into a HIP graph, for the bucket of
-// positions that `pos` lies in; with `multi` also the graph of kStepsPerGraph steps.
-int build_graph(wgml_gpt2 *m, uint32_t pos, bool multi = false) {
+// positions that `pos` lies in, and the graph of kStepsPerGraph such steps where the bucket
+// holds that many positions (both at once, so that a short first run leaves nothing to build
+// for a longer one).
+int build_graph(wgml_gpt2 *m, uint32_t pos) {
     wgml_ctx *ctx = m->ctx;
     const wgml_gpt2_params &p = m->p;
     const uint32_t n = p.n_embd;
@@ -399,6 +429,8 @@ int build_graph(wgml_gpt2 *m, uint32_t pos, bool multi = false) {
     if (m->graph_fusion != m->fusion || m->graph_tuning != ctx->tuning_generation) drop_graph(m);
     int b = 0;
     const uint32_t plan = plan_bucket(pos, p.n_seq, &b);
+    // the bucket's positions are [256 << (b - 1), plan), from 0 for the first bucket
+    const bool multi = plan - (b == 0 ? 0u : 256u << (b - 1)) >= kStepsPerGraph;
     if (m->graph_exec[b]) {
         if (multi && !m->graph_exec_multi[b]) {
             const int rc = capture_steps(m, plan, kStepsPerGraph, &m->graph_multi[b],
@@ -449,6 +481,18 @@ int build_graph(wgml_gpt2 *m, uint32_t pos, bool multi = false) {
     return WGML_OK;
 }
 
+// The recorded steps of every bucket that a run over positions 0 .. n_total - 1 passes through.
+int record_steps(wgml_gpt2 *m, uint32_t n_total) {
+    if (graphs_disabled()) return reserve_all_plans(m);
+    for (uint32_t pos = 0; n_total > 0;) {
+        const uint32_t limit = plan_bucket(pos, m->p.n_seq, nullptr);
+        WGML_TRY(build_graph(m, pos));
+        if (limit >= n_total || limit >= m->p.n_seq) break;
+        pos = limit;
+    }
+    return WGML_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -479,6 +523,15 @@ int wgml_gpt2_read_logits(wgml_gpt2 *m, float *host_out) {
                                   hipMemcpyDeviceToHost, m->ctx->stream));
     WGML_CHECK_HIP(hipStreamSynchronize(m->ctx->stream));
     return WGML_OK;
+}
+
+int wgml_gpt2_record_steps(wgml_gpt2 *m, uint32_t n_total) {
+    WGML_REQUIRE(m, "wgml_gpt2_record_steps: null argument");
+    WGML_REQUIRE(n_total <= m->p.n_seq, "wgml_gpt2_record_steps: %u positions exceed n_seq %u", n_total,
+                 m->p.n_seq);
+    WGML_TRY(check_ready(m));
+    if (m->fusion < 1 || !can_fold(m)) return WGML_OK;  // the unfused loop records nothing
+    return record_steps(m, n_total);
 }
 
 int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_prompt,
@@ -514,18 +567,7 @@ int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_p
     // Recorded step replayed per token: sampling and bookkeeping stay on the device,
     // one synchronisation at the end.
     const bool use_graph = !graphs_disabled();
-    if (use_graph) {
-        // every bucket this run passes through, before the first launch
-        for (uint32_t pos = 0; n_total > 0;) {
-            const uint32_t limit = plan_bucket(pos, m->p.n_seq, nullptr);
-            const uint32_t end = limit < n_total ? limit : n_total;
-            WGML_TRY(build_graph(m, pos, end - pos >= kStepsPerGraph));
-            if (limit >= n_total || limit >= m->p.n_seq) break;
-            pos = limit;
-        }
-    } else {
-        WGML_TRY(reserve_all_plans(m));
-    }
+    WGML_TRY(record_steps(m, n_total));
     const uint32_t np = n_prompt < n_total ? n_prompt : n_total;
     WGML_CHECK_HIP(hipMemcpyAsync(m->d_prompt, prompt, (size_t)np * 4, hipMemcpyHostToDevice,
                                   ctx->stream));

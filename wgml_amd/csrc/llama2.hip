@@ -310,18 +310,50 @@ int capture_steps(wgml_llama2 *m, uint32_t plan, uint32_t steps, hipGraph_t *gra
     if (e != hipSuccess)
         return set_error(WGML_E_HIP, "wgml_llama2: graph instantiate failed: %s",
                          hipGetErrorString(e));
+    if (steps > 1) {
+        // A graph's first replay costs milliseconds (2.2 ms for the eight steps of the 7B
+        // shape; uploading the graph ahead of time does not remove it): do it here, from
+        // position 0, with the cache rows it writes saved and put back.
+        const size_t bytes = (size_t)steps * m->kv_dim * 4;
+        void *saved = nullptr;
+        WGML_CHECK_HIP(hipMalloc(&saved, bytes * 2 * c.n_layers));
+        for (uint32_t l = 0; l < c.n_layers; ++l) {
+            (void)hipMemcpyAsync((char *)saved + bytes * (2 * l), m->layers[l].key_cache, bytes,
+                                 hipMemcpyDeviceToDevice, ctx->stream);
+            (void)hipMemcpyAsync((char *)saved + bytes * (2 * l + 1), m->layers[l].value_cache, bytes,
+                                 hipMemcpyDeviceToDevice, ctx->stream);
+        }
+        const DynState init{0, 0, 0, 0};
+        e = hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipGraphLaunch(*exec, ctx->stream);
+        for (uint32_t l = 0; l < c.n_layers; ++l) {
+            (void)hipMemcpyAsync(m->layers[l].key_cache, (char *)saved + bytes * (2 * l), bytes,
+                                 hipMemcpyDeviceToDevice, ctx->stream);
+            (void)hipMemcpyAsync(m->layers[l].value_cache, (char *)saved + bytes * (2 * l + 1), bytes,
+                                 hipMemcpyDeviceToDevice, ctx->stream);
+        }
+        const hipError_t es = hipStreamSynchronize(ctx->stream);  // `init` is a stack object
+        (void)hipFree(saved);
+        if (e == hipSuccess) e = es;
+        if (e != hipSuccess)
+            return set_error(WGML_E_HIP, "wgml_llama2: first replay failed: %s", hipGetErrorString(e));
+    }
     return WGML_OK;
 }
 
 // Records one step (+ greedy sampling and bookkeeping) into a HIP graph, for the bucket of
-// positions that `pos` lies in; with `multi` also the graph of kStepsPerGraph steps.
-int build_graph(wgml_llama2 *m, uint32_t pos, bool multi = false) {
+// positions that `pos` lies in, and the graph of kStepsPerGraph such steps where the bucket
+// holds that many positions (both at once, so that a short first run leaves nothing to build
+// for a longer one).
+int build_graph(wgml_llama2 *m, uint32_t pos) {
     wgml_ctx *ctx = m->ctx;
     const wgml_llama2_config &c = m->cfg;
     // captures made at another fusion level or under other launch-shape overrides are stale
     if (m->graph_fusion != m->fusion || m->graph_tuning != ctx->tuning_generation) drop_graph(m);
     int b = 0;
     const uint32_t plan = plan_bucket(pos, c.seq_len, &b);
+    // the bucket's positions are [256 << (b - 1), plan), from 0 for the first bucket
+    const bool multi = plan - (b == 0 ? 0u : 256u << (b - 1)) >= kStepsPerGraph;
     if (m->graph_exec[b]) {
         if (multi && !m->graph_exec_multi[b]) {
             const int rc = capture_steps(m, plan, kStepsPerGraph, &m->graph_multi[b],
@@ -374,6 +406,19 @@ int build_graph(wgml_llama2 *m, uint32_t pos, bool multi = false) {
     return WGML_OK;
 }
 
+// The recorded steps of every bucket that a run of n_steps from start_pos passes through,
+// before its first launch.
+int record_steps(wgml_llama2 *m, uint32_t start_pos, uint32_t n_steps) {
+    if (graphs_disabled()) return reserve_all_plans(m);
+    for (uint32_t pos = start_pos; n_steps > 0;) {
+        const uint32_t limit = plan_bucket(pos, m->cfg.seq_len, nullptr);
+        WGML_TRY(build_graph(m, pos));
+        if (limit >= start_pos + n_steps || limit >= m->cfg.seq_len) break;
+        pos = limit;
+    }
+    return WGML_OK;
+}
+
 // Runs n_steps recorded steps from (first_token, start_pos); prompt tokens (if
 // any) are forced.  One synchronisation at the end.
 int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint32_t n_steps,
@@ -381,18 +426,7 @@ int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint3
     wgml_ctx *ctx = m->ctx;
     WGML_TRY(check_ready(m));
     const bool use_graph = !graphs_disabled();
-    if (use_graph) {
-        // every bucket this run passes through, before the first launch
-        for (uint32_t pos = start_pos; n_steps > 0;) {
-            const uint32_t limit = plan_bucket(pos, m->cfg.seq_len, nullptr);
-            const uint32_t end = limit < start_pos + n_steps ? limit : start_pos + n_steps;
-            WGML_TRY(build_graph(m, pos, end - pos >= kStepsPerGraph));
-            if (limit >= start_pos + n_steps || limit >= m->cfg.seq_len) break;
-            pos = limit;
-        }
-    } else {
-        WGML_TRY(reserve_all_plans(m));
-    }
+    WGML_TRY(record_steps(m, start_pos, n_steps));
     if (n_prompt)
         WGML_CHECK_HIP(hipMemcpyAsync(m->d_prompt, prompt, (size_t)n_prompt * 4,
                                       hipMemcpyHostToDevice, ctx->stream));
@@ -781,6 +815,15 @@ int wgml_llama2_decode_greedy(wgml_llama2 *m, uint32_t first_token, uint32_t sta
     WGML_REQUIRE(first_token < m->cfg.vocab_size, "wgml_llama2_decode_greedy: token outside vocabulary");
     if (n_steps == 0) return WGML_OK;
     return run_recorded(m, first_token, start_pos, n_steps, nullptr, 0, out_tokens);
+}
+
+int wgml_llama2_record_steps(wgml_llama2 *m, uint32_t start_pos, uint32_t n_steps) {
+    WGML_REQUIRE(m, "wgml_llama2_record_steps: null argument");
+    WGML_REQUIRE((uint64_t)start_pos + n_steps <= m->cfg.seq_len,
+                 "wgml_llama2_record_steps: %u steps from %u exceed seq_len %u", n_steps, start_pos,
+                 m->cfg.seq_len);
+    WGML_TRY(check_ready(m));
+    return record_steps(m, start_pos, n_steps);
 }
 
 int wgml_llama2_generate_greedy(wgml_llama2 *m, const uint32_t *prompt, uint32_t n_prompt,

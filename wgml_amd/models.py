@@ -203,6 +203,12 @@ class Llama2:
         call("wgml_llama2_decode_greedy", self._h, first_token, start_pos, n_steps, _ptr(out))
         return out
 
+    def record_steps(self, start_pos: int, n_steps: int) -> None:
+        """Records ahead of time the steps the token loops replay for positions
+        start_pos .. start_pos + n_steps - 1 (otherwise the first run through a range of
+        positions does it before its first launch)."""
+        call("wgml_llama2_record_steps", self._h, start_pos, n_steps)
+
     def decode_greedy_sync(self, first_token: int, start_pos: int, n_steps: int) -> np.ndarray:
         """Same as decode_greedy with a host read-back of every token."""
         out = np.empty(n_steps, dtype=np.uint32)
@@ -330,6 +336,11 @@ class Gpt2:
         out = np.empty(n_total, dtype=np.uint32)
         call("wgml_gpt2_generate_greedy", self._h, _ptr(p), p.size, n_total, _ptr(out))
         return out
+
+    def record_steps(self, n_total: int) -> None:
+        """Records ahead of time the steps `generate_greedy` replays for positions
+        0 .. n_total - 1."""
+        call("wgml_gpt2_record_steps", self._h, n_total)
 
     def close(self) -> None:
         if self._h:
