@@ -134,10 +134,17 @@ def test_recording_steps_ahead_of_time(gpu):
     m.record_steps(0, MICRO.seq_len)
     for n in (29, 8, 7, 17):
         assert np.array_equal(m.generate_greedy(prompt, n), want_t[:n]), n
-    # a decode that continues from a cache the caller filled: recording must leave it alone
+    # a decode that continues from a cache the caller filled: recording must leave it, and
+    # the logits of the last step, alone (a changed override drops what was recorded)
     kv0 = m.kv_download(0, 0, 0, 8).copy()
-    m.record_steps(8, 16)
+    logits0 = m.logits().copy()
+    gpu.set_tuning(gpu.TUNE_ATTN_SPLITS, 3)
+    try:
+        m.record_steps(8, 16)
+    finally:
+        gpu.set_tuning(gpu.TUNE_ATTN_SPLITS, 0)
     assert np.array_equal(m.kv_download(0, 0, 0, 8), kv0)
+    assert np.array_equal(m.logits(), logits0)
     with pytest.raises(W.WgmlError):
         m.record_steps(MICRO.seq_len - 1, 2)
 

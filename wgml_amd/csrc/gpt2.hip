@@ -531,7 +531,18 @@ int wgml_gpt2_record_steps(wgml_gpt2 *m, uint32_t n_total) {
                  m->p.n_seq);
     WGML_TRY(check_ready(m));
     if (m->fusion < 1 || !can_fold(m)) return WGML_OK;  // the unfused loop records nothing
-    return record_steps(m, n_total);
+    // recording runs steps of its own: the logits the caller may still want are kept aside
+    const size_t bytes = (size_t)m->p.n_vocab * 4;
+    void *saved = nullptr;
+    WGML_CHECK_HIP(hipMalloc(&saved, bytes));
+    (void)hipMemcpyAsync(saved, m->curr_vocab, bytes, hipMemcpyDeviceToDevice, m->ctx->stream);
+    const int rc = record_steps(m, n_total);
+    (void)hipMemcpyAsync(m->curr_vocab, saved, bytes, hipMemcpyDeviceToDevice, m->ctx->stream);
+    const hipError_t e = hipStreamSynchronize(m->ctx->stream);
+    (void)hipFree(saved);
+    if (rc != WGML_OK) return rc;
+    WGML_CHECK_HIP(e);
+    return WGML_OK;
 }
 
 int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_prompt,

@@ -823,7 +823,19 @@ int wgml_llama2_record_steps(wgml_llama2 *m, uint32_t start_pos, uint32_t n_step
                  "wgml_llama2_record_steps: %u steps from %u exceed seq_len %u", n_steps, start_pos,
                  m->cfg.seq_len);
     WGML_TRY(check_ready(m));
-    return record_steps(m, start_pos, n_steps);
+    // recording runs steps of its own (from position 0, cache rows saved and put back): the
+    // logits the caller may still want to read are kept aside as well
+    const size_t bytes = (size_t)m->cfg.vocab_size * 4;
+    void *saved = nullptr;
+    WGML_CHECK_HIP(hipMalloc(&saved, bytes));
+    (void)hipMemcpyAsync(saved, m->logits, bytes, hipMemcpyDeviceToDevice, m->ctx->stream);
+    const int rc = record_steps(m, start_pos, n_steps);
+    (void)hipMemcpyAsync(m->logits, saved, bytes, hipMemcpyDeviceToDevice, m->ctx->stream);
+    const hipError_t e = hipStreamSynchronize(m->ctx->stream);
+    (void)hipFree(saved);
+    if (rc != WGML_OK) return rc;
+    WGML_CHECK_HIP(e);
+    return WGML_OK;
 }
 
 int wgml_llama2_generate_greedy(wgml_llama2 *m, const uint32_t *prompt, uint32_t n_prompt,
