@@ -282,8 +282,21 @@ struct DynState {
 int launch_embed(wgml_ctx *ctx, float *x, const float *table, uint32_t dim, DynPos token,
                  float *rope_cs, uint32_t head_size, float rope_base, DynPos pos,
                  const float *pos_table = nullptr);
+// What launch_embed does for the token and position that launch_argmax_next has just chosen,
+// done by that same launch: the next step of a token loop then starts with its first layer.
+struct NextEmbed {
+    float *x;
+    const float *table;
+    uint32_t dim;
+    float *rope_cs;  // optional
+    uint32_t head_size;
+    float rope_base;
+    const float *pos_table;  // optional (GPT-2's learned positions)
+    uint32_t n_pos;          // rows of pos_table: no row is read for a position beyond them
+};
 int launch_argmax_next(wgml_ctx *ctx, const float *v, uint32_t n, DynState *dyn,
-                       const uint32_t *prompt, uint32_t *tokens_out);
+                       const uint32_t *prompt, uint32_t *tokens_out,
+                       const NextEmbed *embed = nullptr);
 int launch_dequantize(wgml_ctx *ctx, float *out, const wgml_qmat *m);
 
 // ---- batched products for prompt processing (prefill.hip) ---------------------

@@ -240,8 +240,10 @@ bool can_fold(const wgml_gpt2 *m) {
     return true;
 }
 
+// embed == false: m->layer_input already holds wte[:, token] + wpe[:, pos] (the sampling launch
+// of the step before wrote it).
 int enqueue_step(wgml_gpt2 *m, bool dynamic, uint32_t token, uint32_t pos,
-                 uint32_t plan_positions = 0) {
+                 uint32_t plan_positions = 0, bool embed = true) {
     const wgml_gpt2_params &p = m->p;
     wgml_ctx *ctx = m->ctx;
     const uint32_t n = p.n_embd;
@@ -254,7 +256,7 @@ int enqueue_step(wgml_gpt2 *m, bool dynamic, uint32_t token, uint32_t pos,
         return set_error(WGML_E_UNSUPPORTED, "wgml_gpt2: the recorded step needs fusion 1");
 
     // layer_input = wte[:, token] + wpe[:, pos]   (:277-290)
-    WGML_TRY(launch_embed(ctx, m->layer_input, m->wte, n, dtok, nullptr, 2, 0.f, dpos, m->wpe));
+    if (embed) WGML_TRY(launch_embed(ctx, m->layer_input, m->wte, n, dtok, nullptr, 2, 0.f, dpos, m->wpe));
 
     for (uint32_t l = 0; l < p.n_layer; ++l) {
         const Gpt2Layer &w = m->layers[l];
@@ -365,6 +367,21 @@ int reserve_all_plans(wgml_gpt2 *m) {
 
 constexpr uint32_t kStepsPerGraph = 8;
 
+// A step of the token loop that keeps its state on the device: the layers and the output
+// projection, then the launch that samples (arg-max), does the loop's bookkeeping and writes
+// wte[:, token] + wpe[:, pos] of the token and position it has chosen, for the step that
+// follows.  The loop's first step finds it written by loop_first_embed.
+int enqueue_loop_step(wgml_gpt2 *m, uint32_t plan) {
+    const wgml_gpt2_params &p = m->p;
+    WGML_TRY(enqueue_step(m, true, 0, 0, plan, false));
+    const NextEmbed ne{m->layer_input, m->wte, p.n_embd, nullptr, 2, 0.f, m->wpe, p.n_seq};
+    return launch_argmax_next(m->ctx, m->curr_vocab, p.n_vocab, m->dyn, m->d_prompt, m->d_tokens, &ne);
+}
+int loop_first_embed(wgml_gpt2 *m) {
+    return launch_embed(m->ctx, m->layer_input, m->wte, m->p.n_embd, DynPos{&m->dyn->token, 0}, nullptr, 2,
+                        0.f, DynPos{&m->dyn->pos, 0}, m->wpe);
+}
+
 // Records `steps` consecutive steps (each followed by greedy sampling and the loop's
 // bookkeeping, all on the device) into one HIP graph.
 int capture_steps(wgml_gpt2 *m, uint32_t plan, uint32_t steps, hipGraph_t *graph,
@@ -373,11 +390,7 @@ int capture_steps(wgml_gpt2 *m, uint32_t plan, uint32_t steps, hipGraph_t *graph
     WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     const uint64_t launches0 = ctx->launches;
     int rc = WGML_OK;
-    for (uint32_t k = 0; k < steps && rc == WGML_OK; ++k) {
-        rc = enqueue_step(m, true, 0, 0, plan);
-        if (rc == WGML_OK)
-            rc = launch_argmax_next(ctx, m->curr_vocab, m->p.n_vocab, m->dyn, m->d_prompt, m->d_tokens);
-    }
+    for (uint32_t k = 0; k < steps && rc == WGML_OK; ++k) rc = enqueue_loop_step(m, plan);
     if (launches_per_step) *launches_per_step = (ctx->launches - launches0) / steps;
     hipError_t e = hipStreamEndCapture(ctx->stream, graph);
     if (rc != WGML_OK) return rc;
@@ -401,6 +414,7 @@ int capture_steps(wgml_gpt2 *m, uint32_t plan, uint32_t steps, hipGraph_t *graph
         }
         const DynState init{0, 0, 0, 0};
         e = hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess && loop_first_embed(m) != WGML_OK) e = hipErrorUnknown;
         if (e == hipSuccess) e = hipGraphLaunch(*exec, ctx->stream);
         for (uint32_t l = 0; l < m->p.n_layer; ++l) {
             (void)hipMemcpyAsync(m->layers[l].key_cache, (char *)saved + bytes * (2 * l), bytes,
@@ -454,9 +468,8 @@ int build_graph(wgml_gpt2 *m, uint32_t pos) {
     }
     const DynState init{0, 0, 0, 0};
     hipError_t ew = hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream);
-    int rcw = ew == hipSuccess ? enqueue_step(m, true, 0, 0, plan) : WGML_E_HIP;
-    if (rcw == WGML_OK)
-        rcw = launch_argmax_next(ctx, m->curr_vocab, p.n_vocab, m->dyn, m->d_prompt, m->d_tokens);
+    int rcw = ew == hipSuccess ? loop_first_embed(m) : WGML_E_HIP;
+    if (rcw == WGML_OK) rcw = enqueue_loop_step(m, plan);
     for (uint32_t l = 0; l < p.n_layer; ++l) {
         (void)hipMemcpyAsync(m->layers[l].key_cache, (char *)saved + col * (2 * l), col,
                              hipMemcpyDeviceToDevice, ctx->stream);
@@ -584,6 +597,7 @@ int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_p
                                   ctx->stream));
     const DynState init{0, prompt[0], 0, np};
     WGML_CHECK_HIP(hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream));
+    WGML_TRY(loop_first_embed(m));
     for (uint32_t i = 0; i < n_total; ++i) {
         int b = 0;
         const uint32_t plan = plan_bucket(i, m->p.n_seq, &b);
@@ -599,9 +613,7 @@ int wgml_gpt2_generate_greedy(wgml_gpt2 *m, const uint32_t *prompt, uint32_t n_p
             m->launches_last = m->graph_launches[b];
         } else {
             const uint64_t l0 = ctx->launches;
-            WGML_TRY(enqueue_step(m, true, 0, 0, plan));
-            WGML_TRY(launch_argmax_next(ctx, m->curr_vocab, m->p.n_vocab, m->dyn, m->d_prompt,
-                                        m->d_tokens));
+            WGML_TRY(enqueue_loop_step(m, plan));
             m->launches_last = ctx->launches - l0;
         }
     }

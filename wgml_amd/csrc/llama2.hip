@@ -113,8 +113,10 @@ void drop_graph(wgml_llama2 *m) {
 // fusion 0: one launch per reference op.  1: bias and residual adds folded into
 // the GEMV epilogues.  2: additionally every RMSNorm folded into the staging of
 // the GEMVs that consume it.
+//   embed == false : m->x and the RoPE table already hold the token's embedding and the
+//                     position's angles (the sampling launch of the step before wrote them).
 int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos,
-                 uint32_t plan_positions = 0) {
+                 uint32_t plan_positions = 0, bool embed = true) {
     const wgml_llama2_config &c = m->cfg;
     wgml_ctx *ctx = m->ctx;
     const uint32_t dim = c.dim, kv_dim = m->kv_dim;
@@ -126,8 +128,9 @@ int enqueue_step(wgml_llama2 *m, bool dynamic, uint32_t token, uint32_t pos,
     const uint32_t plan = dynamic ? (plan_positions ? plan_positions : c.seq_len) : pos + 1;
 
     // dim >= head_size / 2, so the embedding launch also covers the RoPE table
-    WGML_TRY(launch_embed(ctx, m->x, m->token_embd, dim, dtok, m->rope_cs, m->head_size,
-                          c.rope_base_freq, dpos));
+    if (embed)
+        WGML_TRY(launch_embed(ctx, m->x, m->token_embd, dim, dtok, m->rope_cs, m->head_size,
+                              c.rope_base_freq, dpos));
 
     for (uint32_t l = 0; l < c.n_layers; ++l) {
         const LlamaLayer &w = m->layers[l];
@@ -287,6 +290,22 @@ int reserve_all_plans(wgml_llama2 *m) {
 
 constexpr uint32_t kStepsPerGraph = 8;
 
+// A step of the token loops that keep their state on the device: the layers and the output
+// projection, then the launch that samples (arg-max), does the loop's bookkeeping and writes the
+// embedding and the RoPE table of the token and position it has chosen, for the step that follows.
+// The loop's first step finds them written by loop_first_embed.
+int enqueue_loop_step(wgml_llama2 *m, uint32_t plan) {
+    const wgml_llama2_config &c = m->cfg;
+    WGML_TRY(enqueue_step(m, true, 0, 0, plan, false));
+    const NextEmbed ne{m->x, m->token_embd, c.dim, m->rope_cs, m->head_size, c.rope_base_freq, nullptr, 0};
+    return launch_argmax_next(m->ctx, m->logits, c.vocab_size, m->dyn, m->d_prompt, m->d_tokens, &ne);
+}
+int loop_first_embed(wgml_llama2 *m) {
+    const wgml_llama2_config &c = m->cfg;
+    return launch_embed(m->ctx, m->x, m->token_embd, c.dim, DynPos{&m->dyn->token, 0}, m->rope_cs,
+                        m->head_size, c.rope_base_freq, DynPos{&m->dyn->pos, 0});
+}
+
 // Records `steps` consecutive steps (each followed by greedy sampling and the loop's
 // bookkeeping, all on the device) into one HIP graph.
 int capture_steps(wgml_llama2 *m, uint32_t plan, uint32_t steps, hipGraph_t *graph,
@@ -296,11 +315,7 @@ int capture_steps(wgml_llama2 *m, uint32_t plan, uint32_t steps, hipGraph_t *gra
     WGML_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     const uint64_t launches0 = ctx->launches;
     int rc = WGML_OK;
-    for (uint32_t k = 0; k < steps && rc == WGML_OK; ++k) {
-        rc = enqueue_step(m, true, 0, 0, plan);
-        if (rc == WGML_OK)
-            rc = launch_argmax_next(ctx, m->logits, c.vocab_size, m->dyn, m->d_prompt, m->d_tokens);
-    }
+    for (uint32_t k = 0; k < steps && rc == WGML_OK; ++k) rc = enqueue_loop_step(m, plan);
     if (launches_per_step) *launches_per_step = (ctx->launches - launches0) / steps;
     hipError_t e = hipStreamEndCapture(ctx->stream, graph);
     if (rc != WGML_OK) return rc;
@@ -325,6 +340,7 @@ int capture_steps(wgml_llama2 *m, uint32_t plan, uint32_t steps, hipGraph_t *gra
         }
         const DynState init{0, 0, 0, 0};
         e = hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess && loop_first_embed(m) != WGML_OK) e = hipErrorUnknown;
         if (e == hipSuccess) e = hipGraphLaunch(*exec, ctx->stream);
         for (uint32_t l = 0; l < c.n_layers; ++l) {
             (void)hipMemcpyAsync(m->layers[l].key_cache, (char *)saved + bytes * (2 * l), bytes,
@@ -379,9 +395,8 @@ int build_graph(wgml_llama2 *m, uint32_t pos) {
     }
     const DynState init{0, 0, 0, 0};
     hipError_t ew = hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream);
-    int rcw = ew == hipSuccess ? enqueue_step(m, true, 0, 0, plan) : WGML_E_HIP;
-    if (rcw == WGML_OK)
-        rcw = launch_argmax_next(ctx, m->logits, c.vocab_size, m->dyn, m->d_prompt, m->d_tokens);
+    int rcw = ew == hipSuccess ? loop_first_embed(m) : WGML_E_HIP;
+    if (rcw == WGML_OK) rcw = enqueue_loop_step(m, plan);
     for (uint32_t l = 0; l < c.n_layers; ++l) {
         (void)hipMemcpyAsync(m->layers[l].key_cache, (char *)saved + col * (2 * l), col,
                              hipMemcpyDeviceToDevice, ctx->stream);
@@ -433,6 +448,8 @@ int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint3
     const DynState init{start_pos, first_token, 0, n_prompt};
     WGML_CHECK_HIP(hipMemcpyAsync(m->dyn, &init, sizeof(init), hipMemcpyHostToDevice, ctx->stream));
     WGML_CHECK_HIP(hipStreamSynchronize(ctx->stream));  // `init` is a stack object
+    uint64_t launches0 = ctx->launches;
+    WGML_TRY(loop_first_embed(m));
     for (uint32_t i = 0; i < n_steps; ++i) {
         int b = 0;
         const uint32_t plan = plan_bucket(start_pos + i, m->cfg.seq_len, &b);
@@ -449,10 +466,8 @@ int run_recorded(wgml_llama2 *m, uint32_t first_token, uint32_t start_pos, uint3
             m->launches_last = m->graph_launches[b];
         } else {
             // the same launches, enqueued one by one (no host synchronisation either)
-            const uint64_t launches0 = ctx->launches;
-            WGML_TRY(enqueue_step(m, true, 0, 0, plan));
-            WGML_TRY(launch_argmax_next(ctx, m->logits, m->cfg.vocab_size, m->dyn, m->d_prompt,
-                                        m->d_tokens));
+            launches0 = ctx->launches;
+            WGML_TRY(enqueue_loop_step(m, plan));
             m->launches_last = ctx->launches - launches0;
         }
     }

@@ -233,6 +233,42 @@ __global__ __launch_bounds__(1024) void argmax_next_kernel(const float *__restri
     }
 }
 
+// argmax_next_kernel followed, in the same launch, by what embed_kernel does for the token and
+// position just chosen (the same expressions, so the same bits): the next step of the loop needs
+// no launch of its own for the embedding.
+__global__ __launch_bounds__(1024) void argmax_next_embed_kernel(const float *__restrict__ v, uint32_t n,
+                                                                 DynState *dyn,
+                                                                 const uint32_t *__restrict__ prompt,
+                                                                 uint32_t *__restrict__ tokens_out,
+                                                                 const NextEmbed e) {
+    __shared__ uint32_t next[2];
+    const uint32_t idx = block_argmax(v, n);
+    if (threadIdx.x == 0) {
+        const uint32_t pos = dyn->pos, cnt = dyn->count;
+        tokens_out[cnt] = idx;
+        const uint32_t tok = (pos + 1 < dyn->n_prompt) ? prompt[pos + 1] : idx;
+        dyn->token = tok;
+        dyn->pos = pos + 1;
+        dyn->count = cnt + 1;
+        next[0] = tok;
+        next[1] = pos + 1;
+    }
+    __syncthreads();
+    const uint32_t tok = next[0], pos = next[1];
+    for (uint32_t i = threadIdx.x; i < e.dim; i += blockDim.x) {
+        float x = e.table[(size_t)tok * e.dim + i];
+        if (e.pos_table && pos < e.n_pos) x += e.pos_table[(size_t)pos * e.dim + i];
+        e.x[i] = x;
+    }
+    if (e.rope_cs && threadIdx.x < e.head_size / 2) {
+        const float head_dim = (float)(2 * threadIdx.x);
+        const float theta = powf(e.rope_base, -head_dim / (float)e.head_size);
+        float sn, cs;
+        sincosf((float)pos * theta, &sn, &cs);
+        reinterpret_cast<float2 *>(e.rope_cs)[threadIdx.x] = make_float2(cs, sn);
+    }
+}
+
 // state.x.copy_from_view(token_embd.column(token)) (wgml-chat/src/chat_llama2.rs:185-187)
 // Also fills the step's RoPE table (if given): (cos, sin) of pos * theta_i for the
 // head_size/2 pairs of a head, with the angle formed exactly as ops/rope.wgsl:38-41.
@@ -338,8 +374,15 @@ int launch_embed(wgml_ctx *ctx, float *x, const float *table, uint32_t dim, DynP
 }
 
 int launch_argmax_next(wgml_ctx *ctx, const float *v, uint32_t n, DynState *dyn,
-                       const uint32_t *prompt, uint32_t *tokens_out) {
-    argmax_next_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(v, n, dyn, prompt, tokens_out);
+                       const uint32_t *prompt, uint32_t *tokens_out, const NextEmbed *embed) {
+    if (embed) {
+        if (embed->rope_cs && embed->head_size / 2 > 1024)
+            return set_error(WGML_E_UNSUPPORTED, "argmax_next: head_size %u too large", embed->head_size);
+        argmax_next_embed_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(v, n, dyn, prompt, tokens_out,
+                                                                         *embed);
+    } else {
+        argmax_next_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(v, n, dyn, prompt, tokens_out);
+    }
     WGML_CHECK_LAUNCH();
     ctx->launches++;
     return WGML_OK;
