@@ -17,9 +17,9 @@
 //
 // Fast kernel (no score output wanted, head size a multiple of 4, 16-byte aligned
 // operands): 16 lanes share a position (float4 loads, 16-lane DPP reductions), a
-// wave works on 4 positions at a time and keeps 16 positions in flight; the chunk
+// wave works on 4 positions at a time (and has those four in flight, no more); the chunk
 // per wave is derived from the current position on the device, so every wave of
-// a recorded launch has work at any position.  Up to 128 positions one 16-wave
+// a recorded launch has work at any position.  Up to 256 positions one 16-wave
 // workgroup per head group does everything and writes the result (one launch, no
 // workspace); beyond that 4-wave workgroups write partials for the merge kernel.
 // (Merging in the workgroup that arrives last was tried twice and dropped.  With
@@ -30,6 +30,8 @@
 // memory (store acknowledgement, counter, loads) cost what the launch costs: +0.6 % on 32
 // heads of 128 beyond position 256, -1.2 % on 12 heads of 64, -16 % at 8192 positions of
 // 8 KV heads, where one workgroup merges the four heads of its group in turn.)
+#include <algorithm>
+
 #include "common.h"
 #include "device_utils.h"
 
@@ -302,10 +304,15 @@ __device__ __forceinline__ float4 axpby4(const float4 a, float sa, const float4 
 }
 __device__ __forceinline__ float shfl_xor_f32(float v, int mask) { return __shfl_xor(v, mask, 64); }
 
-// NS: register sets of two quads each that take turns (NS * 2 quads of a wave in flight; four
-// sets measured slower than two at every context length: 27.2 against 26.1 us at 4096 positions
-// of 32 heads, 23.6 against 22.7 us at 8192 positions of 8 KV heads, merge included).
-template <int NV4, int KM, int NW, int NS = 2>
+// NS register sets of QS quads each take turns (NS * QS quads of a wave in flight).  Less is
+// more here: one set of one quad -- a wave requests the K and V rows of four positions, waits,
+// consumes them and requests the next four; the other waves of the CU cover the wait -- is the
+// fastest at every length measured (per layer, attention + merge, us; sets x quads 1x1 / 2x1 /
+// 1x2 / 2x2 / 1x4: 32 heads of 128 at position 150: 4.38 / 4.62 / 4.54 / 4.84 / 5.94, at 1000:
+// 9.41 / 9.61 / 9.57 / 10.26 / 10.41; 8 KV heads x 4 at 8192: 20.2 / 20.6 / 21.3 / 21.8 / 21.5;
+// four sets of two were slower still), as with the GEMV's weight tiles: requests beyond what
+// keeps the memory system busy only queue.
+template <int NV4, int KM, int NW, int NS = 1, int QS = 1>
 __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
     constexpr int HSP = NV4 * 64;  // dimension capacity: 16 lanes x 4 x NV4
     __shared__ float sm_m[NW][KM], sm_l[NW][KM];
@@ -334,25 +341,25 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
         cv[v] = min(sub + 16 * v, hs / 4 - 1);
     }
 
-    // This wave's quads are gid, gid + total, ...  NS register sets of two quads
-    // each take turns: while one is consumed the others' loads are in flight.  The
-    // quads of the first set are requested before the position is known (`spec_rows` rows
+    // This wave's quads are gid, gid + total, ...  NS register sets of QS quads
+    // each take turns: while one is consumed the others' loads (if NS > 1) are in flight.
+    // The quads of the first set are requested before the position is known (`spec_rows` rows
     // of the caches may be read; rows beyond the position are masked out below),
     // the others once it is, and only those that hold a position <= pos.
-    float4 kS[NS][2][NV4], vS[NS][2][NV4];
+    float4 kS[NS][QS][NV4], vS[NS][QS][NV4];
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < QS; ++u) {
 #pragma unroll
             for (int v = 0; v < NV4; ++v) kS[s][u][v] = vS[s][u][v] = zero4;
         }
     }
-    // requests quads number i0 + u (u_begin <= u < 2) of this wave into a set
-    auto request = [&](float4(&kk)[2][NV4], float4(&vv)[2][NV4], uint32_t i0, uint32_t last,
+    // requests quads number i0 + u (u_begin <= u < QS) of this wave into a set
+    auto request = [&](float4(&kk)[QS][NV4], float4(&vv)[QS][NV4], uint32_t i0, uint32_t last,
                        int u_begin, uint32_t nq_limit) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < QS; ++u) {
             const uint32_t quad = (i0 + u) * total + gid;
             if (u >= u_begin && quad < nq_limit) {  // uniform over the wave
                 const uint32_t tt = min(quad * 4 + quarter, last);
@@ -373,10 +380,13 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
     int n_spec[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-        const uint32_t q0 = (uint32_t)(2 * s) * total + gid;
-        n_spec[s] = ((uint32_t)s < a.spec_sets && q0 < spec_quads) ? (q0 + total < spec_quads ? 2 : 1) : 0;
-        if (n_spec[s])
-            request(kS[s], vS[s], 2 * s, a.spec_rows - 1, 0, n_spec[s] == 2 ? spec_quads : q0 + 1);
+        // the set's leading quads that lie below spec_rows (a wave's quads ascend)
+        n_spec[s] = 0;
+        if ((uint32_t)s < a.spec_sets) {
+#pragma unroll
+            for (int u = 0; u < QS; ++u) n_spec[s] += ((uint32_t)(QS * s + u) * total + gid < spec_quads) ? 1 : 0;
+        }
+        if (n_spec[s]) request(kS[s], vS[s], QS * s, a.spec_rows - 1, 0, spec_quads);
     }
 
     float4 q[KM][NV4], acc[KM][NV4];
@@ -407,10 +417,10 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
         return;
     }
     const uint32_t nq = pos / 4 + 1;
-    // online-softmax update with the two quads of a set
-    auto consume = [&](const float4(&kk)[2][NV4], const float4(&vv)[2][NV4], uint32_t i0) {
+    // online-softmax update with the quads of a set
+    auto consume = [&](const float4(&kk)[QS][NV4], const float4(&vv)[QS][NV4], uint32_t i0) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < QS; ++u) {
             // uniform within each 16-lane row, so the row reductions below see whole rows
             if (((i0 + u) * total + gid) * 4 + quarter <= pos) {
 #pragma unroll
@@ -431,12 +441,12 @@ __global__ __launch_bounds__(NW * 64) void attn_fast_kernel(const AttnArgs a) {
         }
     };
 #pragma unroll
-    for (int s = 0; s < NS; ++s) request(kS[s], vS[s], 2 * s, pos, n_spec[s], nq);
-    for (uint32_t i0 = 0; i0 * total + gid < nq; i0 += 2 * NS) {
+    for (int s = 0; s < NS; ++s) request(kS[s], vS[s], QS * s, pos, n_spec[s], nq);
+    for (uint32_t i0 = 0; i0 * total + gid < nq; i0 += QS * NS) {
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
-            consume(kS[s], vS[s], i0 + 2 * s);
-            request(kS[s], vS[s], i0 + 2 * s + 2 * NS, pos, 0, nq);
+            consume(kS[s], vS[s], i0 + QS * s);
+            request(kS[s], vS[s], i0 + QS * s + QS * NS, pos, 0, nq);
         }
     }
 
@@ -643,9 +653,14 @@ static int make_fast_plan(wgml_ctx *ctx, const wgml_attn_params &p, uint32_t pla
     const uint32_t cu = ctx->n_cu > 0 ? (uint32_t)ctx->n_cu : 256u;
     // about two workgroups per CU, each with at least 64 positions at full length (four
     // quads per wave; measured on 32 x 128 and 12 x 64 heads, shorter shares only add
-    // partial results for the merge to read)
+    // partial results for the merge to read) -- or 32 positions while that keeps the partial
+    // results within the 16 that the merge takes in one round of loads (512 planned positions:
+    // 6.9 against 7.3 us per layer with 16 instead of 8 workgroups per head of 128, 4.95 against
+    // 5.17 with heads of 64; beyond 16 the merge costs 2 us more)
     uint32_t n_wg_y = (2 * cu + pl.groups - 1) / pl.groups;
     uint32_t max_y = (plan_positions + 16 * WAVES - 1) / (16 * WAVES);
+    const uint32_t short_y = std::min<uint32_t>(16u, (plan_positions + 8 * WAVES - 1) / (8 * WAVES));
+    if (max_y < short_y && !folded) max_y = short_y;
     // short contexts of a folded plan: up to one workgroup per CU
     if (folded && plan_positions <= kWidePositions) {
         max_y = (cu + pl.groups - 1) / pl.groups;
