@@ -266,9 +266,12 @@ __global__ __launch_bounds__(256) void attn_merge_fast_kernel(const AttnArgs a, 
     const float ly = lane < ny ? ml[lane * 2 + 1] : 0.f;
     float v[B];
     const bool has_d = tid < a.head_size;  // head sizes up to 256: one dimension per thread
+    // Loads without conditions (a thread beyond the head reads the head's last dimension, a
+    // partial beyond ny the last one: their weights are zero or their results not stored), so
+    // that they leave back to back instead of one branch each.
+    const uint32_t td = has_d ? tid : a.head_size - 1;
 #pragma unroll
-    for (int k = 0; k < B; ++k)
-        v[k] = (has_d && (uint32_t)k < ny) ? base[(size_t)k * stride + tid] : 0.f;
+    for (int k = 0; k < B; ++k) v[k] = base[(size_t)min((uint32_t)k, ny - 1) * stride + td];
     const float M = wave_max(my);
     const float wgt = my == -INFINITY ? 0.f : __expf(my - M);
     const float L = wave_sum(ly * wgt);
@@ -280,8 +283,7 @@ __global__ __launch_bounds__(256) void attn_merge_fast_kernel(const AttnArgs a, 
     }
     for (uint32_t y0 = B; y0 < ny; y0 += B) {
 #pragma unroll
-        for (int k = 0; k < B; ++k)
-            v[k] = (has_d && y0 + k < ny) ? base[(size_t)(y0 + k) * stride + tid] : 0.f;
+        for (int k = 0; k < B; ++k) v[k] = base[(size_t)min(y0 + k, ny - 1) * stride + td];
 #pragma unroll
         for (int k = 0; k < B; ++k) {
             const float wk = __shfl(wgt, (int)(y0 + k), 64);
