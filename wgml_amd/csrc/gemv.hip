@@ -1655,8 +1655,11 @@ int launch_fmt_i8(wgml_ctx *ctx, const GemvParams &p) {
     int R = ctx->tuning[WGML_TUNE_GEMV_ROWS_PER_WAVE], waves = ctx->tuning[WGML_TUNE_GEMV_WAVES_PER_WG],
         depth = ctx->tuning[WGML_TUNE_GEMV_DEPTH];
     const bool q8 = F::TILE == 32;
-    if (!R) R = 1;
-    if (!waves) waves = (q8 && p.ncols <= 1024) ? 8 : 16;  // short rows: less staging per row
+    // (GPT-2 124M's shapes, Q8_0 rows of 768 columns: 16-wave workgroups are as fast as 8-wave
+    // ones or faster -- 3072x768 3.3 against 3.6 us, 50257x768 11.1 against 13.4 -- and the
+    // tall output projection gains again from two rows per wave, 10.7 us)
+    if (!R) R = (q8 && SWEEP && p.ncols <= 1024 && p.nrows >= 16384) ? 2 : 1;
+    if (!waves) waves = 16;
     if (waves == 12) waves = 16;  // 12-wave workgroups exist for the fused launches only
     // Q8_0 rows of five and more steps (over 8192 columns): four tiles in flight per wave
     // (4096x11008: 11.0 us against 13.4); everywhere else one tile is as fast or faster
